@@ -1,0 +1,198 @@
+/*
+ * cahel_hip.h -- C-ABI of the MI355X (gfx950) CKKS kernel library, libcahel_hip.so.
+ *
+ * This is the device boundary of the engine: the C++ host layer (context, encoder, keys, evaluator,
+ * pyCAHEL binding) calls only these functions and never includes a HIP header.  Each entry point
+ * replaces one device routine of the reference (cited per function, paths relative to cahel-main/).
+ *
+ * Conventions
+ *   - every function returns 0 on success, a positive hipError_t value when the HIP runtime failed, or a
+ *     negative HE_E_* code for invalid arguments; nothing throws across this boundary
+ *   - all polynomial pointers are DEVICE pointers to uint64_t residues in [0, q), layout
+ *     [poly][limb][coeff] with the coefficient index fastest (include/ciphertext.h:303-333); outputs
+ *     are always canonical residues
+ *   - "L" is the number of data limbs of the level, K = size_p special limbs; limb t of a Ql u P buffer
+ *     uses modulus table t for t < L and size_q + (t - L) otherwise (src/ntt/ntt_modup.cu:404-406)
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous on it
+ *   - the caller owns every buffer, including the workspaces whose sizes the *_workspace_words functions
+ *     return; the library allocates device memory only in he_context_create / he_context_set_level /
+ *     he_malloc
+ */
+#ifndef CAHEL_HIP_H
+#define CAHEL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HE_OK 0
+#define HE_E_INVALID_ARGUMENT (-1)
+#define HE_E_UNSUPPORTED (-2)
+#define HE_E_LEVEL_NOT_SET (-3)
+#define HE_E_OUT_OF_MEMORY (-4)
+
+typedef struct he_context he_context;
+typedef void *he_stream;
+
+/* Human-readable text for a status code returned by any function below. */
+const char *he_error_string(int status);
+
+/* ---- device memory and streams: what cahel::util::Pointer<T> / MemoryPoolST give the reference's host
+ *      code (include/mempool.cuh:183-280) and its cudaMemcpy/cudaMemset calls ---- */
+int he_device_count(int *count);
+int he_malloc(void **dev_ptr, size_t bytes);
+int he_free(void *dev_ptr);
+int he_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, he_stream stream);
+int he_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, he_stream stream);
+int he_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes, he_stream stream);
+int he_memset_zero(void *dst_dev, size_t bytes, he_stream stream);
+int he_stream_create(he_stream *stream);
+int he_stream_destroy(he_stream stream);
+int he_stream_synchronize(he_stream stream);
+
+/* ---- parameter tables ---- */
+
+/* Host-side description of one parameter set; replaces the uploads of CAHELGPUContext's constructor
+ * (include/gpucontext.h:53-136: DNTTTable, DModulus) and the level-independent part of DRNSTool::init
+ * (src/rns.cu:9-67).  All arrays are HOST pointers, copied during he_context_create. */
+typedef struct {
+    uint32_t log_n;               /* N = 2^log_n, 9 <= log_n <= 16 */
+    uint32_t size_q;              /* Q limbs at the key level */
+    uint32_t size_p;              /* special limbs (alpha); may be 0 when no key switching is used */
+    uint32_t reserved;
+    const uint64_t *moduli;       /* [size_q + size_p] q_0..q_{Q-1}, p_0..p_{K-1}, each < 2^61 */
+    const uint64_t *barrett;      /* [size_qp][2] floor(2^128 / m): low word, high word */
+    const uint64_t *psi;          /* [size_qp][N][2] (psi^bitrev(i), Shoup quotient); src/util/ntt.cu:46-56 */
+    const uint64_t *ipsi_div2;    /* [size_qp][N][2] (psi^-bitrev(i) / 2, Shoup quotient); src/util/ntt.cu:58-71 */
+    const uint64_t *p_mod_q;      /* [size_q][2] (P mod q_i, Shoup quotient)            src/util/rns.cu:497-508 */
+    const uint64_t *pinv_mod_q;   /* [size_q][2] (P^-1 mod q_i, Shoup quotient) */
+    const uint64_t *phat_inv_mod_p; /* [size_p][2] ((P/p_k)^-1 mod p_k, Shoup quotient)  src/util/rns.cu:218-270 */
+    const uint64_t *phat_mod_q;   /* [size_q][size_p] (P/p_k) mod q_j                    src/util/rns.cu:374-392 */
+} he_context_desc;
+
+/* Tables of the data level with L limbs: the hybrid section of RNSTool (src/util/rns.cu:514-551) and
+ * inv_q_last_mod_q (:483-488). */
+typedef struct {
+    uint32_t L;
+    uint32_t beta;                   /* ceil(L / size_p) digits */
+    const uint64_t *part_hat_inv;    /* [L][2] ((Q_d/q_i)^-1 mod q_i, Shoup quotient), d = digit of limb i */
+    const uint64_t *digit_mats;      /* digit d: row-major [L + K - size_d][size_d], (Q_d/q_i) mod m_t over the
+                                        limbs t of Ql u P outside the digit, in order */
+    const uint32_t *digit_mat_off;   /* [beta] word offset of digit d's matrix in digit_mats */
+    const uint64_t *qlast_inv;       /* [L-1][2] (q_{L-1}^-1 mod q_j, Shoup quotient) */
+} he_level_desc;
+
+int he_context_create(const he_context_desc *desc, he_context **out);
+int he_context_set_level(he_context *ctx, const he_level_desc *level);
+int he_context_destroy(he_context *ctx);
+
+/* ---- NTT ---- */
+
+/* Batched forward negacyclic NTT in place.  data: [n_polys][poly_stride_limbs][N]; the first `limbs` limbs
+ * of every polynomial are transformed; limb i uses table first_table + i for i < split and
+ * tail_table + (i - split) for i >= split (pass split = limbs for a plain range).
+ * Replaces nwt_2d_radix8_forward_inplace (src/ntt/fntt_2d.cu:872-910) and its _include_special_mod
+ * variant (src/ntt/ntt_modup.cu:591-643). */
+int he_ntt_forward(const he_context *ctx, uint64_t *data, uint32_t n_polys, uint32_t poly_stride_limbs,
+                   uint32_t limbs, uint32_t first_table, uint32_t split, uint32_t tail_table, he_stream stream);
+
+/* Batched inverse NTT in place (includes the factor 1/N).  Replaces nwt_2d_radix8_backward_inplace
+ * (src/ntt/intt_2d.cu:693-771) and _include_special_mod (:773-815). */
+int he_ntt_inverse(const he_context *ctx, uint64_t *data, uint32_t n_polys, uint32_t poly_stride_limbs,
+                   uint32_t limbs, uint32_t first_table, uint32_t split, uint32_t tail_table, he_stream stream);
+
+/* ---- elementwise polynomial arithmetic (src/polymath.cu:16-180, 227, 349) ----
+ * a, b, c, out: [n_polys][limbs][N], limb i mod q_{first_table + i}; out may alias any input. */
+int he_add(const he_context *ctx, const uint64_t *a, const uint64_t *b, uint64_t *out, uint32_t n_polys,
+           uint32_t limbs, uint32_t first_table, he_stream stream);
+int he_sub(const he_context *ctx, const uint64_t *a, const uint64_t *b, uint64_t *out, uint32_t n_polys,
+           uint32_t limbs, uint32_t first_table, he_stream stream);
+int he_negate(const he_context *ctx, const uint64_t *a, uint64_t *out, uint32_t n_polys, uint32_t limbs,
+              uint32_t first_table, he_stream stream);
+int he_multiply(const he_context *ctx, const uint64_t *a, const uint64_t *b, uint64_t *out, uint32_t n_polys,
+                uint32_t limbs, uint32_t first_table, he_stream stream);
+/* out = a*b + c, or -(a*b + c) when negate != 0 */
+int he_multiply_add(const he_context *ctx, const uint64_t *a, const uint64_t *b, const uint64_t *c, uint64_t *out,
+                    uint32_t n_polys, uint32_t limbs, uint32_t first_table, int negate, he_stream stream);
+
+/* out = a + b * P mod q_i on limbs [first_limb, first_limb + limbs) of Q (a, b, out point at limb first_limb):
+ * the key-generation step that plants [P]_{q_i} s' on one digit of a switching key.
+ * Replaces multiply_temp_mod_and_add_rns_poly (src/polymath.cu:320-338). */
+int he_add_p_multiple(const he_context *ctx, const uint64_t *a, const uint64_t *b, uint64_t *out, uint32_t first_limb,
+                      uint32_t limbs, he_stream stream);
+
+/* (c0,c1) x (c0',c1') -> (d0,d1,d2): ct1, ct2 [2][L][N], out [3][L][N] (out may alias ct1 if it has room).
+ * Replaces tensor_prod_2x2_rns_poly (src/polymath.cu:531-566). */
+int he_tensor(const he_context *ctx, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
+              he_stream stream);
+/* Squaring variant; replaces tensor_square_2x2_rns_poly (src/polymath.cu:568-612). */
+int he_tensor_square(const he_context *ctx, const uint64_t *ct, uint64_t *out, uint32_t L, he_stream stream);
+
+/* NTT-domain Galois automorphism X -> X^galois_elt of `total_limbs` limbs (any moduli): out[l][i] =
+ * in[l][pi(i)]; in and out must not overlap.  Replaces CAHELGPUGaloisTool::apply_galois_ntt
+ * (src/galois.cu:20-30, table of include/galois.cuh:45-57, computed on the fly here). */
+int he_galois_ntt(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_t total_limbs,
+                  uint32_t galois_elt, he_stream stream);
+
+/* ---- rescale ---- */
+
+/* in [n_polys][L][N] -> out [n_polys][L-1][N], out_j = (in_j - NTT_j(INTT(in_{L-1}) mod q_j)) / q_{L-1}.
+ * workspace: n_polys * N words.  in and out must not overlap.
+ * Replaces DRNSTool::divide_and_round_q_last_ntt (src/rns.cu:544-570). */
+int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_t n_polys, uint32_t L,
+               uint64_t *workspace, he_stream stream);
+
+/* ---- hybrid key switching ---- */
+
+/* c [L][N] (NTT) -> out [beta][L+K][N] (NTT).  workspace: L * N words.
+ * Replaces DRNSTool::modup (src/rns_bconv.cu:668-792). */
+int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out, uint64_t *workspace,
+             he_stream stream);
+
+/* y [beta][L+K][N], evk: HOST array of beta DEVICE pointers, each [2][size_q+size_p][N] -> out [2][L+K][N].
+ * galois_elt != 0 applies X -> X^galois_elt to y while loading (the hoisting form, src/evaluate.cu:2492-2497);
+ * accumulate != 0 adds onto out instead of overwriting it (:2571-2576).
+ * Replaces key_switch_inner_prod_c2_and_evk (src/eval_key_switch.cu:13-76). */
+int he_ks_inner_product(const he_context *ctx, uint32_t L, const uint64_t *y, const uint64_t *const *evk,
+                        uint64_t *out, uint32_t galois_elt, int accumulate, he_stream stream);
+
+/* cx [n_polys][L+K][N] (NTT) -> out [n_polys][L][N]: out_j = (cx_j - NTT_j(delta)) * P^-1 mod q_j; with
+ * accumulate != 0 the result is added onto out (the add_to_ct step of src/eval_key_switch.cu:193-215).
+ * cx's special limbs are overwritten.  workspace: n_polys * L * N words.
+ * Replaces DRNSTool::moddown_from_NTT (src/rns_bconv.cu:965-1053) and moddown (:871-944). */
+int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, uint32_t n_polys, int accumulate,
+               uint64_t *workspace, he_stream stream);
+
+/* Words of workspace he_keyswitch needs at level L: beta*(L+K)*N + 2*(L+K)*N + 2*L*N. */
+size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L);
+
+/* ct[0..1] += KeySwitch(c): c [L][N], ct [2][L][N], evk as in he_ks_inner_product.  galois_elt != 0 switches
+ * sigma(c) instead of c (the permutation is fused into the first pass).
+ * Replaces switch_key_inplace (src/eval_key_switch.cu:80-216). */
+int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk, uint64_t *ct,
+                 uint32_t galois_elt, uint64_t *workspace, he_stream stream);
+
+/* ---- encoder support ----
+ * coeffs: DEVICE array of N doubles holding integers (already rounded, |c| < 2^63); out [limbs][N]:
+ * out[l][i] = c_i mod q_{first_table + l} (negative values wrap to q - |c| mod q).
+ * Replaces decompose_array_uint64 (src/rns_base.cu:121-156). */
+int he_decompose_real(const he_context *ctx, const double *coeffs, uint64_t *out, uint32_t limbs,
+                      uint32_t first_table, he_stream stream);
+
+/* ---- samplers (replace sample_ternary_poly / sample_error_poly / sample_uniform_poly, src/prng.cu:143-242,
+ *      and the OpenFHE Gaussian of src/secretkey.cu:632-649) ----
+ * ChaCha20 block function keyed by key[8]; `stream_id` selects an independent stream.  out: [limbs][N],
+ * limb i mod table first_table+i (i < split) / tail_table + i - split.
+ * kind: 0 ternary {-1,0,1}; 1 centred binomial (21 - 21 bits); 2 uniform residues; 3 discrete Gaussian by
+ * the cumulative table cdt[cdt_len] (DEVICE pointer, cdt[i] = floor(2^63 P(|X| <= i))). */
+int he_sample(const he_context *ctx, int kind, const uint32_t key[8], uint64_t stream_id, uint64_t *out,
+              uint32_t limbs, uint32_t first_table, uint32_t split, uint32_t tail_table, const uint64_t *cdt,
+              uint32_t cdt_len, he_stream stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CAHEL_HIP_H */

@@ -1,0 +1,79 @@
+"""ctypes view of libcahel_hip.so (the C-ABI declared in include/cahel_hip.h).
+
+For callers that own their device buffers (torch tensors, the benchmark, the parity tests): every
+function takes raw device pointers as integers.  `check(rc)` turns a non-zero status into RuntimeError.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libcahel_hip.so")
+
+u64 = C.c_uint64
+u32 = C.c_uint32
+vp = C.c_void_p
+
+# name -> (restype, argtypes); one entry per declaration in include/cahel_hip.h
+SIGNATURES = {
+    "he_error_string": (C.c_char_p, [C.c_int]),
+    "he_device_count": (C.c_int, [C.POINTER(C.c_int)]),
+    "he_malloc": (C.c_int, [C.POINTER(vp), C.c_size_t]),
+    "he_free": (C.c_int, [vp]),
+    "he_memcpy_h2d": (C.c_int, [vp, vp, C.c_size_t, vp]),
+    "he_memcpy_d2h": (C.c_int, [vp, vp, C.c_size_t, vp]),
+    "he_memcpy_d2d": (C.c_int, [vp, vp, C.c_size_t, vp]),
+    "he_memset_zero": (C.c_int, [vp, C.c_size_t, vp]),
+    "he_stream_create": (C.c_int, [C.POINTER(vp)]),
+    "he_stream_destroy": (C.c_int, [vp]),
+    "he_stream_synchronize": (C.c_int, [vp]),
+    "he_context_create": (C.c_int, [vp, C.POINTER(vp)]),
+    "he_context_set_level": (C.c_int, [vp, vp]),
+    "he_context_destroy": (C.c_int, [vp]),
+    "he_ntt_forward": (C.c_int, [vp, vp, u32, u32, u32, u32, u32, u32, vp]),
+    "he_ntt_inverse": (C.c_int, [vp, vp, u32, u32, u32, u32, u32, u32, vp]),
+    "he_add": (C.c_int, [vp, vp, vp, vp, u32, u32, u32, vp]),
+    "he_sub": (C.c_int, [vp, vp, vp, vp, u32, u32, u32, vp]),
+    "he_negate": (C.c_int, [vp, vp, vp, u32, u32, u32, vp]),
+    "he_multiply": (C.c_int, [vp, vp, vp, vp, u32, u32, u32, vp]),
+    "he_multiply_add": (C.c_int, [vp, vp, vp, vp, vp, u32, u32, u32, C.c_int, vp]),
+    "he_add_p_multiple": (C.c_int, [vp, vp, vp, vp, u32, u32, vp]),
+    "he_tensor": (C.c_int, [vp, vp, vp, vp, u32, vp]),
+    "he_tensor_square": (C.c_int, [vp, vp, vp, u32, vp]),
+    "he_galois_ntt": (C.c_int, [vp, vp, vp, u32, u32, vp]),
+    "he_rescale": (C.c_int, [vp, vp, vp, u32, u32, vp, vp]),
+    "he_modup": (C.c_int, [vp, u32, vp, vp, vp, vp]),
+    "he_ks_inner_product": (C.c_int, [vp, u32, vp, C.POINTER(vp), vp, u32, C.c_int, vp]),
+    "he_moddown": (C.c_int, [vp, u32, vp, vp, u32, C.c_int, vp, vp]),
+    "he_keyswitch_workspace_words": (C.c_size_t, [vp, u32]),
+    "he_keyswitch": (C.c_int, [vp, u32, vp, C.POINTER(vp), vp, u32, vp, vp]),
+    "he_decompose_real": (C.c_int, [vp, vp, vp, u32, u32, vp]),
+    "he_sample": (C.c_int, [vp, C.c_int, C.POINTER(u32), u64, vp, u32, u32, u32, u32, vp, u32, vp]),
+}
+
+_lib = None
+
+
+def lib():
+    """Loads libcahel_hip.so; raises if it has not been built (there is no fallback)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libcahel_hip.so is missing: run `python -m lancelot_amd.build`")
+        _lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(_lib, name)
+            fn.restype = res
+            fn.argtypes = args
+    return _lib
+
+
+def check(rc: int, what: str = "libcahel_hip"):
+    if rc != 0:
+        raise RuntimeError("%s failed: %s" % (what, lib().he_error_string(rc).decode()))
+
+
+def evk_array(ptrs):
+    """Host array of device pointers for he_ks_inner_product / he_keyswitch."""
+    return (vp * len(ptrs))(*ptrs)

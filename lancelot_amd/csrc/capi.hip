@@ -1,0 +1,521 @@
+// C-ABI of libcahel_hip.so (declared in include/cahel_hip.h): parameter tables on the device and the
+// orchestration of the kernels in ntt.hip / rns.hip into the operations of the CKKS hot path.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "../../include/cahel_hip.h"
+#include "kernels.h"
+
+using namespace he;
+
+namespace {
+
+struct Digit {
+    uint32_t start = 0, size = 0, n_out = 0;
+    uint32_t *d_out_limb = nullptr;   // [n_out] limb of Ql u P each matrix row writes
+    uint32_t *d_out_table = nullptr;  // [n_out] modulus table of that limb
+    size_t mat_off = 0;
+};
+
+struct Level {
+    bool set = false;
+    uint32_t L = 0, beta = 0;
+    uint64_t *d_part_hat_inv = nullptr;  // [L][2]
+    uint64_t *d_mats = nullptr;
+    uint64_t *d_qlast_inv = nullptr;     // [L-1][2]
+    std::vector<Digit> digits;
+    LimbJob *d_modup_jobs = nullptr;     // NTT jobs over the converted limbs of all digits
+    uint32_t n_modup_jobs = 0;
+};
+
+}  // namespace
+
+struct he_context {
+    uint32_t log_n = 0, size_q = 0, size_p = 0, size_qp = 0;
+    int device = 0;
+    uint64_t *d_moduli = nullptr, *d_barrett = nullptr, *d_psi = nullptr, *d_ipsi = nullptr;
+    uint64_t *d_p_mod_q = nullptr, *d_pinv_mod_q = nullptr, *d_phat_inv = nullptr, *d_phat_mod_q = nullptr;
+    uint32_t *d_iota = nullptr;  // 0, 1, 2, ...: row -> limb/table map of the P -> Ql conversion
+    std::vector<Level> levels;   // indexed by L
+    std::vector<void *> owned;
+
+    Tables tables() const { return Tables{d_moduli, d_barrett, log_n}; }
+    size_t n() const { return (size_t)1 << log_n; }
+};
+
+namespace {
+
+#define HE_HIP(expr)                          \
+    do {                                      \
+        hipError_t _e = (expr);               \
+        if (_e != hipSuccess) return (int)_e; \
+    } while (0)
+
+template <typename T>
+int upload(he_context *ctx, T **dst, const T *src, size_t count) {
+    if (count == 0) {
+        *dst = nullptr;
+        return HE_OK;
+    }
+    void *p = nullptr;
+    HE_HIP(hipMalloc(&p, count * sizeof(T)));
+    ctx->owned.push_back(p);
+    HE_HIP(hipMemcpy(p, src, count * sizeof(T), hipMemcpyHostToDevice));
+    *dst = static_cast<T *>(p);
+    return HE_OK;
+}
+
+inline hipStream_t S(he_stream s) { return static_cast<hipStream_t>(s); }
+
+inline uint32_t table_of(const he_context *ctx, uint32_t L, uint32_t t) { return t < L ? t : ctx->size_q + (t - L); }
+
+const Level *level_of(const he_context *ctx, uint32_t L) {
+    if (L == 0 || L >= ctx->levels.size() || !ctx->levels[L].set) return nullptr;
+    return &ctx->levels[L];
+}
+
+NttArgs base_args(const he_context *ctx, bool forward) {
+    NttArgs a;
+    memset(&a, 0, sizeof(a));
+    a.tw = forward ? ctx->d_psi : ctx->d_ipsi;
+    a.moduli = ctx->d_moduli;
+    a.barrett = ctx->d_barrett;
+    a.log_n = ctx->log_n;
+    return a;
+}
+
+int check_map(const he_context *ctx, uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail) {
+    if (split > limbs) return HE_E_INVALID_ARGUMENT;
+    if (first + split > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
+    if (limbs > split && tail + (limbs - split) > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
+    return HE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *he_error_string(int status) {
+    switch (status) {
+        case HE_OK: return "success";
+        case HE_E_INVALID_ARGUMENT: return "invalid argument";
+        case HE_E_UNSUPPORTED: return "unsupported parameter";
+        case HE_E_LEVEL_NOT_SET: return "tables of this level were not provided (he_context_set_level)";
+        case HE_E_OUT_OF_MEMORY: return "out of host memory";
+        default: return status > 0 ? hipGetErrorString((hipError_t)status) : "unknown error";
+    }
+}
+
+int he_device_count(int *count) {
+    if (!count) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(hipGetDeviceCount(count));
+    return HE_OK;
+}
+
+int he_malloc(void **dev_ptr, size_t bytes) {
+    if (!dev_ptr) return HE_E_INVALID_ARGUMENT;
+    *dev_ptr = nullptr;
+    if (bytes == 0) return HE_OK;
+    HE_HIP(hipMalloc(dev_ptr, bytes));
+    return HE_OK;
+}
+
+int he_free(void *dev_ptr) {
+    if (dev_ptr) HE_HIP(hipFree(dev_ptr));
+    return HE_OK;
+}
+
+int he_memcpy_h2d(void *dst, const void *src, size_t bytes, he_stream s) {
+    if (bytes == 0) return HE_OK;
+    HE_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, S(s)));
+    HE_HIP(hipStreamSynchronize(S(s)));  // the host buffer may be pageable and reused by the caller
+    return HE_OK;
+}
+
+int he_memcpy_d2h(void *dst, const void *src, size_t bytes, he_stream s) {
+    if (bytes == 0) return HE_OK;
+    HE_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, S(s)));
+    HE_HIP(hipStreamSynchronize(S(s)));
+    return HE_OK;
+}
+
+int he_memcpy_d2d(void *dst, const void *src, size_t bytes, he_stream s) {
+    if (bytes == 0) return HE_OK;
+    HE_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, S(s)));
+    return HE_OK;
+}
+
+int he_memset_zero(void *dst, size_t bytes, he_stream s) {
+    if (bytes == 0) return HE_OK;
+    HE_HIP(hipMemsetAsync(dst, 0, bytes, S(s)));
+    return HE_OK;
+}
+
+int he_stream_create(he_stream *s) {
+    if (!s) return HE_E_INVALID_ARGUMENT;
+    hipStream_t st;
+    HE_HIP(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+    *s = st;
+    return HE_OK;
+}
+
+int he_stream_destroy(he_stream s) {
+    if (s) HE_HIP(hipStreamDestroy(S(s)));
+    return HE_OK;
+}
+
+int he_stream_synchronize(he_stream s) {
+    HE_HIP(hipStreamSynchronize(S(s)));
+    return HE_OK;
+}
+
+int he_context_create(const he_context_desc *d, he_context **out) {
+    if (!d || !out || !d->moduli || !d->barrett || !d->psi || !d->ipsi_div2) return HE_E_INVALID_ARGUMENT;
+    if (d->log_n < 9 || d->log_n > 16) return HE_E_UNSUPPORTED;
+    if (d->size_q == 0 || d->size_q + d->size_p > 256) return HE_E_INVALID_ARGUMENT;
+    if (d->size_p && (!d->p_mod_q || !d->pinv_mod_q || !d->phat_inv_mod_p || !d->phat_mod_q)) return HE_E_INVALID_ARGUMENT;
+    for (uint32_t i = 0; i < d->size_q + d->size_p; i++)
+        if (d->moduli[i] < 2 || (d->moduli[i] >> 61)) return HE_E_UNSUPPORTED;
+    he_context *ctx = new (std::nothrow) he_context;
+    if (!ctx) return HE_E_OUT_OF_MEMORY;
+    ctx->log_n = d->log_n;
+    ctx->size_q = d->size_q;
+    ctx->size_p = d->size_p;
+    ctx->size_qp = d->size_q + d->size_p;
+    ctx->levels.resize(ctx->size_q + 1);
+    const size_t n = ctx->n(), qp = ctx->size_qp;
+    int rc = hipGetDevice(&ctx->device);
+    if (!rc) rc = upload(ctx, &ctx->d_moduli, d->moduli, qp);
+    if (!rc) rc = upload(ctx, &ctx->d_barrett, d->barrett, 2 * qp);
+    if (!rc) rc = upload(ctx, &ctx->d_psi, d->psi, 2 * qp * n);
+    if (!rc) rc = upload(ctx, &ctx->d_ipsi, d->ipsi_div2, 2 * qp * n);
+    if (!rc && d->size_p) {
+        rc = upload(ctx, &ctx->d_p_mod_q, d->p_mod_q, 2 * (size_t)d->size_q);
+        if (!rc) rc = upload(ctx, &ctx->d_pinv_mod_q, d->pinv_mod_q, 2 * (size_t)d->size_q);
+        if (!rc) rc = upload(ctx, &ctx->d_phat_inv, d->phat_inv_mod_p, 2 * (size_t)d->size_p);
+        if (!rc) rc = upload(ctx, &ctx->d_phat_mod_q, d->phat_mod_q, (size_t)d->size_q * d->size_p);
+    }
+    if (!rc) {
+        std::vector<uint32_t> iota(qp);
+        for (uint32_t i = 0; i < qp; i++) iota[i] = i;
+        rc = upload(ctx, &ctx->d_iota, iota.data(), qp);
+    }
+    if (rc) {
+        he_context_destroy(ctx);
+        return rc;
+    }
+    *out = ctx;
+    return HE_OK;
+}
+
+int he_context_set_level(he_context *ctx, const he_level_desc *d) {
+    if (!ctx || !d || d->L == 0 || d->L > ctx->size_q) return HE_E_INVALID_ARGUMENT;
+    Level &lv = ctx->levels[d->L];
+    if (lv.set) return HE_OK;
+    const uint32_t L = d->L, K = ctx->size_p;
+    lv.L = L;
+    int rc = HE_OK;
+    if (L > 1) {
+        if (!d->qlast_inv) return HE_E_INVALID_ARGUMENT;
+        rc = upload(ctx, &lv.d_qlast_inv, d->qlast_inv, 2 * (size_t)(L - 1));
+        if (rc) return rc;
+    }
+    if (K) {
+        const uint32_t beta = (L + K - 1) / K;
+        if (d->beta != beta || beta > (uint32_t)kMaxDigits || !d->part_hat_inv || !d->digit_mats || !d->digit_mat_off)
+            return HE_E_INVALID_ARGUMENT;
+        lv.beta = beta;
+        rc = upload(ctx, &lv.d_part_hat_inv, d->part_hat_inv, 2 * (size_t)L);
+        if (rc) return rc;
+        size_t mat_words = 0;
+        std::vector<LimbJob> jobs;
+        lv.digits.resize(beta);
+        for (uint32_t dg = 0; dg < beta; dg++) {
+            Digit &g = lv.digits[dg];
+            g.start = dg * K;
+            g.size = (g.start + K <= L) ? K : L - g.start;
+            g.n_out = L + K - g.size;
+            g.mat_off = d->digit_mat_off[dg];
+            mat_words = g.mat_off + (size_t)g.n_out * g.size;
+            std::vector<uint32_t> limb(g.n_out), table(g.n_out);
+            for (uint32_t r = 0; r < g.n_out; r++) {
+                limb[r] = r < g.start ? r : r + g.size;
+                table[r] = table_of(ctx, L, limb[r]);
+                jobs.push_back(LimbJob{dg * (L + K) + limb[r], table[r]});
+            }
+            rc = upload(ctx, &g.d_out_limb, limb.data(), g.n_out);
+            if (!rc) rc = upload(ctx, &g.d_out_table, table.data(), g.n_out);
+            if (rc) return rc;
+        }
+        rc = upload(ctx, &lv.d_mats, d->digit_mats, mat_words);
+        if (rc) return rc;
+        lv.n_modup_jobs = (uint32_t)jobs.size();
+        rc = upload(ctx, &lv.d_modup_jobs, jobs.data(), jobs.size());
+        if (rc) return rc;
+    }
+    lv.set = true;
+    return HE_OK;
+}
+
+int he_context_destroy(he_context *ctx) {
+    if (!ctx) return HE_OK;
+    for (void *p : ctx->owned) (void)hipFree(p);
+    delete ctx;
+    return HE_OK;
+}
+
+int he_ntt_forward(const he_context *ctx, uint64_t *data, uint32_t n_polys, uint32_t poly_stride, uint32_t limbs,
+                   uint32_t first, uint32_t split, uint32_t tail, he_stream s) {
+    if (!ctx || !data || limbs > poly_stride) return HE_E_INVALID_ARGUMENT;
+    if (int rc = check_map(ctx, limbs, first, split, tail)) return rc;
+    NttArgs a = base_args(ctx, true);
+    a.in = data;
+    a.out = data;
+    a.in_poly_stride = a.out_poly_stride = poly_stride;
+    a.map = LimbMap{limbs, first, split, tail};
+    HE_HIP(launch_ntt_forward(a, n_polys, S(s)));
+    return HE_OK;
+}
+
+int he_ntt_inverse(const he_context *ctx, uint64_t *data, uint32_t n_polys, uint32_t poly_stride, uint32_t limbs,
+                   uint32_t first, uint32_t split, uint32_t tail, he_stream s) {
+    if (!ctx || !data || limbs > poly_stride) return HE_E_INVALID_ARGUMENT;
+    if (int rc = check_map(ctx, limbs, first, split, tail)) return rc;
+    NttArgs a = base_args(ctx, false);
+    a.in = data;
+    a.out = data;
+    a.in_poly_stride = a.out_poly_stride = poly_stride;
+    a.map = LimbMap{limbs, first, split, tail};
+    HE_HIP(launch_ntt_inverse(a, n_polys, S(s)));
+    return HE_OK;
+}
+
+static int elementwise(const he_context *ctx, int op, const uint64_t *a, const uint64_t *b, const uint64_t *c,
+                       uint64_t *out, uint32_t n_polys, uint32_t limbs, uint32_t first, he_stream s) {
+    if (!ctx || !a || !out || (op != EW_NEG && !b)) return HE_E_INVALID_ARGUMENT;
+    if (first + limbs > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(launch_elementwise(ctx->tables(), op, a, b, c, out, n_polys, plain_map(limbs, first), S(s)));
+    return HE_OK;
+}
+
+int he_add(const he_context *ctx, const uint64_t *a, const uint64_t *b, uint64_t *out, uint32_t n_polys,
+           uint32_t limbs, uint32_t first, he_stream s) {
+    return elementwise(ctx, EW_ADD, a, b, nullptr, out, n_polys, limbs, first, s);
+}
+
+int he_sub(const he_context *ctx, const uint64_t *a, const uint64_t *b, uint64_t *out, uint32_t n_polys,
+           uint32_t limbs, uint32_t first, he_stream s) {
+    return elementwise(ctx, EW_SUB, a, b, nullptr, out, n_polys, limbs, first, s);
+}
+
+int he_negate(const he_context *ctx, const uint64_t *a, uint64_t *out, uint32_t n_polys, uint32_t limbs,
+              uint32_t first, he_stream s) {
+    return elementwise(ctx, EW_NEG, a, nullptr, nullptr, out, n_polys, limbs, first, s);
+}
+
+int he_multiply(const he_context *ctx, const uint64_t *a, const uint64_t *b, uint64_t *out, uint32_t n_polys,
+                uint32_t limbs, uint32_t first, he_stream s) {
+    return elementwise(ctx, EW_MUL, a, b, nullptr, out, n_polys, limbs, first, s);
+}
+
+int he_multiply_add(const he_context *ctx, const uint64_t *a, const uint64_t *b, const uint64_t *c, uint64_t *out,
+                    uint32_t n_polys, uint32_t limbs, uint32_t first, int negate, he_stream s) {
+    if (!c) return HE_E_INVALID_ARGUMENT;
+    return elementwise(ctx, negate ? EW_MUL_ADD_NEG : EW_MUL_ADD, a, b, c, out, n_polys, limbs, first, s);
+}
+
+int he_add_p_multiple(const he_context *ctx, const uint64_t *a, const uint64_t *b, uint64_t *out, uint32_t first_limb,
+                      uint32_t limbs, he_stream s) {
+    if (!ctx || !a || !b || !out || ctx->size_p == 0 || first_limb + limbs > ctx->size_q) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(launch_scalar_mul_add(ctx->tables(), a, b, out, ctx->d_p_mod_q, first_limb, limbs, S(s)));
+    return HE_OK;
+}
+
+int he_tensor(const he_context *ctx, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
+              he_stream s) {
+    if (!ctx || !ct1 || !ct2 || !out || L == 0 || L > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(launch_tensor(ctx->tables(), ct1, ct2, out, L, false, S(s)));
+    return HE_OK;
+}
+
+int he_tensor_square(const he_context *ctx, const uint64_t *ct, uint64_t *out, uint32_t L, he_stream s) {
+    if (!ctx || !ct || !out || L == 0 || L > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(launch_tensor(ctx->tables(), ct, ct, out, L, true, S(s)));
+    return HE_OK;
+}
+
+int he_galois_ntt(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_t total_limbs, uint32_t elt,
+                  he_stream s) {
+    if (!ctx || !in || !out || in == out || !(elt & 1) || elt >= (2u << ctx->log_n)) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(launch_galois(ctx->tables(), in, out, total_limbs, elt, S(s)));
+    return HE_OK;
+}
+
+int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_t n_polys, uint32_t L,
+               uint64_t *ws, he_stream s) {
+    if (!ctx || !in || !out || !ws || L < 2 || L > ctx->size_q) return HE_E_INVALID_ARGUMENT;
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    const size_t n = ctx->n();
+    // last limb -> coefficient form, one limb per poly in the workspace
+    NttArgs inv = base_args(ctx, false);
+    inv.in = in + (size_t)(L - 1) * n;
+    inv.in_poly_stride = L;
+    inv.out = ws;
+    inv.out_poly_stride = 1;
+    inv.map = plain_map(1, L - 1);
+    HE_HIP(launch_ntt_inverse(inv, n_polys, S(s)));
+    // every remaining limb: NTT_j(ws mod q_j), then (in_j - that) / q_last
+    NttArgs fwd = base_args(ctx, true);
+    fwd.pro_mode = NTT_PRO_BROADCAST_REDUCE;
+    fwd.pro_src = ws;
+    fwd.pro_poly_stride = 1;
+    fwd.out = out;
+    fwd.out_poly_stride = L - 1;
+    fwd.map = plain_map(L - 1, 0);
+    fwd.epi_mode = NTT_EPI_SUB_MUL;
+    fwd.epi_a = in;
+    fwd.epi_a_poly_stride = L;
+    fwd.w = lv->d_qlast_inv;
+    fwd.epi_dst = out;
+    fwd.epi_dst_poly_stride = L - 1;
+    HE_HIP(launch_ntt_forward(fwd, n_polys, S(s)));
+    return HE_OK;
+}
+
+int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out, uint64_t *ws, he_stream s) {
+    if (!ctx || !c || !out || !ws || ctx->size_p == 0) return HE_E_INVALID_ARGUMENT;
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    const size_t n = ctx->n();
+    const uint32_t LK = L + ctx->size_p;
+    // coefficient form scaled by (Q_d / q_i)^-1, out of place into the workspace
+    NttArgs inv = base_args(ctx, false);
+    inv.in = c;
+    inv.out = ws;
+    inv.in_poly_stride = inv.out_poly_stride = L;
+    inv.map = plain_map(L, 0);
+    inv.epi_mode = NTT_EPI_MUL;
+    inv.w = lv->d_part_hat_inv;
+    HE_HIP(launch_ntt_inverse(inv, 1, S(s)));
+    for (uint32_t d = 0; d < lv->beta; d++) {
+        const Digit &g = lv->digits[d];
+        uint64_t *od = out + (size_t)d * LK * n;
+        // the digit's own limbs keep their NTT form
+        HE_HIP(hipMemcpyAsync(od + (size_t)g.start * n, c + (size_t)g.start * n, (size_t)g.size * n * sizeof(uint64_t),
+                              hipMemcpyDeviceToDevice, S(s)));
+        BconvArgs b{ws + (size_t)g.start * n, od, lv->d_mats + g.mat_off, g.d_out_limb, g.d_out_table, g.size, g.n_out};
+        HE_HIP(launch_bconv(ctx->tables(), b, S(s)));
+    }
+    NttArgs fwd = base_args(ctx, true);
+    fwd.in = out;
+    fwd.out = out;
+    fwd.jobs = lv->d_modup_jobs;
+    fwd.n_jobs = lv->n_modup_jobs;
+    HE_HIP(launch_ntt_forward(fwd, 1, S(s)));
+    return HE_OK;
+}
+
+int he_ks_inner_product(const he_context *ctx, uint32_t L, const uint64_t *y, const uint64_t *const *evk,
+                        uint64_t *out, uint32_t galois_elt, int accumulate, he_stream s) {
+    if (!ctx || !y || !evk || !out || ctx->size_p == 0 || L == 0 || L > ctx->size_q) return HE_E_INVALID_ARGUMENT;
+    if (galois_elt && (!(galois_elt & 1) || galois_elt >= (2u << ctx->log_n))) return HE_E_INVALID_ARGUMENT;
+    const uint32_t beta = (L + ctx->size_p - 1) / ctx->size_p;
+    if (beta > (uint32_t)kMaxDigits) return HE_E_UNSUPPORTED;
+    EvkPtrs ptrs;
+    memset(&ptrs, 0, sizeof(ptrs));
+    for (uint32_t d = 0; d < beta; d++) {
+        if (!evk[d]) return HE_E_INVALID_ARGUMENT;
+        ptrs.p[d] = evk[d];
+    }
+    HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, out, L, ctx->size_p, ctx->size_q, beta, galois_elt,
+                                accumulate != 0, S(s)));
+    return HE_OK;
+}
+
+int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, uint32_t n_polys, int accumulate,
+               uint64_t *ws, he_stream s) {
+    if (!ctx || !cx || !out || !ws || ctx->size_p == 0 || L == 0 || L > ctx->size_q) return HE_E_INVALID_ARGUMENT;
+    const size_t n = ctx->n();
+    const uint32_t K = ctx->size_p, LK = L + K;
+    // special limbs -> coefficient form, scaled by (P / p_k)^-1, in place
+    NttArgs inv = base_args(ctx, false);
+    inv.in = cx + (size_t)L * n;
+    inv.out = cx + (size_t)L * n;
+    inv.in_poly_stride = inv.out_poly_stride = LK;
+    inv.map = plain_map(K, ctx->size_q);
+    inv.epi_mode = NTT_EPI_MUL;
+    inv.w = ctx->d_phat_inv;
+    HE_HIP(launch_ntt_inverse(inv, n_polys, S(s)));
+    for (uint32_t p = 0; p < n_polys; p++) {
+        BconvArgs b{cx + ((size_t)p * LK + L) * n, ws + (size_t)p * L * n, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, K, L};
+        HE_HIP(launch_bconv(ctx->tables(), b, S(s)));
+    }
+    NttArgs fwd = base_args(ctx, true);
+    fwd.in = ws;
+    fwd.out = ws;
+    fwd.in_poly_stride = fwd.out_poly_stride = L;
+    fwd.map = plain_map(L, 0);
+    fwd.epi_mode = accumulate ? NTT_EPI_SUB_MUL_ADD : NTT_EPI_SUB_MUL;
+    fwd.epi_a = cx;
+    fwd.epi_a_poly_stride = LK;
+    fwd.epi_b = out;
+    fwd.epi_b_poly_stride = L;
+    fwd.w = ctx->d_pinv_mod_q;
+    fwd.epi_dst = out;
+    fwd.epi_dst_poly_stride = L;
+    HE_HIP(launch_ntt_forward(fwd, n_polys, S(s)));
+    return HE_OK;
+}
+
+size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L) {
+    if (!ctx || ctx->size_p == 0 || L == 0 || L > ctx->size_q) return 0;
+    const size_t n = ctx->n(), K = ctx->size_p, LK = L + K;
+    const size_t beta = (L + K - 1) / K;
+    return beta * LK * n + 2 * LK * n + 2 * (size_t)L * n;
+}
+
+int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk, uint64_t *ct,
+                 uint32_t galois_elt, uint64_t *ws, he_stream s) {
+    if (!ctx || !c || !evk || !ct || !ws || ctx->size_p == 0) return HE_E_INVALID_ARGUMENT;
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    const size_t n = ctx->n(), LK = L + ctx->size_p;
+    uint64_t *y = ws;
+    uint64_t *cx = y + (size_t)lv->beta * LK * n;
+    uint64_t *tmp = cx + 2 * LK * n;
+    const uint64_t *src = c;
+    if (galois_elt) {
+        // sigma(c) is staged in the (not yet used) inner-product buffer
+        if (int rc = he_galois_ntt(ctx, c, cx, L, galois_elt, s)) return rc;
+        src = cx;
+    }
+    if (int rc = he_modup(ctx, L, src, y, tmp, s)) return rc;
+    if (int rc = he_ks_inner_product(ctx, L, y, evk, cx, 0, 0, s)) return rc;
+    return he_moddown(ctx, L, cx, ct, 2, 1, tmp, s);
+}
+
+int he_decompose_real(const he_context *ctx, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,
+                      he_stream s) {
+    if (!ctx || !coeffs || !out || first + limbs > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(launch_decompose_real(ctx->tables(), coeffs, out, limbs, first, S(s)));
+    return HE_OK;
+}
+
+int he_sample(const he_context *ctx, int kind, const uint32_t key[8], uint64_t stream_id, uint64_t *out,
+              uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail, const uint64_t *cdt, uint32_t cdt_len,
+              he_stream s) {
+    if (!ctx || !key || !out || kind < 0 || kind > 3 || (kind == SAMPLE_GAUSS && (!cdt || !cdt_len)))
+        return HE_E_INVALID_ARGUMENT;
+    if (int rc = check_map(ctx, limbs, first, split, tail)) return rc;
+    ChaChaKey k;
+    memcpy(k.k, key, sizeof(k.k));
+    HE_HIP(launch_sample(ctx->tables(), kind, k, stream_id, out, LimbMap{limbs, first, split, tail}, cdt, cdt_len, S(s)));
+    return HE_OK;
+}
+
+}  // extern "C"

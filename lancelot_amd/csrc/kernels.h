@@ -1,0 +1,128 @@
+// Internal interface between the C-ABI layer (capi.hip) and the kernel translation units.
+// Nothing here is visible to callers of the shared library; see include/cahel_hip.h for that.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace he {
+
+// One limb-sized NTT job given explicitly: which limb of the buffer, which modulus table.
+struct LimbJob {
+    uint32_t data_limb;
+    uint32_t table;
+};
+
+// How limb i (0 <= i < limbs) of every polynomial maps to a modulus table:
+//   table(i) = first + i             for i < split
+//   table(i) = tail_first + i - split  otherwise
+// (the second branch is the "special primes after the first L data primes" layout of a Ql u P buffer).
+struct LimbMap {
+    uint32_t limbs;
+    uint32_t first;
+    uint32_t split;
+    uint32_t tail_first;
+};
+
+__host__ __device__ inline uint32_t map_table(const LimbMap &m, uint32_t i) {
+    return i < m.split ? m.first + i : m.tail_first + (i - m.split);
+}
+
+inline LimbMap plain_map(uint32_t limbs, uint32_t first = 0) { return LimbMap{limbs, first, limbs, 0}; }
+
+// Prologue of the first forward pass / epilogue of the last pass of either direction.
+enum : int {
+    NTT_PLAIN = 0,
+    // forward prologue: input value = pro_src[poly][coeff] mod q (one source limb broadcast to every limb)
+    NTT_PRO_BROADCAST_REDUCE = 1,
+    // forward epilogue: dst = (epi_a - v) * w mod q
+    NTT_EPI_SUB_MUL = 2,
+    // forward epilogue: dst = epi_b + (epi_a - v) * w mod q
+    NTT_EPI_SUB_MUL_ADD = 3,
+    // inverse epilogue: out = v * w mod q
+    NTT_EPI_MUL = 4,
+};
+
+struct NttArgs {
+    const uint64_t *in;   // limb (poly, i) at in + (poly * in_poly_stride + i) * N
+    uint64_t *out;
+    uint32_t in_poly_stride;
+    uint32_t out_poly_stride;
+    const uint64_t *tw;       // [tables][N][2] (operand, Shoup quotient)
+    const uint64_t *moduli;   // [tables]
+    const uint64_t *barrett;  // [tables][2]
+    const LimbJob *jobs;      // explicit list (then in/out limbs are absolute, no prologue/epilogue)
+    uint32_t n_jobs;
+    uint32_t log_n;
+    LimbMap map;
+    int pro_mode;
+    int epi_mode;
+    const uint64_t *pro_src;  // [poly][pro_poly_stride limbs], the first limb of each poly is the source
+    uint32_t pro_poly_stride;
+    const uint64_t *epi_a;    // limb (poly, i) like `out`, with its own poly stride
+    uint32_t epi_a_poly_stride;
+    const uint64_t *epi_b;
+    uint32_t epi_b_poly_stride;
+    const uint64_t *w;        // [limbs][2] Shoup constants indexed by limb i of the map
+    uint64_t *epi_dst;        // destination of the forward epilogues
+    uint32_t epi_dst_poly_stride;
+};
+
+// Forward transform: phase 1 (strided rows) then phase 2 (contiguous 256-blocks).  `a.in`/`a.out` and the
+// prologue describe phase 1's input; phase 2 runs in place on a.out unless an epilogue redirects it.
+hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, hipStream_t s);
+// Inverse transform: phase A (contiguous blocks, reads a.in writes a.out) then phase B (rows, in place on
+// a.out, epilogue NTT_EPI_MUL optional).
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, hipStream_t s);
+
+struct Tables {
+    const uint64_t *moduli;
+    const uint64_t *barrett;
+    uint32_t log_n;
+};
+
+// elementwise family, limb i of every poly uses table map_table(map, i)
+enum : int { EW_ADD = 0, EW_SUB = 1, EW_MUL = 2, EW_NEG = 3, EW_MUL_ADD = 4, EW_MUL_ADD_NEG = 5 };
+hipError_t launch_elementwise(const Tables &t, int op, const uint64_t *a, const uint64_t *b, const uint64_t *c,
+                              uint64_t *out, uint32_t n_polys, LimbMap map, hipStream_t s);
+// out = a + b * w[limb] on limbs first .. first+limbs-1 (pointers already offset to limb `first`)
+hipError_t launch_scalar_mul_add(const Tables &t, const uint64_t *a, const uint64_t *b, uint64_t *out,
+                                 const uint64_t *w, uint32_t first, uint32_t limbs, hipStream_t s);
+hipError_t launch_tensor(const Tables &t, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
+                         bool square, hipStream_t s);
+hipError_t launch_galois(const Tables &t, const uint64_t *in, uint64_t *out, uint32_t total_limbs, uint32_t elt,
+                         hipStream_t s);
+
+// out[(row_limb(t))][j] = sum_i x[i][j] * mat[row][i] mod m: base conversion of one digit.
+//   x: [n_in][N] scaled residues; rows: n_out output limbs, output limb r is written to
+//   out + out_limb[r] * N and reduced by table out_table[r] (both small device arrays).
+struct BconvArgs {
+    const uint64_t *x;
+    uint64_t *out;
+    const uint64_t *mat;         // [n_out][n_in]
+    const uint32_t *out_limb;    // [n_out]
+    const uint32_t *out_table;   // [n_out]
+    uint32_t n_in, n_out;
+};
+hipError_t launch_bconv(const Tables &t, const BconvArgs &a, hipStream_t s);
+
+constexpr int kMaxDigits = 64;
+struct EvkPtrs {
+    const uint64_t *p[kMaxDigits];
+};
+// (2, L+K, N) <- sum_d y_d * evk_d ; galois_elt != 0 applies the NTT-domain automorphism to y on load.
+hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
+                                uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
+                                hipStream_t s);
+
+hipError_t launch_decompose_real(const Tables &t, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,
+                                 hipStream_t s);
+
+// samplers (ChaCha20 block function keyed by key[8]; distributions as in the CPU checker)
+enum : int { SAMPLE_TERNARY = 0, SAMPLE_ERROR = 1, SAMPLE_UNIFORM = 2, SAMPLE_GAUSS = 3 };
+struct ChaChaKey {
+    uint32_t k[8];
+};
+hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
+                         const uint64_t *cdt, uint32_t cdt_len, hipStream_t s);
+
+}  // namespace he

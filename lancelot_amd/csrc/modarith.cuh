@@ -1,0 +1,151 @@
+// Device-side 64-bit modular arithmetic for gfx950 (wave64, VALU integer multiplies).
+//
+// All routines work on residues of primes below 2^61.  "lazy" values live in [0, 2q) or [0, 4q) and
+// never leave a kernel: every store to HBM that a caller can observe is the canonical residue, which
+// is what makes limb-for-limb comparison with the CPU checker meaningful.
+//
+// Semantics follow cahel-main/include/uintmodmath.cuh (Shoup :226-245, Barrett :112-218) and
+// cahel-main/src/ntt/butterfly.cuh:10-43 (Harvey butterflies); the code is written for the CDNA4
+// integer pipeline (64x64 products are assembled from v_mad_u64_u32 by the compiler).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace he {
+
+struct Shoup {
+    uint64_t w;   // operand in [0, q)
+    uint64_t wq;  // floor(w * 2^64 / q)
+};
+
+__device__ __forceinline__ uint64_t mulhi64(uint64_t a, uint64_t b) { return __umul64hi(a, b); }
+
+// x * w mod q up to one subtraction of q: result in [0, 2q).  x may be any 64-bit value.
+__device__ __forceinline__ uint64_t mul_shoup_lazy(uint64_t x, Shoup s, uint64_t q) {
+    uint64_t hi = mulhi64(x, s.wq);
+    return x * s.w - hi * q;
+}
+
+__device__ __forceinline__ uint64_t mul_shoup(uint64_t x, Shoup s, uint64_t q) {
+    uint64_t r = mul_shoup_lazy(x, s, q);
+    return r >= q ? r - q : r;
+}
+
+__device__ __forceinline__ uint64_t add_mod(uint64_t a, uint64_t b, uint64_t q) {
+    uint64_t s = a + b;
+    return s >= q ? s - q : s;
+}
+
+__device__ __forceinline__ uint64_t sub_mod(uint64_t a, uint64_t b, uint64_t q) {
+    return a >= b ? a - b : a + q - b;
+}
+
+__device__ __forceinline__ uint64_t neg_mod(uint64_t a, uint64_t q) { return a ? q - a : 0; }
+
+// 128-bit value (hi:lo) mod q with ratio = floor(2^128 / q) = (r1:r0).
+__device__ __forceinline__ uint64_t barrett128(uint64_t lo, uint64_t hi, uint64_t q, uint64_t r0, uint64_t r1) {
+    uint64_t carry = mulhi64(lo, r0);
+    uint64_t t_lo = lo * r1;
+    uint64_t t_hi = mulhi64(lo, r1);
+    uint64_t tmp = t_lo + carry;
+    uint64_t quo = t_hi + (tmp < t_lo);
+    uint64_t u_lo = hi * r0;
+    uint64_t u_hi = mulhi64(hi, r0);
+    uint64_t tmp2 = tmp + u_lo;
+    quo += u_hi + (tmp2 < tmp);
+    quo += hi * r1;
+    uint64_t r = lo - quo * q;
+    return r >= q ? r - q : r;
+}
+
+__device__ __forceinline__ uint64_t mul_mod(uint64_t a, uint64_t b, uint64_t q, uint64_t r0, uint64_t r1) {
+    return barrett128(a * b, mulhi64(a, b), q, r0, r1);
+}
+
+// 64-bit value mod q with r1 = floor(2^64 / q).
+__device__ __forceinline__ uint64_t barrett64(uint64_t x, uint64_t q, uint64_t r1) {
+    uint64_t r = x - mulhi64(r1, x) * q;
+    return r >= q ? r - q : r;
+}
+
+struct U128 {
+    uint64_t lo, hi;
+};
+
+__device__ __forceinline__ void mac128(U128 &acc, uint64_t a, uint64_t b) {
+    uint64_t lo = a * b;
+    uint64_t hi = mulhi64(a, b);
+    acc.lo += lo;
+    acc.hi += hi + (acc.lo < lo);
+}
+
+// Cooley-Tukey butterfly, inputs in [0, 4q), outputs in [0, 4q).
+__device__ __forceinline__ void ct_butterfly(uint64_t &x, uint64_t &y, Shoup tw, uint64_t q) {
+    uint64_t q2 = q << 1;
+    uint64_t t = mul_shoup_lazy(y, tw, q);
+    uint64_t xr = x >= q2 ? x - q2 : x;
+    y = xr + q2 - t;
+    x = xr + t;
+}
+
+// Gentleman-Sande butterfly with the division by two folded in (the inverse twiddles are stored
+// pre-halved), inputs in [0, 2q), outputs in [0, 2q).
+__device__ __forceinline__ void gs_butterfly(uint64_t &x, uint64_t &y, Shoup tw, uint64_t q) {
+    uint64_t q2 = q << 1;
+    uint64_t d = x + q2 - y;
+    uint64_t s = x + y;
+    s = s >= q2 ? s - q2 : s;
+    s += (d & 1) ? q : 0;
+    x = s >> 1;
+    y = mul_shoup_lazy(d, tw, q);
+}
+
+__device__ __forceinline__ uint64_t reduce_4q(uint64_t v, uint64_t q) {
+    uint64_t q2 = q << 1;
+    v = v >= q2 ? v - q2 : v;
+    return v >= q ? v - q : v;
+}
+
+__device__ __forceinline__ uint64_t reduce_2q(uint64_t v, uint64_t q) { return v >= q ? v - q : v; }
+
+__device__ __forceinline__ Shoup load_shoup(const uint64_t *table, size_t idx) {
+    const ulonglong2 v = reinterpret_cast<const ulonglong2 *>(table)[idx];
+    return Shoup{v.x, v.y};
+}
+
+// R = 2^LOGR point decimation-in-time block: LOGR consecutive forward stages on register values.
+// v[j] are the elements whose index differs in the LOGR bits that these stages pair, most significant
+// first; idx = 2^s0 + (group number at the first stage s0); twiddle of local stage l, sub-block b is
+// table[(idx << l) + b].
+template <int LOGR>
+__device__ __forceinline__ void ct_block(uint64_t *v, const uint64_t *table, uint32_t idx, uint64_t q) {
+    constexpr int R = 1 << LOGR;
+#pragma unroll
+    for (int l = 0; l < LOGR; l++) {
+        const int half = R >> (l + 1);
+#pragma unroll
+        for (int b = 0; b < (1 << l); b++) {
+            Shoup tw = load_shoup(table, ((size_t)idx << l) + b);
+#pragma unroll
+            for (int j = 0; j < half; j++) ct_butterfly(v[2 * b * half + j], v[2 * b * half + j + half], tw, q);
+        }
+    }
+}
+
+// The mirror image: the same LOGR stages in inverse order with Gentleman-Sande butterflies.
+template <int LOGR>
+__device__ __forceinline__ void gs_block(uint64_t *v, const uint64_t *table, uint32_t idx, uint64_t q) {
+    constexpr int R = 1 << LOGR;
+#pragma unroll
+    for (int l = LOGR - 1; l >= 0; l--) {
+        const int half = R >> (l + 1);
+#pragma unroll
+        for (int b = 0; b < (1 << l); b++) {
+            Shoup tw = load_shoup(table, ((size_t)idx << l) + b);
+#pragma unroll
+            for (int j = 0; j < half; j++) gs_butterfly(v[2 * b * half + j], v[2 * b * half + j + half], tw, q);
+        }
+    }
+}
+
+}  // namespace he

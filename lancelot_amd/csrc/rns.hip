@@ -1,0 +1,355 @@
+// Streaming RNS kernels for gfx950: elementwise polynomial arithmetic, tensor product, NTT-domain Galois
+// gather, base conversion (the modular matrix-vector product of ModUp / ModDown), the key-switch inner
+// product, and the seeded samplers.  All of them are HBM-bound streams over [limb][coeff] arrays: one
+// coefficient per lane, 256 consecutive coefficients per workgroup, so every access is a full-width
+// coalesced row segment.
+//
+// What they compute follows cahel-main/src/polymath.cu (add :40, sub :108, multiply :160, mad :227/:349,
+// tensor :531-612), src/galois.cu:20-30 + include/galois.cuh:45-57, src/rns_bconv.cu:587-623 and :166-198
+// (base conversion, uncorrected sum, one reduction), src/eval_key_switch.cu:13-76 (inner product) and
+// src/prng.cu:143-242 (distributions of the samplers).
+#include "kernels.h"
+#include "modarith.cuh"
+
+namespace he {
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct EwArgs {
+    const uint64_t *a, *b, *c;
+    uint64_t *out;
+    const uint64_t *moduli, *barrett;
+    LimbMap map;
+    uint32_t log_n;
+    int op;
+};
+
+// grid: (N / 256, limbs, polys)
+__global__ __launch_bounds__(kThreads) void elementwise_kernel(EwArgs p) {
+    const uint32_t limb = blockIdx.y;
+    const uint32_t table = map_table(p.map, limb);
+    const uint64_t q = p.moduli[table];
+    const size_t idx = (((size_t)blockIdx.z * p.map.limbs + limb) << p.log_n) + blockIdx.x * kThreads + threadIdx.x;
+    uint64_t r;
+    switch (p.op) {
+        case EW_ADD: r = add_mod(p.a[idx], p.b[idx], q); break;
+        case EW_SUB: r = sub_mod(p.a[idx], p.b[idx], q); break;
+        case EW_NEG: r = neg_mod(p.a[idx], q); break;
+        case EW_MUL: r = mul_mod(p.a[idx], p.b[idx], q, p.barrett[2 * table], p.barrett[2 * table + 1]); break;
+        default: {
+            r = add_mod(mul_mod(p.a[idx], p.b[idx], q, p.barrett[2 * table], p.barrett[2 * table + 1]), p.c[idx], q);
+            if (p.op == EW_MUL_ADD_NEG) r = neg_mod(r, q);
+        }
+    }
+    p.out[idx] = r;
+}
+
+// grid: (N / 256, limbs): out = a + b * w[first + limb]
+__global__ __launch_bounds__(kThreads) void scalar_mul_add_kernel(const uint64_t *a, const uint64_t *b, uint64_t *out,
+                                                                  const uint64_t *moduli, const uint64_t *w,
+                                                                  uint32_t first, uint32_t log_n) {
+    const uint32_t table = first + blockIdx.y;
+    const uint64_t q = moduli[table];
+    const size_t idx = ((size_t)blockIdx.y << log_n) + blockIdx.x * kThreads + threadIdx.x;
+    out[idx] = add_mod(a[idx], mul_shoup(b[idx], load_shoup(w, table), q), q);
+}
+
+// grid: (N / 256, limbs): residue of a rounded real coefficient
+__global__ __launch_bounds__(kThreads) void decompose_real_kernel(const double *coeffs, uint64_t *out,
+                                                                  const uint64_t *moduli, const uint64_t *barrett,
+                                                                  uint32_t first, uint32_t log_n) {
+    const uint32_t table = first + blockIdx.y;
+    const uint64_t q = moduli[table];
+    const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+    const double c = coeffs[i];
+    const uint64_t r = barrett64((uint64_t)fabs(c), q, barrett[2 * table + 1]);
+    out[((size_t)blockIdx.y << log_n) + i] = c < 0 ? neg_mod(r, q) : r;
+}
+
+struct TensorArgs {
+    const uint64_t *ct1, *ct2;
+    uint64_t *out;
+    const uint64_t *moduli, *barrett;
+    uint32_t L, log_n;
+};
+
+// grid: (N / 256, L).  Reads the four input limbs once, writes the three outputs: (d0, d1, d2) =
+// (a0 b0, a0 b1 + a1 b0, a1 b1); out may alias ct1 (every index is read before it is written).
+template <bool SQUARE>
+__global__ __launch_bounds__(kThreads) void tensor_kernel(TensorArgs p) {
+    const uint32_t limb = blockIdx.y;
+    const uint64_t q = p.moduli[limb], r0 = p.barrett[2 * limb], r1 = p.barrett[2 * limb + 1];
+    const size_t poly = (size_t)p.L << p.log_n;
+    const size_t idx = ((size_t)limb << p.log_n) + blockIdx.x * kThreads + threadIdx.x;
+    const uint64_t a0 = p.ct1[idx], a1 = p.ct1[idx + poly];
+    uint64_t d0, d1, d2;
+    if (SQUARE) {
+        d0 = mul_mod(a0, a0, q, r0, r1);
+        d2 = mul_mod(a1, a1, q, r0, r1);
+        uint64_t m = mul_mod(a0, a1, q, r0, r1);
+        d1 = add_mod(m, m, q);
+    } else {
+        const uint64_t b0 = p.ct2[idx], b1 = p.ct2[idx + poly];
+        d0 = mul_mod(a0, b0, q, r0, r1);
+        d2 = mul_mod(a1, b1, q, r0, r1);
+        // Karatsuba: (a0 + a1)(b0 + b1) - d0 - d2; the sums stay below 2^62
+        uint64_t m = mul_mod(a0 + a1, b0 + b1, q, r0, r1);
+        d1 = sub_mod(sub_mod(m, d0, q), d2, q);
+    }
+    p.out[idx] = d0;
+    p.out[idx + poly] = d1;
+    p.out[idx + 2 * poly] = d2;
+}
+
+// NTT-domain automorphism X -> X^elt as a gather: out[i] = in[pi(i)],
+// pi(i) = bitrev(((elt * (2 bitrev(i) + 1)) >> 1) mod N)
+__device__ __forceinline__ uint32_t galois_index(uint32_t i, uint32_t elt, uint32_t log_n) {
+    const uint32_t r = __brev(i) >> (32 - log_n);
+    const uint32_t raw = (uint32_t)(((uint64_t)elt * (2 * r + 1)) >> 1) & ((1u << log_n) - 1);
+    return __brev(raw) >> (32 - log_n);
+}
+
+// grid: (N / 256, total limbs)
+__global__ __launch_bounds__(kThreads) void galois_kernel(const uint64_t *in, uint64_t *out, uint32_t elt,
+                                                          uint32_t log_n) {
+    const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+    const size_t base = (size_t)blockIdx.y << log_n;
+    out[base + i] = in[base + galois_index(i, elt, log_n)];
+}
+
+// Base conversion of one digit: thread = one coefficient x kRows output limbs.
+constexpr int kRows = 4;
+
+struct BconvKArgs {
+    BconvArgs a;
+    const uint64_t *moduli, *barrett;
+    uint32_t log_n;
+};
+
+template <int NIN>
+__global__ __launch_bounds__(kThreads) void bconv_kernel(BconvKArgs p) {
+    const size_t j = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    const uint32_t n_in = NIN > 0 ? NIN : p.a.n_in;
+    uint64_t x[NIN > 0 ? NIN : 1];
+    if (NIN > 0) {
+#pragma unroll
+        for (int i = 0; i < NIN; i++) x[i] = p.a.x[((size_t)i << p.log_n) + j];
+    }
+    for (uint32_t rr = 0; rr < kRows; rr++) {
+        const uint32_t row = blockIdx.y * kRows + rr;
+        if (row >= p.a.n_out) return;
+        const uint64_t *m = p.a.mat + (size_t)row * n_in;
+        U128 acc{0, 0};
+        if (NIN > 0) {
+#pragma unroll
+            for (int i = 0; i < NIN; i++) mac128(acc, x[i], m[i]);
+        } else {
+            for (uint32_t i = 0; i < n_in; i++) mac128(acc, p.a.x[((size_t)i << p.log_n) + j], m[i]);
+        }
+        const uint32_t t = p.a.out_table[row];
+        p.a.out[((size_t)p.a.out_limb[row] << p.log_n) + j] =
+            barrett128(acc.lo, acc.hi, p.moduli[t], p.barrett[2 * t], p.barrett[2 * t + 1]);
+    }
+}
+
+struct InnerArgs {
+    const uint64_t *y;
+    uint64_t *out;
+    const uint64_t *moduli, *barrett;
+    EvkPtrs evk;
+    uint32_t L, K, size_q, beta, log_n, galois_elt;
+    int accumulate;
+};
+
+// grid: (N / 256, L + K).  Streams beta digit limbs of y and 2 beta key limbs, writes (or accumulates) the
+// two output limbs.  The products are summed in 128 bits and reduced once (beta <= 64 products of
+// 61-bit factors cannot overflow).
+__global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
+    const uint32_t t = blockIdx.y;
+    const uint32_t LK = p.L + p.K;
+    const uint32_t table = t < p.L ? t : p.size_q + (t - p.L);
+    const uint32_t j = blockIdx.x * kThreads + threadIdx.x;
+    const uint32_t src = p.galois_elt ? galois_index(j, p.galois_elt, p.log_n) : j;
+    const size_t key_off = ((size_t)table << p.log_n) + j;
+    const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
+    U128 a0{0, 0}, a1{0, 0};
+    for (uint32_t d = 0; d < p.beta; d++) {
+        const uint64_t v = p.y[(((size_t)d * LK + t) << p.log_n) + src];
+        const uint64_t *k = p.evk.p[d];
+        mac128(a0, v, k[key_off]);
+        mac128(a1, v, k[key_off + key_poly]);
+    }
+    const uint64_t q = p.moduli[table], r0 = p.barrett[2 * table], r1 = p.barrett[2 * table + 1];
+    uint64_t o0 = barrett128(a0.lo, a0.hi, q, r0, r1);
+    uint64_t o1 = barrett128(a1.lo, a1.hi, q, r0, r1);
+    const size_t o = ((size_t)t << p.log_n) + j;
+    const size_t opoly = (size_t)LK << p.log_n;
+    if (p.accumulate) {
+        o0 = add_mod(o0, p.out[o], q);
+        o1 = add_mod(o1, p.out[o + opoly], q);
+    }
+    p.out[o] = o0;
+    p.out[o + opoly] = o1;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// samplers: ChaCha20 block function (RFC 8439 section 2.3), 64-bit block counter in words 12-13,
+// 64-bit stream id in words 14-15
+// ---------------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint32_t rotl32(uint32_t v, int c) { return (v << c) | (v >> (32 - c)); }
+
+#define HE_QR(a, b, c, d) \
+    a += b; d ^= a; d = rotl32(d, 16); \
+    c += d; b ^= c; b = rotl32(b, 12); \
+    a += b; d ^= a; d = rotl32(d, 8);  \
+    c += d; b ^= c; b = rotl32(b, 7);
+
+__device__ void chacha20_block(const ChaChaKey &key, uint64_t counter, uint64_t stream, uint32_t *out) {
+    uint32_t s[16] = {0x61707865u, 0x3320646eu, 0x79622d32u, 0x6b206574u,
+                      key.k[0], key.k[1], key.k[2], key.k[3], key.k[4], key.k[5], key.k[6], key.k[7],
+                      (uint32_t)counter, (uint32_t)(counter >> 32), (uint32_t)stream, (uint32_t)(stream >> 32)};
+    uint32_t x[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) x[i] = s[i];
+    for (int i = 0; i < 10; i++) {
+        HE_QR(x[0], x[4], x[8], x[12]) HE_QR(x[1], x[5], x[9], x[13]) HE_QR(x[2], x[6], x[10], x[14]) HE_QR(x[3], x[7], x[11], x[15])
+        HE_QR(x[0], x[5], x[10], x[15]) HE_QR(x[1], x[6], x[11], x[12]) HE_QR(x[2], x[7], x[8], x[13]) HE_QR(x[3], x[4], x[9], x[14])
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) out[i] = x[i] + s[i];
+}
+
+struct SampleArgs {
+    uint64_t *out;
+    const uint64_t *moduli, *barrett;
+    const uint64_t *cdt;
+    ChaChaKey key;
+    uint64_t stream;
+    LimbMap map;
+    uint32_t log_n, cdt_len;
+    int kind;
+};
+
+// ternary / error / gauss: one thread = one ChaCha block = 16 (ternary) or 8 coefficients, the same
+// signed value written to every limb.  uniform: one thread = one block = 4 residues of one limb.
+__global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
+    const uint32_t n = 1u << p.log_n;
+    const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
+    uint32_t w[16];
+    if (p.kind == SAMPLE_UNIFORM) {
+        const uint32_t per_limb = n / 4;
+        if (b >= per_limb * p.map.limbs) return;
+        const uint32_t limb = b / per_limb, blk = b % per_limb;
+        const uint32_t table = map_table(p.map, limb);
+        const uint64_t q = p.moduli[table], r0 = p.barrett[2 * table], r1 = p.barrett[2 * table + 1];
+        chacha20_block(p.key, b, p.stream, w);
+        for (int e = 0; e < 4; e++) {
+            uint64_t lo = ((uint64_t)w[4 * e + 1] << 32) | w[4 * e];
+            uint64_t hi = ((uint64_t)w[4 * e + 3] << 32) | w[4 * e + 2];
+            p.out[((size_t)limb << p.log_n) + 4 * blk + e] = barrett128(lo, hi, q, r0, r1);
+        }
+        return;
+    }
+    const uint32_t per_block = p.kind == SAMPLE_TERNARY ? 16 : 8;
+    if (b >= n / per_block) return;
+    chacha20_block(p.key, b, p.stream, w);
+    for (uint32_t e = 0; e < per_block; e++) {
+        int v;
+        if (p.kind == SAMPLE_TERNARY) {
+            v = (int)(((uint64_t)w[e] * 3) >> 32) - 1;
+        } else if (p.kind == SAMPLE_ERROR) {
+            v = __popc(w[2 * e] & 0x1FFFFFu) - __popc(w[2 * e + 1] & 0x1FFFFFu);
+        } else {
+            uint64_t u = ((uint64_t)w[2 * e + 1] << 32) | w[2 * e];
+            const bool neg = u >> 63;
+            u &= 0x7FFFFFFFFFFFFFFFull;
+            uint32_t mag = 0;
+            while (mag < p.cdt_len && u >= p.cdt[mag]) mag++;
+            v = neg ? -(int)mag : (int)mag;
+        }
+        for (uint32_t limb = 0; limb < p.map.limbs; limb++) {
+            const uint64_t q = p.moduli[map_table(p.map, limb)];
+            p.out[((size_t)limb << p.log_n) + per_block * b + e] = v < 0 ? q - (uint64_t)(-v) : (uint64_t)v;
+        }
+    }
+}
+
+}  // namespace
+
+hipError_t launch_elementwise(const Tables &t, int op, const uint64_t *a, const uint64_t *b, const uint64_t *c,
+                              uint64_t *out, uint32_t n_polys, LimbMap map, hipStream_t s) {
+    if (n_polys == 0 || map.limbs == 0) return hipSuccess;
+    EwArgs p{a, b, c, out, t.moduli, t.barrett, map, t.log_n, op};
+    hipLaunchKernelGGL(elementwise_kernel, dim3((1u << t.log_n) / kThreads, map.limbs, n_polys), dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_scalar_mul_add(const Tables &t, const uint64_t *a, const uint64_t *b, uint64_t *out,
+                                 const uint64_t *w, uint32_t first, uint32_t limbs, hipStream_t s) {
+    if (limbs == 0) return hipSuccess;
+    hipLaunchKernelGGL(scalar_mul_add_kernel, dim3((1u << t.log_n) / kThreads, limbs), dim3(kThreads), 0, s, a, b, out,
+                       t.moduli, w, first, t.log_n);
+    return hipGetLastError();
+}
+
+hipError_t launch_decompose_real(const Tables &t, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,
+                                 hipStream_t s) {
+    if (limbs == 0) return hipSuccess;
+    hipLaunchKernelGGL(decompose_real_kernel, dim3((1u << t.log_n) / kThreads, limbs), dim3(kThreads), 0, s, coeffs, out,
+                       t.moduli, t.barrett, first, t.log_n);
+    return hipGetLastError();
+}
+
+hipError_t launch_tensor(const Tables &t, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
+                         bool square, hipStream_t s) {
+    TensorArgs p{ct1, ct2, out, t.moduli, t.barrett, L, t.log_n};
+    dim3 grid((1u << t.log_n) / kThreads, L);
+    if (square)
+        hipLaunchKernelGGL(tensor_kernel<true>, grid, dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL(tensor_kernel<false>, grid, dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_galois(const Tables &t, const uint64_t *in, uint64_t *out, uint32_t total_limbs, uint32_t elt,
+                         hipStream_t s) {
+    if (total_limbs == 0) return hipSuccess;
+    hipLaunchKernelGGL(galois_kernel, dim3((1u << t.log_n) / kThreads, total_limbs), dim3(kThreads), 0, s, in, out, elt,
+                       t.log_n);
+    return hipGetLastError();
+}
+
+hipError_t launch_bconv(const Tables &t, const BconvArgs &a, hipStream_t s) {
+    if (a.n_out == 0) return hipSuccess;
+    BconvKArgs p{a, t.moduli, t.barrett, t.log_n};
+    dim3 grid((1u << t.log_n) / kThreads, (a.n_out + kRows - 1) / kRows);
+    switch (a.n_in) {
+#define HE_CASE(NIN) \
+    case NIN: hipLaunchKernelGGL(bconv_kernel<NIN>, grid, dim3(kThreads), 0, s, p); break;
+        HE_CASE(1) HE_CASE(2) HE_CASE(3) HE_CASE(4) HE_CASE(5) HE_CASE(6) HE_CASE(7) HE_CASE(8)
+#undef HE_CASE
+        default: hipLaunchKernelGGL(bconv_kernel<0>, grid, dim3(kThreads), 0, s, p);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
+                                uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
+                                hipStream_t s) {
+    InnerArgs p{y, out, t.moduli, t.barrett, evk, L, K, size_q, beta, t.log_n, galois_elt, accumulate ? 1 : 0};
+    hipLaunchKernelGGL(inner_product_kernel, dim3((1u << t.log_n) / kThreads, L + K), dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
+                         const uint64_t *cdt, uint32_t cdt_len, hipStream_t s) {
+    const uint32_t n = 1u << t.log_n;
+    uint32_t blocks = kind == SAMPLE_UNIFORM ? (n / 4) * map.limbs : (kind == SAMPLE_TERNARY ? n / 16 : n / 8);
+    SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind};
+    hipLaunchKernelGGL(sample_kernel, dim3((blocks + kThreads - 1) / kThreads), dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
+}  // namespace he

@@ -1,0 +1,303 @@
+"""Parity of every HIP kernel against the CPU oracle, called through the C-ABI of libcahel_hip.so.
+
+Bit-exact: every integer stage must reproduce the oracle's limbs word for word on the same seeded inputs.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from gpu_util import DeviceArray, make_pair, rand_limbs
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from lancelot_amd import capi as c
+    c.lib()
+    return c
+
+
+@pytest.fixture(scope="module")
+def small(oracle):
+    # N = 4096, 6 Q limbs (mixed widths) + 2 special: three digits of two limbs
+    return make_pair(oracle, 12, [60, 40, 50, 45, 30, 59, 60, 60], 2)
+
+
+@pytest.fixture(scope="module")
+def full(oracle):
+    # benchmark shape: N = 2^16, 24 Q limbs + 8 special limbs of 50 bits (beta = 3)
+    return make_pair(oracle, 16, [50] * 32, 8)
+
+
+def test_tables_match_oracle(small):
+    cahel, parms, ctx, p = small
+    psi, ipsi = ctx.psi_table(), ctx.ipsi_table()
+    assert (psi[:, :, 0] == p.tw).all() and (psi[:, :, 1] == p.twq).all()
+    assert (ipsi[:, :, 0] == p.itw).all() and (ipsi[:, :, 1] == p.itwq).all()
+    for L in range(1, p.size_q + 1):
+        lt, got = p.level(L), ctx.level_tables(L)
+        assert got["beta"] == lt.beta
+        assert got["part_hat_inv"][0::2] == [int(v) for v in lt.hatinv]
+        assert got["digit_mats"] == [int(v) for v in lt.mats]
+        assert got["digit_mat_off"] == [int(v) for v in lt.mat_off]
+        assert got["qlast_inv"][0::2] == [int(v) for v in lt.qlast_inv]
+        for w, wq, q in zip(got["part_hat_inv"][0::2], got["part_hat_inv"][1::2], p.moduli):
+            assert wq == (w << 64) // q
+
+
+@pytest.mark.parametrize("logn", [9, 10, 11, 12, 13, 14, 15, 16])
+def test_ntt_all_sizes(oracle, capi, logn):
+    cahel, parms, ctx, p = make_pair(oracle, logn, [60, 50, 35, 59], 1)
+    rng = np.random.default_rng(logn)
+    h = ctx.he_handle()
+    x = rand_limbs(p, rng, range(4), n_polys=2)
+    x[0, 0, :8] = 0
+    x[0, 1, :8] = p.moduli[1] - 1
+    d = DeviceArray(capi, host=x)
+    capi.check(capi.lib().he_ntt_forward(h, d.ptr, 2, 4, 4, 0, 4, 0, None))
+    want = np.stack([p.ntt_fwd(x[i].copy()) for i in range(2)])
+    got = d.numpy()
+    assert (got == want).all()
+    capi.check(capi.lib().he_ntt_inverse(h, d.ptr, 2, 4, 4, 0, 4, 0, None))
+    assert (d.numpy() == x).all()
+    # inverse of arbitrary canonical data (not an NTT image of anything special) against the oracle
+    d2 = DeviceArray(capi, host=x)
+    capi.check(capi.lib().he_ntt_inverse(h, d2.ptr, 2, 4, 4, 0, 4, 0, None))
+    assert (d2.numpy() == np.stack([p.ntt_inv(x[i].copy()) for i in range(2)])).all()
+
+
+def test_ntt_limb_maps(small, capi):
+    """Partial limb ranges, the Ql u P table map and poly strides larger than the transformed range."""
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(1)
+    h = ctx.he_handle()
+    L, K, Q = 4, p.size_p, p.size_q
+    tidx = [p.table_index(L, t) for t in range(L + K)]
+    x = rand_limbs(p, rng, tidx, n_polys=3)
+    d = DeviceArray(capi, host=x)
+    capi.check(capi.lib().he_ntt_forward(h, d.ptr, 3, L + K, L + K, 0, L, Q, None))
+    want = np.stack([p.ntt_fwd(x[i].copy(), tidx) for i in range(3)])
+    assert (d.numpy() == want).all()
+    # only the special limbs, in place inside the wider buffer (what ModDown does)
+    capi.check(capi.lib().he_ntt_inverse(h, d.at(L * p.n), 3, L + K, K, Q, K, 0, None))
+    got = d.numpy()
+    assert (got[:, :L] == want[:, :L]).all() and (got[:, L:] == x[:, L:]).all()
+    # a single limb in the middle of Q
+    y = rand_limbs(p, rng, [3])
+    dy = DeviceArray(capi, host=y)
+    capi.check(capi.lib().he_ntt_forward(h, dy.ptr, 1, 1, 1, 3, 1, 0, None))
+    assert (dy.numpy() == p.ntt_fwd(y.copy(), [3])).all()
+
+
+def test_ntt_benchmark_shape(full, capi):
+    """N = 2^16, 24 limbs, 2 polynomials: forward vs oracle, inverse round trip."""
+    cahel, parms, ctx, p = full
+    rng = np.random.default_rng(2)
+    x = rand_limbs(p, rng, range(24), n_polys=2)
+    d = DeviceArray(capi, host=x)
+    h = ctx.he_handle()
+    capi.check(capi.lib().he_ntt_forward(h, d.ptr, 2, 24, 24, 0, 24, 0, None))
+    assert (d.numpy() == np.stack([p.ntt_fwd(x[i].copy()) for i in range(2)])).all()
+    capi.check(capi.lib().he_ntt_inverse(h, d.ptr, 2, 24, 24, 0, 24, 0, None))
+    assert (d.numpy() == x).all()
+
+
+def test_ntt_rejects_bad_arguments(small, capi):
+    cahel, parms, ctx, p = small
+    d = DeviceArray(capi, shape=(1, p.n))
+    lib, h = capi.lib(), ctx.he_handle()
+    assert lib.he_ntt_forward(h, d.ptr, 1, 1, 1, p.size_qp, 1, 0, None) == -1      # table out of range
+    assert lib.he_ntt_forward(h, d.ptr, 1, 1, 2, 0, 2, 0, None) == -1              # limbs > stride
+    assert lib.he_ntt_forward(h, None, 1, 1, 1, 0, 1, 0, None) == -1
+    with pytest.raises(RuntimeError):
+        capi.check(-1)
+
+
+def test_elementwise(small, capi):
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(3)
+    lib, h = capi.lib(), ctx.he_handle()
+    limbs = p.size_qp
+    a, b, c = (rand_limbs(p, rng, range(limbs), n_polys=2) for _ in range(3))
+    a[0, :, 0], b[0, :, 0] = 0, [q - 1 for q in p.moduli]
+    da, db, dc, do = (DeviceArray(capi, host=v) for v in (a, b, c, a))
+    flat = lambda f, *xs: np.stack([f(*(x[i] for x in xs)) for i in range(2)])
+    capi.check(lib.he_add(h, da.ptr, db.ptr, do.ptr, 2, limbs, 0, None))
+    assert (do.numpy() == flat(p.add, a, b)).all()
+    capi.check(lib.he_sub(h, da.ptr, db.ptr, do.ptr, 2, limbs, 0, None))
+    assert (do.numpy() == flat(p.sub, a, b)).all()
+    capi.check(lib.he_negate(h, da.ptr, do.ptr, 2, limbs, 0, None))
+    assert (do.numpy() == flat(p.negate, a)).all()
+    capi.check(lib.he_multiply(h, da.ptr, db.ptr, do.ptr, 2, limbs, 0, None))
+    assert (do.numpy() == flat(p.mul, a, b)).all()
+    capi.check(lib.he_multiply_add(h, da.ptr, db.ptr, dc.ptr, do.ptr, 2, limbs, 0, 0, None))
+    assert (do.numpy() == flat(p.mul_add, a, b, c)).all()
+    capi.check(lib.he_multiply_add(h, da.ptr, db.ptr, dc.ptr, do.ptr, 2, limbs, 0, 1, None))
+    assert (do.numpy() == flat(lambda x, y, z: p.mul_add(x, y, z, True), a, b, c)).all()
+    # in place (out aliases a)
+    capi.check(lib.he_add(h, da.ptr, db.ptr, da.ptr, 2, limbs, 0, None))
+    assert (da.numpy() == flat(p.add, a, b)).all()
+
+
+def test_tensor_and_square(small, capi):
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(4)
+    lib, h = capi.lib(), ctx.he_handle()
+    for L in (6, 3, 1):
+        a, b = (rand_limbs(p, rng, range(L), n_polys=2) for _ in range(2))
+        a[:, :, 0] = [q - 1 for q in p.moduli[:L]]
+        b[:, :, 0] = [q - 1 for q in p.moduli[:L]]
+        da, db = DeviceArray(capi, host=a), DeviceArray(capi, host=b)
+        do = DeviceArray(capi, shape=(3, L, p.n))
+        capi.check(lib.he_tensor(h, da.ptr, db.ptr, do.ptr, L, None))
+        assert (do.numpy() == p.tensor(a, b)).all()
+        capi.check(lib.he_tensor_square(h, da.ptr, do.ptr, L, None))
+        assert (do.numpy() == p.square(a)).all()
+        # in place on a 3-poly buffer whose first two polys hold the operand
+        buf = np.zeros((3, L, p.n), dtype=np.uint64)
+        buf[:2] = a
+        dbuf = DeviceArray(capi, host=buf)
+        capi.check(lib.he_tensor(h, dbuf.ptr, db.ptr, dbuf.ptr, L, None))
+        assert (dbuf.numpy() == p.tensor(a, b)).all()
+
+
+@pytest.mark.parametrize("step", [1, -1, 7, 0, 1000])
+def test_galois(small, capi, oracle, step):
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(5)
+    elt = oracle.galois_elt_from_step(step, p.n)
+    assert cahel.get_elts_from_steps([step], p.n) == [elt]
+    a = rand_limbs(p, rng, range(p.size_qp))
+    da, do = DeviceArray(capi, host=a), DeviceArray(capi, shape=a.shape)
+    capi.check(capi.lib().he_galois_ntt(ctx.he_handle(), da.ptr, do.ptr, p.size_qp, elt, None))
+    assert (do.numpy() == p.galois_ntt(a, elt)).all()
+    assert capi.lib().he_galois_ntt(ctx.he_handle(), da.ptr, do.ptr, 1, 4, None) == -1      # even element
+    assert capi.lib().he_galois_ntt(ctx.he_handle(), da.ptr, da.ptr, 1, elt, None) == -1    # in place
+
+
+@pytest.mark.parametrize("L", [6, 5, 2])
+def test_rescale(small, capi, L):
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(6 + L)
+    ct = rand_limbs(p, rng, range(L), n_polys=3)
+    din = DeviceArray(capi, host=ct)
+    dout = DeviceArray(capi, shape=(3, L - 1, p.n))
+    ws = DeviceArray(capi, shape=(3, p.n))
+    capi.check(capi.lib().he_rescale(ctx.he_handle(), din.ptr, dout.ptr, 3, L, ws.ptr, None))
+    assert (dout.numpy() == p.rescale(ct)).all()
+    assert (din.numpy() == ct).all()                      # the input is left untouched
+    assert capi.lib().he_rescale(ctx.he_handle(), din.ptr, dout.ptr, 3, 1, ws.ptr, None) == -1
+
+
+def _evk(p, rng, capi):
+    dnum = p.size_q // p.size_p
+    host = [rand_limbs(p, rng, range(p.size_qp), n_polys=2) for _ in range(dnum)]
+    dev = [DeviceArray(capi, host=k) for k in host]
+    return host, dev, capi.evk_array([d.ptr for d in dev])
+
+
+@pytest.mark.parametrize("L", [6, 5, 4, 3, 1])
+def test_modup_inner_moddown(small, capi, L):
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(10 + L)
+    lib, h = capi.lib(), ctx.he_handle()
+    K, n = p.size_p, p.n
+    beta = -(-L // K)
+    c = rand_limbs(p, rng, range(L))
+    dc = DeviceArray(capi, host=c)
+    dy = DeviceArray(capi, shape=(beta, L + K, n))
+    ws = DeviceArray(capi, shape=(2 * L, n))
+    capi.check(lib.he_modup(h, L, dc.ptr, dy.ptr, ws.ptr, None))
+    y = p.modup(c)
+    assert (dy.numpy() == y).all()
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    dcx = DeviceArray(capi, shape=(2, L + K, n))
+    capi.check(lib.he_ks_inner_product(h, L, dy.ptr, ptrs, dcx.ptr, 0, 0, None))
+    cx = p.inner_prod(y, host_evk)
+    assert (dcx.numpy() == cx).all()
+    # accumulate + automorphism on load (the hoisting form)
+    elt = 25
+    capi.check(lib.he_ks_inner_product(h, L, dy.ptr, ptrs, dcx.ptr, elt, 1, None))
+    tidx = [p.table_index(L, t) for t in range(L + K)]
+    cx2 = p.inner_prod(p.galois_ntt(y, elt), host_evk)
+    acc = np.stack([p._add_tidx(cx[b], cx2[b], tidx) for b in range(2)])
+    assert (dcx.numpy() == acc).all()
+    # ModDown: plain and accumulating
+    dcx = DeviceArray(capi, host=cx)
+    dout = DeviceArray(capi, shape=(2, L, n))
+    capi.check(lib.he_moddown(h, L, dcx.ptr, dout.ptr, 2, 0, ws.ptr, None))
+    md = np.stack([p.moddown(cx[0]), p.moddown(cx[1])])
+    assert (dout.numpy() == md).all()
+    base = rand_limbs(p, rng, range(L), n_polys=2)
+    dcx, dacc = DeviceArray(capi, host=cx), DeviceArray(capi, host=base)
+    capi.check(lib.he_moddown(h, L, dcx.ptr, dacc.ptr, 2, 1, ws.ptr, None))
+    assert (dacc.numpy() == np.stack([p.add(base[b], md[b]) for b in range(2)])).all()
+
+
+@pytest.mark.parametrize("L,elt", [(6, 0), (5, 0), (6, 5), (3, 125)])
+def test_keyswitch(small, capi, L, elt):
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(20 + L)
+    lib, h = capi.lib(), ctx.he_handle()
+    c = rand_limbs(p, rng, range(L))
+    ct = rand_limbs(p, rng, range(L), n_polys=2)
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    words = lib.he_keyswitch_workspace_words(h, L)
+    beta = -(-L // p.size_p)
+    assert words == (beta + 2) * (L + p.size_p) * p.n + 2 * L * p.n
+    dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
+    ws = DeviceArray(capi, shape=(words,))
+    capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, elt, ws.ptr, None))
+    src = p.galois_ntt(c, elt) if elt else c
+    ks = p.key_switch(src, host_evk)
+    assert (dct.numpy() == np.stack([p.add(ct[b], ks[b]) for b in range(2)])).all()
+    assert (dc.numpy() == c).all()
+
+
+def test_keyswitch_benchmark_shape(full, capi):
+    """Key switch at N = 2^16, L = 24, K = 8, beta = 3 against the oracle."""
+    cahel, parms, ctx, p = full
+    rng = np.random.default_rng(30)
+    lib, h = capi.lib(), ctx.he_handle()
+    L = 24
+    c = rand_limbs(p, rng, range(L))
+    ct = rand_limbs(p, rng, range(L), n_polys=2)
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
+    ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, 0, ws.ptr, None))
+    ks = p.key_switch(c, host_evk)
+    assert (dct.numpy() == np.stack([p.add(ct[b], ks[b]) for b in range(2)])).all()
+
+
+def test_samplers(small, capi, oracle):
+    cahel, parms, ctx, p = small
+    lib, h = capi.lib(), ctx.he_handle()
+    key = oracle.chacha_key(77)
+    kp = key.ctypes.data_as(C.POINTER(C.c_uint32))
+    limbs = p.size_qp
+    out = DeviceArray(capi, shape=(limbs, p.n))
+    cdt = oracle.gauss_cdt()
+    dcdt = DeviceArray(capi, host=cdt)
+    for kind, fn in ((0, p.sample_ternary), (1, p.sample_error), (2, p.sample_uniform)):
+        capi.check(lib.he_sample(h, kind, kp, 5, out.ptr, limbs, 0, limbs, 0, None, 0, None))
+        assert (out.numpy() == fn(key, 5, limbs)).all(), kind
+    capi.check(lib.he_sample(h, 3, kp, 9, out.ptr, limbs, 0, limbs, 0, dcdt.ptr, len(cdt), None))
+    assert (out.numpy() == p.sample_gauss(key, 9, limbs, cdt)).all()
+    assert lib.he_sample(h, 3, kp, 9, out.ptr, limbs, 0, limbs, 0, None, 0, None) == -1
+
+
+def test_decompose_real(small, capi, oracle):
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(40)
+    coeffs = np.round(rng.uniform(-2.0 ** 62, 2.0 ** 62, p.n))
+    coeffs[:4] = [0.0, -0.0, 1.0, -1.0]
+    dco = DeviceArray(capi, host=coeffs)
+    out = DeviceArray(capi, shape=(p.size_q, p.n))
+    capi.check(capi.lib().he_decompose_real(ctx.he_handle(), dco.ptr, out.ptr, p.size_q, 0, None))
+    want = np.empty((p.size_q, p.n), dtype=np.uint64)
+    oracle.lib().orc_decompose_coeffs(C.byref(p.c), coeffs.ctypes.data_as(C.POINTER(C.c_double)),
+                                      want.ctypes.data_as(oracle.u64p), C.c_uint32(p.size_q))
+    assert (out.numpy() == want).all()
