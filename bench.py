@@ -1,0 +1,256 @@
+#!/usr/bin/env python3
+"""Benchmark of the CKKS hot path on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+One "step" is one homomorphic multiplication with relinearisation and rescale (tensor product -> hybrid key
+switch with dnum = 3 digits -> rescale) of two fresh ciphertexts at N = 2^16, L = 24 data limbs and 8 special
+limbs of 50 bits, scale 2^40, on buffers that are resident in HBM before the timed region starts; the step goes
+through the C-ABI of libcahel_hip.so exactly as the pyCAHEL evaluator drives it.  Prints ONE JSON line.
+
+Extra objects on the line:
+  roofline      the dominant kernel of the step (forward NTT, blocks pass, as launched by the key switch's
+                ModUp) timed alone with HIP events: algorithmic bytes = limbs * N * 8 read + written
+  ntt           config "batched forward + inverse NTT, 24 limbs x 2 polynomials": GB/s of limb data
+  rotate        one rotation with key switch; hoisted and plain rotate-and-sum over 15 steps
+  cpu_baseline  the CPU checker (oracle/, OpenMP) on the same HMult+relin+rescale workload, bounded sample
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+LOG_N, SIZE_Q, SIZE_P, BITS, SCALE = 16, 24, 8, 50, 2.0 ** 40
+HBM_PEAK_GBS = 8000.0
+
+
+def sync(capi):
+    capi.check(capi.lib().he_stream_synchronize(None), "sync")
+
+
+class Timer:
+    """HIP-event timer on the null stream (the stream every kernel here is launched on)."""
+
+    def __init__(self, capi):
+        self.capi, self.lib = capi, capi.lib()
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        capi.check(self.lib.he_event_create(C.byref(self.e0)))
+        capi.check(self.lib.he_event_create(C.byref(self.e1)))
+
+    def time(self, fn, iters, warmup=3):
+        for _ in range(warmup):
+            fn()
+        sync(self.capi)
+        self.capi.check(self.lib.he_event_record(self.e0, None))
+        for _ in range(iters):
+            fn()
+        self.capi.check(self.lib.he_event_record(self.e1, None))
+        self.capi.check(self.lib.he_event_synchronize(self.e1))
+        ms = C.c_float()
+        self.capi.check(self.lib.he_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
+        return ms.value / iters
+
+
+class Buf:
+    def __init__(self, capi, words):
+        self.capi = capi
+        p = C.c_void_p()
+        capi.check(capi.lib().he_malloc(C.byref(p), 8 * words), "he_malloc")
+        self.ptr, self.words = p.value, words
+
+    def at(self, word):
+        return self.ptr + 8 * word
+
+
+def cpu_baseline(seconds_budget=12.0):
+    """HMult + relinearise + rescale on the CPU checker at the benchmark's own shape (random residues)."""
+    from oracle import ckks_oracle as O
+    n = 1 << LOG_N
+    mods = O.coeff_modulus_create(n, [BITS] * (SIZE_Q + SIZE_P))
+    p = O.Params(LOG_N, mods, SIZE_P)
+    rng = np.random.default_rng(1)
+
+    def rnd(limbs, polys):
+        out = np.empty((polys, limbs, n), dtype=np.uint64)
+        for i in range(limbs):
+            out[:, i] = rng.integers(0, mods[i], size=(polys, n), dtype=np.uint64)
+        return out
+
+    a, b = rnd(SIZE_Q, 2), rnd(SIZE_Q, 2)
+    evk = [rnd(SIZE_Q + SIZE_P, 2) for _ in range(SIZE_Q // SIZE_P)]
+
+    def op():
+        return p.rescale(p.relinearize(p.tensor(a, b), evk))
+
+    op()
+    t0, iters = time.time(), 0
+    while True:
+        op()
+        iters += 1
+        if time.time() - t0 > seconds_budget or iters >= 200:
+            break
+    dt = (time.time() - t0) / iters
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    return {"value": 1.0 / dt, "unit": "HMult+relin+rescale ops/s", "cores": threads, "kind": "port",
+            "sample": "%d iterations of the same workload (N=2^16, L=24, K=8, dnum=3, random residues) on "
+                      "oracle/ckks_oracle.c with OpenMP" % iters,
+            "ms_per_op": dt * 1e3}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", choices=["all", "roofline"], default="all",
+                    help="roofline: run just the kernel the roofline object describes (for rocprofv3)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import lancelot_amd  # noqa: F401  (raises if the native libraries are missing)
+    import pyCAHEL as cahel
+    from lancelot_amd import capi
+    lib = capi.lib()
+
+    n = 1 << LOG_N
+    parms = cahel.params(cahel.scheme_type.ckks)
+    parms.set_poly_modulus_degree(n)
+    parms.set_coeff_modulus(cahel.coeff_modulus_create(n, [BITS] * (SIZE_Q + SIZE_P)))
+    parms.set_special_modulus_size(SIZE_P)
+    steps_pow2 = [1 << k for k in range(15)]
+    parms.set_galois_elts(cahel.get_elts_from_steps(steps_pow2, n))
+    ctx = cahel.context(parms, True, cahel.sec_level_type.tc128)
+    ctx.set_seed(2025)
+    if args.only == "roofline":
+        h, n_ = ctx.he_handle(), n
+        big = Buf(capi, 3 * (SIZE_Q + SIZE_P) * n_)
+        capi.check(lib.he_memset_zero(big.ptr, 8 * 3 * (SIZE_Q + SIZE_P) * n_, None))
+        ms = Timer(capi).time(lambda: capi.check(lib.he_ntt_forward(h, big.ptr, 3, SIZE_Q + SIZE_P, SIZE_Q, 0, SIZE_Q, 0,
+                                                                    None)), args.steps, args.warmup)
+        print(json.dumps({"kernel": "forward NTT, 72 limbs", "ms_per_launch": ms,
+                          "GBps": 72 * 8 * n_ * 2 / (ms * 1e-3) / 1e9}))
+        return
+    sk = cahel.secret_key(parms)
+    sk.gen_secretkey(ctx)
+    pk = cahel.public_key(ctx)
+    sk.gen_publickey(ctx, pk)
+    rlk = cahel.relin_key(ctx)
+    sk.gen_relinkey(ctx, rlk)
+    glk = cahel.galois_key(ctx)
+    sk.create_galois_keys(ctx, glk)
+    enc = cahel.ckks_encoder(ctx)
+    rng = np.random.default_rng(2025)
+    x, y = rng.uniform(-1, 1, n // 2), rng.uniform(-1, 1, n // 2)
+    ct1 = pk.encrypt_asymmetric(ctx, enc.encode(ctx, x, SCALE))
+    ct2 = pk.encrypt_asymmetric(ctx, enc.encode(ctx, y, SCALE))
+
+    h = ctx.he_handle()
+    L, K = SIZE_Q, SIZE_P
+    LK = L + K
+    limb_bytes = 8 * n
+    evk = capi.evk_array([rlk.digit_ptr(d) for d in range(rlk.digit_count())])
+    ws = Buf(capi, lib.he_keyswitch_workspace_words(h, L))
+    t3 = Buf(capi, 3 * L * n)
+    res = Buf(capi, 2 * (L - 1) * n)
+    rs_ws = Buf(capi, 2 * n)
+    a_ptr, b_ptr = ct1.data_ptr(), ct2.data_ptr()
+
+    def step():
+        capi.check(lib.he_tensor(h, a_ptr, b_ptr, t3.ptr, L, None))
+        capi.check(lib.he_keyswitch(h, L, t3.at(2 * L * n), evk, t3.ptr, 0, ws.ptr, None))
+        capi.check(lib.he_rescale(h, t3.ptr, res.ptr, 2, L, rs_ws.ptr, None))
+
+    for _ in range(args.warmup):
+        step()
+    sync(capi)
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    sync(capi)
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # the evaluator path must give the same limbs, and decrypt to x * y
+    prod = cahel.ciphertext(ctx)
+    cahel.multiply(ctx, ct1, ct2, prod)
+    cahel.relinearize_inplace(ctx, prod, rlk)
+    cahel.rescale_to_next_inplace(ctx, prod)
+    got = np.empty((2, L - 1, n), dtype=np.uint64)
+    capi.check(lib.he_memcpy_d2h(got.ctypes.data, res.ptr, got.nbytes, None))
+    same = bool((got == prod.to_numpy()).all())
+    dec = np.array(enc.decode(ctx, sk.decrypt(ctx, prod)))
+    max_err = float(np.max(np.abs(dec - x * y)))
+
+    timer = Timer(capi)
+    # dominant kernel: the forward NTT over the 72 converted limbs of ModUp (beta = 3 digits x 24 limbs); the same
+    # two kernels also run in ModDown and rescale.  Timed alone on a 72-limb buffer.
+    big = Buf(capi, 3 * LK * n)
+    capi.check(lib.he_memset_zero(big.ptr, 8 * 3 * LK * n, None))
+    fwd72 = timer.time(lambda: capi.check(lib.he_ntt_forward(h, big.ptr, 3, LK, L, 0, L, 0, None)), 50)
+    ntt_bytes = 72 * limb_bytes * 2          # each limb read once and written once
+    roof_gbs = ntt_bytes / (fwd72 * 1e-3) / 1e9
+
+    # config "NTT alone": 24 limbs x 2 polynomials, forward + inverse
+    two = Buf(capi, 2 * L * n)
+    capi.check(lib.he_memcpy_d2d(two.ptr, a_ptr, 8 * 2 * L * n, None))
+    f = timer.time(lambda: capi.check(lib.he_ntt_forward(h, two.ptr, 2, L, L, 0, L, 0, None)), 100)
+    i = timer.time(lambda: capi.check(lib.he_ntt_inverse(h, two.ptr, 2, L, L, 0, L, 0, None)), 100)
+    ntt = {"forward_ms": f, "inverse_ms": i, "bytes_fwd_plus_inv": 4 * 2 * L * limb_bytes,
+           "GBps": 4 * 2 * L * limb_bytes / ((f + i) * 1e-3) / 1e9}
+    ntt["frac_of_hbm_peak"] = ntt["GBps"] / HBM_PEAK_GBS
+
+    # rotations (config "rotate-and-sum"): one keyed rotation; 15 dependent rotations + adds; hoisted form
+    rot_in = ct1.copy()
+    rot_out = cahel.ciphertext(ctx)
+
+    def one_rot():
+        cahel.rotate_vector(ctx, rot_in, 1, glk, rot_out)
+
+    rot_ms = timer.time(one_rot, 20)
+
+    def rotate_and_sum():
+        acc = ct1.copy()
+        tmp = cahel.ciphertext(ctx)
+        for s in steps_pow2:
+            cahel.rotate_vector(ctx, acc, s, glk, tmp)
+            cahel.add_inplace(ctx, acc, tmp)
+        return acc
+
+    ras_ms = timer.time(rotate_and_sum, 5, warmup=1)
+    total = np.array(enc.decode(ctx, sk.decrypt(ctx, rotate_and_sum())))
+    rotate = {"one_rotation_ms": rot_ms, "rotate_and_sum_15_ms": ras_ms,
+              "one_rotation_GBps": 288 * limb_bytes / (rot_ms * 1e-3) / 1e9,
+              "rotate_and_sum_GBps": 15 * 432 * limb_bytes / (ras_ms * 1e-3) / 1e9,
+              "slot_sum_rel_err": float(np.max(np.abs(total - x.sum())) / abs(x.sum()))}
+
+    alg_bytes = 334 * limb_bytes
+    line = {
+        "metric": "HMult+relin+rescale ops/s at N=2^16, L=24 (dnum=3, 8 special primes)",
+        "value": 1e3 / ms_per_step, "unit": "ops/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u64", "data": "synthetic",
+        "config": {"workload": "HMult+relinearize+rescale, N=2^16, L=24 limbs of 50 bits, K=8, dnum=3, scale 2^40, "
+                               "two fresh ciphertexts of 32768 uniform[-1,1] slots (BASELINE.json configs[2])"},
+        "hmult_frac_of_hbm_roofline": alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "hmult_algorithmic_bytes": alg_bytes,
+        "check": {"c_abi_equals_evaluator": same, "decrypt_max_abs_err_vs_xy": max_err},
+        "roofline": {"bound": "hbm", "kernel": "ntt_rows_kernel + ntt_blocks_kernel (forward NTT, 72 limbs of ModUp)",
+                     "achieved": roof_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": roof_gbs / HBM_PEAK_GBS,
+                     "traffic": None, "ms_per_launch": fwd72, "algorithmic_bytes_per_launch": ntt_bytes},
+        "ntt": ntt, "rotate": rotate,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -53,6 +53,14 @@ int he_stream_create(he_stream *stream);
 int he_stream_destroy(he_stream stream);
 int he_stream_synchronize(he_stream stream);
 
+/* Events for timing work on a stream (the role of CUDATimer, include/util.cuh:66-157). */
+typedef void *he_event;
+int he_event_create(he_event *event);
+int he_event_destroy(he_event event);
+int he_event_record(he_event event, he_stream stream);
+int he_event_synchronize(he_event event);
+int he_event_elapsed_ms(he_event start, he_event stop, float *ms);
+
 /* ---- parameter tables ---- */
 
 /* Host-side description of one parameter set; replaces the uploads of CAHELGPUContext's constructor

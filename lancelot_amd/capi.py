@@ -28,6 +28,11 @@ SIGNATURES = {
     "he_stream_create": (C.c_int, [C.POINTER(vp)]),
     "he_stream_destroy": (C.c_int, [vp]),
     "he_stream_synchronize": (C.c_int, [vp]),
+    "he_event_create": (C.c_int, [C.POINTER(vp)]),
+    "he_event_destroy": (C.c_int, [vp]),
+    "he_event_record": (C.c_int, [vp, vp]),
+    "he_event_synchronize": (C.c_int, [vp]),
+    "he_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
     "he_context_create": (C.c_int, [vp, C.POINTER(vp)]),
     "he_context_set_level": (C.c_int, [vp, vp]),
     "he_context_destroy": (C.c_int, [vp]),

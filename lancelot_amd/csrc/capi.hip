@@ -173,6 +173,35 @@ int he_stream_synchronize(he_stream s) {
     return HE_OK;
 }
 
+int he_event_create(he_event *e) {
+    if (!e) return HE_E_INVALID_ARGUMENT;
+    hipEvent_t ev;
+    HE_HIP(hipEventCreate(&ev));
+    *e = ev;
+    return HE_OK;
+}
+
+int he_event_destroy(he_event e) {
+    if (e) HE_HIP(hipEventDestroy(static_cast<hipEvent_t>(e)));
+    return HE_OK;
+}
+
+int he_event_record(he_event e, he_stream s) {
+    HE_HIP(hipEventRecord(static_cast<hipEvent_t>(e), S(s)));
+    return HE_OK;
+}
+
+int he_event_synchronize(he_event e) {
+    HE_HIP(hipEventSynchronize(static_cast<hipEvent_t>(e)));
+    return HE_OK;
+}
+
+int he_event_elapsed_ms(he_event start, he_event stop, float *ms) {
+    if (!ms) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+    return HE_OK;
+}
+
 int he_context_create(const he_context_desc *d, he_context **out) {
     if (!d || !out || !d->moduli || !d->barrett || !d->psi || !d->ipsi_div2) return HE_E_INVALID_ARGUMENT;
     if (d->log_n < 9 || d->log_n > 16) return HE_E_UNSUPPORTED;
