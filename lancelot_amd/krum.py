@@ -1,0 +1,191 @@
+"""Encrypted Krum distance computation over pyCAHEL: the caller side of the hot path.
+
+Restates the protocol of lancelot-main-GPU/utils/byzantine_fl.py (GPU_init :432-462,
+GPU_compute_pair_distance :173-321, GPU_computing_distance_cipher :466-514, GPU_decrypt_sort_mask :327-369,
+GPU_krum :517-525) on top of the same pyCAHEL calls, with two differences that do not change the result:
+every client chunk is encoded and encrypted once (the reference re-encrypts both operands for every pair) and
+the i == j pairs, whose distance is zero, are not evaluated.
+
+Per pair (i, j): for every chunk  d = ct_j - ct_i ; d = d^2 (size 3) ; acc += d   ("lazy relinearisation"),
+then one relinearise + rescale, then rotate-and-sum so that every slot holds sum_k (u_i[k] - u_j[k])^2.
+The score of a client is the plain row sum of its distances (no nearest-neighbour truncation), as in
+byzantine_fl.py:344-353 and :531-533; the chosen client is the argmin.
+"""
+from __future__ import annotations
+
+import math
+import time
+from dataclasses import dataclass, field
+
+import numpy as np
+
+
+@dataclass
+class KrumConfig:
+    log_n: int = 16
+    modulus_bits: tuple = (60, 40, 40, 60)   # GPU_init: modulus_chain = [60, 40, 40, 60]
+    special_modulus_size: int = 1            # GPU_init: size_P = 1
+    scale: float = 2.0 ** 40
+    hoisting: bool = True                    # byzantine_fl.py: Hoisting_flag = 1
+    sec_level: str = "tc128"
+    seed: int | None = None
+
+
+@dataclass
+class KrumState:
+    cahel: object
+    config: KrumConfig
+    context: object
+    pk: object
+    sk: object
+    glk: object
+    rlk: object
+    encoder: object
+    slots: int
+    timings: dict = field(default_factory=lambda: {"encode": 0.0, "encrypt": 0.0, "evaluate": 0.0, "decrypt": 0.0})
+
+
+def _sync(cahel):
+    cahel._synchronize()
+
+
+def gpu_init(config: KrumConfig | None = None) -> KrumState:
+    """Context, keys and encoder (byzantine_fl.py:432-462)."""
+    import lancelot_amd  # noqa: F401
+    import pyCAHEL as cahel
+    config = config or KrumConfig()
+    n = 1 << config.log_n
+    log_slots = config.log_n - 1
+    if config.hoisting:
+        steps = list(range(1, 16)) + [2 ** i for i in range(4, log_slots)]
+    else:
+        steps = [2 ** i for i in range(0, log_slots)]
+    steps = [s for s in steps if s < n // 2]
+    params = cahel.params(cahel.scheme_type.ckks)
+    params.set_poly_modulus_degree(n)
+    params.set_coeff_modulus(cahel.coeff_modulus_create(n, list(config.modulus_bits)))
+    params.set_special_modulus_size(config.special_modulus_size)
+    params.set_galois_elts(cahel.get_elts_from_steps(steps, n))
+    context = cahel.context(params, True, getattr(cahel.sec_level_type, config.sec_level))
+    if config.seed is not None:
+        context.set_seed(config.seed)
+    sk = cahel.secret_key(params)
+    sk.gen_secretkey(context)
+    pk = cahel.public_key(context)
+    sk.gen_publickey(context, pk)
+    rlk = cahel.relin_key(context)
+    sk.gen_relinkey(context, rlk)
+    glk = cahel.galois_key(context)
+    sk.create_galois_keys(context, glk)
+    encoder = cahel.ckks_encoder(context)
+    return KrumState(cahel, config, context, pk, sk, glk, rlk, encoder, encoder.slot_count())
+
+
+def split_updates(vectors, slots: int):
+    """Zero-pad every flattened update to a multiple of `slots` and split it (byzantine_fl.py:474-490)."""
+    vectors = [np.asarray(v, dtype=np.float64).reshape(-1) for v in vectors]
+    length = len(vectors[0])
+    if any(len(v) != length for v in vectors):
+        raise ValueError("all client updates must have the same length")
+    whole = length if length % slots == 0 else (length // slots + 1) * slots
+    return [np.array_split(np.pad(v, (0, whole - length)), whole // slots) for v in vectors]
+
+
+def encrypt_updates(state: KrumState, chunks):
+    """One ciphertext per (client, chunk)."""
+    c, ctx = state.cahel, state.context
+    out = []
+    for client in chunks:
+        row = []
+        for chunk in client:
+            t0 = time.perf_counter()
+            pt = state.encoder.encode(ctx, chunk, state.config.scale)
+            t1 = time.perf_counter()
+            row.append(state.pk.encrypt_asymmetric(ctx, pt))
+            _sync(c)
+            t2 = time.perf_counter()
+            state.timings["encode"] += t1 - t0
+            state.timings["encrypt"] += t2 - t1
+        out.append(row)
+    return out
+
+
+def pair_distance(state: KrumState, cts_i, cts_j):
+    """Ciphertext whose every slot holds ||u_i - u_j||^2 (byzantine_fl.py:173-321)."""
+    c, ctx, cfg = state.cahel, state.context, state.config
+    acc = None
+    tmp = c.ciphertext(ctx)
+    for ct1, ct2 in zip(cts_i, cts_j):
+        c.sub(ctx, ct2, ct1, tmp)
+        c.square_inplace(ctx, tmp)
+        if acc is None:
+            acc = tmp
+            tmp = c.ciphertext(ctx)
+        else:
+            c.add_inplace(ctx, acc, tmp)
+    c.relinearize_inplace(ctx, acc, state.rlk)
+    c.rescale_to_next_inplace(ctx, acc)
+    acc.set_scale(cfg.scale)
+    log_slots = int(math.log2(state.slots))
+    rot = c.ciphertext(ctx)
+    if cfg.hoisting and log_slots > 4:
+        hoisted = c.hoisting(ctx, acc, state.glk, list(range(1, 16)))
+        c.add_inplace(ctx, acc, hoisted)
+        first = 4
+    else:
+        first = 0
+    for k in range(first, log_slots):
+        c.rotate_vector(ctx, acc, 2 ** k, state.glk, rot)
+        c.add_inplace(ctx, acc, rot)
+    return acc
+
+
+def distance_matrix(state: KrumState, updates):
+    """Encrypted pairwise squared distances and their decryptions (slot 0 of every pair)."""
+    c = state.cahel
+    chunks = split_updates(updates, state.slots)
+    cts = encrypt_updates(state, chunks)
+    n_clients = len(updates)
+    enc = [[None] * n_clients for _ in range(n_clients)]
+    t0 = time.perf_counter()
+    for i in range(n_clients):
+        for j in range(i + 1, n_clients):
+            enc[i][j] = enc[j][i] = pair_distance(state, cts[i], cts[j])
+    _sync(c)
+    state.timings["evaluate"] += time.perf_counter() - t0
+    t0 = time.perf_counter()
+    dist = np.zeros((n_clients, n_clients))
+    for i in range(n_clients):
+        for j in range(i + 1, n_clients):
+            value = state.encoder.decode(state.context, state.sk.decrypt(state.context, enc[i][j]))[0]
+            dist[i, j] = dist[j, i] = value
+    state.timings["decrypt"] += time.perf_counter() - t0
+    return dist, enc
+
+
+def plain_distance_matrix(updates):
+    """float64 closed form ||u_i - u_j||^2 (byzantine_fl.py:129-131, 162-171)."""
+    v = [np.asarray(u, dtype=np.float64).reshape(-1) for u in updates]
+    n = len(v)
+    d = np.zeros((n, n))
+    for i in range(n):
+        for j in range(i + 1, n):
+            d[i, j] = d[j, i] = float(np.sum((v[i] - v[j]) ** 2))
+    return d
+
+
+def krum_select(dist: np.ndarray) -> int:
+    """Row sums, argsort, first entry (byzantine_fl.py:531-533)."""
+    return int(np.argsort(dist.sum(axis=0), kind="stable")[0])
+
+
+def gpu_krum(updates, config: KrumConfig | None = None, state: KrumState | None = None):
+    """One encrypted Krum round: returns (chosen client index, distance matrix, timings in seconds)."""
+    state = state or gpu_init(config)
+    for k in state.timings:
+        state.timings[k] = 0.0
+    t0 = time.perf_counter()
+    dist, _ = distance_matrix(state, updates)
+    total = time.perf_counter() - t0
+    timings = dict(state.timings, total=total)
+    return krum_select(dist), dist, timings

@@ -1,0 +1,341 @@
+"""pyCAHEL-level parity on the GPU: keys, encryption, evaluator and decryption against the CPU oracle.
+
+Product and oracle draw the same seeded ChaCha20 streams in the same order, so every key and ciphertext limb
+must agree word for word (integer stages: bit-exact).  Decoded slots are compared with the oracle's decode
+to 2^-20 relative (encode/decode use FP64 transforms whose operation order differs), and with the plaintext
+truth to the scheme's own precision.
+"""
+import numpy as np
+import pytest
+
+from gpu_util import make_pair
+
+pytestmark = pytest.mark.gpu
+
+REL = 2.0 ** -20
+SEED = 2025
+
+
+def rel_err(a, b):
+    return float(np.max(np.abs(np.asarray(a) - np.asarray(b))) / max(1.0, float(np.max(np.abs(b)))))
+
+
+@pytest.fixture(scope="module")
+def world(oracle):
+    """N = 2^12, 6 Q limbs + 2 special (3 digits), Galois keys for steps 1, 2, 3, -1, 4 and conjugation."""
+    O = oracle
+    import lancelot_amd  # noqa: F401
+    import pyCAHEL as cahel
+    logn, n = 12, 4096
+    bits = [50, 40, 40, 40, 40, 40, 50, 50]
+    steps = [1, 2, 3, -1, 0, 4]
+    mods = cahel.coeff_modulus_create(n, bits)
+    parms = cahel.params(cahel.scheme_type.ckks)
+    parms.set_poly_modulus_degree(n)
+    parms.set_coeff_modulus(mods)
+    parms.set_special_modulus_size(2)
+    elts = cahel.get_elts_from_steps(steps, n)
+    parms.set_galois_elts(elts)
+    ctx = cahel.context(parms, True, cahel.sec_level_type.none)
+    ctx.set_seed(SEED)
+    p = O.Params(logn, [m.value() for m in mods], 2)
+    ks = O.KeySet(p, seed=SEED)
+    sk = cahel.secret_key(parms)
+    sk.gen_secretkey(ctx)
+    o_sk = ks.gen_secret()
+    pk = cahel.public_key(ctx)
+    sk.gen_publickey(ctx, pk)
+    o_pk = ks.gen_public()
+    rlk = cahel.relin_key(ctx)
+    sk.gen_relinkey(ctx, rlk)
+    o_rlk = ks.gen_relin()
+    glk = cahel.galois_key(ctx)
+    sk.create_galois_keys(ctx, glk)
+    o_glk = [ks.gen_galois(e) for e in elts]
+    enc = cahel.ckks_encoder(ctx)
+    return dict(cahel=cahel, parms=parms, ctx=ctx, p=p, ks=ks, sk=sk, o_sk=o_sk, pk=pk, o_pk=o_pk, rlk=rlk,
+                o_rlk=o_rlk, glk=glk, o_glk=o_glk, enc=enc, o_enc=O.Encoder(p), elts=elts, steps=steps, O=O)
+
+
+def test_keys_match_oracle(world):
+    w = world
+    assert (w["sk"].to_numpy(w["ctx"]) == w["o_sk"]).all()
+    assert (w["pk"].to_numpy() == w["o_pk"]).all()
+    assert w["rlk"].digit_count() == 3
+    for d in range(3):
+        assert (w["rlk"].digit_to_numpy(d) == w["o_rlk"][d]).all()
+    assert w["glk"].key_count() == len(w["elts"])
+    for i in range(len(w["elts"])):
+        for d in range(3):
+            assert (w["glk"].key(i).digit_to_numpy(d) == w["o_glk"][i][d]).all()
+
+
+def _encrypt_both(w, values, scale=2.0 ** 40):
+    pt = w["enc"].encode(w["ctx"], values, scale)
+    o_pt = w["o_enc"].encode(values, scale, w["p"].size_q)
+    ct = w["pk"].encrypt_asymmetric(w["ctx"], pt)
+    o_ct = w["ks"].encrypt_asymmetric(w["o_pk"], pt.to_numpy())   # same plaintext limbs on both sides
+    return pt, o_pt, ct, o_ct
+
+
+def _encrypt_product_only(w, values, scale=2.0 ** 40):
+    """Encrypts on the GPU only and advances the oracle's stream counter by the three streams it used."""
+    ct = w["pk"].encrypt_asymmetric(w["ctx"], w["enc"].encode(w["ctx"], values, scale))
+    w["ks"].stream += 3
+    return ct
+
+
+def test_encode_matches_oracle(world):
+    w = world
+    rng = np.random.default_rng(1)
+    z = rng.uniform(-1, 1, w["p"].n // 2)
+    pt = w["enc"].encode(w["ctx"], z, 2.0 ** 40)
+    o_pt = w["o_enc"].encode(z, 2.0 ** 40, w["p"].size_q)
+    # rounding of the FP64 transform may differ by one unit in a coefficient; compare decoded values
+    got = np.array(w["enc"].decode(w["ctx"], pt))
+    assert rel_err(got, w["o_enc"].decode(o_pt, 2.0 ** 40).real) < REL
+    assert rel_err(got, z) < REL
+    coeff_diff = w["p"].ntt_inv(pt.to_numpy().copy())[0].astype(np.int64) - w["p"].ntt_inv(o_pt.copy())[0].astype(np.int64)
+    assert np.max(np.abs(coeff_diff)) <= 1
+
+
+def test_encrypt_multiply_relin_rescale_bit_exact(world):
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    rng = np.random.default_rng(2)
+    x, y = rng.uniform(-1, 1, p.n // 2), rng.uniform(-1, 1, p.n // 2)
+    _, _, cx, o_cx = _encrypt_both(w, x)
+    _, _, cy, o_cy = _encrypt_both(w, y)
+    assert (cx.to_numpy() == o_cx).all() and (cy.to_numpy() == o_cy).all()
+    prod = c.ciphertext(ctx)
+    c.multiply(ctx, cx, cy, prod)
+    o_t = p.tensor(o_cx, o_cy)
+    assert prod.size() == 3 and (prod.to_numpy() == o_t).all()
+    c.relinearize_inplace(ctx, prod, w["rlk"])
+    o_r = p.relinearize(o_t, w["o_rlk"])
+    assert prod.size() == 2 and (prod.to_numpy() == o_r).all()
+    c.rescale_to_next_inplace(ctx, prod)
+    o_s = p.rescale(o_r)
+    assert prod.chain_index() == 2 and (prod.to_numpy() == o_s).all()
+    assert prod.scale() == (2.0 ** 80) / p.moduli[p.size_q - 1]
+    # decrypt (with the seeded flooding noise) and decode
+    pt = w["sk"].decrypt(ctx, prod)
+    o_pt = w["ks"].decrypt(o_s, w["O"].gauss_cdt())
+    assert (pt.to_numpy() == o_pt).all()
+    got = np.array(w["enc"].decode(ctx, pt))
+    want = w["o_enc"].decode(o_pt, prod.scale()).real
+    assert rel_err(got, want) < REL
+    assert np.max(np.abs(got - x * y)) < 1e-5          # cahel-main/unittest/evaluator.cu:419-472 bound
+    # square, multiply_and_relin_inplace
+    sq = c.ciphertext(ctx)
+    c.square(ctx, cx, sq)
+    assert (sq.to_numpy() == p.square(o_cx)).all()
+    c.multiply_and_relin_inplace(ctx, cx, cy, w["rlk"])
+    assert (cx.to_numpy() == o_r).all()
+
+
+def test_add_sub_negate_plain_ops(world):
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    rng = np.random.default_rng(3)
+    x, y = rng.uniform(-1, 1, p.n // 2), rng.uniform(-1, 1, p.n // 2)
+    pt_x, _, cx, o_cx = _encrypt_both(w, x)
+    pt_y, _, cy, o_cy = _encrypt_both(w, y)
+    out = c.ciphertext(ctx)
+    both = lambda f: np.stack([f(o_cx[i], o_cy[i]) for i in range(2)])
+    c.add(ctx, cx, cy, out)
+    assert (out.to_numpy() == both(p.add)).all()
+    c.sub(ctx, cx, cy, out)
+    assert (out.to_numpy() == both(p.sub)).all()
+    # sub with destination aliasing the second operand (include/evaluate.h:52-61)
+    alias = cy.copy()
+    c.sub(ctx, cx, alias, alias)
+    assert (alias.to_numpy() == both(p.sub)).all()
+    c.negate(ctx, cx, out)
+    assert (out.to_numpy() == np.stack([p.negate(o_cx[i]) for i in range(2)])).all()
+    c.add_many(ctx, [cx, cy, cx], out)
+    assert (out.to_numpy() == np.stack([p.add(p.add(o_cx[i], o_cy[i]), o_cx[i]) for i in range(2)])).all()
+    c.add_plain(ctx, cx, pt_y, out)
+    assert (out.to_numpy() == np.stack([p.add(o_cx[0], pt_y.to_numpy()), o_cx[1]])).all()
+    c.sub_plain(ctx, cx, pt_y, out)
+    assert (out.to_numpy() == np.stack([p.sub(o_cx[0], pt_y.to_numpy()), o_cx[1]])).all()
+    c.multiply_plain(ctx, cx, pt_y, out)
+    assert (out.to_numpy() == np.stack([p.mul(o_cx[i], pt_y.to_numpy()) for i in range(2)])).all()
+    assert out.scale() == 2.0 ** 80
+    # size-3 accumulation used by the lazy relinearisation of the Krum protocol
+    s1, s2 = c.ciphertext(ctx), c.ciphertext(ctx)
+    c.square(ctx, cx, s1)
+    c.square(ctx, cy, s2)
+    c.add_inplace(ctx, s1, s2)
+    o3 = np.stack([p.add(p.square(o_cx)[i], p.square(o_cy)[i]) for i in range(3)])
+    assert (s1.to_numpy() == o3).all()
+
+
+@pytest.mark.parametrize("step", [1, 3, -1])
+def test_rotate_bit_exact(world, step):
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    rng = np.random.default_rng(4)
+    z = rng.uniform(-1, 1, p.n // 2)
+    _, _, ct, o_ct = _encrypt_both(w, z)
+    out = c.ciphertext(ctx)
+    c.rotate_vector(ctx, ct, step, w["glk"], out)
+    idx = w["steps"].index(step)
+    o_out = p.apply_galois(o_ct, w["elts"][idx], w["o_glk"][idx])
+    assert (out.to_numpy() == o_out).all()
+    w["sk"].set_noise_flooding(False)
+    got = np.array(w["enc"].decode(ctx, w["sk"].decrypt(ctx, out)))
+    w["sk"].set_noise_flooding(True)
+    assert np.max(np.abs(got - np.roll(z, -step))) < 1e-6
+
+
+def test_rotate_after_rescale_and_conjugate(world):
+    """Key switching at a lower level (L = 5: digits of 2, 2 and 1 limbs) and the conjugation key."""
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    rng = np.random.default_rng(5)
+    z = rng.uniform(-1, 1, p.n // 2)
+    _, _, ct, o_ct = _encrypt_both(w, z)
+    c.mod_switch_to_next_inplace(ctx, ct)
+    o_ct = np.ascontiguousarray(o_ct[:, :5])
+    assert ct.chain_index() == 2 and (ct.to_numpy() == o_ct).all()
+    c.rotate_vector_inplace(ctx, ct, 2, w["glk"])
+    idx = w["steps"].index(2)
+    assert (ct.to_numpy() == p.apply_galois(o_ct, w["elts"][idx], w["o_glk"][idx])).all()
+    conj = c.ciphertext(ctx)
+    c.complex_conjugate(ctx, ct, w["glk"], conj)
+    ci = w["steps"].index(0)
+    assert (conj.to_numpy() == p.apply_galois(ct.to_numpy(), w["elts"][ci], w["o_glk"][ci])).all()
+
+
+def test_rotate_naf_fallback(world):
+    """No key for step 5: the rotation is split into the signed powers of two 1 + 4 (src/evaluate.cu:2395-2408)."""
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    assert c._naf(5) == [1, 4] and c._naf(-3) == [1, -4] and c._naf(127) == [-1, 128] and c._naf(0) == []
+    rng = np.random.default_rng(8)
+    z = rng.uniform(-1, 1, p.n // 2)
+    _, _, ct, o_ct = _encrypt_both(w, z)
+    out = c.ciphertext(ctx)
+    c.rotate_vector(ctx, ct, 5, w["glk"], out)
+    for s in (1, 4):
+        i = w["steps"].index(s)
+        o_ct = p.apply_galois(o_ct, w["elts"][i], w["o_glk"][i])
+    assert (out.to_numpy() == o_ct).all()
+
+
+def test_rotate_missing_power_of_two_raises(world):
+    w = world
+    c, ctx = w["cahel"], w["ctx"]
+    ct = _encrypt_product_only(w, np.zeros(w["p"].n // 2))
+    with pytest.raises(ValueError, match="Galois key not present"):
+        c.rotate_vector_inplace(ctx, ct, 64, w["glk"])
+
+
+def test_hoisting_bit_exact(world):
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    rng = np.random.default_rng(6)
+    z = rng.uniform(-1, 1, p.n // 2)
+    _, _, ct, o_ct = _encrypt_both(w, z)
+    assert (ct.to_numpy() == o_ct).all()
+    steps = [1, 2, 3]
+    out = c.hoisting(ctx, ct, w["glk"], steps)
+    idxs = [w["steps"].index(s) for s in steps]
+    o_out = p.hoisting(o_ct, [w["elts"][i] for i in idxs], [w["o_glk"][i] for i in idxs])
+    assert (out.to_numpy() == o_out).all()
+    w["sk"].set_noise_flooding(False)
+    got = np.array(w["enc"].decode(ctx, w["sk"].decrypt(ctx, out)))
+    w["sk"].set_noise_flooding(True)
+    assert np.max(np.abs(got - sum(np.roll(z, -s) for s in steps))) < 1e-6
+    with pytest.raises(RuntimeError, match="Galois key not present in hoisting"):
+        c.hoisting(ctx, ct, w["glk"], [7])
+
+
+def test_error_behaviour(world):
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    z = np.ones(p.n // 2)
+    a = _encrypt_product_only(w, z)
+    b = _encrypt_product_only(w, z, 2.0 ** 30)
+    with pytest.raises(ValueError, match="scale mismatch"):
+        c.add_inplace(ctx, a, b)
+    with pytest.raises(ValueError, match="destination_size must be 3"):
+        c.relinearize_inplace(ctx, a, w["rlk"])
+    lower = a.copy()
+    c.mod_switch_to_inplace(ctx, lower, 3)
+    assert lower.chain_index() == 3 and lower.coeff_modulus_size() == 4
+    with pytest.raises(ValueError, match="parameter mismatch"):
+        c.add_inplace(ctx, a, lower)
+    with pytest.raises(ValueError, match="cannot switch to higher level modulus"):
+        c.mod_switch_to_inplace(ctx, lower, 1)
+    with pytest.raises(RuntimeError, match="unsupported scheme"):
+        c.rotate_rows_inplace(ctx, a, 1, w["glk"])
+    with pytest.raises(RuntimeError, match="unsupported scheme"):
+        c.multiply_many(ctx, [a, a], w["rlk"], a)
+    last = a.copy()
+    c.mod_switch_to_inplace(ctx, last, 6)
+    with pytest.raises(ValueError, match="end of modulus switching chain reached"):
+        c.rescale_to_next_inplace(ctx, last)
+    sq = a.copy()
+    c.square_inplace(ctx, sq)
+    with pytest.raises(ValueError, match="ciphertext size must be 2"):
+        c.hoisting(ctx, sq, w["glk"], [1])
+    with pytest.raises(ValueError, match="values_size is too large"):
+        w["enc"].encode(ctx, np.zeros(p.n), 2.0 ** 40)
+
+
+def test_lancelot_smoke_script_flow(oracle):
+    """The sequence of lancelot-main-GPU/ckks.py:1-57 with its parameters, checked against the closed form."""
+    import lancelot_amd  # noqa: F401
+    import pyCAHEL as cahel
+    n = 2 ** 13
+    scale = 2.0 ** 40
+    params = cahel.params(cahel.scheme_type.ckks)
+    params.set_poly_modulus_degree(n)
+    params.set_coeff_modulus(cahel.coeff_modulus_create(n, [60, 40, 40, 60]))
+    params.set_special_modulus_size(1)
+    params.set_galois_elts(cahel.get_elts_from_steps([-2], n))
+    context = cahel.context(params, True, cahel.sec_level_type.tc128)
+    sk = cahel.secret_key(params)
+    sk.gen_secretkey(context)
+    pk = cahel.public_key(context)
+    sk.gen_publickey(context, pk)
+    rlk = cahel.relin_key(context)
+    sk.gen_relinkey(context, rlk)
+    glk = cahel.galois_key(context)
+    sk.create_galois_keys(context, glk)
+    encoder = cahel.ckks_encoder(context)
+    slot_count = encoder.slot_count()
+    msg = [1.0, 2.0, 3.0, 4.0] + [0.0] * (slot_count - 4)
+    ct = pk.encrypt_asymmetric(context, encoder.encode(context, msg, scale))
+    cahel.square_inplace(context, ct)
+    cahel.relinearize_inplace(context, ct, rlk)
+    cahel.rescale_to_next_inplace(context, ct)
+    pt_2 = encoder.encode_to(context, [2.0] * slot_count, 2, scale)
+    ct.set_scale(scale)
+    cahel.multiply_plain_inplace(context, ct, pt_2)
+    cahel.rescale_to_next_inplace(context, ct)
+    cahel.add_inplace(context, ct, ct)
+    cahel.rotate_vector_inplace(context, ct, -2, glk)
+    result = encoder.decode(context, sk.decrypt(context, ct))
+    want = np.roll(4.0 * np.array(msg) ** 2, 2)
+    assert np.max(np.abs(np.array(result) - want)) < 1e-3
+    assert ["%.1f" % abs(v) for v in result[:6]] == ["0.0", "0.0", "4.0", "16.0", "36.0", "64.0"]
+
+
+def test_encrypted_krum_small(oracle):
+    """Encrypted Krum distances on 4 clients x 5000 parameters (2 chunks at N = 2^13) against float64."""
+    from lancelot_amd import krum
+    rng = np.random.default_rng(7)
+    updates = [rng.normal(0, 0.01, 5000).astype(np.float32) for _ in range(4)]
+    updates[3] = updates[3] * 10
+    cfg = krum.KrumConfig(log_n=13, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=11)
+    chosen, dist, timings = krum.gpu_krum(updates, cfg)
+    want = krum.plain_distance_matrix(updates)
+    assert rel_err(dist, want) < 1e-3
+    assert chosen == krum.krum_select(want) and chosen != 3
+    plain = krum.KrumConfig(log_n=13, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=11, hoisting=False)
+    chosen2, dist2, _ = krum.gpu_krum(updates, plain)
+    assert chosen2 == chosen and rel_err(dist2, want) < 1e-3
+    assert set(timings) == {"encode", "encrypt", "evaluate", "decrypt", "total"}

@@ -1,0 +1,123 @@
+"""CPU-only checks of the product: the C-ABI library loads and exports every declared symbol, and the host
+number theory agrees with the reference's known answers and with the oracle.  No GPU calls."""
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def cahel():
+    import lancelot_amd  # noqa: F401
+    import pyCAHEL
+    return pyCAHEL
+
+
+def test_library_exports_every_declared_symbol():
+    from lancelot_amd import capi
+    header = open(os.path.join(ROOT, "include", "cahel_hip.h")).read()
+    declared = set(re.findall(r"\b(he_[a-z0-9_]+)\s*\(", header))
+    declared -= {"he_context", "he_stream", "he_event"}
+    assert len(declared) >= 35
+    lib = capi.lib()
+    for name in sorted(declared):
+        assert hasattr(lib, name), name
+    assert declared == set(capi.SIGNATURES), declared ^ set(capi.SIGNATURES)
+    assert lib.he_error_string(0) == b"success" and lib.he_error_string(-3).startswith(b"tables of this level")
+
+
+def test_pycahel_exports_the_reference_names(cahel):
+    # cahel-main/python/src/binding.cu:8-156
+    names = """scheme_type mul_tech_type sec_level_type modulus coeff_modulus_create params context secret_key
+    public_key relin_key galois_key get_elts_from_steps ckks_encoder plaintext ciphertext negate negate_inplace add
+    add_inplace add_plain add_plain_inplace add_many sub sub_inplace sub_plain sub_plain_inplace multiply
+    multiply_inplace multiply_and_relin_inplace multiply_plain multiply_plain_inplace multiply_many square
+    square_inplace exponentiate exponentiate_inplace relinearize relinearize_inplace mod_switch_to
+    mod_switch_to_inplace mod_switch_to_next mod_switch_to_next_inplace rescale_to_next rescale_to_next_inplace
+    apply_galois apply_galois_inplace rotate_rows rotate_rows_inplace rotate_columns rotate_columns_inplace
+    rotate_vector rotate_vector_inplace hoisting hoisting_inplace complex_conjugate complex_conjugate_inplace""".split()
+    for name in names:
+        assert hasattr(cahel, name), name
+    for cls, methods in {"params": ["set_mul_tech", "set_poly_modulus_degree", "set_special_modulus_size",
+                                    "set_galois_elts", "set_coeff_modulus"],
+                         "secret_key": ["gen_secretkey", "gen_publickey", "gen_relinkey", "create_galois_keys",
+                                        "encrypt_symmetric", "decrypt"],
+                         "public_key": ["encrypt_asymmetric"],
+                         "ckks_encoder": ["slot_count", "encode", "encode_to", "decode"],
+                         "ciphertext": ["set_scale"]}.items():
+        for m in methods:
+            assert hasattr(getattr(cahel, cls), m), (cls, m)
+    assert cahel.scheme_type.ckks != cahel.scheme_type.bfv and int(cahel.sec_level_type.tc128) == 128
+
+
+def test_host_number_theory_known_answers(cahel, oracle):
+    # cahel-main/unittest/util/numth.cu:197-216, :112-150; src/util/globals.cu:77-101
+    assert cahel._minimal_primitive_root(2, 11) == 10 and cahel._minimal_primitive_root(4, 29) == 12
+    assert cahel._minimal_primitive_root(8, 1234565441) == 249725733
+    assert cahel._get_primes(16384, 48, 3) == [0xfffffffd8001, 0xfffffffa0001, 0xfffffff00001]
+    assert cahel._get_primes(8192, 44, 3) == [0xfffffffc001, 0xffffff6c001, 0xfffffebc001]
+    for v in (0, 1, -1, 2, -2, 3, -3, 127, -127, 123, -123):
+        parts = cahel._naf(v)
+        assert sum(parts) == v
+        assert len(parts) == {0: 0, 1: 1, 2: 1, 3: 2, 127: 2}.get(abs(v), len(parts))
+    for n, bits in ((8192, [60, 40, 40, 60]), (65536, [50] * 32), (4096, [30, 30, 36])):
+        assert [m.value() for m in cahel.coeff_modulus_create(n, bits)] == oracle.coeff_modulus_create(n, bits)
+    for q in oracle.get_primes(65536, 50, 3):
+        assert cahel._minimal_primitive_root(131072, q) == oracle.minimal_primitive_root(131072, q)
+
+
+def test_galois_elements(cahel, oracle):
+    n = 65536
+    steps = [0, 1, 2, 15, -1, -7, 16384]
+    assert cahel.get_elts_from_steps(steps, n) == [oracle.galois_elt_from_step(s, n) for s in steps]
+    with pytest.raises(ValueError, match="step count too large"):
+        cahel.get_elts_from_steps([n // 2], n)
+
+
+def test_parameter_errors(cahel):
+    with pytest.raises(ValueError):
+        cahel.modulus(1)
+    with pytest.raises(ValueError):
+        cahel.modulus(1 << 61)
+    with pytest.raises(ValueError, match="bit_sizes is invalid"):
+        cahel.coeff_modulus_create(8192, [61])
+    with pytest.raises(ValueError, match="poly_modulus_degree is invalid"):
+        cahel.coeff_modulus_create(1000, [40])
+    p = cahel.params(cahel.scheme_type.ckks)
+    with pytest.raises(ValueError, match="only supported for BFV"):
+        p.set_mul_tech(cahel.mul_tech_type.hps)
+    none = cahel.params(cahel.scheme_type.none)
+    with pytest.raises(RuntimeError):
+        none.set_poly_modulus_degree(4096)
+    # parameter validation happens before any device work
+    p.set_poly_modulus_degree(8192)
+    p.set_coeff_modulus(cahel.coeff_modulus_create(8192, [60, 60, 60, 60]))
+    with pytest.raises(ValueError, match="insecure"):
+        cahel.context(p, True, cahel.sec_level_type.tc128)
+    p.set_coeff_modulus(cahel.coeff_modulus_create(8192, [40, 40, 40, 40, 40]))
+    p.set_special_modulus_size(2)
+    with pytest.raises(ValueError, match="multiple of the special modulus size"):
+        cahel.context(p, True, cahel.sec_level_type.none)
+    bfv = cahel.params(cahel.scheme_type.bfv)
+    bfv.set_poly_modulus_degree(8192)
+    bfv.set_coeff_modulus(cahel.coeff_modulus_create(8192, [40, 40]))
+    with pytest.raises(ValueError, match="implements CKKS"):
+        cahel.context(bfv, True, cahel.sec_level_type.none)
+
+
+def test_krum_host_logic():
+    import numpy as np
+    from lancelot_amd import krum
+    rng = np.random.default_rng(0)
+    ups = [rng.normal(0, 0.01, 1000) for _ in range(5)]
+    ups[4] = ups[4] * 10
+    chunks = krum.split_updates(ups, 256)
+    assert len(chunks) == 5 and len(chunks[0]) == 4 and all(len(c) == 256 for c in chunks[0])
+    assert np.allclose(np.concatenate(chunks[2])[:1000], ups[2]) and not np.concatenate(chunks[2])[1000:].any()
+    d = krum.plain_distance_matrix(ups)
+    assert d.shape == (5, 5) and np.allclose(d, d.T) and abs(d[0, 1] - np.sum((ups[0] - ups[1]) ** 2)) < 1e-12
+    assert krum.krum_select(d) != 4
+    with pytest.raises(ValueError):
+        krum.split_updates([np.zeros(3), np.zeros(4)], 2)
