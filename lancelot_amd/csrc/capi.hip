@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -40,6 +41,9 @@ struct he_context {
     uint64_t *d_moduli = nullptr, *d_barrett = nullptr, *d_psi = nullptr, *d_ipsi = nullptr;
     uint64_t *d_p_mod_q = nullptr, *d_pinv_mod_q = nullptr, *d_phat_inv = nullptr, *d_phat_mod_q = nullptr;
     uint32_t *d_iota = nullptr;  // 0, 1, 2, ...: row -> limb/table map of the P -> Ql conversion
+    double *d_psi_fp = nullptr, *d_ipsi_fp = nullptr, *d_fp_consts = nullptr;  // FP64 back end tables
+    std::vector<uint8_t> fp_ok;  // per table: prime below 2^50
+    bool use_fp = true;          // environment CAHEL_HIP_NO_FP64=1 forces the integer back end
     std::vector<Level> levels;   // indexed by L
     std::vector<void *> owned;
 
@@ -82,10 +86,27 @@ NttArgs base_args(const he_context *ctx, bool forward) {
     NttArgs a;
     memset(&a, 0, sizeof(a));
     a.tw = forward ? ctx->d_psi : ctx->d_ipsi;
+    a.tw_fp = forward ? ctx->d_psi_fp : ctx->d_ipsi_fp;
+    a.fp_consts = ctx->d_fp_consts;
     a.moduli = ctx->d_moduli;
     a.barrett = ctx->d_barrett;
     a.log_n = ctx->log_n;
     return a;
+}
+
+// the FP64 back end applies when every table of the launch has a prime below 2^50
+bool fp_for(const he_context *ctx, const LimbMap &m) {
+    if (!ctx->use_fp) return false;
+    for (uint32_t i = 0; i < m.limbs; i++)
+        if (!ctx->fp_ok[map_table(m, i)]) return false;
+    return true;
+}
+
+bool fp_for_level(const he_context *ctx, uint32_t L) {
+    if (!ctx->use_fp) return false;
+    for (uint32_t t = 0; t < L + ctx->size_p; t++)
+        if (!ctx->fp_ok[table_of(ctx, L, t)]) return false;
+    return true;
 }
 
 int check_map(const he_context *ctx, uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail) {
@@ -229,6 +250,36 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         if (!rc) rc = upload(ctx, &ctx->d_phat_mod_q, d->phat_mod_q, (size_t)d->size_q * d->size_p);
     }
     if (!rc) {
+        // FP64 back end: (w, w/q) twiddles, un-halved inverse twiddles, per-table constants
+        const char *env = getenv("CAHEL_HIP_NO_FP64");
+        ctx->use_fp = !(env && env[0] == '1');
+        ctx->fp_ok.assign(qp, 0);
+        std::vector<double> psi_fp(2 * qp * n, 0.0), ipsi_fp(2 * qp * n, 0.0), consts(4 * qp, 0.0);
+        for (size_t t = 0; t < qp; t++) {
+            const uint64_t q = d->moduli[t];
+            if (q >> 50) continue;
+            ctx->fp_ok[t] = 1;
+            const double qd = (double)q;
+            for (size_t i = 0; i < n; i++) {
+                const uint64_t w = d->psi[2 * (t * n + i)];
+                uint64_t iw = 2 * d->ipsi_div2[2 * (t * n + i)];
+                if (iw >= q) iw -= q;
+                psi_fp[2 * (t * n + i)] = (double)w;
+                psi_fp[2 * (t * n + i) + 1] = (double)w / qd;
+                ipsi_fp[2 * (t * n + i)] = (double)iw;
+                ipsi_fp[2 * (t * n + i) + 1] = (double)iw / qd;
+            }
+            const uint64_t ninv = q - (q - 1) / n;  // q = 1 mod 2N, so N * (q - (q-1)/N) = 1 mod q
+            consts[4 * t] = qd;
+            consts[4 * t + 1] = 1.0 / qd;
+            consts[4 * t + 2] = (double)ninv;
+            consts[4 * t + 3] = (double)ninv / qd;
+        }
+        rc = upload(ctx, &ctx->d_psi_fp, psi_fp.data(), psi_fp.size());
+        if (!rc) rc = upload(ctx, &ctx->d_ipsi_fp, ipsi_fp.data(), ipsi_fp.size());
+        if (!rc) rc = upload(ctx, &ctx->d_fp_consts, consts.data(), consts.size());
+    }
+    if (!rc) {
         std::vector<uint32_t> iota(qp);
         for (uint32_t i = 0; i < qp; i++) iota[i] = i;
         rc = upload(ctx, &ctx->d_iota, iota.data(), qp);
@@ -306,7 +357,7 @@ int he_ntt_forward(const he_context *ctx, uint64_t *data, uint32_t n_polys, uint
     a.out = data;
     a.in_poly_stride = a.out_poly_stride = poly_stride;
     a.map = LimbMap{limbs, first, split, tail};
-    HE_HIP(launch_ntt_forward(a, n_polys, S(s)));
+    HE_HIP(launch_ntt_forward(a, n_polys, fp_for(ctx, a.map), S(s)));
     return HE_OK;
 }
 
@@ -319,7 +370,7 @@ int he_ntt_inverse(const he_context *ctx, uint64_t *data, uint32_t n_polys, uint
     a.out = data;
     a.in_poly_stride = a.out_poly_stride = poly_stride;
     a.map = LimbMap{limbs, first, split, tail};
-    HE_HIP(launch_ntt_inverse(a, n_polys, S(s)));
+    HE_HIP(launch_ntt_inverse(a, n_polys, fp_for(ctx, a.map), S(s)));
     return HE_OK;
 }
 
@@ -397,7 +448,7 @@ int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_
     inv.out = ws;
     inv.out_poly_stride = 1;
     inv.map = plain_map(1, L - 1);
-    HE_HIP(launch_ntt_inverse(inv, n_polys, S(s)));
+    HE_HIP(launch_ntt_inverse(inv, n_polys, fp_for(ctx, inv.map), S(s)));
     // every remaining limb: NTT_j(ws mod q_j), then (in_j - that) / q_last
     NttArgs fwd = base_args(ctx, true);
     fwd.pro_mode = NTT_PRO_BROADCAST_REDUCE;
@@ -412,7 +463,8 @@ int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_
     fwd.w = lv->d_qlast_inv;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L - 1;
-    HE_HIP(launch_ntt_forward(fwd, n_polys, S(s)));
+    // the broadcast source is a residue of q_{L-1}: the FP64 back end needs it below 2^50 as well
+    HE_HIP(launch_ntt_forward(fwd, n_polys, fp_for(ctx, plain_map(L, 0)), S(s)));
     return HE_OK;
 }
 
@@ -430,7 +482,7 @@ int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out
     inv.map = plain_map(L, 0);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_part_hat_inv;
-    HE_HIP(launch_ntt_inverse(inv, 1, S(s)));
+    HE_HIP(launch_ntt_inverse(inv, 1, fp_for(ctx, inv.map), S(s)));
     for (uint32_t d = 0; d < lv->beta; d++) {
         const Digit &g = lv->digits[d];
         uint64_t *od = out + (size_t)d * LK * n;
@@ -445,7 +497,7 @@ int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out
     fwd.out = out;
     fwd.jobs = lv->d_modup_jobs;
     fwd.n_jobs = lv->n_modup_jobs;
-    HE_HIP(launch_ntt_forward(fwd, 1, S(s)));
+    HE_HIP(launch_ntt_forward(fwd, 1, fp_for_level(ctx, L), S(s)));
     return HE_OK;
 }
 
@@ -479,7 +531,7 @@ int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, u
     inv.map = plain_map(K, ctx->size_q);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = ctx->d_phat_inv;
-    HE_HIP(launch_ntt_inverse(inv, n_polys, S(s)));
+    HE_HIP(launch_ntt_inverse(inv, n_polys, fp_for(ctx, inv.map), S(s)));
     for (uint32_t p = 0; p < n_polys; p++) {
         BconvArgs b{cx + ((size_t)p * LK + L) * n, ws + (size_t)p * L * n, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, K, L};
         HE_HIP(launch_bconv(ctx->tables(), b, S(s)));
@@ -497,7 +549,7 @@ int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, u
     fwd.w = ctx->d_pinv_mod_q;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L;
-    HE_HIP(launch_ntt_forward(fwd, n_polys, S(s)));
+    HE_HIP(launch_ntt_forward(fwd, n_polys, fp_for(ctx, fwd.map), S(s)));
     return HE_OK;
 }
 

@@ -48,6 +48,8 @@ struct NttArgs {
     uint32_t in_poly_stride;
     uint32_t out_poly_stride;
     const uint64_t *tw;       // [tables][N][2] (operand, Shoup quotient)
+    const double *tw_fp;      // [tables][N][2] (w, w/q) for the FP64 back end (primes below 2^50)
+    const double *fp_consts;  // [tables][4]: q, 1/q, N^-1 mod q, (N^-1 mod q)/q
     const uint64_t *moduli;   // [tables]
     const uint64_t *barrett;  // [tables][2]
     const LimbJob *jobs;      // explicit list (then in/out limbs are absolute, no prologue/epilogue)
@@ -69,10 +71,11 @@ struct NttArgs {
 
 // Forward transform: phase 1 (strided rows) then phase 2 (contiguous 256-blocks).  `a.in`/`a.out` and the
 // prologue describe phase 1's input; phase 2 runs in place on a.out unless an epilogue redirects it.
-hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, hipStream_t s);
+// fp selects the FP64 back end; every table the launch touches must then hold a prime below 2^50.
+hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s);
 // Inverse transform: phase A (contiguous blocks, reads a.in writes a.out) then phase B (rows, in place on
 // a.out, epilogue NTT_EPI_MUL optional).
-hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, hipStream_t s);
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s);
 
 struct Tables {
     const uint64_t *moduli;

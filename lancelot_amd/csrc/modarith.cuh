@@ -149,3 +149,117 @@ __device__ __forceinline__ void gs_block(uint64_t *v, const uint64_t *table, uin
 }
 
 }  // namespace he
+
+// ---------------------------------------------------------------------------------------------------
+// FP64 modular arithmetic for primes below 2^50.
+//
+// v_fma_f64 / v_mul_f64 / v_add_f64 run at full rate on CDNA4, so a modular product costs six
+// operations instead of the ~20 of a 64-bit Shoup product.  Every value is an integer held exactly
+// in a double; residues are signed and lazy (|v| < 2^53).  All steps below are exact integer
+// computations, so the canonical result equals the integer path's bit for bit.
+//
+//   x * w = h + l exactly (h = fl(x w), l = fma(x, w, -h)); k = rint(x * fl(w/q)) differs from
+//   x w / q by at most 1/2 + |x| 2^-52; h - k q and (h - k q) + l are integers below 2^52 in
+//   magnitude, hence exact; the result is congruent to x w with |r| <= (1/2 + |x| 2^-52) q.
+// ---------------------------------------------------------------------------------------------------
+namespace he {
+
+struct FpMod {
+    double q, qinv;
+};
+
+struct FpTw {
+    double w, winv;
+};
+
+// canonical residue (< 2^52) <-> exact double, through the exponent-bias trick
+__device__ __forceinline__ double fp_from_u64(uint64_t x) {
+    return __longlong_as_double((long long)(x | 0x4330000000000000ull)) - 4503599627370496.0;
+}
+
+__device__ __forceinline__ uint64_t fp_to_u64(double c) {  // 0 <= c < 2^52, integer
+    return (uint64_t)__double_as_longlong(c + 4503599627370496.0) & 0x000FFFFFFFFFFFFFull;
+}
+
+__device__ __forceinline__ double fp_mulmod(double x, FpTw t, FpMod m) {
+    const double k = __builtin_rint(x * t.winv);
+    const double h = x * t.w;
+    const double l = __builtin_fma(x, t.w, -h);
+    return __builtin_fma(-k, m.q, h) + l;
+}
+
+// centred representative, |result| <= (1/2 + 2^-49) q for |v| < 2^53
+__device__ __forceinline__ double fp_reduce(double v, FpMod m) {
+    const double k = __builtin_rint(v * m.qinv);
+    return __builtin_fma(-k, m.q, v);
+}
+
+// canonical residue in [0, q) as an exact double
+__device__ __forceinline__ double fp_canonical(double v, FpMod m) {
+    const double c = fp_reduce(v, m);
+    return c < 0.0 ? c + m.q : c;
+}
+
+__device__ __forceinline__ FpTw load_fptw(const double *table, size_t idx) {
+    const double2 v = reinterpret_cast<const double2 *>(table)[idx];
+    return FpTw{v.x, v.y};
+}
+
+// Forward block on lazy signed doubles.  REDUCE_FIRST brings every input back to |v| <= q/2; from there
+// (or from canonical inputs) the bound grows by 1.25 b + 0.5 per stage: below 5.4 q after four stages.
+template <int LOGR, bool REDUCE_FIRST>
+__device__ __forceinline__ void fp_ct_block(double *v, const double *table, uint32_t idx, FpMod m) {
+    constexpr int R = 1 << LOGR;
+    if (REDUCE_FIRST) {
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = fp_reduce(v[j], m);
+    }
+#pragma unroll
+    for (int l = 0; l < LOGR; l++) {
+        const int half = R >> (l + 1);
+#pragma unroll
+        for (int b = 0; b < (1 << l); b++) {
+            const FpTw tw = load_fptw(table, ((size_t)idx << l) + b);
+#pragma unroll
+            for (int j = 0; j < half; j++) {
+                const double x = v[2 * b * half + j];
+                const double t = fp_mulmod(v[2 * b * half + j + half], tw, m);
+                v[2 * b * half + j] = x + t;
+                v[2 * b * half + j + half] = x - t;
+            }
+        }
+    }
+}
+
+// Inverse block (no halving: the factor 1/N is applied once at the end of the transform).  Sums double
+// per stage, so after two stages the sum outputs are reduced again; outputs stay below 6 q.
+template <int LOGR, bool REDUCE_FIRST>
+__device__ __forceinline__ void fp_gs_block(double *v, const double *table, uint32_t idx, FpMod m) {
+    constexpr int R = 1 << LOGR;
+    if (REDUCE_FIRST) {
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = fp_reduce(v[j], m);
+    }
+#pragma unroll
+    for (int l = LOGR - 1; l >= 0; l--) {
+        const int half = R >> (l + 1);
+#pragma unroll
+        for (int b = 0; b < (1 << l); b++) {
+            const FpTw tw = load_fptw(table, ((size_t)idx << l) + b);
+#pragma unroll
+            for (int j = 0; j < half; j++) {
+                const double x = v[2 * b * half + j], y = v[2 * b * half + j + half];
+                v[2 * b * half + j] = x + y;
+                v[2 * b * half + j + half] = fp_mulmod(x - y, tw, m);
+            }
+        }
+        if (LOGR == 4 && l == 2) {
+#pragma unroll
+            for (int b = 0; b < (1 << l); b++)
+#pragma unroll
+                for (int j = 0; j < half; j++) v[2 * b * half + j] = fp_reduce(v[2 * b * half + j], m);
+        }
+    }
+}
+
+}  // namespace he

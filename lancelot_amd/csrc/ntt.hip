@@ -3,8 +3,7 @@
 // Mathematics (what the CPU checker and the reference compute; cahel-main/src/ntt/fntt_2d.cu:8-246,
 // src/ntt/intt_2d.cu:8-198, src/ntt/butterfly.cuh): forward = log2(N) Cooley-Tukey stages m = 1, 2, ..., N/2
 // with twiddle psi^bitrev(m+k) for group k, output in bit-reversed order, canonical residues; inverse =
-// the Gentleman-Sande stages in the opposite order with pre-halved inverse twiddles, so that no final
-// multiplication by 1/N is needed.
+// the Gentleman-Sande stages in the opposite order including the factor 1/N.
 //
 // Decomposition for the GPU: N = R x 256.  A limb is an R x 256 row-major matrix.
 //   rows pass   : the first log2(R) stages pair elements that are whole rows apart.  A workgroup owns a
@@ -16,6 +15,14 @@
 // radix-16) and writes them back; 8 stages cost two LDS round trips.  LDS indices are skewed by one word
 // per 16 so that both the stride-16 and the stride-256 gathers of a wave hit distinct banks.
 // The forward transform runs rows pass then blocks pass, the inverse the other way round.
+//
+// Two arithmetic back ends share this skeleton:
+//   integer : 64-bit Shoup/Harvey butterflies, any prime below 2^61 (~35 VALU instructions per butterfly);
+//             inverse twiddles are pre-halved so that 1/N comes for free
+//   FP64    : exact integer arithmetic in doubles for primes below 2^50 (8 full-rate operations per
+//             butterfly, see modarith.cuh); values between the two passes are lazy signed doubles stored
+//             in the same 8-byte words; the factor 1/N is folded into the last multiplication
+// A launch uses the FP64 back end when every limb it touches has a prime below 2^50.
 #include "kernels.h"
 #include "modarith.cuh"
 
@@ -66,11 +73,31 @@ __device__ __forceinline__ Job decode_job(const NttArgs &a, uint32_t job) {
     return j;
 }
 
+// Per-limb constants of one back end.
+struct IntCtx {
+    uint64_t q;
+    const uint64_t *tw;
+};
+
+struct FpCtx {
+    FpMod m;
+    const double *tw;
+};
+
+__device__ __forceinline__ IntCtx int_ctx(const NttArgs &a, uint32_t table) {
+    return IntCtx{a.moduli[table], a.tw + ((size_t)table << (a.log_n + 1))};
+}
+
+__device__ __forceinline__ FpCtx fp_ctx(const NttArgs &a, uint32_t table) {
+    const double *c = a.fp_consts + 4 * (size_t)table;
+    return FpCtx{FpMod{c[0], c[1]}, a.tw_fp + ((size_t)table << (a.log_n + 1))};
+}
+
 // r stages on a tile held in LDS.  Tile index bits: [upper][mid: r bits][lower: low_bits]; the 2^r
 // elements of a group differ in `mid`.  idx_base + upper is the twiddle index of the group's first stage.
 template <int LOGR, bool FWD>
 __device__ __forceinline__ void tile_pass(uint64_t *lds, uint32_t tile_elems, uint32_t low_bits, uint32_t idx_base,
-                                          const uint64_t *tw, uint64_t q) {
+                                          IntCtx c) {
     constexpr int R = 1 << LOGR;
     const uint32_t groups = tile_elems >> LOGR;
     const uint32_t low_mask = (1u << low_bits) - 1;
@@ -81,11 +108,33 @@ __device__ __forceinline__ void tile_pass(uint64_t *lds, uint32_t tile_elems, ui
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = lds[skew(base + ((uint32_t)j << low_bits))];
         if (FWD)
-            ct_block<LOGR>(v, tw, idx_base + upper, q);
+            ct_block<LOGR>(v, c.tw, idx_base + upper, c.q);
         else
-            gs_block<LOGR>(v, tw, idx_base + upper, q);
+            gs_block<LOGR>(v, c.tw, idx_base + upper, c.q);
 #pragma unroll
         for (int j = 0; j < R; j++) lds[skew(base + ((uint32_t)j << low_bits))] = v[j];
+    }
+}
+
+template <int LOGR, bool FWD, bool REDUCE_FIRST>
+__device__ __forceinline__ void tile_pass_fp(uint64_t *lds, uint32_t tile_elems, uint32_t low_bits, uint32_t idx_base,
+                                             FpCtx c) {
+    constexpr int R = 1 << LOGR;
+    double *ld = reinterpret_cast<double *>(lds);
+    const uint32_t groups = tile_elems >> LOGR;
+    const uint32_t low_mask = (1u << low_bits) - 1;
+    for (uint32_t g = threadIdx.x; g < groups; g += kThreads) {
+        const uint32_t upper = g >> low_bits;
+        const uint32_t base = (upper << (low_bits + LOGR)) | (g & low_mask);
+        double v[R];
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = ld[skew(base + ((uint32_t)j << low_bits))];
+        if (FWD)
+            fp_ct_block<LOGR, REDUCE_FIRST>(v, c.tw, idx_base + upper, c.m);
+        else
+            fp_gs_block<LOGR, REDUCE_FIRST>(v, c.tw, idx_base + upper, c.m);
+#pragma unroll
+        for (int j = 0; j < R; j++) ld[skew(base + ((uint32_t)j << low_bits))] = v[j];
     }
 }
 
@@ -100,24 +149,81 @@ __device__ __forceinline__ constexpr int log_cols() {
     return (kTileLog - LD) < 8 ? (kTileLog - LD) : 8;
 }
 
+// (N^-1 [* w]) as an FP twiddle for the last multiplication of the inverse transform
+__device__ __forceinline__ FpTw inverse_scale(const NttArgs &a, const Job &job, FpMod m) {
+    const double *c = a.fp_consts + 4 * (size_t)job.table;
+    FpTw ninv{c[2], c[3]};
+    if (a.epi_mode != NTT_EPI_MUL) return ninv;
+    const double w = fp_canonical(fp_mulmod(fp_from_u64(a.w[2 * job.limb]), ninv, m), m);
+    return FpTw{w, w * m.qinv};
+}
+
 // ---------------------------------------------------------------------------------------------------
 // rows pass: stages 0 .. LD-1 (forward) over an R = 2^LD rows x 256 matrix
 // ---------------------------------------------------------------------------------------------------
-template <int LD, bool FWD>
+template <int LD, bool FWD, bool FP>
 __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
     __shared__ uint64_t lds[kLdsWords];
     constexpr int LOGC = log_cols<LD>();
     constexpr uint32_t C = 1u << LOGC;
     constexpr uint32_t tile_elems = 1u << (LD + LOGC);
     constexpr uint32_t tiles_per_limb = 256u >> LOGC;
+    constexpr int p0 = Split<LD>::p0, p1 = Split<LD>::p1;
 
     const uint32_t lb = logical_block();
     const Job job = decode_job(a, lb / tiles_per_limb);
     const uint32_t col0 = (lb % tiles_per_limb) << LOGC;
-    const uint64_t q = a.moduli[job.table];
-    const uint64_t *tw = a.tw + ((size_t)job.table << (a.log_n + 1));
+    double *ld = reinterpret_cast<double *>(lds);
 
-    // load
+    if (FP) {
+        const FpCtx c = fp_ctx(a, job.table);
+        if (FWD) {
+            // input: canonical residues (or one broadcast source limb); output: lazy signed doubles
+            const uint64_t *src =
+                a.pro_mode == NTT_PRO_BROADCAST_REDUCE ? a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n) : job.in;
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+                uint32_t row = e >> LOGC, col = e & (C - 1);
+                ld[skew(e)] = fp_from_u64(src[(size_t)row * 256 + col0 + col]);
+            }
+            __syncthreads();
+            // a broadcast source may exceed this limb's prime: reduce first in that case
+            if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE)
+                tile_pass_fp<p0, true, true>(lds, tile_elems, LD - p0 + LOGC, 1u, c);
+            else
+                tile_pass_fp<p0, true, false>(lds, tile_elems, LD - p0 + LOGC, 1u, c);
+            __syncthreads();
+            if (p1 > 0) {
+                tile_pass_fp<(p1 > 0 ? p1 : 1), true, true>(lds, tile_elems, LOGC, 1u << p0, c);
+                __syncthreads();
+            }
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+                uint32_t row = e >> LOGC, col = e & (C - 1);
+                job.out[(size_t)row * 256 + col0 + col] = lds[skew(e)];
+            }
+        } else {
+            // input: lazy signed doubles from the blocks pass; output: canonical residues
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+                uint32_t row = e >> LOGC, col = e & (C - 1);
+                lds[skew(e)] = job.in[(size_t)row * 256 + col0 + col];
+            }
+            __syncthreads();
+            if (p1 > 0) {
+                tile_pass_fp<(p1 > 0 ? p1 : 1), false, true>(lds, tile_elems, LOGC, 1u << p0, c);
+                __syncthreads();
+            }
+            tile_pass_fp<p0, false, true>(lds, tile_elems, LD - p0 + LOGC, 1u, c);
+            __syncthreads();
+            const FpTw scale = inverse_scale(a, job, c.m);
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+                uint32_t row = e >> LOGC, col = e & (C - 1);
+                job.out[(size_t)row * 256 + col0 + col] = fp_to_u64(fp_canonical(fp_mulmod(ld[skew(e)], scale, c.m), c.m));
+            }
+        }
+        return;
+    }
+
+    const IntCtx c = int_ctx(a, job.table);
+    const uint64_t q = c.q;
     if (FWD && a.pro_mode == NTT_PRO_BROADCAST_REDUCE) {
         const uint64_t r1 = a.barrett[2 * job.table + 1];
         const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
@@ -133,12 +239,11 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
     }
     __syncthreads();
 
-    constexpr int p0 = Split<LD>::p0, p1 = Split<LD>::p1;
     if (FWD) {
-        tile_pass<p0, true>(lds, tile_elems, LD - p0 + LOGC, 1u, tw, q);
+        tile_pass<p0, true>(lds, tile_elems, LD - p0 + LOGC, 1u, c);
         __syncthreads();
         if (p1 > 0) {
-            tile_pass<(p1 > 0 ? p1 : 1), true>(lds, tile_elems, LOGC, 1u << p0, tw, q);
+            tile_pass<(p1 > 0 ? p1 : 1), true>(lds, tile_elems, LOGC, 1u << p0, c);
             __syncthreads();
         }
         // lazy values in [0, 4q) go to the blocks pass
@@ -148,10 +253,10 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
         }
     } else {
         if (p1 > 0) {
-            tile_pass<(p1 > 0 ? p1 : 1), false>(lds, tile_elems, LOGC, 1u << p0, tw, q);
+            tile_pass<(p1 > 0 ? p1 : 1), false>(lds, tile_elems, LOGC, 1u << p0, c);
             __syncthreads();
         }
-        tile_pass<p0, false>(lds, tile_elems, LD - p0 + LOGC, 1u, tw, q);
+        tile_pass<p0, false>(lds, tile_elems, LD - p0 + LOGC, 1u, c);
         __syncthreads();
         if (a.epi_mode == NTT_EPI_MUL) {
             const Shoup w = load_shoup(a.w, job.limb);
@@ -169,9 +274,9 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// blocks pass: the 8 stages that stay inside 256 consecutive words; LR = log2(rows of the limb)
+// blocks pass: the 8 stages that stay inside 256 consecutive words
 // ---------------------------------------------------------------------------------------------------
-template <bool FWD>
+template <bool FWD, bool FP>
 __global__ __launch_bounds__(kThreads) void ntt_blocks_kernel(NttArgs a) {
     __shared__ uint64_t lds[kLdsWords];
     const uint32_t lr = a.log_n - 8;                       // log2(number of 256-blocks per limb)
@@ -183,27 +288,63 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_kernel(NttArgs a) {
     const Job job = decode_job(a, lb / tiles_per_limb);
     const uint32_t tile = lb % tiles_per_limb;
     const size_t off = (size_t)tile * tile_elems;
-    const uint64_t q = a.moduli[job.table];
-    const uint64_t *tw = a.tw + ((size_t)job.table << (a.log_n + 1));
     const uint32_t blk0 = tile << log_b;                   // first 256-block of this tile within the limb
+    const size_t n = (size_t)1 << a.log_n;
+    double *ld = reinterpret_cast<double *>(lds);
 
     const uint64_t *src = FWD ? job.out : job.in;  // the forward blocks pass continues on the rows pass's output
-    for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) lds[skew(e)] = src[off + e];
+    if (FP && !FWD) {
+        for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) ld[skew(e)] = fp_from_u64(src[off + e]);
+    } else {
+        for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) lds[skew(e)] = src[off + e];
+    }
     __syncthreads();
 
+    const bool epi = a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD;
+    const uint64_t *minuend = epi ? a.epi_a + ((size_t)job.poly * a.epi_a_poly_stride + job.limb) * n + off : nullptr;
+    const uint64_t *addend =
+        a.epi_mode == NTT_EPI_SUB_MUL_ADD ? a.epi_b + ((size_t)job.poly * a.epi_b_poly_stride + job.limb) * n + off : nullptr;
+    uint64_t *dst = epi ? a.epi_dst + ((size_t)job.poly * a.epi_dst_poly_stride + job.limb) * n + off : job.out + off;
+
+    if (FP) {
+        const FpCtx c = fp_ctx(a, job.table);
+        if (FWD) {
+            tile_pass_fp<4, true, true>(lds, tile_elems, 4, (1u << lr) + blk0, c);
+            __syncthreads();
+            tile_pass_fp<4, true, true>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), c);
+            __syncthreads();
+            if (epi) {
+                const double wd = fp_from_u64(a.w[2 * job.limb]);
+                const FpTw w{wd, wd * c.m.qinv};
+                for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+                    const double v = fp_canonical(ld[skew(e)], c.m);
+                    double r = fp_mulmod(fp_from_u64(minuend[e]) - v, w, c.m);
+                    if (addend) r += fp_from_u64(addend[e]);
+                    dst[e] = fp_to_u64(fp_canonical(r, c.m));
+                }
+            } else {
+                for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads)
+                    dst[e] = fp_to_u64(fp_canonical(ld[skew(e)], c.m));
+            }
+        } else {
+            tile_pass_fp<4, false, false>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), c);
+            __syncthreads();
+            tile_pass_fp<4, false, true>(lds, tile_elems, 4, (1u << lr) + blk0, c);
+            __syncthreads();
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) job.out[off + e] = lds[skew(e)];
+        }
+        return;
+    }
+
+    const IntCtx c = int_ctx(a, job.table);
+    const uint64_t q = c.q;
     if (FWD) {
-        tile_pass<4, true>(lds, tile_elems, 4, (1u << lr) + blk0, tw, q);
+        tile_pass<4, true>(lds, tile_elems, 4, (1u << lr) + blk0, c);
         __syncthreads();
-        tile_pass<4, true>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), tw, q);
+        tile_pass<4, true>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), c);
         __syncthreads();
-        if (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD) {
-            const size_t n = (size_t)1 << a.log_n;
+        if (epi) {
             const Shoup w = load_shoup(a.w, job.limb);
-            const uint64_t *minuend = a.epi_a + ((size_t)job.poly * a.epi_a_poly_stride + job.limb) * n + off;
-            const uint64_t *addend =
-                a.epi_mode == NTT_EPI_SUB_MUL_ADD ? a.epi_b + ((size_t)job.poly * a.epi_b_poly_stride + job.limb) * n + off
-                                              : nullptr;
-            uint64_t *dst = a.epi_dst + ((size_t)job.poly * a.epi_dst_poly_stride + job.limb) * n + off;
             for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
                 uint64_t v = reduce_4q(lds[skew(e)], q);
                 uint64_t r = mul_shoup(sub_mod(minuend[e], v, q), w, q);
@@ -211,19 +352,19 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_kernel(NttArgs a) {
                 dst[e] = r;
             }
         } else {
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) job.out[off + e] = reduce_4q(lds[skew(e)], q);
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) dst[e] = reduce_4q(lds[skew(e)], q);
         }
     } else {
-        tile_pass<4, false>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), tw, q);
+        tile_pass<4, false>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), c);
         __syncthreads();
-        tile_pass<4, false>(lds, tile_elems, 4, (1u << lr) + blk0, tw, q);
+        tile_pass<4, false>(lds, tile_elems, 4, (1u << lr) + blk0, c);
         __syncthreads();
         // lazy values in [0, 2q) go to the rows pass
         for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) job.out[off + e] = lds[skew(e)];
     }
 }
 
-template <bool FWD>
+template <bool FWD, bool FP>
 hipError_t launch_rows(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
     const int ld = (int)a.log_n - 8;
     auto grid = [&](int ldv) {
@@ -231,9 +372,9 @@ hipError_t launch_rows(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
         return dim3(n_jobs * (256u >> logc));
     };
     switch (ld) {
-#define HE_CASE(LD)                                                                      \
-    case LD:                                                                             \
-        hipLaunchKernelGGL((ntt_rows_kernel<LD, FWD>), grid(LD), dim3(kThreads), 0, s, a); \
+#define HE_CASE(LD)                                                                          \
+    case LD:                                                                                 \
+        hipLaunchKernelGGL((ntt_rows_kernel<LD, FWD, FP>), grid(LD), dim3(kThreads), 0, s, a); \
         break;
         HE_CASE(1) HE_CASE(2) HE_CASE(3) HE_CASE(4) HE_CASE(5) HE_CASE(6) HE_CASE(7) HE_CASE(8)
 #undef HE_CASE
@@ -243,35 +384,35 @@ hipError_t launch_rows(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
     return hipGetLastError();
 }
 
-template <bool FWD>
+template <bool FWD, bool FP>
 hipError_t launch_blocks(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
     const uint32_t lr = a.log_n - 8;
     const uint32_t log_b = lr < 4 ? lr : 4;
-    hipLaunchKernelGGL((ntt_blocks_kernel<FWD>), dim3(n_jobs << (lr - log_b)), dim3(kThreads), 0, s, a);
+    hipLaunchKernelGGL((ntt_blocks_kernel<FWD, FP>), dim3(n_jobs << (lr - log_b)), dim3(kThreads), 0, s, a);
     return hipGetLastError();
 }
 
 }  // namespace
 
-hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, hipStream_t s) {
+hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s) {
     if (a.log_n < 9 || a.log_n > 16) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
-    hipError_t e = launch_rows<true>(a, n_jobs, s);
+    hipError_t e = fp ? launch_rows<true, true>(a, n_jobs, s) : launch_rows<true, false>(a, n_jobs, s);
     if (e != hipSuccess) return e;
-    return launch_blocks<true>(a, n_jobs, s);
+    return fp ? launch_blocks<true, true>(a, n_jobs, s) : launch_blocks<true, false>(a, n_jobs, s);
 }
 
-hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, hipStream_t s) {
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s) {
     if (a.log_n < 9 || a.log_n > 16) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
-    hipError_t e = launch_blocks<false>(a, n_jobs, s);
+    hipError_t e = fp ? launch_blocks<false, true>(a, n_jobs, s) : launch_blocks<false, false>(a, n_jobs, s);
     if (e != hipSuccess) return e;
     NttArgs rows = a;
     rows.in = a.out;  // the rows pass continues in place on the output buffer
     rows.in_poly_stride = a.out_poly_stride;
-    return launch_rows<false>(rows, n_jobs, s);
+    return fp ? launch_rows<false, true>(rows, n_jobs, s) : launch_rows<false, false>(rows, n_jobs, s);
 }
 
 }  // namespace he

@@ -47,14 +47,18 @@ def test_tables_match_oracle(small):
             assert wq == (w << 64) // q
 
 
+# [60, 50, 35, 59]: a prime above 2^50 keeps the launch on the integer back end; [50, 49, 35, 50]: all below
+# 2^50, the FP64 back end
+@pytest.mark.parametrize("bits", [[60, 50, 35, 59], [50, 49, 35, 50]])
 @pytest.mark.parametrize("logn", [9, 10, 11, 12, 13, 14, 15, 16])
-def test_ntt_all_sizes(oracle, capi, logn):
-    cahel, parms, ctx, p = make_pair(oracle, logn, [60, 50, 35, 59], 1)
+def test_ntt_all_sizes(oracle, capi, logn, bits):
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, 1)
     rng = np.random.default_rng(logn)
     h = ctx.he_handle()
     x = rand_limbs(p, rng, range(4), n_polys=2)
     x[0, 0, :8] = 0
-    x[0, 1, :8] = p.moduli[1] - 1
+    x[0, 1, :] = p.moduli[1] - 1          # a whole limb of q - 1: the largest lazy values
+    x[1, 2, :] = 1
     d = DeviceArray(capi, host=x)
     capi.check(capi.lib().he_ntt_forward(h, d.ptr, 2, 4, 4, 0, 4, 0, None))
     want = np.stack([p.ntt_fwd(x[i].copy()) for i in range(2)])
@@ -102,6 +106,33 @@ def test_ntt_benchmark_shape(full, capi):
     assert (d.numpy() == np.stack([p.ntt_fwd(x[i].copy()) for i in range(2)])).all()
     capi.check(capi.lib().he_ntt_inverse(h, d.ptr, 2, 24, 24, 0, 24, 0, None))
     assert (d.numpy() == x).all()
+
+
+def test_integer_and_fp64_back_ends_agree(oracle, capi, monkeypatch):
+    """The same 50-bit parameter set with the FP64 back end and, forced by the environment, the integer one."""
+    results = []
+    for no_fp in ("0", "1"):
+        monkeypatch.setenv("CAHEL_HIP_NO_FP64", no_fp)
+        cahel, parms, ctx, p = make_pair(oracle, 13, [50, 50, 49, 50, 50, 50], 2)
+        rng = np.random.default_rng(11)
+        lib, h = capi.lib(), ctx.he_handle()
+        L = 4
+        c = rand_limbs(p, rng, range(L))
+        ct = rand_limbs(p, rng, range(L), n_polys=2)
+        host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+        dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
+        ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+        capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, 5, ws.ptr, None))
+        ks = p.key_switch(p.galois_ntt(c, 5), host_evk)
+        want = np.stack([p.add(ct[b], ks[b]) for b in range(2)])
+        got = dct.numpy()
+        assert (got == want).all(), no_fp
+        dres = DeviceArray(capi, shape=(2, L - 1, p.n))
+        rws = DeviceArray(capi, shape=(2, p.n))
+        capi.check(lib.he_rescale(h, dct.ptr, dres.ptr, 2, L, rws.ptr, None))
+        assert (dres.numpy() == p.rescale(want)).all(), no_fp
+        results.append(dres.numpy())
+    assert (results[0] == results[1]).all()
 
 
 def test_ntt_rejects_bad_arguments(small, capi):
