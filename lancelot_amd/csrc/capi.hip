@@ -2,6 +2,7 @@
 // orchestration of the kernels in ntt.hip / rns.hip into the operations of the CKKS hot path.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -31,6 +32,11 @@ struct Level {
     std::vector<Digit> digits;
     LimbJob *d_modup_jobs = nullptr;     // NTT jobs over the converted limbs of all digits
     uint32_t n_modup_jobs = 0;
+    // batched base conversion (all digits of ModUp / all polynomials of ModDown in one launch)
+    BconvDesc *d_modup_descs = nullptr, *d_moddown_descs = nullptr;
+    uint32_t *d_modup_limb = nullptr, *d_modup_table = nullptr;
+    uint32_t modup_max_rows = 0, modup_max_copy = 0;
+    bool batched = false;
 };
 
 }  // namespace
@@ -333,6 +339,45 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
         }
         rc = upload(ctx, &lv.d_mats, d->digit_mats, mat_words);
         if (rc) return rc;
+        if (K <= 8) {
+            const size_t n = ctx->n();
+            std::vector<BconvDesc> up(beta), down(4);
+            std::vector<uint32_t> limb_all, table_all;
+            for (uint32_t dg = 0; dg < beta; dg++) {
+                const Digit &g = lv.digits[dg];
+                BconvDesc &bd = up[dg];
+                memset(&bd, 0, sizeof(bd));
+                bd.x_off = (uint64_t)g.start * n;
+                bd.out_off = (uint64_t)dg * (L + K) * n;
+                bd.mat_off = g.mat_off;
+                bd.map_off = (uint32_t)limb_all.size();
+                bd.n_in = g.size;
+                bd.n_out = g.n_out;
+                bd.copy_first = g.start;
+                bd.copy_count = g.size;
+                for (uint32_t r = 0; r < g.n_out; r++) {
+                    const uint32_t lim = r < g.start ? r : r + g.size;
+                    limb_all.push_back(lim);
+                    table_all.push_back(table_of(ctx, L, lim));
+                }
+                lv.modup_max_rows = std::max(lv.modup_max_rows, g.n_out);
+                lv.modup_max_copy = std::max(lv.modup_max_copy, g.size);
+            }
+            for (uint32_t p = 0; p < 4; p++) {
+                BconvDesc &bd = down[p];
+                memset(&bd, 0, sizeof(bd));
+                bd.x_off = ((uint64_t)p * (L + K) + L) * n;
+                bd.out_off = (uint64_t)p * L * n;
+                bd.n_in = K;
+                bd.n_out = L;
+            }
+            rc = upload(ctx, &lv.d_modup_descs, up.data(), up.size());
+            if (!rc) rc = upload(ctx, &lv.d_moddown_descs, down.data(), down.size());
+            if (!rc) rc = upload(ctx, &lv.d_modup_limb, limb_all.data(), limb_all.size());
+            if (!rc) rc = upload(ctx, &lv.d_modup_table, table_all.data(), table_all.size());
+            if (rc) return rc;
+            lv.batched = true;
+        }
         lv.n_modup_jobs = (uint32_t)jobs.size();
         rc = upload(ctx, &lv.d_modup_jobs, jobs.data(), jobs.size());
         if (rc) return rc;
@@ -483,7 +528,12 @@ int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_part_hat_inv;
     HE_HIP(launch_ntt_inverse(inv, 1, fp_for(ctx, inv.map), S(s)));
-    for (uint32_t d = 0; d < lv->beta; d++) {
+    if (lv->batched) {
+        BconvBatch b{ws, out, c, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
+                     lv->beta, lv->modup_max_rows, lv->modup_max_copy};
+        HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+    }
+    for (uint32_t d = 0; d < lv->beta && !lv->batched; d++) {
         const Digit &g = lv->digits[d];
         uint64_t *od = out + (size_t)d * LK * n;
         // the digit's own limbs keep their NTT form
@@ -532,7 +582,13 @@ int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, u
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = ctx->d_phat_inv;
     HE_HIP(launch_ntt_inverse(inv, n_polys, fp_for(ctx, inv.map), S(s)));
-    for (uint32_t p = 0; p < n_polys; p++) {
+    const Level *lv = level_of(ctx, L);
+    const bool batched = lv && lv->batched && n_polys <= 4;
+    if (batched) {
+        BconvBatch b{cx, ws, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, n_polys, L, 0};
+        HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+    }
+    for (uint32_t p = 0; p < n_polys && !batched; p++) {
         BconvArgs b{cx + ((size_t)p * LK + L) * n, ws + (size_t)p * L * n, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, K, L};
         HE_HIP(launch_bconv(ctx->tables(), b, S(s)));
     }

@@ -108,6 +108,29 @@ struct BconvArgs {
 };
 hipError_t launch_bconv(const Tables &t, const BconvArgs &a, hipStream_t s);
 
+// Batched form: every unit (a ModUp digit or a ModDown polynomial) in one launch, together with the limbs
+// that are copied unchanged (a digit's own limbs keep their NTT form).  Requires n_in <= 8.
+struct BconvDesc {
+    uint64_t x_off;      // words from x_base to this unit's first input limb
+    uint64_t out_off;    // words from out_base to limb 0 of this unit's output buffer
+    uint64_t mat_off;    // words from mat_base to this unit's row-major [n_out][n_in] matrix
+    uint32_t map_off;    // offset into out_limb / out_table
+    uint32_t n_in, n_out;
+    uint32_t copy_first, copy_count;  // limbs copied from copy_base (same limb index in the unit's output)
+    uint32_t pad;
+};
+struct BconvBatch {
+    const uint64_t *x_base;
+    uint64_t *out_base;
+    const uint64_t *copy_base;
+    const uint64_t *mat_base;
+    const uint32_t *out_limb;
+    const uint32_t *out_table;
+    const BconvDesc *descs;  // device memory
+    uint32_t n_units, max_rows, max_copy;
+};
+hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s);
+
 constexpr int kMaxDigits = 64;
 struct EvkPtrs {
     const uint64_t *p[kMaxDigits];

@@ -305,6 +305,17 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_kernel(NttArgs a) {
     const uint64_t *addend =
         a.epi_mode == NTT_EPI_SUB_MUL_ADD ? a.epi_b + ((size_t)job.poly * a.epi_b_poly_stride + job.limb) * n + off : nullptr;
     uint64_t *dst = epi ? a.epi_dst + ((size_t)job.poly * a.epi_dst_poly_stride + job.limb) * n + off : job.out + off;
+    // the epilogue operands are fetched now so that their latency hides behind the butterflies
+    constexpr int kPer = kTile / kThreads;
+    uint64_t pre_a[kPer], pre_b[kPer];
+    if (FWD && epi) {
+#pragma unroll
+        for (int i = 0; i < kPer; i++) {
+            const uint32_t e = threadIdx.x + i * kThreads;
+            pre_a[i] = e < tile_elems ? minuend[e] : 0;
+            pre_b[i] = (addend && e < tile_elems) ? addend[e] : 0;
+        }
+    }
 
     if (FP) {
         const FpCtx c = fp_ctx(a, job.table);
@@ -316,11 +327,15 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_kernel(NttArgs a) {
             if (epi) {
                 const double wd = fp_from_u64(a.w[2 * job.limb]);
                 const FpTw w{wd, wd * c.m.qinv};
-                for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
-                    const double v = fp_canonical(ld[skew(e)], c.m);
-                    double r = fp_mulmod(fp_from_u64(minuend[e]) - v, w, c.m);
-                    if (addend) r += fp_from_u64(addend[e]);
-                    dst[e] = fp_to_u64(fp_canonical(r, c.m));
+#pragma unroll
+                for (int i = 0; i < kPer; i++) {
+                    const uint32_t e = threadIdx.x + i * kThreads;
+                    if (e < tile_elems) {
+                        const double v = fp_canonical(ld[skew(e)], c.m);
+                        double r = fp_mulmod(fp_from_u64(pre_a[i]) - v, w, c.m);
+                        if (addend) r += fp_from_u64(pre_b[i]);
+                        dst[e] = fp_to_u64(fp_canonical(r, c.m));
+                    }
                 }
             } else {
                 for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads)
@@ -345,11 +360,15 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_kernel(NttArgs a) {
         __syncthreads();
         if (epi) {
             const Shoup w = load_shoup(a.w, job.limb);
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
-                uint64_t v = reduce_4q(lds[skew(e)], q);
-                uint64_t r = mul_shoup(sub_mod(minuend[e], v, q), w, q);
-                if (addend) r = add_mod(r, addend[e], q);
-                dst[e] = r;
+#pragma unroll
+            for (int i = 0; i < kPer; i++) {
+                const uint32_t e = threadIdx.x + i * kThreads;
+                if (e < tile_elems) {
+                    uint64_t v = reduce_4q(lds[skew(e)], q);
+                    uint64_t r = mul_shoup(sub_mod(pre_a[i], v, q), w, q);
+                    if (addend) r = add_mod(r, pre_b[i], q);
+                    dst[e] = r;
+                }
             }
         } else {
             for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) dst[e] = reduce_4q(lds[skew(e)], q);

@@ -154,6 +154,48 @@ __global__ __launch_bounds__(kThreads) void bconv_kernel(BconvKArgs p) {
     }
 }
 
+constexpr int kBatchRows = 8;
+constexpr int kBatchIn = 8;
+
+struct BconvBatchK {
+    BconvBatch b;
+    const uint64_t *moduli, *barrett;
+    uint32_t log_n, compute_groups;
+};
+
+// grid: (N / 256, compute groups + copy groups, units); thread = one coefficient x kBatchRows output limbs
+__global__ __launch_bounds__(kThreads) void bconv_batched_kernel(BconvBatchK p) {
+    const BconvDesc d = p.b.descs[blockIdx.z];
+    const size_t j = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    uint64_t *out = p.b.out_base + d.out_off;
+    if (blockIdx.y >= p.compute_groups) {
+        // limbs that pass through unchanged
+        const uint32_t first = (blockIdx.y - p.compute_groups) * kBatchRows;
+        for (uint32_t r = first; r < first + kBatchRows && r < d.copy_count; r++) {
+            const size_t idx = ((size_t)(d.copy_first + r) << p.log_n) + j;
+            out[idx] = p.b.copy_base[idx];
+        }
+        return;
+    }
+    const uint32_t row0 = blockIdx.y * kBatchRows;
+    if (row0 >= d.n_out) return;
+    const uint64_t *x = p.b.x_base + d.x_off;
+    uint64_t xv[kBatchIn];
+#pragma unroll
+    for (int i = 0; i < kBatchIn; i++) xv[i] = (uint32_t)i < d.n_in ? x[((size_t)i << p.log_n) + j] : 0;
+    const uint64_t *mat = p.b.mat_base + d.mat_off;
+    for (uint32_t row = row0; row < row0 + kBatchRows && row < d.n_out; row++) {
+        const uint64_t *m = mat + (size_t)row * d.n_in;
+        U128 acc{0, 0};
+#pragma unroll
+        for (int i = 0; i < kBatchIn; i++)
+            if ((uint32_t)i < d.n_in) mac128(acc, xv[i], m[i]);
+        const uint32_t t = p.b.out_table[d.map_off + row];
+        out[((size_t)p.b.out_limb[d.map_off + row] << p.log_n) + j] =
+            barrett128(acc.lo, acc.hi, p.moduli[t], p.barrett[2 * t], p.barrett[2 * t + 1]);
+    }
+}
+
 struct InnerArgs {
     const uint64_t *y;
     uint64_t *out;
@@ -332,6 +374,14 @@ hipError_t launch_bconv(const Tables &t, const BconvArgs &a, hipStream_t s) {
 #undef HE_CASE
         default: hipLaunchKernelGGL(bconv_kernel<0>, grid, dim3(kThreads), 0, s, p);
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s) {
+    if (b.n_units == 0) return hipSuccess;
+    const uint32_t cg = (b.max_rows + kBatchRows - 1) / kBatchRows, kg = (b.max_copy + kBatchRows - 1) / kBatchRows;
+    BconvBatchK p{b, t.moduli, t.barrett, t.log_n, cg};
+    hipLaunchKernelGGL(bconv_batched_kernel, dim3((1u << t.log_n) / kThreads, cg + kg, b.n_units), dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
 
