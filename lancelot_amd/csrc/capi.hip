@@ -37,6 +37,7 @@ struct Level {
     uint32_t *d_modup_limb = nullptr, *d_modup_table = nullptr;
     uint32_t modup_max_rows = 0, modup_max_copy = 0;
     bool batched = false;
+    double *d_mats_fp = nullptr;         // (M, M/m) pairs of the digit matrices, when every prime is below 2^50
 };
 
 }  // namespace
@@ -48,6 +49,8 @@ struct he_context {
     uint64_t *d_p_mod_q = nullptr, *d_pinv_mod_q = nullptr, *d_phat_inv = nullptr, *d_phat_mod_q = nullptr;
     uint32_t *d_iota = nullptr;  // 0, 1, 2, ...: row -> limb/table map of the P -> Ql conversion
     double *d_psi_fp = nullptr, *d_ipsi_fp = nullptr, *d_fp_consts = nullptr;  // FP64 back end tables
+    double *d_phat_mod_q_fp = nullptr;   // (M, M/q_j) pairs of the P -> Ql matrix
+    std::vector<uint64_t> h_moduli;
     std::vector<uint8_t> fp_ok;  // per table: prime below 2^50
     bool use_fp = true;          // environment CAHEL_HIP_NO_FP64=1 forces the integer back end
     std::vector<Level> levels;   // indexed by L
@@ -243,6 +246,7 @@ int he_context_create(const he_context_desc *d, he_context **out) {
     ctx->size_p = d->size_p;
     ctx->size_qp = d->size_q + d->size_p;
     ctx->levels.resize(ctx->size_q + 1);
+    ctx->h_moduli.assign(d->moduli, d->moduli + ctx->size_qp);
     const size_t n = ctx->n(), qp = ctx->size_qp;
     int rc = hipGetDevice(&ctx->device);
     if (!rc) rc = upload(ctx, &ctx->d_moduli, d->moduli, qp);
@@ -281,7 +285,16 @@ int he_context_create(const he_context_desc *d, he_context **out) {
             consts[4 * t + 2] = (double)ninv;
             consts[4 * t + 3] = (double)ninv / qd;
         }
-        rc = upload(ctx, &ctx->d_psi_fp, psi_fp.data(), psi_fp.size());
+        if (d->size_p) {
+            std::vector<double> pfp(2 * (size_t)d->size_q * d->size_p);
+            for (size_t jq = 0; jq < d->size_q; jq++)
+                for (size_t k = 0; k < d->size_p; k++) {
+                    pfp[2 * (jq * d->size_p + k)] = (double)d->phat_mod_q[jq * d->size_p + k];
+                    pfp[2 * (jq * d->size_p + k) + 1] = (double)d->phat_mod_q[jq * d->size_p + k] / (double)d->moduli[jq];
+                }
+            rc = upload(ctx, &ctx->d_phat_mod_q_fp, pfp.data(), pfp.size());
+        }
+        if (!rc) rc = upload(ctx, &ctx->d_psi_fp, psi_fp.data(), psi_fp.size());
         if (!rc) rc = upload(ctx, &ctx->d_ipsi_fp, ipsi_fp.data(), ipsi_fp.size());
         if (!rc) rc = upload(ctx, &ctx->d_fp_consts, consts.data(), consts.size());
     }
@@ -377,6 +390,23 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
             if (!rc) rc = upload(ctx, &lv.d_modup_table, table_all.data(), table_all.size());
             if (rc) return rc;
             lv.batched = true;
+            if (fp_for_level(ctx, L)) {
+                std::vector<double> mfp(2 * mat_words);
+                for (uint32_t dg = 0; dg < beta; dg++) {
+                    const Digit &g = lv.digits[dg];
+                    for (uint32_t r = 0; r < g.n_out; r++) {
+                        const uint32_t lim = r < g.start ? r : r + g.size;
+                        const double m = (double)ctx->h_moduli[table_of(ctx, L, lim)];
+                        for (uint32_t i = 0; i < g.size; i++) {
+                            const size_t idx = g.mat_off + (size_t)r * g.size + i;
+                            mfp[2 * idx] = (double)d->digit_mats[idx];
+                            mfp[2 * idx + 1] = (double)d->digit_mats[idx] / m;
+                        }
+                    }
+                }
+                rc = upload(ctx, &lv.d_mats_fp, mfp.data(), mfp.size());
+                if (rc) return rc;
+            }
         }
         lv.n_modup_jobs = (uint32_t)jobs.size();
         rc = upload(ctx, &lv.d_modup_jobs, jobs.data(), jobs.size());
@@ -530,7 +560,7 @@ int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out
     HE_HIP(launch_ntt_inverse(inv, 1, fp_for(ctx, inv.map), S(s)));
     if (lv->batched) {
         BconvBatch b{ws, out, c, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                     lv->beta, lv->modup_max_rows, lv->modup_max_copy};
+                     lv->beta, lv->modup_max_rows, lv->modup_max_copy, lv->d_mats_fp, ctx->d_fp_consts};
         HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
     }
     for (uint32_t d = 0; d < lv->beta && !lv->batched; d++) {
@@ -585,7 +615,8 @@ int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, u
     const Level *lv = level_of(ctx, L);
     const bool batched = lv && lv->batched && n_polys <= 4;
     if (batched) {
-        BconvBatch b{cx, ws, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, n_polys, L, 0};
+        BconvBatch b{cx, ws, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, n_polys, L, 0,
+                     fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts};
         HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
     }
     for (uint32_t p = 0; p < n_polys && !batched; p++) {

@@ -128,6 +128,10 @@ struct BconvBatch {
     const uint32_t *out_table;
     const BconvDesc *descs;  // device memory
     uint32_t n_units, max_rows, max_copy;
+    // FP64 back end (all primes involved below 2^50): the matrix as (M, M/m) pairs at the same offsets * 2,
+    // per-table constants as in NttArgs::fp_consts; null selects the integer kernel
+    const double *mat_fp;
+    const double *fp_consts;
 };
 hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s);
 

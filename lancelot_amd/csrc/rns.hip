@@ -8,6 +8,8 @@
 // tensor :531-612), src/galois.cu:20-30 + include/galois.cuh:45-57, src/rns_bconv.cu:587-623 and :166-198
 // (base conversion, uncorrected sum, one reduction), src/eval_key_switch.cu:13-76 (inner product) and
 // src/prng.cu:143-242 (distributions of the samplers).
+#include <cstdlib>
+
 #include "kernels.h"
 #include "modarith.cuh"
 
@@ -154,13 +156,14 @@ __global__ __launch_bounds__(kThreads) void bconv_kernel(BconvKArgs p) {
     }
 }
 
-constexpr int kBatchRows = 8;
+// output limbs per thread in the batched base conversion: the inputs are re-read once per row group
+
 constexpr int kBatchIn = 8;
 
 struct BconvBatchK {
     BconvBatch b;
     const uint64_t *moduli, *barrett;
-    uint32_t log_n, compute_groups;
+    uint32_t log_n, compute_groups, rows_per;
 };
 
 // grid: (N / 256, compute groups + copy groups, units); thread = one coefficient x kBatchRows output limbs
@@ -170,21 +173,21 @@ __global__ __launch_bounds__(kThreads) void bconv_batched_kernel(BconvBatchK p) 
     uint64_t *out = p.b.out_base + d.out_off;
     if (blockIdx.y >= p.compute_groups) {
         // limbs that pass through unchanged
-        const uint32_t first = (blockIdx.y - p.compute_groups) * kBatchRows;
-        for (uint32_t r = first; r < first + kBatchRows && r < d.copy_count; r++) {
+        const uint32_t first = (blockIdx.y - p.compute_groups) * p.rows_per;
+        for (uint32_t r = first; r < first + p.rows_per && r < d.copy_count; r++) {
             const size_t idx = ((size_t)(d.copy_first + r) << p.log_n) + j;
             out[idx] = p.b.copy_base[idx];
         }
         return;
     }
-    const uint32_t row0 = blockIdx.y * kBatchRows;
+    const uint32_t row0 = blockIdx.y * p.rows_per;
     if (row0 >= d.n_out) return;
     const uint64_t *x = p.b.x_base + d.x_off;
     uint64_t xv[kBatchIn];
 #pragma unroll
     for (int i = 0; i < kBatchIn; i++) xv[i] = (uint32_t)i < d.n_in ? x[((size_t)i << p.log_n) + j] : 0;
     const uint64_t *mat = p.b.mat_base + d.mat_off;
-    for (uint32_t row = row0; row < row0 + kBatchRows && row < d.n_out; row++) {
+    for (uint32_t row = row0; row < row0 + p.rows_per && row < d.n_out; row++) {
         const uint64_t *m = mat + (size_t)row * d.n_in;
         U128 acc{0, 0};
 #pragma unroll
@@ -193,6 +196,39 @@ __global__ __launch_bounds__(kThreads) void bconv_batched_kernel(BconvBatchK p) 
         const uint32_t t = p.b.out_table[d.map_off + row];
         out[((size_t)p.b.out_limb[d.map_off + row] << p.log_n) + j] =
             barrett128(acc.lo, acc.hi, p.moduli[t], p.barrett[2 * t], p.barrett[2 * t + 1]);
+    }
+}
+
+// FP64 variant: every product is reduced on the fly to |r| <= 0.75 m, so the sum of up to 8 terms stays an
+// exact integer below 6 m < 2^53; one canonicalisation per output.
+__global__ __launch_bounds__(kThreads) void bconv_batched_fp_kernel(BconvBatchK p) {
+    const BconvDesc d = p.b.descs[blockIdx.z];
+    const size_t j = (size_t)blockIdx.x * kThreads + threadIdx.x;
+    uint64_t *out = p.b.out_base + d.out_off;
+    if (blockIdx.y >= p.compute_groups) {
+        const uint32_t first = (blockIdx.y - p.compute_groups) * p.rows_per;
+        for (uint32_t r = first; r < first + p.rows_per && r < d.copy_count; r++) {
+            const size_t idx = ((size_t)(d.copy_first + r) << p.log_n) + j;
+            out[idx] = p.b.copy_base[idx];
+        }
+        return;
+    }
+    const uint32_t row0 = blockIdx.y * p.rows_per;
+    if (row0 >= d.n_out) return;
+    const uint64_t *x = p.b.x_base + d.x_off;
+    double xv[kBatchIn];
+#pragma unroll
+    for (int i = 0; i < kBatchIn; i++) xv[i] = (uint32_t)i < d.n_in ? fp_from_u64(x[((size_t)i << p.log_n) + j]) : 0.0;
+    const double *mat = p.b.mat_fp + 2 * d.mat_off;
+    for (uint32_t row = row0; row < row0 + p.rows_per && row < d.n_out; row++) {
+        const double *m = mat + 2 * (size_t)row * d.n_in;
+        const uint32_t t = p.b.out_table[d.map_off + row];
+        const FpMod mod{p.b.fp_consts[4 * t], p.b.fp_consts[4 * t + 1]};
+        double acc = 0.0;
+#pragma unroll
+        for (int i = 0; i < kBatchIn; i++)
+            if ((uint32_t)i < d.n_in) acc += fp_mulmod(xv[i], FpTw{m[2 * i], m[2 * i + 1]}, mod);
+        out[((size_t)p.b.out_limb[d.map_off + row] << p.log_n) + j] = fp_to_u64(fp_canonical(acc, mod));
     }
 }
 
@@ -379,9 +415,19 @@ hipError_t launch_bconv(const Tables &t, const BconvArgs &a, hipStream_t s) {
 
 hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s) {
     if (b.n_units == 0) return hipSuccess;
-    const uint32_t cg = (b.max_rows + kBatchRows - 1) / kBatchRows, kg = (b.max_copy + kBatchRows - 1) / kBatchRows;
-    BconvBatchK p{b, t.moduli, t.barrett, t.log_n, cg};
-    hipLaunchKernelGGL(bconv_batched_kernel, dim3((1u << t.log_n) / kThreads, cg + kg, b.n_units), dim3(kThreads), 0, s, p);
+    static const uint32_t target = [] {
+        const char *e = getenv("CAHEL_HIP_BCONV_ROWS");
+        return e ? (uint32_t)atoi(e) : 6u;
+    }();
+    const uint32_t cg = (b.max_rows + target - 1) / target;
+    const uint32_t rows_per = (b.max_rows + cg - 1) / cg;
+    const uint32_t kg = (b.max_copy + rows_per - 1) / rows_per;
+    BconvBatchK p{b, t.moduli, t.barrett, t.log_n, cg, rows_per};
+    const dim3 grid((1u << t.log_n) / kThreads, cg + kg, b.n_units);
+    if (b.mat_fp)
+        hipLaunchKernelGGL(bconv_batched_fp_kernel, grid, dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL(bconv_batched_kernel, grid, dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
 
