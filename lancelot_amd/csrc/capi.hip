@@ -260,11 +260,11 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         if (!rc) rc = upload(ctx, &ctx->d_phat_mod_q, d->phat_mod_q, (size_t)d->size_q * d->size_p);
     }
     if (!rc) {
-        // FP64 back end: (w, w/q) twiddles, un-halved inverse twiddles, per-table constants
+        // FP64 back end: twiddles as doubles (inverse ones un-halved), per-table constants
         const char *env = getenv("CAHEL_HIP_NO_FP64");
         ctx->use_fp = !(env && env[0] == '1');
         ctx->fp_ok.assign(qp, 0);
-        std::vector<double> psi_fp(2 * qp * n, 0.0), ipsi_fp(2 * qp * n, 0.0), consts(4 * qp, 0.0);
+        std::vector<double> psi_fp(qp * n, 0.0), ipsi_fp(qp * n, 0.0), consts(4 * qp, 0.0);
         for (size_t t = 0; t < qp; t++) {
             const uint64_t q = d->moduli[t];
             if (q >> 50) continue;
@@ -274,10 +274,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
                 const uint64_t w = d->psi[2 * (t * n + i)];
                 uint64_t iw = 2 * d->ipsi_div2[2 * (t * n + i)];
                 if (iw >= q) iw -= q;
-                psi_fp[2 * (t * n + i)] = (double)w;
-                psi_fp[2 * (t * n + i) + 1] = (double)w / qd;
-                ipsi_fp[2 * (t * n + i)] = (double)iw;
-                ipsi_fp[2 * (t * n + i) + 1] = (double)iw / qd;
+                psi_fp[t * n + i] = (double)w;
+                ipsi_fp[t * n + i] = (double)iw;
             }
             const uint64_t ninv = q - (q - 1) / n;  // q = 1 mod 2N, so N * (q - (q-1)/N) = 1 mod q
             consts[4 * t] = qd;

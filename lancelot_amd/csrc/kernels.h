@@ -48,7 +48,7 @@ struct NttArgs {
     uint32_t in_poly_stride;
     uint32_t out_poly_stride;
     const uint64_t *tw;       // [tables][N][2] (operand, Shoup quotient)
-    const double *tw_fp;      // [tables][N][2] (w, w/q) for the FP64 back end (primes below 2^50)
+    const double *tw_fp;      // [tables][N] twiddles as exact doubles for the FP64 back end (primes below 2^50)
     const double *fp_consts;  // [tables][4]: q, 1/q, N^-1 mod q, (N^-1 mod q)/q
     const uint64_t *moduli;   // [tables]
     const uint64_t *barrett;  // [tables][2]

@@ -158,9 +158,10 @@ __device__ __forceinline__ void gs_block(uint64_t *v, const uint64_t *table, uin
 // in a double; residues are signed and lazy (|v| < 2^53).  All steps below are exact integer
 // computations, so the canonical result equals the integer path's bit for bit.
 //
-//   x * w = h + l exactly (h = fl(x w), l = fma(x, w, -h)); k = rint(x * fl(w/q)) differs from
-//   x w / q by at most 1/2 + |x| 2^-52; h - k q and (h - k q) + l are integers below 2^52 in
-//   magnitude, hence exact; the result is congruent to x w with |r| <= (1/2 + |x| 2^-52) q.
+//   x * w = h + l exactly (h = fl(x w), l = fma(x, w, -h)); k = rint(x * winv), winv ~ w/q with
+//   relative error at most 2^-52, differs from x w / q by at most 1/2 + 1.5 |x| 2^-52; h - k q and
+//   (h - k q) + l are integers below 2^53 in magnitude, hence exact; the result is congruent to x w
+//   with |r| <= (1/2 + 1.5 |x| 2^-52) q, i.e. (1/2 + 0.375 b) q for |x| <= b q, q < 2^50.
 // ---------------------------------------------------------------------------------------------------
 namespace he {
 
@@ -200,13 +201,17 @@ __device__ __forceinline__ double fp_canonical(double v, FpMod m) {
     return c < 0.0 ? c + m.q : c;
 }
 
-__device__ __forceinline__ FpTw load_fptw(const double *table, size_t idx) {
-    const double2 v = reinterpret_cast<const double2 *>(table)[idx];
-    return FpTw{v.x, v.y};
+// Twiddle tables hold w only (8 bytes per entry: the tables are as large as the data they transform, so
+// their size is HBM traffic); the quotient estimate w * fl(1/q) has relative error 2^-52, which with the
+// rounding of x * winv puts k within 1/2 + 1.5 |x| 2^-52 of x w / q.
+__device__ __forceinline__ FpTw load_fptw(const double *table, size_t idx, FpMod m) {
+    const double w = table[idx];
+    return FpTw{w, w * m.qinv};
 }
 
 // Forward block on lazy signed doubles.  REDUCE_FIRST brings every input back to |v| <= q/2; from there
-// (or from canonical inputs) the bound grows by 1.25 b + 0.5 per stage: below 5.4 q after four stages.
+// (or from canonical inputs) the bound grows by 1.375 b + 0.5 per stage: 5.3 q after four stages, 7.1 q from
+// canonical inputs, always below 8 q < 2^53.
 template <int LOGR, bool REDUCE_FIRST>
 __device__ __forceinline__ void fp_ct_block(double *v, const double *table, uint32_t idx, FpMod m) {
     constexpr int R = 1 << LOGR;
@@ -219,7 +224,7 @@ __device__ __forceinline__ void fp_ct_block(double *v, const double *table, uint
         const int half = R >> (l + 1);
 #pragma unroll
         for (int b = 0; b < (1 << l); b++) {
-            const FpTw tw = load_fptw(table, ((size_t)idx << l) + b);
+            const FpTw tw = load_fptw(table, ((size_t)idx << l) + b, m);
 #pragma unroll
             for (int j = 0; j < half; j++) {
                 const double x = v[2 * b * half + j];
@@ -232,7 +237,8 @@ __device__ __forceinline__ void fp_ct_block(double *v, const double *table, uint
 }
 
 // Inverse block (no halving: the factor 1/N is applied once at the end of the transform).  Sums double
-// per stage, so after two stages the sum outputs are reduced again; outputs stay below 6 q.
+// per stage, so after two stages the sum outputs are reduced again; outputs stay at or below 5 q (8 q from
+// canonical inputs without REDUCE_FIRST), which is below 2^53.
 template <int LOGR, bool REDUCE_FIRST>
 __device__ __forceinline__ void fp_gs_block(double *v, const double *table, uint32_t idx, FpMod m) {
     constexpr int R = 1 << LOGR;
@@ -245,7 +251,7 @@ __device__ __forceinline__ void fp_gs_block(double *v, const double *table, uint
         const int half = R >> (l + 1);
 #pragma unroll
         for (int b = 0; b < (1 << l); b++) {
-            const FpTw tw = load_fptw(table, ((size_t)idx << l) + b);
+            const FpTw tw = load_fptw(table, ((size_t)idx << l) + b, m);
 #pragma unroll
             for (int j = 0; j < half; j++) {
                 const double x = v[2 * b * half + j], y = v[2 * b * half + j + half];

@@ -90,7 +90,7 @@ __device__ __forceinline__ IntCtx int_ctx(const NttArgs &a, uint32_t table) {
 
 __device__ __forceinline__ FpCtx fp_ctx(const NttArgs &a, uint32_t table) {
     const double *c = a.fp_consts + 4 * (size_t)table;
-    return FpCtx{FpMod{c[0], c[1]}, a.tw_fp + ((size_t)table << (a.log_n + 1))};
+    return FpCtx{FpMod{c[0], c[1]}, a.tw_fp + ((size_t)table << a.log_n)};
 }
 
 // r stages on a tile held in LDS.  Tile index bits: [upper][mid: r bits][lower: low_bits]; the 2^r
