@@ -32,6 +32,8 @@ struct Level {
     std::vector<Digit> digits;
     LimbJob *d_modup_jobs = nullptr;     // NTT jobs over the converted limbs of all digits
     uint32_t n_modup_jobs = 0;
+    LimbGroup *d_modup_groups = nullptr; // runs of those jobs that share a modulus table
+    uint32_t n_modup_groups = 0;
     // batched base conversion (all digits of ModUp / all polynomials of ModDown in one launch)
     BconvDesc *d_modup_descs = nullptr, *d_moddown_descs = nullptr;
     uint32_t *d_modup_limb = nullptr, *d_modup_table = nullptr;
@@ -406,8 +408,18 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
                 if (rc) return rc;
             }
         }
+        // limbs with the same modulus sit together so that one set of workgroups can share the twiddle table
+        std::stable_sort(jobs.begin(), jobs.end(), [](const LimbJob &x, const LimbJob &y) { return x.table < y.table; });
+        std::vector<LimbGroup> groups;
+        for (uint32_t j = 0; j < jobs.size(); j++) {
+            if (groups.empty() || jobs[groups.back().first].table != jobs[j].table || groups.back().count == 4)
+                groups.push_back(LimbGroup{j, 0});
+            groups.back().count++;
+        }
         lv.n_modup_jobs = (uint32_t)jobs.size();
+        lv.n_modup_groups = (uint32_t)groups.size();
         rc = upload(ctx, &lv.d_modup_jobs, jobs.data(), jobs.size());
+        if (!rc) rc = upload(ctx, &lv.d_modup_groups, groups.data(), groups.size());
         if (rc) return rc;
     }
     lv.set = true;
@@ -575,6 +587,8 @@ int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out
     fwd.out = out;
     fwd.jobs = lv->d_modup_jobs;
     fwd.n_jobs = lv->n_modup_jobs;
+    fwd.groups = lv->d_modup_groups;
+    fwd.n_groups = lv->n_modup_groups;
     HE_HIP(launch_ntt_forward(fwd, 1, fp_for_level(ctx, L), S(s)));
     return HE_OK;
 }

@@ -12,6 +12,13 @@ struct LimbJob {
     uint32_t table;
 };
 
+// Consecutive jobs of an explicit list that share a modulus table: the blocks pass of the NTT gives each
+// group to one set of workgroups so that the table is read once.
+struct LimbGroup {
+    uint32_t first;
+    uint32_t count;
+};
+
 // How limb i (0 <= i < limbs) of every polynomial maps to a modulus table:
 //   table(i) = first + i             for i < split
 //   table(i) = tail_first + i - split  otherwise
@@ -54,6 +61,9 @@ struct NttArgs {
     const uint64_t *barrett;  // [tables][2]
     const LimbJob *jobs;      // explicit list (then in/out limbs are absolute, no prologue/epilogue)
     uint32_t n_jobs;
+    const LimbGroup *groups;  // partition of `jobs` into runs with one table each (required with `jobs`)
+    uint32_t n_groups;
+    uint32_t batch, n_polys;  // filled in by the launcher
     uint32_t log_n;
     LimbMap map;
     int pro_mode;

@@ -268,4 +268,71 @@ __device__ __forceinline__ void fp_gs_block(double *v, const double *table, uint
     }
 }
 
+// The same blocks with the 2^LOGR - 1 twiddles already in registers (tw[2^l - 1 + b] for stage l, sub-block b):
+// a workgroup that transforms several limbs of one modulus loads them once.
+template <int LOGR>
+__device__ __forceinline__ void fp_load_block_tw(double *tw, const double *table, uint32_t idx) {
+#pragma unroll
+    for (int l = 0; l < LOGR; l++)
+#pragma unroll
+        for (int b = 0; b < (1 << l); b++) tw[(1 << l) - 1 + b] = table[((size_t)idx << l) + b];
+}
+
+template <int LOGR, bool REDUCE_FIRST>
+__device__ __forceinline__ void fp_ct_block_tw(double *v, const double *tw, FpMod m) {
+    constexpr int R = 1 << LOGR;
+    if (REDUCE_FIRST) {
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = fp_reduce(v[j], m);
+    }
+#pragma unroll
+    for (int l = 0; l < LOGR; l++) {
+        const int half = R >> (l + 1);
+#pragma unroll
+        for (int b = 0; b < (1 << l); b++) {
+            double w = tw[(1 << l) - 1 + b];
+            asm volatile("" : "+v"(w));  // keeps w * qinv out of the caller's loop-invariant registers
+            const FpTw t{w, w * m.qinv};
+#pragma unroll
+            for (int j = 0; j < half; j++) {
+                const double x = v[2 * b * half + j];
+                const double p = fp_mulmod(v[2 * b * half + j + half], t, m);
+                v[2 * b * half + j] = x + p;
+                v[2 * b * half + j + half] = x - p;
+            }
+        }
+    }
+}
+
+template <int LOGR, bool REDUCE_FIRST>
+__device__ __forceinline__ void fp_gs_block_tw(double *v, const double *tw, FpMod m) {
+    constexpr int R = 1 << LOGR;
+    if (REDUCE_FIRST) {
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = fp_reduce(v[j], m);
+    }
+#pragma unroll
+    for (int l = LOGR - 1; l >= 0; l--) {
+        const int half = R >> (l + 1);
+#pragma unroll
+        for (int b = 0; b < (1 << l); b++) {
+            double w = tw[(1 << l) - 1 + b];
+            asm volatile("" : "+v"(w));  // keeps w * qinv out of the caller's loop-invariant registers
+            const FpTw t{w, w * m.qinv};
+#pragma unroll
+            for (int j = 0; j < half; j++) {
+                const double x = v[2 * b * half + j], y = v[2 * b * half + j + half];
+                v[2 * b * half + j] = x + y;
+                v[2 * b * half + j + half] = fp_mulmod(x - y, t, m);
+            }
+        }
+        if (LOGR == 4 && l == 2) {
+#pragma unroll
+            for (int b = 0; b < (1 << l); b++)
+#pragma unroll
+                for (int j = 0; j < half; j++) v[2 * b * half + j] = fp_reduce(v[2 * b * half + j], m);
+        }
+    }
+}
+
 }  // namespace he

@@ -37,6 +37,10 @@ constexpr uint32_t kLdsWords = kTile + (kTile >> 4);
 
 __device__ __forceinline__ uint32_t skew(uint32_t e) { return e + (e >> 4); }
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global load and
+// store of the wave, which would serialise a prefetch issued before it with the butterflies after it.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Workgroups are dealt round-robin to the 8 XCDs; give every XCD a contiguous range of logical ids so
 // that the tiles of one limb (which share a twiddle table) meet in one L2.
 __device__ __forceinline__ uint32_t logical_block() {
@@ -101,7 +105,7 @@ __device__ __forceinline__ void tile_pass(uint64_t *lds, uint32_t tile_elems, ui
     constexpr int R = 1 << LOGR;
     const uint32_t groups = tile_elems >> LOGR;
     const uint32_t low_mask = (1u << low_bits) - 1;
-    for (uint32_t g = threadIdx.x; g < groups; g += kThreads) {
+    for (uint32_t g = threadIdx.x; g < groups; g += blockDim.x) {
         const uint32_t upper = g >> low_bits;
         const uint32_t base = (upper << (low_bits + LOGR)) | (g & low_mask);
         uint64_t v[R];
@@ -123,7 +127,7 @@ __device__ __forceinline__ void tile_pass_fp(uint64_t *lds, uint32_t tile_elems,
     double *ld = reinterpret_cast<double *>(lds);
     const uint32_t groups = tile_elems >> LOGR;
     const uint32_t low_mask = (1u << low_bits) - 1;
-    for (uint32_t g = threadIdx.x; g < groups; g += kThreads) {
+    for (uint32_t g = threadIdx.x; g < groups; g += blockDim.x) {
         const uint32_t upper = g >> low_bits;
         const uint32_t base = (upper << (low_bits + LOGR)) | (g & low_mask);
         double v[R];
@@ -275,111 +279,256 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
 
 // ---------------------------------------------------------------------------------------------------
 // blocks pass: the 8 stages that stay inside 256 consecutive words
+//
+// A workgroup of T threads owns a tile of 16 T consecutive words (T = 128 or 256) and walks through every
+// limb of its unit: the limbs of one unit share a modulus, hence a twiddle table, and the table is as large
+// as a limb, so reading it once per unit instead of once per limb removes up to half of the pass's HBM
+// traffic.  The next limb's tile is fetched into registers while the current one is transformed.
 // ---------------------------------------------------------------------------------------------------
-template <bool FWD, bool FP>
-__global__ __launch_bounds__(kThreads) void ntt_blocks_kernel(NttArgs a) {
-    __shared__ uint64_t lds[kLdsWords];
-    const uint32_t lr = a.log_n - 8;                       // log2(number of 256-blocks per limb)
-    const uint32_t log_b = lr < 4 ? lr : 4;                // blocks per tile = 2^log_b
-    const uint32_t tile_elems = 256u << log_b;
-    const uint32_t tiles_per_limb = 1u << (lr - log_b);
+struct Unit {
+    uint32_t j0, jstride, count;
+};
 
+// map mode: unit = (limb i, group of `batch` polynomials); list mode: unit = group of consecutive jobs
+__device__ __forceinline__ Unit decode_unit(const NttArgs &a, uint32_t u) {
+    if (a.jobs) {
+        const LimbGroup g = a.groups[u];
+        return Unit{g.first, 1u, g.count};
+    }
+    const uint32_t limb = u % a.map.limbs, pg = u / a.map.limbs;
+    const uint32_t p0 = pg * a.batch;
+    const uint32_t cnt = a.n_polys - p0 < a.batch ? a.n_polys - p0 : a.batch;
+    return Unit{p0 * a.map.limbs + limb, a.map.limbs, cnt};
+}
+
+// A workgroup of T threads owns 16 T consecutive words: T = 256 or 128 for N >= 2048, N / 16 below that, so
+// that every thread moves exactly 16 words and no access needs a bounds check (straight-line code lets the
+// compiler count the loads and stores in flight instead of draining them at every step).
+struct BlocksGeom {
+    uint32_t idx0, idx1;
+    size_t off;
+    Unit unit;
+};
+
+__device__ __forceinline__ BlocksGeom blocks_geom(const NttArgs &a) {
+    const uint32_t lr = a.log_n - 8;                       // log2(number of 256-blocks per limb)
+    const uint32_t tile_elems = blockDim.x << 4;
+    const uint32_t log_b = 31 - __builtin_clz(tile_elems >> 8);  // blocks per tile = 2^log_b
+    const uint32_t tiles_per_limb = 1u << (lr - log_b);
     const uint32_t lb = logical_block();
-    const Job job = decode_job(a, lb / tiles_per_limb);
+    BlocksGeom g;
+    g.unit = decode_unit(a, lb / tiles_per_limb);
     const uint32_t tile = lb % tiles_per_limb;
-    const size_t off = (size_t)tile * tile_elems;
+    g.off = (size_t)tile * tile_elems;
     const uint32_t blk0 = tile << log_b;                   // first 256-block of this tile within the limb
+    g.idx0 = (1u << lr) + blk0;
+    g.idx1 = (1u << (lr + 4)) + (blk0 << 4);
+    return g;
+}
+
+constexpr int kPer = 16;  // words per thread in the blocks pass
+constexpr int kMaxGroup = 4;  // most jobs in one LimbGroup
+
+// FP64 back end.  EPI compiles the fused forward epilogues in (they cost 64 registers).
+template <bool FWD, bool EPI>
+__global__ __launch_bounds__(kThreads) void ntt_blocks_fp_kernel(NttArgs a) {
+    __shared__ uint64_t lds[kLdsWords];
+    const uint32_t nthreads = blockDim.x;
+    const BlocksGeom g = blocks_geom(a);
+    const size_t off = g.off;
     const size_t n = (size_t)1 << a.log_n;
     double *ld = reinterpret_cast<double *>(lds);
+    const bool has_addend = EPI && a.epi_mode == NTT_EPI_SUB_MUL_ADD;
 
-    const uint64_t *src = FWD ? job.out : job.in;  // the forward blocks pass continues on the rows pass's output
-    if (FP && !FWD) {
-        for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) ld[skew(e)] = fp_from_u64(src[off + e]);
-    } else {
-        for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) lds[skew(e)] = src[off + e];
-    }
-    __syncthreads();
+    Job job = decode_job(a, g.unit.j0);
+    const FpCtx fc = fp_ctx(a, job.table);
+    const FpMod m = fc.m;
 
-    const bool epi = a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD;
-    const uint64_t *minuend = epi ? a.epi_a + ((size_t)job.poly * a.epi_a_poly_stride + job.limb) * n + off : nullptr;
-    const uint64_t *addend =
-        a.epi_mode == NTT_EPI_SUB_MUL_ADD ? a.epi_b + ((size_t)job.poly * a.epi_b_poly_stride + job.limb) * n + off : nullptr;
-    uint64_t *dst = epi ? a.epi_dst + ((size_t)job.poly * a.epi_dst_poly_stride + job.limb) * n + off : job.out + off;
-    // the epilogue operands are fetched now so that their latency hides behind the butterflies
-    constexpr int kPer = kTile / kThreads;
-    uint64_t pre_a[kPer], pre_b[kPer];
-    if (FWD && epi) {
+    // this thread's group in either register pass, and its twiddles (the same for every limb of the unit)
+    const uint32_t gi = threadIdx.x;
+    const uint32_t base0 = ((gi >> 4) << 8) | (gi & 15);   // pass with stride 16
+    const uint32_t base1 = gi << 4;                        // pass with stride 1
+    double tw0[15], tw1[15];
+    fp_load_block_tw<4>(tw0, fc.tw, g.idx0 + (gi >> 4));
+    fp_load_block_tw<4>(tw1, fc.tw, g.idx1 + gi);
+
+    // list mode: the unit's jobs are read before the first store, so that they stay scalar loads
+    LimbJob pre[kMaxGroup];
+#pragma unroll
+    for (int i = 0; i < kMaxGroup; i++) pre[i] = (a.jobs && (uint32_t)i < g.unit.count) ? a.jobs[g.unit.j0 + i] : LimbJob{0, 0};
+    auto entry = [&](uint32_t b) {
+        if (!a.jobs) return decode_job(a, g.unit.j0 + b * g.unit.jstride);
+        LimbJob lj = pre[0];
+#pragma unroll
+        for (int i = 1; i < kMaxGroup; i++) lj = b == (uint32_t)i ? pre[i] : lj;
+        return Job{a.in + (size_t)lj.data_limb * n, a.out + (size_t)lj.data_limb * n, lj.table, 0, 0};
+    };
+
+    uint64_t nx[kPer];
+    auto stage = [&]() {  // prefetched words -> LDS
 #pragma unroll
         for (int i = 0; i < kPer; i++) {
-            const uint32_t e = threadIdx.x + i * kThreads;
-            pre_a[i] = e < tile_elems ? minuend[e] : 0;
-            pre_b[i] = (addend && e < tile_elems) ? addend[e] : 0;
+            const uint32_t e = threadIdx.x + i * nthreads;
+            if (!FWD)
+                ld[skew(e)] = fp_from_u64(nx[i]);
+            else
+                lds[skew(e)] = nx[i];
         }
-    }
-
-    if (FP) {
-        const FpCtx c = fp_ctx(a, job.table);
-        if (FWD) {
-            tile_pass_fp<4, true, true>(lds, tile_elems, 4, (1u << lr) + blk0, c);
-            __syncthreads();
-            tile_pass_fp<4, true, true>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), c);
-            __syncthreads();
-            if (epi) {
-                const double wd = fp_from_u64(a.w[2 * job.limb]);
-                const FpTw w{wd, wd * c.m.qinv};
+        lds_barrier();
+    };
+    {
+        const uint64_t *src = (FWD ? job.out : job.in) + off;  // the forward blocks pass continues on the rows pass's output
 #pragma unroll
-                for (int i = 0; i < kPer; i++) {
-                    const uint32_t e = threadIdx.x + i * kThreads;
-                    if (e < tile_elems) {
-                        const double v = fp_canonical(ld[skew(e)], c.m);
-                        double r = fp_mulmod(fp_from_u64(pre_a[i]) - v, w, c.m);
-                        if (addend) r += fp_from_u64(pre_b[i]);
-                        dst[e] = fp_to_u64(fp_canonical(r, c.m));
-                    }
-                }
-            } else {
-                for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads)
-                    dst[e] = fp_to_u64(fp_canonical(ld[skew(e)], c.m));
-            }
-        } else {
-            tile_pass_fp<4, false, false>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), c);
-            __syncthreads();
-            tile_pass_fp<4, false, true>(lds, tile_elems, 4, (1u << lr) + blk0, c);
-            __syncthreads();
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) job.out[off + e] = lds[skew(e)];
-        }
-        return;
+        for (int i = 0; i < kPer; i++) nx[i] = src[threadIdx.x + i * nthreads];
     }
+    // the twiddles have arrived before the loop starts: inside it only the prefetch is in flight
+#pragma unroll
+    for (int i = 0; i < 15; i++) asm volatile("" ::"v"(tw0[i]), "v"(tw1[i]));
+    stage();
 
-    const IntCtx c = int_ctx(a, job.table);
-    const uint64_t q = c.q;
-    if (FWD) {
-        tile_pass<4, true>(lds, tile_elems, 4, (1u << lr) + blk0, c);
-        __syncthreads();
-        tile_pass<4, true>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), c);
-        __syncthreads();
-        if (epi) {
-            const Shoup w = load_shoup(a.w, job.limb);
+    for (uint32_t b = 0;; b++) {
+        // the next limb's tile and this limb's epilogue operands travel while the butterflies run
+        const bool more = b + 1 < g.unit.count;
+        // (with a fused epilogue the registers go to its operands instead and the next tile is fetched late)
+        Job next = job;
+        if (more) next = entry(b + 1);
+        if (more && !EPI) {
+            const uint64_t *src = (FWD ? next.out : next.in) + off;
+#pragma unroll
+            for (int i = 0; i < kPer; i++) nx[i] = src[threadIdx.x + i * nthreads];
+        }
+        const size_t epi_off = off + (size_t)job.limb * n;
+        uint64_t *dst = (FWD && EPI) ? a.epi_dst + (size_t)job.poly * a.epi_dst_poly_stride * n + epi_off : job.out + off;
+        uint64_t pre_a[EPI ? kPer : 1], pre_b[EPI ? kPer : 1];
+        if (FWD && EPI) {
+            const uint64_t *minuend = a.epi_a + (size_t)job.poly * a.epi_a_poly_stride * n + epi_off;
+            const uint64_t *addend = has_addend ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
 #pragma unroll
             for (int i = 0; i < kPer; i++) {
-                const uint32_t e = threadIdx.x + i * kThreads;
-                if (e < tile_elems) {
-                    uint64_t v = reduce_4q(lds[skew(e)], q);
-                    uint64_t r = mul_shoup(sub_mod(pre_a[i], v, q), w, q);
-                    if (addend) r = add_mod(r, pre_b[i], q);
+                pre_a[EPI ? i : 0] = minuend[threadIdx.x + i * nthreads];
+                pre_b[EPI ? i : 0] = addend[threadIdx.x + i * nthreads];
+            }
+        }
+
+        double v[16];
+        if (FWD) {
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[skew(base0 + (j << 4))];
+            fp_ct_block_tw<4, true>(v, tw0, m);
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
+            lds_barrier();
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[skew(base1 + j)];
+            fp_ct_block_tw<4, true>(v, tw1, m);
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[skew(base1 + j)] = v[j];
+            lds_barrier();
+#pragma unroll
+            for (int i = 0; i < kPer; i++) v[i] = fp_canonical(ld[skew(threadIdx.x + i * nthreads)], m);
+            if (EPI) {
+                const double wd = fp_from_u64(a.w[2 * job.limb]);
+                const FpTw w{wd, wd * m.qinv};
+#pragma unroll
+                for (int i = 0; i < kPer; i++) {
+                    double r = fp_mulmod(fp_from_u64(pre_a[EPI ? i : 0]) - v[i], w, m);
+                    if (has_addend) r += fp_from_u64(pre_b[EPI ? i : 0]);
+                    v[i] = fp_canonical(r, m);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kPer; i++) dst[threadIdx.x + i * nthreads] = fp_to_u64(v[i]);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[skew(base1 + j)];
+            fp_gs_block_tw<4, false>(v, tw1, m);
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[skew(base1 + j)] = v[j];
+            lds_barrier();
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[skew(base0 + (j << 4))];
+            fp_gs_block_tw<4, true>(v, tw0, m);
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
+            lds_barrier();
+            // lazy signed doubles go to the rows pass
+            uint64_t o[kPer];
+#pragma unroll
+            for (int i = 0; i < kPer; i++) o[i] = lds[skew(threadIdx.x + i * nthreads)];
+#pragma unroll
+            for (int i = 0; i < kPer; i++) dst[threadIdx.x + i * nthreads] = o[i];
+        }
+        if (!more) break;
+        if (EPI) {
+            const uint64_t *src = (FWD ? next.out : next.in) + off;
+#pragma unroll
+            for (int i = 0; i < kPer; i++) nx[i] = src[threadIdx.x + i * nthreads];
+        }
+        lds_barrier();  // every read of this tile is done before the next one overwrites it
+        stage();
+        job = next;
+    }
+}
+
+// Integer back end (twiddles stay in the table: 30 Shoup pairs per thread do not fit in registers).
+template <bool FWD>
+__global__ __launch_bounds__(kThreads) void ntt_blocks_int_kernel(NttArgs a) {
+    __shared__ uint64_t lds[kLdsWords];
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t tile_elems = nthreads << 4;
+    const BlocksGeom g = blocks_geom(a);
+    const size_t off = g.off;
+    const size_t n = (size_t)1 << a.log_n;
+    const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD);
+    const bool has_addend = FWD && a.epi_mode == NTT_EPI_SUB_MUL_ADD;
+
+    for (uint32_t b = 0; b < g.unit.count; b++) {
+        const Job job = decode_job(a, g.unit.j0 + b * g.unit.jstride);
+        const IntCtx ic = int_ctx(a, job.table);
+        const uint64_t q = ic.q;
+        const uint64_t *src = (FWD ? job.out : job.in) + off;
+#pragma unroll
+        for (int i = 0; i < kPer; i++) lds[skew(threadIdx.x + i * nthreads)] = src[threadIdx.x + i * nthreads];
+        __syncthreads();
+        const size_t epi_off = off + (size_t)job.limb * n;
+        if (FWD) {
+            tile_pass<4, true>(lds, tile_elems, 4, g.idx0, ic);
+            __syncthreads();
+            tile_pass<4, true>(lds, tile_elems, 0, g.idx1, ic);
+            __syncthreads();
+            if (epi) {
+                const uint64_t *minuend = a.epi_a + (size_t)job.poly * a.epi_a_poly_stride * n + epi_off;
+                const uint64_t *addend = has_addend ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
+                uint64_t *dst = a.epi_dst + (size_t)job.poly * a.epi_dst_poly_stride * n + epi_off;
+                const Shoup w = load_shoup(a.w, job.limb);
+#pragma unroll
+                for (int i = 0; i < kPer; i++) {
+                    const uint32_t e = threadIdx.x + i * nthreads;
+                    const uint64_t c = reduce_4q(lds[skew(e)], q);
+                    uint64_t r = mul_shoup(sub_mod(minuend[e], c, q), w, q);
+                    if (has_addend) r = add_mod(r, addend[e], q);
                     dst[e] = r;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < kPer; i++) {
+                    const uint32_t e = threadIdx.x + i * nthreads;
+                    job.out[off + e] = reduce_4q(lds[skew(e)], q);
                 }
             }
         } else {
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) dst[e] = reduce_4q(lds[skew(e)], q);
+            tile_pass<4, false>(lds, tile_elems, 0, g.idx1, ic);
+            __syncthreads();
+            tile_pass<4, false>(lds, tile_elems, 4, g.idx0, ic);
+            __syncthreads();
+            // lazy values in [0, 2q) go to the rows pass
+#pragma unroll
+            for (int i = 0; i < kPer; i++) {
+                const uint32_t e = threadIdx.x + i * nthreads;
+                job.out[off + e] = lds[skew(e)];
+            }
         }
-    } else {
-        tile_pass<4, false>(lds, tile_elems, 0, (1u << (lr + 4)) + (blk0 << 4), c);
-        __syncthreads();
-        tile_pass<4, false>(lds, tile_elems, 4, (1u << lr) + blk0, c);
-        __syncthreads();
-        // lazy values in [0, 2q) go to the rows pass
-        for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) job.out[off + e] = lds[skew(e)];
+        __syncthreads();  // every read of this tile is done before the next one overwrites it
     }
 }
 
@@ -403,11 +552,45 @@ hipError_t launch_rows(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
     return hipGetLastError();
 }
 
+// Geometry of the blocks pass: polynomials per unit (map mode) and workgroup size, chosen so that the grid
+// still fills 256 CUs a few times over.
+struct BlocksPlan {
+    uint32_t batch, threads, grid;
+};
+
+BlocksPlan plan_blocks(const NttArgs &a, uint32_t n_polys) {
+    const uint32_t n = 1u << a.log_n;
+    // threads of a workgroup for a wished tile of `want` words (a limb may be smaller than that)
+    auto threads = [&](uint32_t want) { return (n < want ? n : want) >> 4; };
+    auto tiles = [&](uint32_t want) { return n / (threads(want) << 4); };
+    BlocksPlan p;
+    uint32_t units;
+    if (a.jobs) {
+        p.batch = 1;
+        units = a.n_groups;
+    } else {
+        // batching pays once the launch has enough workgroups without splitting the polynomials
+        p.batch = (n_polys > 1 && a.map.limbs * tiles(2048) >= 512) ? n_polys : 1;
+        units = a.map.limbs * ((n_polys + p.batch - 1) / p.batch);
+    }
+    const uint32_t want = units * tiles(4096) >= 1024 ? 4096 : 2048;
+    p.threads = threads(want);
+    p.grid = units * tiles(want);
+    return p;
+}
+
 template <bool FWD, bool FP>
-hipError_t launch_blocks(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
-    const uint32_t lr = a.log_n - 8;
-    const uint32_t log_b = lr < 4 ? lr : 4;
-    hipLaunchKernelGGL((ntt_blocks_kernel<FWD, FP>), dim3(n_jobs << (lr - log_b)), dim3(kThreads), 0, s, a);
+hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
+    const BlocksPlan p = plan_blocks(a, n_polys);
+    a.batch = p.batch;
+    a.n_polys = n_polys;
+    const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD);
+    if (!FP)
+        hipLaunchKernelGGL((ntt_blocks_int_kernel<FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
+    else if (epi)
+        hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
+    else
+        hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, false>), dim3(p.grid), dim3(p.threads), 0, s, a);
     return hipGetLastError();
 }
 
@@ -419,14 +602,14 @@ hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, bool fp, hipSt
     if (n_jobs == 0) return hipSuccess;
     hipError_t e = fp ? launch_rows<true, true>(a, n_jobs, s) : launch_rows<true, false>(a, n_jobs, s);
     if (e != hipSuccess) return e;
-    return fp ? launch_blocks<true, true>(a, n_jobs, s) : launch_blocks<true, false>(a, n_jobs, s);
+    return fp ? launch_blocks<true, true>(a, n_polys, s) : launch_blocks<true, false>(a, n_polys, s);
 }
 
 hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s) {
     if (a.log_n < 9 || a.log_n > 16) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
-    hipError_t e = fp ? launch_blocks<false, true>(a, n_jobs, s) : launch_blocks<false, false>(a, n_jobs, s);
+    hipError_t e = fp ? launch_blocks<false, true>(a, n_polys, s) : launch_blocks<false, false>(a, n_polys, s);
     if (e != hipSuccess) return e;
     NttArgs rows = a;
     rows.in = a.out;  // the rows pass continues in place on the output buffer
