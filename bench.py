@@ -28,6 +28,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 LOG_N, SIZE_Q, SIZE_P, BITS, SCALE = 16, 24, 8, 50, 2.0 ** 40
+# HBM bytes of one 72-limb forward NTT call, from the FETCH_SIZE / WRITE_SIZE counters scaled by a copy of known
+# size (profiles/ntt_forward_72limbs_n65536.md)
+NTT72_TRAFFIC_BYTES = 164_006_912
 HBM_PEAK_GBS = 8000.0
 
 
@@ -248,7 +251,7 @@ def main():
         "check": {"c_abi_equals_evaluator": same, "decrypt_max_abs_err_vs_xy": max_err},
         "roofline": {"bound": "hbm", "kernel": "ntt_rows_kernel + ntt_blocks_kernel (forward NTT, 72 limbs of ModUp)",
                      "achieved": roof_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": roof_gbs / HBM_PEAK_GBS,
-                     "traffic": None, "ms_per_launch": fwd72, "algorithmic_bytes_per_launch": ntt_bytes},
+                     "traffic": NTT72_TRAFFIC_BYTES, "ms_per_launch": fwd72, "algorithmic_bytes_per_launch": ntt_bytes},
         "ntt": ntt, "rotate": rotate,
     }
     if not args.no_cpu_baseline:
