@@ -107,13 +107,33 @@ def cpu_baseline(seconds_budget=12.0):
             "ms_per_op": dt * 1e3}
 
 
+def krum_round(seed: int = 2025):
+    """One encrypted Krum round at its real shape (10 clients x 62,006 parameters, N = 2^16, moduli
+    [60, 40, 40, 60], one special prime): seconds per phase and the error against the float64 closed form."""
+    from lancelot_amd import krum
+    rng = np.random.default_rng(seed)
+    updates = [rng.normal(0.0, 0.01, 62006).astype(np.float32) for _ in range(10)]
+    for k in (8, 9):
+        updates[k] = updates[k] * 10
+    t0 = time.perf_counter()
+    state = krum.gpu_init(krum.KrumConfig(seed=seed))
+    setup = time.perf_counter() - t0
+    krum.gpu_krum(updates, state=state)  # warm-up round (pool growth, first-touch of the keys)
+    chosen, dist, timings = krum.gpu_krum(updates, state=state)
+    plain = krum.plain_distance_matrix(updates)
+    off = ~np.eye(10, dtype=bool)
+    return {"workload": "Krum distance round, 10 clients x 62006 parameters, 2 ciphertexts per client, 45 pairs, N=2^16",
+            "setup_s": setup, "round_s": timings, "chosen": chosen, "chosen_plain": krum.krum_select(plain),
+            "max_rel_err_vs_float64": float(np.max(np.abs(dist[off] - plain[off]) / plain[off]))}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--only", choices=["all", "roofline"], default="all",
+    ap.add_argument("--only", choices=["all", "roofline", "krum"], default="all",
                     help="roofline: run just the kernel the roofline object describes (for rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -133,6 +153,9 @@ def main():
     parms.set_galois_elts(cahel.get_elts_from_steps(steps_pow2, n))
     ctx = cahel.context(parms, True, cahel.sec_level_type.tc128)
     ctx.set_seed(2025)
+    if args.only == "krum":
+        print(json.dumps(krum_round()))
+        return
     if args.only == "roofline":
         # just the kernels the roofline object describes, plus one device-to-device copy of known size that
         # calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run
