@@ -1,0 +1,161 @@
+"""Full-size configurations on the GPU.
+
+C1 (N = 2^14, 4 + 1 primes of 50 bits) is small enough for the CPU oracle: HMult + relinearise + rescale is compared
+limb for limb.  At the benchmark sizes (N = 2^16, L = 24, K = 8 and Lancelot's [60, 40, 40, 60] chain) the oracle
+would take minutes, so the checks are properties that do not depend on the size: commutativity of the product
+(bit-exact), decryption of a size-3 ciphertext against its relinearisation, rotation = roll of the slots,
+rotate-and-sum = sum of all slots, and the encrypted Krum distances against the float64 closed form.
+"""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+REL = 2.0 ** -20
+
+
+def _context(logn, bits, size_p, steps=(), seed=2025, sec="none"):
+    import lancelot_amd  # noqa: F401
+    import pyCAHEL as cahel
+    n = 1 << logn
+    mods = cahel.coeff_modulus_create(n, list(bits))
+    parms = cahel.params(cahel.scheme_type.ckks)
+    parms.set_poly_modulus_degree(n)
+    parms.set_coeff_modulus(mods)
+    parms.set_special_modulus_size(size_p)
+    if steps:
+        parms.set_galois_elts(cahel.get_elts_from_steps(list(steps), n))
+    ctx = cahel.context(parms, True, getattr(cahel.sec_level_type, sec))
+    ctx.set_seed(seed)
+    return cahel, parms, ctx, mods
+
+
+def test_c1_hmult_relin_rescale_bit_exact(oracle):
+    """Config C1: N = 2^14, Q = 4 x 50 bits, P = 1 x 50 bits, scale 2^40, 8192 slots."""
+    O = oracle
+    logn, bits = 14, [50] * 5
+    cahel, parms, ctx, mods = _context(logn, bits, 1)
+    p = O.Params(logn, [m.value() for m in mods], 1)
+    ks = O.KeySet(p, seed=2025)
+    sk = cahel.secret_key(parms)
+    sk.gen_secretkey(ctx)
+    ks.gen_secret()
+    pk = cahel.public_key(ctx)
+    sk.gen_publickey(ctx, pk)
+    o_pk = ks.gen_public()
+    rlk = cahel.relin_key(ctx)
+    sk.gen_relinkey(ctx, rlk)
+    o_rlk = ks.gen_relin()
+    enc = cahel.ckks_encoder(ctx)
+    rng = np.random.default_rng(2025)
+    x, y = rng.uniform(-1, 1, p.n // 2), rng.uniform(-1, 1, p.n // 2)
+    px, py = enc.encode(ctx, x, 2.0 ** 40), enc.encode(ctx, y, 2.0 ** 40)
+    cx = pk.encrypt_asymmetric(ctx, px)
+    o_cx = ks.encrypt_asymmetric(o_pk, px.to_numpy())
+    cy = pk.encrypt_asymmetric(ctx, py)
+    o_cy = ks.encrypt_asymmetric(o_pk, py.to_numpy())
+    assert (cx.to_numpy() == o_cx).all() and (cy.to_numpy() == o_cy).all()
+    cahel.multiply_and_relin_inplace(ctx, cx, cy, rlk)
+    cahel.rescale_to_next_inplace(ctx, cx)
+    want = p.rescale(p.relinearize(p.tensor(o_cx, o_cy), o_rlk))
+    assert (cx.to_numpy() == want).all()
+    pt = sk.decrypt(ctx, cx)
+    assert (pt.to_numpy() == ks.decrypt(want, O.gauss_cdt())).all()
+    got = np.array(enc.decode(ctx, pt))
+    assert np.max(np.abs(got - x * y)) < 1e-2           # scale 2^40 after a 50-bit rescale: about 2^30 left
+
+
+@pytest.fixture(scope="module")
+def bench_world():
+    """The benchmark shape: N = 2^16, 24 + 8 primes of 50 bits, keys for the 15 power-of-two steps."""
+    steps = [1 << k for k in range(15)]
+    cahel, parms, ctx, _ = _context(16, [50] * 32, 8, steps, sec="tc128")
+    sk = cahel.secret_key(parms)
+    sk.gen_secretkey(ctx)
+    pk = cahel.public_key(ctx)
+    sk.gen_publickey(ctx, pk)
+    rlk = cahel.relin_key(ctx)
+    sk.gen_relinkey(ctx, rlk)
+    glk = cahel.galois_key(ctx)
+    sk.create_galois_keys(ctx, glk)
+    enc = cahel.ckks_encoder(ctx)
+    rng = np.random.default_rng(2025)
+    n = 1 << 16
+    x, y = rng.uniform(-1, 1, n // 2), rng.uniform(-1, 1, n // 2)
+    cx = pk.encrypt_asymmetric(ctx, enc.encode(ctx, x, 2.0 ** 40))
+    cy = pk.encrypt_asymmetric(ctx, enc.encode(ctx, y, 2.0 ** 40))
+    return dict(cahel=cahel, ctx=ctx, sk=sk, pk=pk, rlk=rlk, glk=glk, enc=enc, x=x, y=y, cx=cx, cy=cy, steps=steps)
+
+
+def _decode(w, ct):
+    return np.array(w["enc"].decode(w["ctx"], w["sk"].decrypt(w["ctx"], ct)))
+
+
+def test_c3_hmult_properties(bench_world):
+    w = bench_world
+    c, ctx = w["cahel"], w["ctx"]
+    xy, yx = c.ciphertext(ctx), c.ciphertext(ctx)
+    c.multiply(ctx, w["cx"], w["cy"], xy)
+    c.multiply(ctx, w["cy"], w["cx"], yx)
+    assert xy.size() == 3 and (xy.to_numpy() == yx.to_numpy()).all()        # the tensor product commutes exactly
+    three = _decode(w, xy)                                                    # size-3 decryption: c0 + c1 s + c2 s^2
+    c.relinearize_inplace(ctx, xy, w["rlk"])
+    c.relinearize_inplace(ctx, yx, w["rlk"])
+    assert xy.size() == 2 and (xy.to_numpy() == yx.to_numpy()).all()
+    two = _decode(w, xy)
+    assert np.max(np.abs(two - three)) < 2.0 ** -20 * max(1.0, np.max(np.abs(three)))   # key-switch noise only
+    # scale 2^80 before the rescale.  The uncorrected base conversion of the encryption's ModDown leaves an error
+    # in [0, K) on every coefficient of c1; times the ternary secret that is a random walk over the coefficient
+    # index, i.e. a low-frequency error of a few 10^-5 in the first slots and about 10^-8 elsewhere.
+    assert np.max(np.abs(three - w["x"] * w["y"])) < 2e-4
+    assert np.median(np.abs(three - w["x"] * w["y"])) < 1e-7
+    c.rescale_to_next_inplace(ctx, xy)
+    assert xy.chain_index() == 2
+    got = _decode(w, xy)
+    assert np.max(np.abs(got - w["x"] * w["y"])) < 1e-2                       # about 2^30 of scale left
+    # the same product through the fused call
+    fused = c.ciphertext(ctx)
+    c.multiply(ctx, w["cx"], w["cy"], fused)
+    c.relinearize_inplace(ctx, fused, w["rlk"])
+    c.rescale_to_next_inplace(ctx, fused)
+    assert (fused.to_numpy() == xy.to_numpy()).all()
+
+
+def test_c4_rotations(bench_world):
+    w = bench_world
+    c, ctx = w["cahel"], w["ctx"]
+    base = _decode(w, w["cx"])
+    for step in (1, 64, 16384):
+        rot = c.ciphertext(ctx)
+        c.rotate_vector(ctx, w["cx"], step, w["glk"], rot)
+        err = np.abs(_decode(w, rot) - np.roll(base, -step))      # key-switch noise at scale 2^40, K = 8
+        assert np.max(err) < 1e-3 and np.median(err) < 1e-6
+    acc = c.ciphertext(ctx)
+    c.add(ctx, w["cx"], w["cx"], acc)
+    c.sub_inplace(ctx, acc, w["cx"])                     # acc = cx, as a fresh object
+    tmp = c.ciphertext(ctx)
+    for step in w["steps"]:
+        c.rotate_vector(ctx, acc, step, w["glk"], tmp)
+        c.add_inplace(ctx, acc, tmp)
+    total = _decode(w, acc)
+    want = float(np.sum(w["x"]))
+    assert np.max(np.abs(total - want)) < 2.0 ** -10 * max(1.0, abs(want))
+    # hoisted rotations of one ciphertext: sum of the rotated copies
+    hoisted = c.hoisting(ctx, w["cx"], w["glk"], [1, 2, 4])
+    ref = sum(np.roll(base, -s) for s in (1, 2, 4))
+    assert np.max(np.abs(_decode(w, hoisted) - ref)) < 1e-3 and np.median(np.abs(_decode(w, hoisted) - ref)) < 1e-6
+
+
+def test_c5_krum_round_full_shape():
+    """10 clients x 62,006 parameters at N = 2^16 with Lancelot's chain [60, 40, 40, 60], one special prime."""
+    from lancelot_amd import krum
+    rng = np.random.default_rng(2025)
+    updates = [rng.normal(0.0, 0.01, 62006).astype(np.float32) for _ in range(10)]
+    for k in (8, 9):
+        updates[k] = updates[k] * 10
+    chosen, dist, timings = krum.gpu_krum(updates, krum.KrumConfig(seed=2025))
+    want = krum.plain_distance_matrix(updates)
+    off = ~np.eye(10, dtype=bool)
+    assert np.max(np.abs(dist[off] - want[off]) / want[off]) < 1e-4
+    assert chosen == krum.krum_select(want) and chosen not in (8, 9)
+    assert timings["total"] > 0
