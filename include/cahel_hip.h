@@ -190,6 +190,26 @@ int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uin
 int he_decompose_real(const he_context *ctx, const double *coeffs, uint64_t *out, uint32_t limbs,
                       uint32_t first_table, he_stream stream);
 
+/* CKKS encode on the device: `count` <= `slots` values (DEVICE arrays re, im; im may be NULL), zero padded to
+ * `slots` (a power of two, 2 <= slots <= N/2) -> inverse special FFT over the orbit 5^j mod 2N -> times
+ * scale / slots -> rounded to integers -> residues of the first `limbs` primes -> NTT form in out [limbs][N].
+ * workspace: DEVICE, he_ckks_workspace_words(ctx, limbs) words; after the call word 0 of the workspace holds, as
+ * a double, the largest |coefficient| (the caller compares it with the modulus size, as src/ckks.cu:163-181 does).
+ * Replaces CAHELGPUCKKSEncoder::encode_internal (src/ckks.cu:104-209), special_fft_backward (src/fft.cu:350-453)
+ * and decompose_array (src/rns_base.cu:306-323). */
+int he_ckks_encode(const he_context *ctx, const double *re, const double *im, uint32_t count, uint32_t slots,
+                   double scale, uint32_t limbs, uint64_t *out, uint64_t *workspace, he_stream stream);
+
+/* CKKS decode on the device: plain [limbs][N] (NTT form, first `limbs` primes) -> inverse NTT -> CRT
+ * composition centred around zero, as doubles divided by `scale` -> forward special FFT.
+ * out: DEVICE, 2 * slots doubles, value i = (out[2 i], out[2 i + 1]).  workspace as above.
+ * Replaces CAHELGPUCKKSEncoder::decode_internal (src/ckks.cu:292-465), special_fft_forward (src/fft.cu:350-453)
+ * and compose_array (src/rns_base.cu:325-459). */
+int he_ckks_decode(const he_context *ctx, const uint64_t *plain, uint32_t limbs, uint32_t slots, double scale,
+                   double *out, uint64_t *workspace, he_stream stream);
+
+size_t he_ckks_workspace_words(const he_context *ctx, uint32_t limbs);
+
 /* ---- samplers (replace sample_ternary_poly / sample_error_poly / sample_uniform_poly, src/prng.cu:143-242,
  *      and the OpenFHE Gaussian of src/secretkey.cu:632-649) ----
  * ChaCha20 block function keyed by key[8]; `stream_id` selects an independent stream.  out: [limbs][N],

@@ -54,6 +54,9 @@ SIGNATURES = {
     "he_keyswitch_workspace_words": (C.c_size_t, [vp, u32]),
     "he_keyswitch": (C.c_int, [vp, u32, vp, C.POINTER(vp), vp, u32, vp, vp]),
     "he_decompose_real": (C.c_int, [vp, vp, vp, u32, u32, vp]),
+    "he_ckks_encode": (C.c_int, [vp, vp, vp, u32, u32, C.c_double, u32, vp, vp, vp]),
+    "he_ckks_decode": (C.c_int, [vp, vp, u32, u32, C.c_double, vp, vp, vp]),
+    "he_ckks_workspace_words": (C.c_size_t, [vp, u32]),
     "he_sample": (C.c_int, [vp, C.c_int, C.POINTER(u32), u64, vp, u32, u32, u32, u32, vp, u32, vp]),
 }
 

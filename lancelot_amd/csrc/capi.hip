@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -52,6 +53,9 @@ struct he_context {
     uint32_t *d_iota = nullptr;  // 0, 1, 2, ...: row -> limb/table map of the P -> Ql conversion
     double *d_psi_fp = nullptr, *d_ipsi_fp = nullptr, *d_fp_consts = nullptr;  // FP64 back end tables
     double *d_phat_mod_q_fp = nullptr;   // (M, M/q_j) pairs of the P -> Ql matrix
+    uint32_t *d_rot_group = nullptr;     // encoder: 5^j mod 2N
+    double2 *d_ksi = nullptr;            // encoder: e^{2 pi i k / 2N}, k <= 2N
+    uint64_t *d_garner_inv = nullptr;    // decoder: [size_q][size_q], q_j^-1 mod q_i for j < i
     std::vector<uint64_t> h_moduli;
     std::vector<uint8_t> fp_ok;  // per table: prime below 2^50
     bool use_fp = true;          // environment CAHEL_HIP_NO_FP64=1 forces the integer back end
@@ -260,6 +264,38 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         if (!rc) rc = upload(ctx, &ctx->d_pinv_mod_q, d->pinv_mod_q, 2 * (size_t)d->size_q);
         if (!rc) rc = upload(ctx, &ctx->d_phat_inv, d->phat_inv_mod_p, 2 * (size_t)d->size_p);
         if (!rc) rc = upload(ctx, &ctx->d_phat_mod_q, d->phat_mod_q, (size_t)d->size_q * d->size_p);
+    }
+    if (!rc) {
+        // encoder tables (cahel-main/src/ckks.cu:34-102): rotation group and the 2N-th roots of unity
+        const size_t m = 2 * n;
+        std::vector<uint32_t> rot(n / 2);
+        uint32_t pos = 1;
+        for (size_t i = 0; i < n / 2; i++) {
+            rot[i] = pos;
+            pos = (uint32_t)(((uint64_t)pos * 5) & (m - 1));
+        }
+        std::vector<double2> ksi(m + 1);
+        const double pi = 3.14159265358979323846264338327950288;
+        for (size_t k = 0; k <= m; k++) {
+            const double angle = 2.0 * pi * (double)k / (double)m;
+            ksi[k] = double2{std::cos(angle), std::sin(angle)};
+        }
+        // Garner constants of the data primes
+        const size_t sq = d->size_q;
+        std::vector<uint64_t> ginv(sq * sq, 0);
+        for (size_t i = 0; i < sq; i++)
+            for (size_t j = 0; j < i; j++) {
+                const uint64_t qi = d->moduli[i];
+                unsigned __int128 base = d->moduli[j] % qi, acc = 1;
+                for (uint64_t e = qi - 2; e; e >>= 1) {  // q_i is prime: a^(q_i - 2) = a^-1
+                    if (e & 1) acc = acc * base % qi;
+                    base = base * base % qi;
+                }
+                ginv[i * sq + j] = (uint64_t)acc;
+            }
+        rc = upload(ctx, &ctx->d_rot_group, rot.data(), rot.size());
+        if (!rc) rc = upload(ctx, &ctx->d_ksi, ksi.data(), ksi.size());
+        if (!rc) rc = upload(ctx, &ctx->d_garner_inv, ginv.data(), ginv.size());
     }
     if (!rc) {
         // FP64 back end: twiddles as doubles (inverse ones un-halved), per-table constants
@@ -683,6 +719,42 @@ int he_decompose_real(const he_context *ctx, const double *coeffs, uint64_t *out
                       he_stream s) {
     if (!ctx || !coeffs || !out || first + limbs > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
     HE_HIP(launch_decompose_real(ctx->tables(), coeffs, out, limbs, first, S(s)));
+    return HE_OK;
+}
+
+size_t he_ckks_workspace_words(const he_context *ctx, uint32_t limbs) {
+    if (!ctx) return 0;
+    const size_t n = ctx->n();
+    // encode: [8 words, the first holds the maximum] [N words: complex scratch] [N words: coefficients]
+    // decode: [limbs * N words: coefficient-form copy]
+    const size_t enc = 8 + 2 * n, dec = (size_t)limbs * n;
+    return enc > dec ? enc : dec;
+}
+
+int he_ckks_encode(const he_context *ctx, const double *re, const double *im, uint32_t count, uint32_t slots,
+                   double scale, uint32_t limbs, uint64_t *out, uint64_t *ws, he_stream s) {
+    if (!ctx || !re || !out || !ws || limbs == 0 || limbs > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
+    if (slots < 2 || (slots & (slots - 1)) || slots > ctx->n() / 2 || count > slots || !(scale > 0))
+        return HE_E_INVALID_ARGUMENT;
+    const size_t n = ctx->n();
+    double2 *v = reinterpret_cast<double2 *>(ws + 8);
+    double *coeffs = reinterpret_cast<double *>(ws + 8 + n);
+    const FftTables ft{ctx->d_rot_group, ctx->d_ksi, ctx->log_n};
+    HE_HIP(launch_ckks_encode(ft, re, im, count, slots, scale, v, coeffs, ws, S(s)));
+    HE_HIP(launch_decompose_real(ctx->tables(), coeffs, out, limbs, 0, S(s)));
+    return he_ntt_forward(ctx, out, 1, limbs, limbs, 0, limbs, 0, s);
+}
+
+int he_ckks_decode(const he_context *ctx, const uint64_t *plain, uint32_t limbs, uint32_t slots, double scale,
+                   double *out, uint64_t *ws, he_stream s) {
+    if (!ctx || !plain || !out || !ws || limbs == 0 || limbs > ctx->size_q) return HE_E_INVALID_ARGUMENT;
+    if (slots < 2 || (slots & (slots - 1)) || slots > ctx->n() / 2 || !(scale > 0)) return HE_E_INVALID_ARGUMENT;
+    const size_t n = ctx->n();
+    HE_HIP(hipMemcpyAsync(ws, plain, (size_t)limbs * n * sizeof(uint64_t), hipMemcpyDeviceToDevice, S(s)));
+    if (int rc = he_ntt_inverse(ctx, ws, 1, limbs, limbs, 0, limbs, 0, s)) return rc;
+    const FftTables ft{ctx->d_rot_group, ctx->d_ksi, ctx->log_n};
+    HE_HIP(launch_ckks_decode(ft, ctx->tables(), ws, limbs, slots, scale, ctx->d_garner_inv, ctx->size_q,
+                              reinterpret_cast<double2 *>(out), S(s)));
     return HE_OK;
 }
 

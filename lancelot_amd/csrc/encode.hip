@@ -1,0 +1,200 @@
+// CKKS encoding and decoding on the device: the special FFT over the orbit 5^j mod 2N (HEAAN's fftSpecial /
+// fftSpecialInv butterfly network, cahel-main/src/fft.cu:194-453), rounding to integer coefficients
+// (src/rns_base.cu:121-156) and the CRT composition of a decrypted plaintext (src/rns_base.cu:325-459).
+//
+// All floating-point steps are plain IEEE double operations in a fixed order (this file is compiled without
+// contraction): a butterfly is u = a + b, t = (a - b) * w with the four-multiplication complex product, so
+// the result does not depend on how the butterflies are spread over threads.
+//
+// Layout: v = `slots` complex values as double2.  Stages whose span exceeds one tile of 2048 values run as
+// one kernel each over global memory; all the others run inside LDS in a single kernel.
+#include "kernels.h"
+#include "modarith.cuh"
+
+namespace he {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr uint32_t kFftTile = 2048;  // complex values per workgroup in the LDS kernel (32 KiB)
+
+__device__ __forceinline__ double2 cmul(double2 a, double2 w) {
+    return double2{a.x * w.x - a.y * w.y, a.x * w.y + a.y * w.x};
+}
+
+// twiddle of butterfly j in a stage of span len: e^{+-2 pi i (5^j mod 4 len) / (4 len)}
+template <bool INVERSE>
+__device__ __forceinline__ double2 stage_twiddle(const FftTables &t, uint32_t len, uint32_t j) {
+    const uint32_t lenq = len << 2, gap = (2u << t.log_n) / lenq;
+    const uint32_t r = t.rot_group[j] & (lenq - 1);
+    return t.ksi[(INVERSE ? lenq - r : r) * gap];
+}
+
+// INVERSE (encode): decimation in frequency,  (a, b) -> (a + b, (a - b) w)
+// forward (decode): decimation in time,       (a, b) -> (a + b w, a - b w)
+template <bool INVERSE>
+__device__ __forceinline__ void butterfly(double2 &a, double2 &b, double2 w) {
+    if (INVERSE) {
+        const double2 u{a.x + b.x, a.y + b.y};
+        const double2 d{a.x - b.x, a.y - b.y};
+        a = u;
+        b = cmul(d, w);
+    } else {
+        const double2 t = cmul(b, w);
+        const double2 u = a;
+        a = double2{u.x + t.x, u.y + t.y};
+        b = double2{u.x - t.x, u.y - t.y};
+    }
+}
+
+// one stage over global memory; thread = one butterfly
+template <bool INVERSE>
+__global__ __launch_bounds__(kThreads) void cfft_stage_kernel(double2 *v, uint32_t len, FftTables t) {
+    const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
+    const uint32_t lenh = len >> 1;
+    const uint32_t j = b & (lenh - 1), pos = ((b / lenh) * len) + j;
+    double2 x = v[pos], y = v[pos + lenh];
+    butterfly<INVERSE>(x, y, stage_twiddle<INVERSE>(t, len, j));
+    v[pos] = x;
+    v[pos + lenh] = y;
+}
+
+// every stage of span <= tile inside LDS; tile = min(slots, kFftTile) values per workgroup
+template <bool INVERSE>
+__global__ __launch_bounds__(kThreads) void cfft_lds_kernel(double2 *v, uint32_t tile, FftTables t) {
+    __shared__ double2 s[kFftTile];
+    double2 *g = v + (size_t)blockIdx.x * tile;
+    for (uint32_t i = threadIdx.x; i < tile; i += kThreads) s[i] = g[i];
+    __syncthreads();
+    for (uint32_t k = 2; k <= tile; k <<= 1) {
+        const uint32_t len = INVERSE ? (tile << 1) / k : k;   // tile, tile/2, ..., 2  or  2, 4, ..., tile
+        const uint32_t lenh = len >> 1;
+        for (uint32_t b = threadIdx.x; b < (tile >> 1); b += kThreads) {
+            const uint32_t j = b & (lenh - 1), pos = ((b / lenh) * len) + j;
+            double2 x = s[pos], y = s[pos + lenh];
+            butterfly<INVERSE>(x, y, stage_twiddle<INVERSE>(t, len, j));
+            s[pos] = x;
+            s[pos + lenh] = y;
+        }
+        __syncthreads();
+    }
+    for (uint32_t i = threadIdx.x; i < tile; i += kThreads) g[i] = s[i];
+}
+
+// values -> complex vector, zero padded; also clears the maximum that the rounding kernel accumulates
+__global__ __launch_bounds__(kThreads) void encode_load_kernel(const double *re, const double *im, uint32_t count,
+                                                               uint32_t slots, double2 *v,
+                                                               unsigned long long *max_bits) {
+    const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+    if (i == 0) *max_bits = 0;
+    if (i < slots) v[i] = i < count ? double2{re[i], im ? im[i] : 0.0} : double2{0.0, 0.0};
+}
+
+// coefficient c of the plaintext: real parts fill the first half, imaginary parts the second, `gap` apart;
+// value i comes from position bitrev(i) of the transformed vector
+__global__ __launch_bounds__(kThreads) void encode_round_kernel(const double2 *v, uint32_t log_slots, uint32_t gap,
+                                                                uint32_t half, double fix, double *coeffs,
+                                                                unsigned long long *max_bits) {
+    const uint32_t c = blockIdx.x * kThreads + threadIdx.x;
+    const bool imag = c >= half;
+    const uint32_t k = imag ? c - half : c;
+    double val = 0.0;
+    if (k % gap == 0) {
+        const uint32_t i = k / gap;
+        const double2 z = v[__brev(i) >> (32 - log_slots)];
+        val = round((imag ? z.y : z.x) * fix);
+        atomicMax(max_bits, (unsigned long long)__double_as_longlong(fabs(val)));
+    }
+    coeffs[c] = val;
+}
+
+constexpr int kMaxComposeLimbs = 64;
+
+// Garner's mixed-radix composition of one coefficient, centred around zero, as a double divided by the scale.
+// thread s < slots: real part of value s, else imaginary part of value s - slots; stored at position bitrev.
+__global__ __launch_bounds__(kThreads) void decode_compose_kernel(const uint64_t *res, uint32_t limbs, uint32_t log_n,
+                                                                  uint32_t log_slots, uint32_t gap, double inv_scale,
+                                                                  const uint64_t *moduli, const uint64_t *barrett,
+                                                                  const uint64_t *garner_inv, uint32_t garner_stride,
+                                                                  double2 *v) {
+    const uint32_t s = blockIdx.x * kThreads + threadIdx.x;
+    const uint32_t slots = 1u << log_slots, half = 1u << (log_n - 1);
+    if (s >= 2 * slots) return;
+    const bool imag = s >= slots;
+    const uint32_t i0 = imag ? s - slots : s;
+    const size_t coeff = (imag ? half : 0) + (size_t)i0 * gap;
+    uint64_t d[kMaxComposeLimbs];
+    for (uint32_t i = 0; i < limbs; i++) {
+        const uint64_t q = moduli[i], r0 = barrett[2 * i], r1 = barrett[2 * i + 1];
+        uint64_t t = res[((size_t)i << log_n) + coeff];
+        for (uint32_t j = 0; j < i; j++) {
+            const uint64_t dj = barrett64(d[j], q, r1);
+            t = mul_mod(sub_mod(t, dj, q), garner_inv[(size_t)i * garner_stride + j], q, r0, r1);
+        }
+        d[i] = t;
+    }
+    // negative iff the digits, read from the top, exceed those of (Q - 1) / 2, whose digits are (q_i - 1) / 2
+    bool negative = false;
+    for (uint32_t i = limbs; i-- > 0;) {
+        const uint64_t h = (moduli[i] - 1) >> 1;
+        if (d[i] != h) {
+            negative = d[i] > h;
+            break;
+        }
+    }
+    if (negative) {
+        // Q - v = (Q - 1 - v) + 1: digit-wise complement, then increment
+        for (uint32_t i = 0; i < limbs; i++) d[i] = moduli[i] - 1 - d[i];
+        for (uint32_t i = 0; i < limbs; i++) {
+            if (++d[i] < moduli[i]) break;
+            d[i] = 0;
+        }
+    }
+    double acc = 0.0;
+    for (uint32_t i = limbs; i-- > 0;) acc = acc * (double)moduli[i] + (double)d[i];
+    const double val = (negative ? -acc : acc) * inv_scale;
+    double *slot = reinterpret_cast<double *>(&v[__brev(i0) >> (32 - log_slots)]);
+    slot[imag ? 1 : 0] = val;
+}
+
+template <bool INVERSE>
+hipError_t run_fft(double2 *v, uint32_t slots, const FftTables &t, hipStream_t s) {
+    const uint32_t tile = slots < kFftTile ? slots : kFftTile;
+    if (INVERSE) {
+        for (uint32_t len = slots; len > tile; len >>= 1)
+            hipLaunchKernelGGL(cfft_stage_kernel<true>, dim3(slots / 2 / kThreads), dim3(kThreads), 0, s, v, len, t);
+        hipLaunchKernelGGL(cfft_lds_kernel<true>, dim3(slots / tile), dim3(kThreads), 0, s, v, tile, t);
+    } else {
+        hipLaunchKernelGGL(cfft_lds_kernel<false>, dim3(slots / tile), dim3(kThreads), 0, s, v, tile, t);
+        for (uint32_t len = tile << 1; len <= slots; len <<= 1)
+            hipLaunchKernelGGL(cfft_stage_kernel<false>, dim3(slots / 2 / kThreads), dim3(kThreads), 0, s, v, len, t);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace
+
+hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double *im, uint32_t count, uint32_t slots,
+                              double scale, double2 *v, double *coeffs, uint64_t *max_bits, hipStream_t s) {
+    const uint32_t n = 1u << t.log_n, log_slots = 31 - __builtin_clz(slots);
+    auto blocks = [](uint32_t items) { return dim3((items + kThreads - 1) / kThreads); };
+    hipLaunchKernelGGL(encode_load_kernel, blocks(slots), dim3(kThreads), 0, s, re, im, count, slots, v,
+                       reinterpret_cast<unsigned long long *>(max_bits));
+    hipError_t e = run_fft<true>(v, slots, t, s);
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(encode_round_kernel, blocks(n), dim3(kThreads), 0, s, v, log_slots, (n / 2) / slots, n / 2,
+                       scale / (double)slots, coeffs, reinterpret_cast<unsigned long long *>(max_bits));
+    return hipGetLastError();
+}
+
+hipError_t launch_ckks_decode(const FftTables &t, const Tables &tab, const uint64_t *res, uint32_t limbs,
+                              uint32_t slots, double scale, const uint64_t *garner_inv, uint32_t garner_stride,
+                              double2 *v, hipStream_t s) {
+    const uint32_t n = 1u << t.log_n, log_slots = 31 - __builtin_clz(slots);
+    if (limbs == 0 || limbs > (uint32_t)kMaxComposeLimbs) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(decode_compose_kernel, dim3((2 * slots + kThreads - 1) / kThreads), dim3(kThreads), 0, s, res, limbs, t.log_n,
+                       log_slots, (n / 2) / slots, 1.0 / scale, tab.moduli, tab.barrett, garner_inv, garner_stride, v);
+    return run_fft<false>(v, slots, t, s);
+}
+
+}  // namespace he

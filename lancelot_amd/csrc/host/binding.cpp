@@ -145,6 +145,28 @@ PYBIND11_MODULE(pyCAHEL, m) {
         .def(py::init<CAHELGPUContext &>())
         .def("slot_count", &CAHELGPUCKKSEncoder::slot_count)
         .def("reset_sparse_slots", &CAHELGPUCKKSEncoder::reset_sparse_slots)
+        // numpy fast paths (no per-element conversion); lists fall through to the reference's signatures
+        .def("encode",
+             [](CAHELGPUCKKSEncoder &e, const CAHELGPUContext &c, py::array_t<double, py::array::c_style> v, double scale) {
+                 CAHELGPUPlaintext p(c);
+                 e.encode_complex(c, v.data(), nullptr, (std::size_t)v.size(), e.first_chain_index(), scale, p);
+                 return p;
+             },
+             py::arg("context"), py::arg("values").noconvert(), py::arg("scale"))
+        .def("encode_to",
+             [](CAHELGPUCKKSEncoder &e, const CAHELGPUContext &c, py::array_t<double, py::array::c_style> v,
+                std::size_t chain_index, double scale) {
+                 CAHELGPUPlaintext p(c);
+                 e.encode_complex(c, v.data(), nullptr, (std::size_t)v.size(), chain_index, scale, p);
+                 return p;
+             },
+             py::arg("context"), py::arg("values").noconvert(), py::arg("chain_index"), py::arg("scale"))
+        .def("decode_array",
+             [](CAHELGPUCKKSEncoder &e, const CAHELGPUContext &c, const CAHELGPUPlaintext &p) {
+                 std::vector<double> out;
+                 e.decode(c, p, out);
+                 return py::array_t<double>((py::ssize_t)out.size(), out.data());
+             })
         .def("encode", py::overload_cast<const CAHELGPUContext &, const std::vector<double> &, double>(
                            &CAHELGPUCKKSEncoder::encode))
         .def("encode_to", py::overload_cast<const CAHELGPUContext &, const std::vector<double> &, std::size_t, double>(

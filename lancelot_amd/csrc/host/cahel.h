@@ -291,6 +291,7 @@ public:
     explicit CAHELGPUCKKSEncoder(const CAHELGPUContext &context);
     std::size_t slot_count() const { return slots_; }
     void reset_sparse_slots() { sparse_slots_ = 0; }
+    std::size_t first_chain_index() const { return first_chain_index_; }
     void encode(const CAHELGPUContext &context, const std::vector<double> &values, std::size_t chain_index, double scale,
                 CAHELGPUPlaintext &destination);
     void encode(const CAHELGPUContext &context, const std::vector<double> &values, double scale,
@@ -322,8 +323,6 @@ public:
 private:
     std::size_t slots_ = 0, sparse_slots_ = 0;
     std::size_t first_chain_index_ = 1;  // include/ckks.h:325
-    std::vector<uint32_t> rot_group_;
-    std::vector<double> ksi_re_, ksi_im_;  // e^(2 pi i k / M), k <= M
 };
 
 // ---- evaluator: include/evaluate.h:15-600 ----

@@ -165,4 +165,20 @@ struct ChaChaKey {
 hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
                          const uint64_t *cdt, uint32_t cdt_len, hipStream_t s);
 
+// CKKS encoder tables: 5^j mod 2N for j < N/2 and e^{2 pi i k / 2N} for k <= 2N.
+struct FftTables {
+    const uint32_t *rot_group;
+    const double2 *ksi;
+    uint32_t log_n;
+};
+// values (count <= slots, zero padded) -> rounded real coefficients [N]; *max_bits receives the bit pattern of the
+// largest |coefficient| (a non-negative double).  v: scratch of `slots` complex values.
+hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double *im, uint32_t count, uint32_t slots,
+                              double scale, double2 *v, double *coeffs, uint64_t *max_bits, hipStream_t s);
+// res: [limbs][N] coefficient-form residues of the first `limbs` primes -> v: `slots` complex values.
+// garner_inv[i * stride + j] = q_j^-1 mod q_i for j < i.
+hipError_t launch_ckks_decode(const FftTables &t, const Tables &tab, const uint64_t *res, uint32_t limbs,
+                              uint32_t slots, double scale, const uint64_t *garner_inv, uint32_t garner_stride,
+                              double2 *v, hipStream_t s);
+
 }  // namespace he

@@ -99,7 +99,7 @@ def encrypt_updates(state: KrumState, chunks):
         row = []
         for chunk in client:
             t0 = time.perf_counter()
-            pt = state.encoder.encode(ctx, chunk, state.config.scale)
+            pt = state.encoder.encode(ctx, np.ascontiguousarray(chunk, dtype=np.float64), state.config.scale)
             t1 = time.perf_counter()
             row.append(state.pk.encrypt_asymmetric(ctx, pt))
             _sync(c)
@@ -157,7 +157,7 @@ def distance_matrix(state: KrumState, updates):
     dist = np.zeros((n_clients, n_clients))
     for i in range(n_clients):
         for j in range(i + 1, n_clients):
-            value = state.encoder.decode(state.context, state.sk.decrypt(state.context, enc[i][j]))[0]
+            value = state.encoder.decode_array(state.context, state.sk.decrypt(state.context, enc[i][j]))[0]
             dist[i, j] = dist[j, i] = value
     state.timings["decrypt"] += time.perf_counter() - t0
     return dist, enc

@@ -332,3 +332,73 @@ def test_decompose_real(small, capi, oracle):
     oracle.lib().orc_decompose_coeffs(C.byref(p.c), coeffs.ctypes.data_as(C.POINTER(C.c_double)),
                                       want.ctypes.data_as(oracle.u64p), C.c_uint32(p.size_q))
     assert (out.numpy() == want).all()
+
+
+# ---- CKKS encode / decode on the device ----
+
+@pytest.mark.parametrize("slots,complex_values", [(None, False), (None, True), (64, True), (2, False)])
+def test_ckks_encode_decode(small, capi, oracle, slots, complex_values):
+    """he_ckks_encode / he_ckks_decode against the oracle's encoder: coefficients within one unit (the FP64
+    transforms differ in operation order only), decoded values to 2^-20, full and sparse slot counts."""
+    cahel, parms, ctx, p = small
+    lib, h = capi.lib(), ctx.he_handle()
+    ss = slots or p.n // 2
+    rng = np.random.default_rng(50 + ss)
+    count = ss if ss < 8 else ss - 3                      # ragged: the tail is zero padded
+    z = rng.uniform(-1, 1, count) + (1j * rng.uniform(-1, 1, count) if complex_values else 0)
+    scale, limbs = 2.0 ** 40, p.size_q
+    o_enc = oracle.Encoder(p)
+    re = DeviceArray(capi, host=np.ascontiguousarray(np.real(z), dtype=np.float64))
+    im = DeviceArray(capi, host=np.ascontiguousarray(np.imag(z), dtype=np.float64)) if complex_values else None
+    ws = DeviceArray(capi, shape=(lib.he_ckks_workspace_words(h, limbs),))
+    out = DeviceArray(capi, shape=(limbs, p.n))
+    capi.check(lib.he_ckks_encode(h, re.ptr, im.ptr if im else None, count, ss, scale, limbs, out.ptr, ws.ptr, None))
+    got = out.numpy()
+    want = o_enc.encode(z, scale, limbs, ss)
+    coeff_got = p.ntt_inv(got.copy()).astype(np.int64)
+    coeff_want = p.ntt_inv(want.copy()).astype(np.int64)
+    q0 = p.moduli[0]
+    diff = (coeff_got[0] - coeff_want[0]) % q0
+    diff = np.minimum(diff, q0 - diff)
+    assert diff.max() <= 1
+    max_coeff = ws.numpy().view(np.float64)[0]
+    centred = np.where(coeff_got[0] > q0 // 2, coeff_got[0] - q0, coeff_got[0])
+    assert max_coeff == np.abs(centred).max()
+    # decode what was encoded
+    dec = DeviceArray(capi, shape=(2 * ss,), dtype=np.float64)
+    capi.check(lib.he_ckks_decode(h, out.ptr, limbs, ss, scale, dec.ptr, ws.ptr, None))
+    v = dec.numpy().reshape(ss, 2)
+    got_z = v[:, 0] + 1j * v[:, 1]
+    want_z = o_enc.decode(got, scale, ss)
+    assert np.max(np.abs(got_z - want_z)) < 2.0 ** -20
+    full = np.zeros(ss, dtype=np.complex128)
+    full[:count] = z
+    assert np.max(np.abs(got_z - full)) < 2.0 ** -20
+
+
+def test_ckks_decode_large_values(small, capi, oracle):
+    """Composition over several limbs: random residues, i.e. coefficients spread over (-Q/2, Q/2)."""
+    cahel, parms, ctx, p = small
+    lib, h = capi.lib(), ctx.he_handle()
+    limbs, ss = p.size_q, p.n // 2
+    rng = np.random.default_rng(60)
+    plain = rand_limbs(p, rng, list(range(limbs)))
+    scale = float(np.prod([float(q) for q in p.moduli[:limbs]])) / 2.0 ** 20
+    d_plain = DeviceArray(capi, host=plain)
+    ws = DeviceArray(capi, shape=(lib.he_ckks_workspace_words(h, limbs),))
+    dec = DeviceArray(capi, shape=(2 * ss,), dtype=np.float64)
+    capi.check(lib.he_ckks_decode(h, d_plain.ptr, limbs, ss, scale, dec.ptr, ws.ptr, None))
+    v = dec.numpy().reshape(ss, 2)
+    want = oracle.Encoder(p).decode(plain, scale, ss)
+    got = v[:, 0] + 1j * v[:, 1]
+    assert np.max(np.abs(got - want)) < 2.0 ** -20 * np.max(np.abs(want))
+
+
+def test_ckks_encode_bad_arguments(small, capi):
+    cahel, parms, ctx, p = small
+    lib, h = capi.lib(), ctx.he_handle()
+    buf = DeviceArray(capi, shape=(lib.he_ckks_workspace_words(h, p.size_q),))
+    out = DeviceArray(capi, shape=(p.size_q, p.n))
+    for slots, count in ((3, 2), (p.n, 4), (8, 9), (1, 1)):
+        assert lib.he_ckks_encode(h, buf.ptr, None, count, slots, 2.0 ** 30, p.size_q, out.ptr, buf.ptr, None) == -1
+    assert lib.he_ckks_decode(h, out.ptr, p.size_q + 1, 8, 2.0 ** 30, buf.ptr, buf.ptr, None) == -1
