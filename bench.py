@@ -118,12 +118,15 @@ def krum_round(seed: int = 2025):
     t0 = time.perf_counter()
     state = krum.gpu_init(krum.KrumConfig(seed=seed))
     setup = time.perf_counter() - t0
-    krum.gpu_krum(updates, state=state)  # warm-up round (pool growth, first-touch of the keys)
+    krum.gpu_krum_aggregate(updates, state=state)  # warm-up round (pool growth, first-touch of the keys)
+    chosen_full, weights, full_timings = krum.gpu_krum_aggregate(updates, state=state)
     chosen, dist, timings = krum.gpu_krum(updates, state=state)
     plain = krum.plain_distance_matrix(updates)
     off = ~np.eye(10, dtype=bool)
     return {"workload": "Krum distance round, 10 clients x 62006 parameters, 2 ciphertexts per client, 45 pairs, N=2^16",
             "setup_s": setup, "round_s": timings, "chosen": chosen, "chosen_plain": krum.krum_select(plain),
+            "full_round_s": full_timings, "full_round_chosen": chosen_full,
+            "aggregate_max_abs_err": float(np.max(np.abs(weights - updates[chosen_full].astype(np.float64)))),
             "max_rel_err_vs_float64": float(np.max(np.abs(dist[off] - plain[off]) / plain[off]))}
 
 

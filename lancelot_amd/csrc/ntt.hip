@@ -148,9 +148,10 @@ struct Split {
     static constexpr int p1 = LD - p0;
 };
 
-template <int LD>
+// TL = log2(words per tile): 12, or 10 when a launch has too few limbs to give every CU a 4096-word tile
+template <int LD, int TL>
 __device__ __forceinline__ constexpr int log_cols() {
-    return (kTileLog - LD) < 8 ? (kTileLog - LD) : 8;
+    return (TL - LD) < 8 ? (TL - LD) : 8;
 }
 
 // (N^-1 [* w]) as an FP twiddle for the last multiplication of the inverse transform
@@ -165,10 +166,11 @@ __device__ __forceinline__ FpTw inverse_scale(const NttArgs &a, const Job &job, 
 // ---------------------------------------------------------------------------------------------------
 // rows pass: stages 0 .. LD-1 (forward) over an R = 2^LD rows x 256 matrix
 // ---------------------------------------------------------------------------------------------------
-template <int LD, bool FWD, bool FP>
-__global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
-    __shared__ uint64_t lds[kLdsWords];
-    constexpr int LOGC = log_cols<LD>();
+template <int LD, bool FWD, bool FP, int TL>
+__global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
+    __shared__ uint64_t lds[(1 << TL) + (1 << (TL - 4))];
+    constexpr uint32_t kRowThreads = (1u << TL) / 16;
+    constexpr int LOGC = log_cols<LD, TL>();
     constexpr uint32_t C = 1u << LOGC;
     constexpr uint32_t tile_elems = 1u << (LD + LOGC);
     constexpr uint32_t tiles_per_limb = 256u >> LOGC;
@@ -185,7 +187,7 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
             // input: canonical residues (or one broadcast source limb); output: lazy signed doubles
             const uint64_t *src =
                 a.pro_mode == NTT_PRO_BROADCAST_REDUCE ? a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n) : job.in;
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                 uint32_t row = e >> LOGC, col = e & (C - 1);
                 ld[skew(e)] = fp_from_u64(src[(size_t)row * 256 + col0 + col]);
             }
@@ -200,13 +202,13 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
                 tile_pass_fp<(p1 > 0 ? p1 : 1), true, true>(lds, tile_elems, LOGC, 1u << p0, c);
                 __syncthreads();
             }
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                 uint32_t row = e >> LOGC, col = e & (C - 1);
                 job.out[(size_t)row * 256 + col0 + col] = lds[skew(e)];
             }
         } else {
             // input: lazy signed doubles from the blocks pass; output: canonical residues
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                 uint32_t row = e >> LOGC, col = e & (C - 1);
                 lds[skew(e)] = job.in[(size_t)row * 256 + col0 + col];
             }
@@ -218,7 +220,7 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
             tile_pass_fp<p0, false, true>(lds, tile_elems, LD - p0 + LOGC, 1u, c);
             __syncthreads();
             const FpTw scale = inverse_scale(a, job, c.m);
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                 uint32_t row = e >> LOGC, col = e & (C - 1);
                 job.out[(size_t)row * 256 + col0 + col] = fp_to_u64(fp_canonical(fp_mulmod(ld[skew(e)], scale, c.m), c.m));
             }
@@ -231,12 +233,12 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
     if (FWD && a.pro_mode == NTT_PRO_BROADCAST_REDUCE) {
         const uint64_t r1 = a.barrett[2 * job.table + 1];
         const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
-        for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+        for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
             uint32_t row = e >> LOGC, col = e & (C - 1);
             lds[skew(e)] = barrett64(src[(size_t)row * 256 + col0 + col], q, r1);
         }
     } else {
-        for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+        for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
             uint32_t row = e >> LOGC, col = e & (C - 1);
             lds[skew(e)] = job.in[(size_t)row * 256 + col0 + col];
         }
@@ -251,7 +253,7 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
             __syncthreads();
         }
         // lazy values in [0, 4q) go to the blocks pass
-        for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+        for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
             uint32_t row = e >> LOGC, col = e & (C - 1);
             job.out[(size_t)row * 256 + col0 + col] = lds[skew(e)];
         }
@@ -264,12 +266,12 @@ __global__ __launch_bounds__(kThreads) void ntt_rows_kernel(NttArgs a) {
         __syncthreads();
         if (a.epi_mode == NTT_EPI_MUL) {
             const Shoup w = load_shoup(a.w, job.limb);
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                 uint32_t row = e >> LOGC, col = e & (C - 1);
                 job.out[(size_t)row * 256 + col0 + col] = mul_shoup(lds[skew(e)], w, q);
             }
         } else {
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kThreads) {
+            for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                 uint32_t row = e >> LOGC, col = e & (C - 1);
                 job.out[(size_t)row * 256 + col0 + col] = reduce_2q(lds[skew(e)], q);
             }
@@ -535,17 +537,27 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_int_kernel(NttArgs a) {
 template <bool FWD, bool FP>
 hipError_t launch_rows(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
     const int ld = (int)a.log_n - 8;
-    auto grid = [&](int ldv) {
-        int logc = (kTileLog - ldv) < 8 ? (kTileLog - ldv) : 8;
+    auto grid = [&](int ldv, int tl) {
+        int logc = (tl - ldv) < 8 ? (tl - ldv) : 8;
         return dim3(n_jobs * (256u >> logc));
     };
+    // small launches (fewer 4096-word tiles than CUs) are bound by the latency of one workgroup: quarter tiles
+    const bool small = ld >= 5 && n_jobs * (256u >> (kTileLog - ld < 8 ? kTileLog - ld : 8)) < 256;
     switch (ld) {
-#define HE_CASE(LD)                                                                          \
-    case LD:                                                                                 \
-        hipLaunchKernelGGL((ntt_rows_kernel<LD, FWD, FP>), grid(LD), dim3(kThreads), 0, s, a); \
+#define HE_CASE(LD)                                                                               \
+    case LD:                                                                                      \
+        hipLaunchKernelGGL((ntt_rows_kernel<LD, FWD, FP, 12>), grid(LD, 12), dim3(256), 0, s, a); \
         break;
-        HE_CASE(1) HE_CASE(2) HE_CASE(3) HE_CASE(4) HE_CASE(5) HE_CASE(6) HE_CASE(7) HE_CASE(8)
+#define HE_CASE2(LD)                                                                                  \
+    case LD:                                                                                          \
+        if (small)                                                                                    \
+            hipLaunchKernelGGL((ntt_rows_kernel<LD, FWD, FP, 10>), grid(LD, 10), dim3(64), 0, s, a);  \
+        else                                                                                          \
+            hipLaunchKernelGGL((ntt_rows_kernel<LD, FWD, FP, 12>), grid(LD, 12), dim3(256), 0, s, a); \
+        break;
+        HE_CASE(1) HE_CASE(2) HE_CASE(3) HE_CASE(4) HE_CASE2(5) HE_CASE2(6) HE_CASE2(7) HE_CASE2(8)
 #undef HE_CASE
+#undef HE_CASE2
         default:
             return hipErrorInvalidValue;
     }
@@ -573,7 +585,7 @@ BlocksPlan plan_blocks(const NttArgs &a, uint32_t n_polys) {
         p.batch = (n_polys > 1 && a.map.limbs * tiles(2048) >= 512) ? n_polys : 1;
         units = a.map.limbs * ((n_polys + p.batch - 1) / p.batch);
     }
-    const uint32_t want = units * tiles(4096) >= 1024 ? 4096 : 2048;
+    const uint32_t want = units * tiles(4096) >= 1024 ? 4096 : (units * tiles(2048) >= 256 ? 2048 : 1024);
     p.threads = threads(want);
     p.grid = units * tiles(want);
     return p;

@@ -2,7 +2,7 @@
 
 Restates the protocol of lancelot-main-GPU/utils/byzantine_fl.py (GPU_init :432-462,
 GPU_compute_pair_distance :173-321, GPU_computing_distance_cipher :466-514, GPU_decrypt_sort_mask :327-369,
-GPU_krum :517-525) on top of the same pyCAHEL calls, with two differences that do not change the result:
+GPU_mul_mask_weight :371-429, GPU_krum :517-525) on top of the same pyCAHEL calls, with two differences that do not change the result:
 every client chunk is encoded and encrypted once (the reference re-encrypts both operands for every pair) and
 the i == j pairs, whose distance is zero, are not evaluated.
 
@@ -163,6 +163,60 @@ def distance_matrix(state: KrumState, updates):
     return dist, enc
 
 
+def _encrypt_constant(state: KrumState, value: float):
+    c = state.cahel
+    pt = state.encoder.encode(state.context, np.full(state.slots, value, dtype=np.float64), state.config.scale)
+    return state.pk.encrypt_asymmetric(state.context, pt)
+
+
+def decrypt_sort_mask(state: KrumState, enc):
+    """Row sums of the encrypted distances, decrypted scores, and the one-hot mask ciphertexts
+    (byzantine_fl.py:327-369): mask[r][k] encrypts 1 when client k has the r-th smallest score, else 0.
+    Returns (mask, order, scores)."""
+    c, ctx = state.cahel, state.context
+    n_clients = len(enc)
+    level = enc[0][1].chain_index()
+    scores = []
+    t0 = time.perf_counter()
+    for i in range(n_clients):
+        total = _encrypt_constant(state, 0.0)
+        c.mod_switch_to_inplace(ctx, total, level)
+        for j in range(n_clients):
+            if enc[i][j] is not None:          # the i == j distance is zero and was never evaluated
+                c.add_inplace(ctx, total, enc[i][j])
+        scores.append(state.encoder.decode_array(ctx, state.sk.decrypt(ctx, total))[0])
+    order = np.argsort(np.asarray(scores), kind="stable")
+    zero, one = _encrypt_constant(state, 0.0), _encrypt_constant(state, 1.0)
+    mask = [[one if order[r] == k else zero for k in range(n_clients)] for r in range(n_clients)]
+    _sync(c)
+    state.timings["mask"] = state.timings.get("mask", 0.0) + time.perf_counter() - t0
+    return mask, order, np.asarray(scores)
+
+
+def mul_mask_weight(state: KrumState, cts, mask_row):
+    """sum_k mask_row[k] * update_k chunk by chunk with lazy relinearisation: the products stay size-3
+    ciphertexts, are added, and are decrypted as such (byzantine_fl.py:371-429, lazy_relin_flag branch).
+    `cts[k][chunk]` are the cached client ciphertexts.  Returns the decoded weights (all chunks, padded)."""
+    c, ctx = state.cahel, state.context
+    t0 = time.perf_counter()
+    n_chunks = len(cts[0])
+    out = []
+    prod = c.ciphertext(ctx)
+    for chunk in range(n_chunks):
+        acc = None
+        for k, ct_mask in enumerate(mask_row):
+            c.multiply(ctx, cts[k][chunk], ct_mask, prod)
+            if acc is None:
+                acc = prod
+                prod = c.ciphertext(ctx)
+            else:
+                c.add_inplace(ctx, acc, prod)
+        out.append(state.encoder.decode_array(ctx, state.sk.decrypt(ctx, acc)))
+    _sync(c)
+    state.timings["mask_multiply"] = state.timings.get("mask_multiply", 0.0) + time.perf_counter() - t0
+    return np.concatenate(out)
+
+
 def plain_distance_matrix(updates):
     """float64 closed form ||u_i - u_j||^2 (byzantine_fl.py:129-131, 162-171)."""
     v = [np.asarray(u, dtype=np.float64).reshape(-1) for u in updates]
@@ -189,3 +243,28 @@ def gpu_krum(updates, config: KrumConfig | None = None, state: KrumState | None 
     total = time.perf_counter() - t0
     timings = dict(state.timings, total=total)
     return krum_select(dist), dist, timings
+
+
+def gpu_krum_aggregate(updates, config: KrumConfig | None = None, state: KrumState | None = None):
+    """The full round of the reference's driver: encrypted distances, decrypt-sort-mask, and the masked sum of
+    the encrypted updates, which is the update of the chosen client (byzantine_fl.py:517-525 followed by
+    :327-429).  Returns (chosen client index, aggregated weights of len(updates[0]), timings in seconds)."""
+    state = state or gpu_init(config)
+    for k in list(state.timings):
+        state.timings[k] = 0.0
+    t0 = time.perf_counter()
+    chunks = split_updates(updates, state.slots)
+    cts = encrypt_updates(state, chunks)
+    n_clients = len(updates)
+    enc = [[None] * n_clients for _ in range(n_clients)]
+    t1 = time.perf_counter()
+    for i in range(n_clients):
+        for j in range(i + 1, n_clients):
+            enc[i][j] = enc[j][i] = pair_distance(state, cts[i], cts[j])
+    _sync(state.cahel)
+    state.timings["evaluate"] += time.perf_counter() - t1
+    mask, order, _ = decrypt_sort_mask(state, enc)
+    weights = mul_mask_weight(state, cts, mask[0])
+    total = time.perf_counter() - t0
+    length = len(np.asarray(updates[0]).reshape(-1))
+    return int(order[0]), weights[:length], dict(state.timings, total=total)

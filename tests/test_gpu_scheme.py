@@ -339,3 +339,18 @@ def test_encrypted_krum_small(oracle):
     chosen2, dist2, _ = krum.gpu_krum(updates, plain)
     assert chosen2 == chosen and rel_err(dist2, want) < 1e-3
     assert set(timings) == {"encode", "encrypt", "evaluate", "decrypt", "total"}
+
+
+def test_encrypted_krum_aggregate_small(oracle):
+    """Distances, decrypt-sort-mask and the masked sum: the aggregate is the chosen client's update."""
+    from lancelot_amd import krum
+    rng = np.random.default_rng(8)
+    updates = [rng.normal(0, 0.01, 5000).astype(np.float32) for _ in range(4)]
+    updates[1] = updates[1] * 10
+    cfg = krum.KrumConfig(log_n=13, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=12)
+    chosen, weights, timings = krum.gpu_krum_aggregate(updates, cfg)
+    want = krum.krum_select(krum.plain_distance_matrix(updates))
+    assert chosen == want and chosen != 1
+    assert weights.shape == (5000,)
+    assert np.max(np.abs(weights - updates[chosen].astype(np.float64))) < 1e-5
+    assert {"mask", "mask_multiply", "evaluate", "total"} <= set(timings)
