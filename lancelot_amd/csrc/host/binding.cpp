@@ -18,7 +18,7 @@ py::array_t<uint64_t> to_host(const uint64_t *dev, std::vector<py::ssize_t> shap
     py::array_t<uint64_t> out(shape);
     std::size_t words = 1;
     for (auto s : shape) words *= (std::size_t)s;
-    if (words) check_status(he_memcpy_d2h(out.mutable_data(), dev, words * sizeof(uint64_t), nullptr), "download");
+    if (words) check_status(he_memcpy_d2h(out.mutable_data(), dev, words * sizeof(uint64_t), cahel::current_stream()), "download");
     return out;
 }
 
@@ -273,5 +273,8 @@ PYBIND11_MODULE(pyCAHEL, m) {
         return r;
     });
     m.def("_trim_pool", &DeviceBuffer::trim_pool);
-    m.def("_synchronize", []() { check_status(he_stream_synchronize(nullptr), "sync"); });
+    m.def("_synchronize", []() { cahel::synchronize_lanes(); });
+    m.def("_set_lane", &cahel::set_lane);
+    m.def("_current_lane", &cahel::current_lane);
+    m.def("_lane_count", &cahel::lane_count);
 }

@@ -62,7 +62,10 @@ public:
     DeviceBuffer() = default;
     explicit DeviceBuffer(std::size_t words) { allocate(words); }
     DeviceBuffer(const DeviceBuffer &o);
-    DeviceBuffer(DeviceBuffer &&o) noexcept : ptr_(o.ptr_), words_(o.words_) { o.ptr_ = nullptr; o.words_ = 0; }
+    DeviceBuffer(DeviceBuffer &&o) noexcept : ptr_(o.ptr_), words_(o.words_), lane_(o.lane_) {
+        o.ptr_ = nullptr;
+        o.words_ = 0;
+    }
     DeviceBuffer &operator=(const DeviceBuffer &o);
     DeviceBuffer &operator=(DeviceBuffer &&o) noexcept;
     ~DeviceBuffer() { release(); }
@@ -75,7 +78,18 @@ public:
 private:
     uint64_t *ptr_ = nullptr;
     std::size_t words_ = 0;
+    int lane_ = 0;  // the lane whose stream orders the reuse of this block
 };
+
+// Lanes (not in the reference, which runs everything on the legacy default stream): lane 0 is the null stream,
+// lanes 1 .. lane_count() are non-blocking streams.  Every evaluator, encoder and key function enqueues on the
+// current lane, and temporaries are recycled per lane, so independent ciphertext pipelines given different lanes
+// overlap on the GPU.  An object produced on one lane may be used on another only after synchronize_lanes().
+he_stream current_stream();
+int current_lane();
+int lane_count();
+void set_lane(int lane);
+void synchronize_lanes();
 
 }  // namespace cahel
 
@@ -115,7 +129,7 @@ public:
     long find_galois_elt(uint32_t elt) const;
 
     he_context *handle() const { return he_; }
-    he_stream stream() const { return nullptr; }
+    he_stream stream() const { return cahel::current_stream(); }
 
     // Seeded randomness: every sampled polynomial takes the next stream id of the context's ChaCha20 key.
     // The default key comes from /dev/urandom (include/prng.cuh:12-23); set_seed makes runs reproducible.

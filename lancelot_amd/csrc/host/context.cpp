@@ -53,16 +53,24 @@ void EncryptionParameters::set_coeff_modulus(const std::vector<Modulus> &coeff_m
 // ---------------------------------------------------------------------------------------------------
 namespace {
 
+// Lanes: lane 0 is the null stream (what the reference uses for everything); lanes 1 .. kMaxLanes are
+// non-blocking streams created on first use.  Work of different lanes may overlap on the GPU.
+constexpr int kMaxLanes = 8;
+int g_lane = 0;
+he_stream g_lane_streams[kMaxLanes + 1] = {};
+
 struct Pool {
     std::mutex mu;
-    std::multimap<std::size_t, void *> free_blocks;  // bytes -> block
+    // (lane, bytes) -> block.  A block returns to the lane that took it, so that reuse is ordered by that lane's
+    // stream however the owning object travelled.
+    std::multimap<std::pair<int, std::size_t>, void *> free_blocks;
     ~Pool() {
         // the HIP runtime may already be gone at static destruction; leave the blocks to process exit
     }
-    void *take(std::size_t bytes) {
+    void *take(std::size_t bytes, int lane) {
         {
             std::lock_guard<std::mutex> g(mu);
-            auto it = free_blocks.find(bytes);
+            auto it = free_blocks.find({lane, bytes});
             if (it != free_blocks.end()) {
                 void *p = it->second;
                 free_blocks.erase(it);
@@ -78,9 +86,9 @@ struct Pool {
         check_status(rc, "device allocation failed");
         return p;
     }
-    void give(void *p, std::size_t bytes) {
+    void give(void *p, std::size_t bytes, int lane) {
         std::lock_guard<std::mutex> g(mu);
-        free_blocks.emplace(bytes, p);
+        free_blocks.emplace(std::make_pair(lane, bytes), p);
     }
     void trim() {
         std::lock_guard<std::mutex> g(mu);
@@ -99,25 +107,26 @@ Pool &pool() {
 void DeviceBuffer::allocate(std::size_t words) {
     release();
     if (words == 0) return;
-    ptr_ = static_cast<uint64_t *>(pool().take(words * sizeof(uint64_t)));
+    lane_ = g_lane;
+    ptr_ = static_cast<uint64_t *>(pool().take(words * sizeof(uint64_t), lane_));
     words_ = words;
 }
 
 void DeviceBuffer::release() {
-    if (ptr_) pool().give(ptr_, words_ * sizeof(uint64_t));
+    if (ptr_) pool().give(ptr_, words_ * sizeof(uint64_t), lane_);
     ptr_ = nullptr;
     words_ = 0;
 }
 
 DeviceBuffer::DeviceBuffer(const DeviceBuffer &o) {
     allocate(o.words_);
-    if (words_) check_status(he_memcpy_d2d(ptr_, o.ptr_, words_ * sizeof(uint64_t), nullptr), "device copy failed");
+    if (words_) check_status(he_memcpy_d2d(ptr_, o.ptr_, words_ * sizeof(uint64_t), current_stream()), "device copy failed");
 }
 
 DeviceBuffer &DeviceBuffer::operator=(const DeviceBuffer &o) {
     if (this == &o) return *this;
     if (words_ != o.words_) allocate(o.words_);
-    if (words_) check_status(he_memcpy_d2d(ptr_, o.ptr_, words_ * sizeof(uint64_t), nullptr), "device copy failed");
+    if (words_) check_status(he_memcpy_d2d(ptr_, o.ptr_, words_ * sizeof(uint64_t), current_stream()), "device copy failed");
     return *this;
 }
 
@@ -126,6 +135,7 @@ DeviceBuffer &DeviceBuffer::operator=(DeviceBuffer &&o) noexcept {
         release();
         ptr_ = o.ptr_;
         words_ = o.words_;
+        lane_ = o.lane_;
         o.ptr_ = nullptr;
         o.words_ = 0;
     }
@@ -133,6 +143,23 @@ DeviceBuffer &DeviceBuffer::operator=(DeviceBuffer &&o) noexcept {
 }
 
 void DeviceBuffer::trim_pool() { pool().trim(); }
+
+he_stream current_stream() { return g_lane_streams[g_lane]; }
+
+int current_lane() { return g_lane; }
+
+int lane_count() { return kMaxLanes; }
+
+void set_lane(int lane) {
+    if (lane < 0 || lane > kMaxLanes) throw std::invalid_argument("lane out of range");
+    if (lane > 0 && !g_lane_streams[lane]) check_status(he_stream_create(&g_lane_streams[lane]), "stream creation failed");
+    g_lane = lane;
+}
+
+void synchronize_lanes() {
+    for (int i = 0; i <= kMaxLanes; i++)
+        if (i == 0 || g_lane_streams[i]) check_status(he_stream_synchronize(g_lane_streams[i]), "synchronisation failed");
+}
 
 }  // namespace cahel
 
@@ -177,7 +204,7 @@ void CAHELGPUCiphertext::resize(std::size_t size, std::size_t coeff_modulus_size
         DeviceBuffer fresh(new_words);
         const std::size_t keep = old_words < new_words ? old_words : new_words;
         if (keep && data_.get())
-            check_status(he_memcpy_d2d(fresh.get(), data_.get(), keep * sizeof(uint64_t), nullptr), "device copy failed");
+            check_status(he_memcpy_d2d(fresh.get(), data_.get(), keep * sizeof(uint64_t), current_stream()), "device copy failed");
         data_ = std::move(fresh);
     }
     size_ = size;

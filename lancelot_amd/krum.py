@@ -27,6 +27,7 @@ class KrumConfig:
     special_modulus_size: int = 1            # GPU_init: size_P = 1
     scale: float = 2.0 ** 40
     hoisting: bool = True                    # byzantine_fl.py: Hoisting_flag = 1
+    lanes: int = 4                           # independent pairs are spread over this many streams (0: null stream)
     sec_level: str = "tc128"
     seed: int | None = None
 
@@ -140,6 +141,27 @@ def pair_distance(state: KrumState, cts_i, cts_j):
     return acc
 
 
+def all_pair_distances(state: KrumState, cts, enc):
+    """enc[i][j] = enc[j][i] = pair_distance(i, j) for every i < j.  The pairs are independent, and at Lancelot's
+    sizes (three or four limbs) one of them does not fill the GPU, so they are dealt round-robin to the lanes
+    (streams) of the host layer; everything is synchronised before returning."""
+    c = state.cahel
+    n_clients = len(cts)
+    lanes = min(state.config.lanes, c._lane_count())
+    _sync(c)
+    k = 0
+    try:
+        for i in range(n_clients):
+            for j in range(i + 1, n_clients):
+                if lanes > 0:
+                    c._set_lane(1 + k % lanes)
+                enc[i][j] = enc[j][i] = pair_distance(state, cts[i], cts[j])
+                k += 1
+    finally:
+        c._set_lane(0)
+    _sync(c)
+
+
 def distance_matrix(state: KrumState, updates):
     """Encrypted pairwise squared distances and their decryptions (slot 0 of every pair)."""
     c = state.cahel
@@ -148,10 +170,7 @@ def distance_matrix(state: KrumState, updates):
     n_clients = len(updates)
     enc = [[None] * n_clients for _ in range(n_clients)]
     t0 = time.perf_counter()
-    for i in range(n_clients):
-        for j in range(i + 1, n_clients):
-            enc[i][j] = enc[j][i] = pair_distance(state, cts[i], cts[j])
-    _sync(c)
+    all_pair_distances(state, cts, enc)
     state.timings["evaluate"] += time.perf_counter() - t0
     t0 = time.perf_counter()
     dist = np.zeros((n_clients, n_clients))
@@ -258,10 +277,7 @@ def gpu_krum_aggregate(updates, config: KrumConfig | None = None, state: KrumSta
     n_clients = len(updates)
     enc = [[None] * n_clients for _ in range(n_clients)]
     t1 = time.perf_counter()
-    for i in range(n_clients):
-        for j in range(i + 1, n_clients):
-            enc[i][j] = enc[j][i] = pair_distance(state, cts[i], cts[j])
-    _sync(state.cahel)
+    all_pair_distances(state, cts, enc)
     state.timings["evaluate"] += time.perf_counter() - t1
     mask, order, _ = decrypt_sort_mask(state, enc)
     weights = mul_mask_weight(state, cts, mask[0])
