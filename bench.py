@@ -97,7 +97,7 @@ def cpu_baseline(seconds_budget=12.0):
     while True:
         op()
         iters += 1
-        if time.time() - t0 > seconds_budget or iters >= 200:
+        if time.time() - t0 > seconds_budget or iters >= 2000:
             break
     dt = (time.time() - t0) / iters
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
