@@ -59,6 +59,8 @@ int he_event_create(he_event *event);
 int he_event_destroy(he_event event);
 int he_event_record(he_event event, he_stream stream);
 int he_event_synchronize(he_event event);
+/* Work enqueued on `stream` after this call starts only when `event` (recorded on another stream) has completed. */
+int he_stream_wait_event(he_stream stream, he_event event);
 int he_event_elapsed_ms(he_event start, he_event stop, float *ms);
 
 /* ---- parameter tables ---- */

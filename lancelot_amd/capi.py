@@ -32,6 +32,7 @@ SIGNATURES = {
     "he_event_destroy": (C.c_int, [vp]),
     "he_event_record": (C.c_int, [vp, vp]),
     "he_event_synchronize": (C.c_int, [vp]),
+    "he_stream_wait_event": (C.c_int, [vp, vp]),
     "he_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
     "he_context_create": (C.c_int, [vp, C.POINTER(vp)]),
     "he_context_set_level": (C.c_int, [vp, vp]),

@@ -227,6 +227,12 @@ int he_event_record(he_event e, he_stream s) {
     return HE_OK;
 }
 
+int he_stream_wait_event(he_stream s, he_event e) {
+    if (!e) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(hipStreamWaitEvent(S(s), static_cast<hipEvent_t>(e), 0));
+    return HE_OK;
+}
+
 int he_event_synchronize(he_event e) {
     HE_HIP(hipEventSynchronize(static_cast<hipEvent_t>(e)));
     return HE_OK;
