@@ -218,52 +218,55 @@ PYBIND11_MODULE(pyCAHEL, m) {
                                       (py::ssize_t)c.poly_modulus_degree()});
         });
 
-    m.def("negate", &negate);
-    m.def("negate_inplace", &negate_inplace);
-    m.def("add", &add);
-    m.def("add_inplace", &add_inplace);
-    m.def("add_plain", &add_plain);
-    m.def("add_plain_inplace", &add_plain_inplace);
-    m.def("add_many", &add_many);
-    m.def("sub", &sub);
+    // The evaluator only enqueues device work and touches no Python state: the interpreter lock is released so
+    // that several Python threads, each on its own lane, can issue independent pipelines concurrently.
+    const py::call_guard<py::gil_scoped_release> nogil;
+    m.def("negate", &negate, nogil);
+    m.def("negate_inplace", &negate_inplace, nogil);
+    m.def("add", &add, nogil);
+    m.def("add_inplace", &add_inplace, nogil);
+    m.def("add_plain", &add_plain, nogil);
+    m.def("add_plain_inplace", &add_plain_inplace, nogil);
+    m.def("add_many", &add_many, nogil);
+    m.def("sub", &sub, nogil);
     m.def("sub_inplace", &sub_inplace, py::arg("context"), py::arg("encrypted1"), py::arg("encrypted2"),
-          py::arg("negate") = false);
-    m.def("sub_plain", &sub_plain);
-    m.def("sub_plain_inplace", &sub_plain_inplace);
-    m.def("multiply", &multiply);
-    m.def("multiply_inplace", &multiply_inplace);
-    m.def("multiply_and_relin_inplace", &multiply_and_relin_inplace);
-    m.def("multiply_plain", &multiply_plain);
-    m.def("multiply_plain_inplace", &multiply_plain_inplace);
-    m.def("multiply_many", &multiply_many);
-    m.def("square", &square);
-    m.def("square_inplace", &square_inplace);
-    m.def("exponentiate", &exponentiate);
-    m.def("exponentiate_inplace", &exponentiate_inplace);
-    m.def("relinearize", &relinearize);
-    m.def("relinearize_inplace", &relinearize_inplace);
-    m.def("mod_switch_to", py::overload_cast<const CAHELGPUContext &, const CAHELGPUPlaintext &, CAHELGPUPlaintext &, std::size_t>(&mod_switch_to));
-    m.def("mod_switch_to", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &, CAHELGPUCiphertext &, std::size_t>(&mod_switch_to));
-    m.def("mod_switch_to_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUPlaintext &, std::size_t>(&mod_switch_to_inplace));
-    m.def("mod_switch_to_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUCiphertext &, std::size_t>(&mod_switch_to_inplace));
-    m.def("mod_switch_to_next", py::overload_cast<const CAHELGPUContext &, const CAHELGPUPlaintext &, CAHELGPUPlaintext &>(&mod_switch_to_next));
-    m.def("mod_switch_to_next", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &, CAHELGPUCiphertext &>(&mod_switch_to_next));
-    m.def("mod_switch_to_next_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUPlaintext &>(&mod_switch_to_next_inplace));
-    m.def("mod_switch_to_next_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUCiphertext &>(&mod_switch_to_next_inplace));
-    m.def("rescale_to_next", &rescale_to_next);
-    m.def("rescale_to_next_inplace", &rescale_to_next_inplace);
-    m.def("apply_galois", &apply_galois);
-    m.def("apply_galois_inplace", &apply_galois_inplace);
-    m.def("rotate_rows", &rotate_rows);
-    m.def("rotate_rows_inplace", &rotate_rows_inplace);
-    m.def("rotate_columns", &rotate_columns);
-    m.def("rotate_columns_inplace", &rotate_columns_inplace);
-    m.def("rotate_vector", &rotate_vector);
-    m.def("rotate_vector_inplace", &rotate_vector_inplace);
-    m.def("hoisting", &hoisting);
-    m.def("hoisting_inplace", &hoisting_inplace);
-    m.def("complex_conjugate", &complex_conjugate);
-    m.def("complex_conjugate_inplace", &complex_conjugate_inplace);
+          py::arg("negate") = false, nogil);
+    m.def("sub_plain", &sub_plain, nogil);
+    m.def("sub_plain_inplace", &sub_plain_inplace, nogil);
+    m.def("multiply", &multiply, nogil);
+    m.def("multiply_inplace", &multiply_inplace, nogil);
+    m.def("multiply_and_relin_inplace", &multiply_and_relin_inplace, nogil);
+    m.def("multiply_plain", &multiply_plain, nogil);
+    m.def("multiply_plain_inplace", &multiply_plain_inplace, nogil);
+    m.def("multiply_many", &multiply_many, nogil);
+    m.def("square", &square, nogil);
+    m.def("square_inplace", &square_inplace, nogil);
+    m.def("exponentiate", &exponentiate, nogil);
+    m.def("exponentiate_inplace", &exponentiate_inplace, nogil);
+    m.def("relinearize", &relinearize, nogil);
+    m.def("relinearize_inplace", &relinearize_inplace, nogil);
+    m.def("mod_switch_to", py::overload_cast<const CAHELGPUContext &, const CAHELGPUPlaintext &, CAHELGPUPlaintext &, std::size_t>(&mod_switch_to), nogil);
+    m.def("mod_switch_to", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &, CAHELGPUCiphertext &, std::size_t>(&mod_switch_to), nogil);
+    m.def("mod_switch_to_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUPlaintext &, std::size_t>(&mod_switch_to_inplace), nogil);
+    m.def("mod_switch_to_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUCiphertext &, std::size_t>(&mod_switch_to_inplace), nogil);
+    m.def("mod_switch_to_next", py::overload_cast<const CAHELGPUContext &, const CAHELGPUPlaintext &, CAHELGPUPlaintext &>(&mod_switch_to_next), nogil);
+    m.def("mod_switch_to_next", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &, CAHELGPUCiphertext &>(&mod_switch_to_next), nogil);
+    m.def("mod_switch_to_next_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUPlaintext &>(&mod_switch_to_next_inplace), nogil);
+    m.def("mod_switch_to_next_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUCiphertext &>(&mod_switch_to_next_inplace), nogil);
+    m.def("rescale_to_next", &rescale_to_next, nogil);
+    m.def("rescale_to_next_inplace", &rescale_to_next_inplace, nogil);
+    m.def("apply_galois", &apply_galois, nogil);
+    m.def("apply_galois_inplace", &apply_galois_inplace, nogil);
+    m.def("rotate_rows", &rotate_rows, nogil);
+    m.def("rotate_rows_inplace", &rotate_rows_inplace, nogil);
+    m.def("rotate_columns", &rotate_columns, nogil);
+    m.def("rotate_columns_inplace", &rotate_columns_inplace, nogil);
+    m.def("rotate_vector", &rotate_vector, nogil);
+    m.def("rotate_vector_inplace", &rotate_vector_inplace, nogil);
+    m.def("hoisting", &hoisting, nogil);
+    m.def("hoisting_inplace", &hoisting_inplace, nogil);
+    m.def("complex_conjugate", &complex_conjugate, nogil);
+    m.def("complex_conjugate_inplace", &complex_conjugate_inplace, nogil);
 
     m.def("_naf", &naf);
     m.def("_get_primes", &get_primes);

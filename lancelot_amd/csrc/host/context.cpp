@@ -56,8 +56,9 @@ namespace {
 // Lanes: lane 0 is the null stream (what the reference uses for everything); lanes 1 .. kMaxLanes are
 // non-blocking streams created on first use.  Work of different lanes may overlap on the GPU.
 constexpr int kMaxLanes = 8;
-int g_lane = 0;
+thread_local int g_lane = 0;  // every host thread has its own current lane
 he_stream g_lane_streams[kMaxLanes + 1] = {};
+std::mutex g_lane_mu;
 
 struct Pool {
     std::mutex mu;
@@ -152,7 +153,10 @@ int lane_count() { return kMaxLanes; }
 
 void set_lane(int lane) {
     if (lane < 0 || lane > kMaxLanes) throw std::invalid_argument("lane out of range");
-    if (lane > 0 && !g_lane_streams[lane]) check_status(he_stream_create(&g_lane_streams[lane]), "stream creation failed");
+    if (lane > 0) {
+        std::lock_guard<std::mutex> g(g_lane_mu);
+        if (!g_lane_streams[lane]) check_status(he_stream_create(&g_lane_streams[lane]), "stream creation failed");
+    }
     g_lane = lane;
 }
 

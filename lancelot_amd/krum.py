@@ -27,7 +27,8 @@ class KrumConfig:
     special_modulus_size: int = 1            # GPU_init: size_P = 1
     scale: float = 2.0 ** 40
     hoisting: bool = True                    # byzantine_fl.py: Hoisting_flag = 1
-    lanes: int = 4                           # independent pairs are spread over this many streams (0: null stream)
+    lanes: int = 3                           # host threads / streams that the pairs are dealt to (0: null stream);
+                                             # three streams and the null stream fill the four hardware queues
     sec_level: str = "tc128"
     seed: int | None = None
 
@@ -143,22 +144,29 @@ def pair_distance(state: KrumState, cts_i, cts_j):
 
 def all_pair_distances(state: KrumState, cts, enc):
     """enc[i][j] = enc[j][i] = pair_distance(i, j) for every i < j.  The pairs are independent, and at Lancelot's
-    sizes (three or four limbs) one of them does not fill the GPU, so they are dealt round-robin to the lanes
-    (streams) of the host layer; everything is synchronised before returning."""
+    sizes (three or four limbs) one of them neither fills the GPU nor keeps one host thread's launch rate busy, so
+    they are dealt round-robin to `lanes` host threads, each issuing on its own lane (stream) of the host layer
+    (the evaluator calls release the interpreter lock); everything is synchronised before returning."""
     c = state.cahel
     n_clients = len(cts)
-    lanes = min(state.config.lanes, c._lane_count())
+    pairs = [(i, j) for i in range(n_clients) for j in range(i + 1, n_clients)]
+    lanes = min(state.config.lanes, c._lane_count(), max(len(pairs), 1))
     _sync(c)
-    k = 0
-    try:
-        for i in range(n_clients):
-            for j in range(i + 1, n_clients):
-                if lanes > 0:
-                    c._set_lane(1 + k % lanes)
-                enc[i][j] = enc[j][i] = pair_distance(state, cts[i], cts[j])
-                k += 1
-    finally:
-        c._set_lane(0)
+    if lanes <= 0:
+        for i, j in pairs:
+            enc[i][j] = enc[j][i] = pair_distance(state, cts[i], cts[j])
+        _sync(c)
+        return
+
+    def worker(w):
+        c._set_lane(1 + w)          # the current lane is per host thread
+        return [(i, j, pair_distance(state, cts[i], cts[j])) for i, j in pairs[w::lanes]]
+
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=lanes) as pool:
+        for part in pool.map(worker, range(lanes)):
+            for i, j, ct in part:
+                enc[i][j] = enc[j][i] = ct
     _sync(c)
 
 
