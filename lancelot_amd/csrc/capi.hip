@@ -59,6 +59,7 @@ struct he_context {
     std::vector<uint64_t> h_moduli;
     std::vector<uint8_t> fp_ok;  // per table: prime below 2^50
     bool use_fp = true;          // environment CAHEL_HIP_NO_FP64=1 forces the integer back end
+    bool fuse_inner = true;      // environment CAHEL_HIP_NO_FUSED_KS=1: separate NTT and inner-product kernels
     std::vector<Level> levels;   // indexed by L
     std::vector<void *> owned;
 
@@ -307,6 +308,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         // FP64 back end: twiddles as doubles (inverse ones un-halved), per-table constants
         const char *env = getenv("CAHEL_HIP_NO_FP64");
         ctx->use_fp = !(env && env[0] == '1');
+        const char *nf = getenv("CAHEL_HIP_NO_FUSED_KS");
+        ctx->fuse_inner = !(nf && nf[0] == '1');
         ctx->fp_ok.assign(qp, 0);
         std::vector<double> psi_fp(qp * n, 0.0), ipsi_fp(qp * n, 0.0), consts(4 * qp, 0.0);
         for (size_t t = 0; t < qp; t++) {
@@ -712,12 +715,51 @@ int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uin
     uint64_t *tmp = cx + 2 * LK * n;
     const uint64_t *src = c;
     if (galois_elt) {
-        // sigma(c) is staged in the (not yet used) inner-product buffer
-        if (int rc = he_galois_ntt(ctx, c, cx, L, galois_elt, s)) return rc;
-        src = cx;
+        // sigma(c) is staged in the second half of the ModDown workspace, which ModUp leaves alone and ModDown
+        // only touches after the inner product has read it
+        uint64_t *staged = tmp + (size_t)L * n;
+        if (int rc = he_galois_ntt(ctx, c, staged, L, galois_elt, s)) return rc;
+        src = staged;
     }
-    if (int rc = he_modup(ctx, L, src, y, tmp, s)) return rc;
-    if (int rc = he_ks_inner_product(ctx, L, y, evk, cx, 0, 0, s)) return rc;
+    if (ctx->fuse_inner && lv->batched && fp_for_level(ctx, L)) {
+        // ModUp without the copy of a digit's own limbs, then the forward NTT fused with the inner product: the
+        // transformed digits are never written (216 limb transfers less at L = 24, K = 8)
+        NttArgs inv = base_args(ctx, false);
+        inv.in = src;
+        inv.out = tmp;
+        inv.in_poly_stride = inv.out_poly_stride = L;
+        inv.map = plain_map(L, 0);
+        inv.epi_mode = NTT_EPI_MUL;
+        inv.w = lv->d_part_hat_inv;
+        HE_HIP(launch_ntt_inverse(inv, 1, true, S(s)));
+        BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
+                     lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts};
+        HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+        NttArgs fwd = base_args(ctx, true);
+        fwd.in = y;
+        fwd.out = y;
+        fwd.jobs = lv->d_modup_jobs;
+        fwd.n_jobs = lv->n_modup_jobs;
+        fwd.groups = lv->d_modup_groups;
+        fwd.n_groups = lv->n_modup_groups;
+        KsFuseArgs x;
+        memset(&x, 0, sizeof(x));
+        for (uint32_t d = 0; d < lv->beta; d++) {
+            if (!evk[d]) return HE_E_INVALID_ARGUMENT;
+            x.evk.p[d] = evk[d];
+        }
+        x.own = src;
+        x.out = cx;
+        x.L = L;
+        x.K = ctx->size_p;
+        x.size_q = ctx->size_q;
+        x.size_qp = ctx->size_qp;
+        x.beta = lv->beta;
+        HE_HIP(launch_ntt_forward_inner(fwd, x, S(s)));
+    } else {
+        if (int rc = he_modup(ctx, L, src, y, tmp, s)) return rc;
+        if (int rc = he_ks_inner_product(ctx, L, y, evk, cx, 0, 0, s)) return rc;
+    }
     return he_moddown(ctx, L, cx, ct, 2, 1, tmp, s);
 }
 

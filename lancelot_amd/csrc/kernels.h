@@ -154,6 +154,19 @@ hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtr
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
                                 hipStream_t s);
 
+// Forward NTT of ModUp's converted limbs fused with the key-switch inner product (FP64 back end only).
+// `a` describes the converted limbs as launch_ntt_forward's job list does (a.out = the beta x (L+K) x N digit
+// buffer, whose own-digit limbs are never touched); the blocks pass multiplies every transformed tile by the
+// matching key tile and accumulates over the digits, so the transformed limbs are never written:
+//   out[k][t] = sum_d y_d[t] * evk_d[k][t],  y_d[t] = own[t] for the limbs t of digit d itself.
+struct KsFuseArgs {
+    EvkPtrs evk;          // per digit: [2][size_qp][N], NTT form
+    const uint64_t *own;  // the key-switch input c, [L][N], NTT form
+    uint64_t *out;        // [2][L+K][N]
+    uint32_t L, K, size_q, size_qp, beta;
+};
+hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s);
+
 hipError_t launch_decompose_real(const Tables &t, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,
                                  hipStream_t s);
 

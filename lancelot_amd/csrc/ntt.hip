@@ -472,6 +472,101 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_fp_kernel(NttArgs a) {
     }
 }
 
+// Forward blocks pass of ModUp fused with the key-switch inner product.  Workgroup = (limb t of Ql u P, tile of
+// 16 T words): its first T threads transform that tile of every digit in turn; all 2 T threads then multiply
+// it by a key polynomial (threads below T by the first, the others by the second) and accumulate in registers.
+// The key tiles are fetched before the butterflies start, so that they travel meanwhile; the digit that owns
+// limb t contributes the input itself.
+template <uint32_t T>
+__global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, KsFuseArgs x) {
+    __shared__ uint64_t lds[16 * T + T];
+    constexpr uint32_t half = T, tile_elems = half << 4;
+    const uint32_t role = threadIdx.x >= half ? 1u : 0u;       // which key polynomial this thread accumulates
+    const uint32_t tid = threadIdx.x - role * half;
+    const uint32_t lr = a.log_n - 8;
+    const uint32_t log_b = 31 - __builtin_clz(tile_elems >> 8);
+    const uint32_t tiles_per_limb = 1u << (lr - log_b);
+    const uint32_t lb = logical_block();
+    const uint32_t t = lb / tiles_per_limb, tile = lb % tiles_per_limb;
+    const size_t n = (size_t)1 << a.log_n;
+    const size_t off = (size_t)tile * tile_elems;
+    const uint32_t blk0 = tile << log_b;
+    const uint32_t LK = x.L + x.K;
+    const uint32_t table = t < x.L ? t : x.size_q + (t - x.L);
+    const uint32_t own = t < x.L ? t / x.K : 0xffffffffu;
+    double *ld = reinterpret_cast<double *>(lds);
+    const FpCtx fc = fp_ctx(a, table);
+    const FpMod m = fc.m;
+
+    const uint32_t base0 = ((tid >> 4) << 8) | (tid & 15);
+    const uint32_t base1 = tid << 4;
+    // the twiddles stay in the table (the digits after the first find them in cache)
+    const uint32_t idx0 = (1u << lr) + blk0 + (tid >> 4), idx1 = (1u << (lr + 4)) + (blk0 << 4) + tid;
+
+    const size_t key_off = ((size_t)role * x.size_qp + table) * n + off;
+    double acc[kPer];
+    if (own != 0xffffffffu) {
+        const uint64_t *src = x.own + (size_t)t * n + off;
+        const uint64_t *key = x.evk.p[own] + key_off;
+#pragma unroll
+        for (int i = 0; i < kPer; i++) {
+            const double w = fp_from_u64(key[tid + i * half]);
+            acc[i] = fp_mulmod(fp_from_u64(src[tid + i * half]), FpTw{w, w * m.qinv}, m);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < kPer; i++) acc[i] = 0.0;
+    }
+
+    uint32_t terms = 1;
+    for (uint32_t d = 0; d < x.beta; d++) {
+        if (d == own) continue;
+        const uint64_t *key = x.evk.p[d] + key_off;
+        uint64_t pk[kPer];
+#pragma unroll
+        for (int i = 0; i < kPer; i++) pk[i] = key[tid + i * half];
+        if (!role) {
+            const uint64_t *src = a.out + ((size_t)d * LK + t) * n + off;  // lazy values left by the rows pass
+#pragma unroll
+            for (int i = 0; i < kPer; i++) lds[skew(tid + i * half)] = src[tid + i * half];
+        }
+        lds_barrier();
+        if (!role) {
+            double v[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[skew(base0 + (j << 4))];
+            fp_ct_block<4, true>(v, fc.tw, idx0, m);
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
+        }
+        lds_barrier();
+        if (!role) {
+            double v[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[skew(base1 + j)];
+            fp_ct_block<4, true>(v, fc.tw, idx1, m);
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[skew(base1 + j)] = v[j];
+        }
+        lds_barrier();
+        // every term is below 0.7 q, so eight of them fit between two reductions of the accumulators
+#pragma unroll
+        for (int i = 0; i < kPer; i++) {
+            const double y = fp_reduce(ld[skew(tid + i * half)], m);
+            const double w = fp_from_u64(pk[i]);
+            acc[i] += fp_mulmod(y, FpTw{w, w * m.qinv}, m);
+        }
+        if ((++terms & 7) == 0) {
+#pragma unroll
+            for (int i = 0; i < kPer; i++) acc[i] = fp_reduce(acc[i], m);
+        }
+        lds_barrier();  // every read of this tile is done before the next one overwrites it
+    }
+    uint64_t *o = x.out + ((size_t)role * LK + t) * n + off;
+#pragma unroll
+    for (int i = 0; i < kPer; i++) o[tid + i * half] = fp_to_u64(fp_canonical(acc[i], m));
+}
+
 // Integer back end (twiddles stay in the table: 30 Shoup pairs per thread do not fit in registers).
 template <bool FWD>
 __global__ __launch_bounds__(kThreads) void ntt_blocks_int_kernel(NttArgs a) {
@@ -615,6 +710,24 @@ hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, bool fp, hipSt
     hipError_t e = fp ? launch_rows<true, true>(a, n_jobs, s) : launch_rows<true, false>(a, n_jobs, s);
     if (e != hipSuccess) return e;
     return fp ? launch_blocks<true, true>(a, n_polys, s) : launch_blocks<true, false>(a, n_polys, s);
+}
+
+hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s) {
+    if (a.log_n < 9 || a.log_n > 16 || !a.jobs) return hipErrorInvalidValue;
+    if (a.n_jobs) {
+        hipError_t e = launch_rows<true, true>(a, a.n_jobs, s);
+        if (e != hipSuccess) return e;
+    }
+    const uint32_t n = 1u << a.log_n;
+    const uint32_t tile = n < 2048 ? n : 2048;
+    const dim3 grid((x.L + x.K) * (n / tile));
+    if (tile == 2048)
+        hipLaunchKernelGGL(ntt_blocks_fp_inner_kernel<128>, grid, dim3(256), 0, s, a, x);
+    else if (tile == 1024)
+        hipLaunchKernelGGL(ntt_blocks_fp_inner_kernel<64>, grid, dim3(128), 0, s, a, x);
+    else
+        hipLaunchKernelGGL(ntt_blocks_fp_inner_kernel<32>, grid, dim3(64), 0, s, a, x);
+    return hipGetLastError();
 }
 
 hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s) {
