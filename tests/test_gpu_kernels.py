@@ -135,6 +135,29 @@ def test_integer_and_fp64_back_ends_agree(oracle, capi, monkeypatch):
     assert (results[0] == results[1]).all()
 
 
+@pytest.mark.parametrize("logn,bits,size_p,L", [(13, [50, 50, 49, 50, 50, 50], 2, 4), (13, [50, 50, 49, 50, 50, 50], 2, 3),
+                                                 (11, [45, 40, 40, 50], 1, 3), (9, [40, 40, 45, 45], 2, 2)])
+def test_fused_and_separate_key_switch_agree(oracle, capi, monkeypatch, logn, bits, size_p, L):
+    """he_keyswitch with the inner product inside the forward NTT (default for primes below 2^50) and, forced by the
+    environment, with the separate kernels: both equal the oracle, with and without a Galois element, with a
+    partial last digit (L = 3 over two special primes) and at the smallest degree."""
+    for no_fuse in ("0", "1"):
+        monkeypatch.setenv("CAHEL_HIP_NO_FUSED_KS", no_fuse)
+        cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+        rng = np.random.default_rng(12)
+        lib, h = capi.lib(), ctx.he_handle()
+        host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+        ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+        for elt in (0, 5):
+            c = rand_limbs(p, rng, range(L))
+            ct = rand_limbs(p, rng, range(L), n_polys=2)
+            dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
+            capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, elt, ws.ptr, None))
+            ks = p.key_switch(p.galois_ntt(c, elt) if elt else c, host_evk)
+            want = np.stack([p.add(ct[b], ks[b]) for b in range(2)])
+            assert (dct.numpy() == want).all(), (no_fuse, elt)
+
+
 def test_ntt_rejects_bad_arguments(small, capi):
     cahel, parms, ctx, p = small
     d = DeviceArray(capi, shape=(1, p.n))
