@@ -136,7 +136,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--lanes", type=int, default=4, help="streams that the timed operations are dealt to")
+    ap.add_argument("--lanes", type=int, default=3,
+                    help="streams that the timed operations are dealt to (three and the null stream fill the four "
+                         "hardware queues of a process; four measured slower than three or six)")
     ap.add_argument("--only", choices=["all", "roofline", "krum"], default="all",
                     help="roofline: run just the kernel the roofline object describes (for rocprofv3)")
     args = ap.parse_args()
