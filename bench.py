@@ -139,6 +139,8 @@ def main():
     ap.add_argument("--lanes", type=int, default=3,
                     help="streams that the timed operations are dealt to (three and the null stream fill the four "
                          "hardware queues of a process; four measured slower than three or six)")
+    ap.add_argument("--separate-rescale", action="store_true",
+                    help="he_keyswitch then he_rescale instead of the merged he_keyswitch_rescale")
     ap.add_argument("--only", choices=["all", "roofline", "krum"], default="all",
                     help="roofline: run just the kernel the roofline object describes (for rocprofv3)")
     args = ap.parse_args()
@@ -200,10 +202,18 @@ def main():
     rs_ws = Buf(capi, 2 * n)
     a_ptr, b_ptr = ct1.data_ptr(), ct2.data_ptr()
 
+    # relinearise + rescale: one C-ABI call (ModDown's and the rescale's forward transforms merged, same limbs), or,
+    # with --separate-rescale, the two calls that the evaluator's relinearize_inplace / rescale_to_next_inplace make
+    def relin_rescale(t3_, res_, ws_, rs_, st):
+        if args.separate_rescale:
+            capi.check(lib.he_keyswitch(h, L, t3_.at(2 * L * n), evk, t3_.ptr, 0, ws_.ptr, st))
+            capi.check(lib.he_rescale(h, t3_.ptr, res_.ptr, 2, L, rs_.ptr, st))
+        else:
+            capi.check(lib.he_keyswitch_rescale(h, L, t3_.at(2 * L * n), evk, t3_.ptr, res_.ptr, 0, ws_.ptr, st))
+
     def step():
         capi.check(lib.he_tensor(h, a_ptr, b_ptr, t3.ptr, L, None))
-        capi.check(lib.he_keyswitch(h, L, t3.at(2 * L * n), evk, t3.ptr, 0, ws.ptr, None))
-        capi.check(lib.he_rescale(h, t3.ptr, res.ptr, 2, L, rs_ws.ptr, None))
+        relin_rescale(t3, res, ws, rs_ws, None)
 
     # (1) one operation after the other on the null stream: the latency of a single HMult + relin + rescale
     for _ in range(args.warmup):
@@ -230,8 +240,7 @@ def main():
         lws, lt3, lres, lrs = lane_bufs[k]
         st = lane_streams[k]
         capi.check(lib.he_tensor(h, a_ptr, b_ptr, lt3.ptr, L, st))
-        capi.check(lib.he_keyswitch(h, L, lt3.at(2 * L * n), evk, lt3.ptr, 0, lws.ptr, st))
-        capi.check(lib.he_rescale(h, lt3.ptr, lres.ptr, 2, L, lrs.ptr, st))
+        relin_rescale(lt3, lres, lws, lrs, st)
 
     def lanes_sync():
         for st in lane_streams:

@@ -176,7 +176,8 @@ int he_ks_inner_product(const he_context *ctx, uint32_t L, const uint64_t *y, co
 int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, uint32_t n_polys, int accumulate,
                uint64_t *workspace, he_stream stream);
 
-/* Words of workspace he_keyswitch needs at level L: beta*(L+K)*N + 2*(L+K)*N + 2*L*N. */
+/* Words of workspace he_keyswitch and he_keyswitch_rescale need at level L:
+ * beta*(L+K)*N + 2*(L+K)*N + 2*L*N + 2*N. */
 size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L);
 
 /* ct[0..1] += KeySwitch(c): c [L][N], ct [2][L][N], evk as in he_ks_inner_product.  galois_elt != 0 switches
@@ -184,6 +185,15 @@ size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L);
  * Replaces switch_key_inplace (src/eval_key_switch.cu:80-216). */
 int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk, uint64_t *ct,
                  uint32_t galois_elt, uint64_t *workspace, he_stream stream);
+
+/* out [2][L-1][N] = rescale(ct + KeySwitch(c)): he_keyswitch followed by he_rescale with the same limbs, in one
+ * pass less over the data (ModDown's and the rescale's forward transforms are merged: the NTT is linear).
+ * ct [2][L][N] is only read.  workspace as for he_keyswitch.
+ * Replaces the sequence switch_key_inplace (src/eval_key_switch.cu:80-216) + rescale_to_next
+ * (src/evaluate.cu:2058-2085) that relinearize_inplace + rescale_to_next_inplace run back to back. */
+int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk,
+                         const uint64_t *ct, uint64_t *out, uint32_t galois_elt, uint64_t *workspace,
+                         he_stream stream);
 
 /* ---- encoder support ----
  * coeffs: DEVICE array of N doubles holding integers (already rounded, |c| < 2^63); out [limbs][N]:

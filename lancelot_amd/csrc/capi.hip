@@ -701,14 +701,17 @@ size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L) {
     if (!ctx || ctx->size_p == 0 || L == 0 || L > ctx->size_q) return 0;
     const size_t n = ctx->n(), K = ctx->size_p, LK = L + K;
     const size_t beta = (L + K - 1) / K;
-    return beta * LK * n + 2 * LK * n + 2 * (size_t)L * n;
+    // digits | inner product | ModDown scratch | last limb of both polynomials (he_keyswitch_rescale)
+    return beta * LK * n + 2 * LK * n + 2 * (size_t)L * n + 2 * n;
 }
 
-int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk, uint64_t *ct,
-                 uint32_t galois_elt, uint64_t *ws, he_stream s) {
-    if (!ctx || !c || !evk || !ct || !ws || ctx->size_p == 0) return HE_E_INVALID_ARGUMENT;
-    const Level *lv = level_of(ctx, L);
-    if (!lv) return HE_E_LEVEL_NOT_SET;
+}  // extern "C"
+
+namespace {
+
+// ModUp and inner product of a key switch: ws -> cx [2][L+K][N] (the layout of he_keyswitch_workspace_words)
+int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint64_t *c, const uint64_t *const *evk,
+                  uint32_t galois_elt, uint64_t *ws, he_stream s) {
     const size_t n = ctx->n(), LK = L + ctx->size_p;
     uint64_t *y = ws;
     uint64_t *cx = y + (size_t)lv->beta * LK * n;
@@ -760,7 +763,97 @@ int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uin
         if (int rc = he_modup(ctx, L, src, y, tmp, s)) return rc;
         if (int rc = he_ks_inner_product(ctx, L, y, evk, cx, 0, 0, s)) return rc;
     }
+    return HE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk, uint64_t *ct,
+                 uint32_t galois_elt, uint64_t *ws, he_stream s) {
+    if (!ctx || !c || !evk || !ct || !ws || ctx->size_p == 0) return HE_E_INVALID_ARGUMENT;
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    const size_t n = ctx->n(), LK = L + ctx->size_p;
+    uint64_t *cx = ws + (size_t)lv->beta * LK * n;
+    uint64_t *tmp = cx + 2 * LK * n;
+    if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, ws, s)) return rc;
     return he_moddown(ctx, L, cx, ct, 2, 1, tmp, s);
+}
+
+int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk,
+                         const uint64_t *ct, uint64_t *out, uint32_t galois_elt, uint64_t *ws, he_stream s) {
+    if (!ctx || !c || !evk || !ct || !out || !ws || ctx->size_p == 0 || L < 2) return HE_E_INVALID_ARGUMENT;
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    const size_t n = ctx->n();
+    const uint32_t K = ctx->size_p, LK = L + K;
+    uint64_t *cx = ws + (size_t)lv->beta * LK * n;
+    uint64_t *delta = cx + 2 * LK * n;             // [2][L][N]
+    uint64_t *last = delta + 2 * (size_t)L * n;    // [2][N]
+    if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, ws, s)) return rc;
+    // ModDown up to the base conversion: delta = P -> Ql conversion of the special limbs, coefficient form
+    NttArgs inv = base_args(ctx, false);
+    inv.in = cx + (size_t)L * n;
+    inv.out = cx + (size_t)L * n;
+    inv.in_poly_stride = inv.out_poly_stride = LK;
+    inv.map = plain_map(K, ctx->size_q);
+    inv.epi_mode = NTT_EPI_MUL;
+    inv.w = ctx->d_phat_inv;
+    HE_HIP(launch_ntt_inverse(inv, 2, fp_for(ctx, inv.map), S(s)));
+    if (lv->batched) {
+        BconvBatch b{cx, delta, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
+                     fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts};
+        HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+    } else {
+        for (uint32_t p = 0; p < 2; p++) {
+            BconvArgs b{cx + ((size_t)p * LK + L) * n, delta + (size_t)p * L * n, ctx->d_phat_mod_q, ctx->d_iota,
+                        ctx->d_iota, K, L};
+            HE_HIP(launch_bconv(ctx->tables(), b, S(s)));
+        }
+    }
+    const bool fp = fp_for(ctx, plain_map(L, 0));
+    // the last limb of the switched ciphertext, c'_{L-1} = (cx - NTT(delta)) P^-1 + ct, then its coefficients
+    NttArgs one = base_args(ctx, true);
+    one.in = one.out = delta + (size_t)(L - 1) * n;
+    one.in_poly_stride = one.out_poly_stride = L;
+    one.map = plain_map(1, L - 1);
+    one.epi_mode = NTT_EPI_SUB_MUL_ADD;
+    one.epi_a = cx + (size_t)(L - 1) * n;
+    one.epi_a_poly_stride = LK;
+    one.epi_b = ct + (size_t)(L - 1) * n;
+    one.epi_b_poly_stride = L;
+    one.w = ctx->d_pinv_mod_q + 2 * (size_t)(L - 1);
+    one.epi_dst = last;
+    one.epi_dst_poly_stride = 1;
+    HE_HIP(launch_ntt_forward(one, 2, fp, S(s)));
+    NttArgs linv = base_args(ctx, false);
+    linv.in = linv.out = last;
+    linv.in_poly_stride = linv.out_poly_stride = 1;
+    linv.map = plain_map(1, L - 1);
+    HE_HIP(launch_ntt_inverse(linv, 2, fp, S(s)));
+    // every other limb j: rescale(c')_j = ((cx_j P^-1 + ct_j) - NTT_j(delta_j P^-1 + [last]_{q_j})) q_last^-1.
+    // One transform serves ModDown and rescale because the NTT is linear; every step is exact modular
+    // arithmetic, so the limbs equal he_keyswitch followed by he_rescale.
+    NttArgs fwd = base_args(ctx, true);
+    fwd.in = fwd.out = delta;
+    fwd.in_poly_stride = fwd.out_poly_stride = L;
+    fwd.map = plain_map(L - 1, 0);
+    fwd.pro_mode = NTT_PRO_SCALE_ADD_BROADCAST;
+    fwd.pro_src = last;
+    fwd.pro_poly_stride = 1;
+    fwd.pro_w = ctx->d_pinv_mod_q;
+    fwd.epi_mode = NTT_EPI_FMA_SUB_MUL;
+    fwd.epi_a = cx;
+    fwd.epi_a_poly_stride = LK;
+    fwd.epi_b = ct;
+    fwd.epi_b_poly_stride = L;
+    fwd.w = lv->d_qlast_inv;
+    fwd.epi_dst = out;
+    fwd.epi_dst_poly_stride = L - 1;
+    HE_HIP(launch_ntt_forward(fwd, 2, fp, S(s)));
+    return HE_OK;
 }
 
 int he_decompose_real(const he_context *ctx, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,

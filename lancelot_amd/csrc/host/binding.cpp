@@ -245,6 +245,7 @@ PYBIND11_MODULE(pyCAHEL, m) {
     m.def("exponentiate_inplace", &exponentiate_inplace, nogil);
     m.def("relinearize", &relinearize, nogil);
     m.def("relinearize_inplace", &relinearize_inplace, nogil);
+    m.def("relinearize_rescale_inplace", &relinearize_rescale_inplace, nogil);
     m.def("mod_switch_to", py::overload_cast<const CAHELGPUContext &, const CAHELGPUPlaintext &, CAHELGPUPlaintext &, std::size_t>(&mod_switch_to), nogil);
     m.def("mod_switch_to", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &, CAHELGPUCiphertext &, std::size_t>(&mod_switch_to), nogil);
     m.def("mod_switch_to_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUPlaintext &, std::size_t>(&mod_switch_to_inplace), nogil);

@@ -374,6 +374,8 @@ void exponentiate_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &en
 void exponentiate(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, uint64_t exponent,
                   CAHELGPUCiphertext &destination, CAHELGPURelinKey &relin_key);
 void relinearize_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, const CAHELGPURelinKey &relin_keys);
+void relinearize_rescale_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted,
+                                 const CAHELGPURelinKey &relin_keys);  // this build's addition
 void relinearize(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, CAHELGPUCiphertext &destination,
                  const CAHELGPURelinKey &relin_keys);
 void mod_switch_to_next_inplace(const CAHELGPUContext &context, CAHELGPUPlaintext &plain);

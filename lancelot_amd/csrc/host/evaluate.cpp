@@ -238,6 +238,39 @@ void relinearize_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &enc
     encrypted.resize(2, encrypted.coeff_modulus_size(), encrypted.poly_modulus_degree());
 }
 
+// relinearize_inplace followed by rescale_to_next_inplace in one device call (he_keyswitch_rescale): the same limbs,
+// one forward transform less.  Not in the reference; its callers run the two back to back
+// (lancelot-main-GPU/utils/byzantine_fl.py:254-256).
+void relinearize_rescale_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted,
+                                 const CAHELGPURelinKey &relin_keys) {
+    require_ckks(context);
+    if (encrypted.size() != 3) throw std::invalid_argument("destination_size must be 3");
+    if (!encrypted.is_ntt_form()) throw std::invalid_argument("CKKS encrypted must be in NTT form");
+    if (relin_keys.parms_id() != context.key_parms_id())
+        throw std::invalid_argument("relin_keys is not valid for encryption parameters");
+    if (!context.using_keyswitching()) throw std::logic_error("keyswitching is not supported by the context");
+    const std::size_t chain = encrypted.chain_index();
+    if (chain == 0) throw std::invalid_argument("key switching needs a data-level ciphertext");
+    if (chain == context.max_chain_index()) throw std::invalid_argument("end of modulus switching chain reached");
+    const std::size_t n = context.poly_degree();
+    const uint32_t L = (uint32_t)encrypted.coeff_modulus_size();
+    auto ptrs = relin_keys.key_ptrs();
+    const std::size_t beta = (L + context.size_p() - 1) / context.size_p();
+    if (ptrs.size() < beta) throw std::invalid_argument("key_poly_num != 2");
+    DeviceBuffer ws(he_keyswitch_workspace_words(context.handle(), L)), out(2 * (std::size_t)(L - 1) * n);
+    check_status(he_keyswitch_rescale(context.handle(), L, encrypted.data() + 2 * (std::size_t)L * n, ptrs.data(),
+                                      encrypted.data(), out.get(), 0, ws.get(), context.stream()),
+                 "he_keyswitch_rescale");
+    const double scale = encrypted.scale() / static_cast<double>(context.key_modulus()[L - 1].value());
+    encrypted.data_ = std::move(out);
+    encrypted.size_ = 2;
+    encrypted.coeff_modulus_size_ = L - 1;
+    encrypted.poly_modulus_degree_ = n;
+    encrypted.chain_index() = chain + 1;
+    encrypted.parms_id() = context.parms_id_at(chain + 1);
+    encrypted.scale() = scale;
+}
+
 void relinearize(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, CAHELGPUCiphertext &destination,
                  const CAHELGPURelinKey &relin_keys) {
     if (&encrypted != &destination) destination = encrypted;

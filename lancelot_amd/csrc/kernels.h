@@ -47,6 +47,11 @@ enum : int {
     NTT_EPI_SUB_MUL_ADD = 3,
     // inverse epilogue: out = v * w mod q
     NTT_EPI_MUL = 4,
+    // forward prologue: input value = in * pro_w + (pro_src mod q)  (ModDown's delta * P^-1 plus the broadcast
+    // last limb of a rescale: one transform serves both, because the NTT is linear)
+    NTT_PRO_SCALE_ADD_BROADCAST = 5,
+    // forward epilogue: dst = ((epi_a * pro_w + epi_b) - v) * w mod q
+    NTT_EPI_FMA_SUB_MUL = 6,
 };
 
 struct NttArgs {
@@ -74,6 +79,7 @@ struct NttArgs {
     uint32_t epi_a_poly_stride;
     const uint64_t *epi_b;
     uint32_t epi_b_poly_stride;
+    const uint64_t *pro_w;    // [limbs][2] Shoup constants of the scaling prologue / epilogue, indexed like w
     const uint64_t *w;        // [limbs][2] Shoup constants indexed by limb i of the map
     uint64_t *epi_dst;        // destination of the forward epilogues
     uint32_t epi_dst_poly_stride;

@@ -185,15 +185,25 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
         const FpCtx c = fp_ctx(a, job.table);
         if (FWD) {
             // input: canonical residues (or one broadcast source limb); output: lazy signed doubles
-            const uint64_t *src =
-                a.pro_mode == NTT_PRO_BROADCAST_REDUCE ? a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n) : job.in;
-            for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
-                uint32_t row = e >> LOGC, col = e & (C - 1);
-                ld[skew(e)] = fp_from_u64(src[(size_t)row * 256 + col0 + col]);
+            const uint64_t *bsrc = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+            const uint64_t *src = a.pro_mode == NTT_PRO_BROADCAST_REDUCE ? bsrc : job.in;
+            if (a.pro_mode == NTT_PRO_SCALE_ADD_BROADCAST) {
+                const double wd = fp_from_u64(a.pro_w[2 * job.limb]);
+                const FpTw w{wd, wd * c.m.qinv};
+                for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
+                    uint32_t row = e >> LOGC, col = e & (C - 1);
+                    const size_t g = (size_t)row * 256 + col0 + col;
+                    ld[skew(e)] = fp_mulmod(fp_from_u64(src[g]), w, c.m) + fp_reduce(fp_from_u64(bsrc[g]), c.m);
+                }
+            } else {
+                for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
+                    uint32_t row = e >> LOGC, col = e & (C - 1);
+                    ld[skew(e)] = fp_from_u64(src[(size_t)row * 256 + col0 + col]);
+                }
             }
             __syncthreads();
             // a broadcast source may exceed this limb's prime: reduce first in that case
-            if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE)
+            if (a.pro_mode != NTT_PLAIN)
                 tile_pass_fp<p0, true, true>(lds, tile_elems, LD - p0 + LOGC, 1u, c);
             else
                 tile_pass_fp<p0, true, false>(lds, tile_elems, LD - p0 + LOGC, 1u, c);
@@ -236,6 +246,15 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
         for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
             uint32_t row = e >> LOGC, col = e & (C - 1);
             lds[skew(e)] = barrett64(src[(size_t)row * 256 + col0 + col], q, r1);
+        }
+    } else if (FWD && a.pro_mode == NTT_PRO_SCALE_ADD_BROADCAST) {
+        const uint64_t r1 = a.barrett[2 * job.table + 1];
+        const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+        const Shoup w = load_shoup(a.pro_w, job.limb);
+        for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
+            uint32_t row = e >> LOGC, col = e & (C - 1);
+            const size_t g = (size_t)row * 256 + col0 + col;
+            lds[skew(e)] = add_mod(mul_shoup(job.in[g], w, q), barrett64(src[g], q, r1), q);
         }
     } else {
         for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
@@ -340,7 +359,8 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_fp_kernel(NttArgs a) {
     const size_t off = g.off;
     const size_t n = (size_t)1 << a.log_n;
     double *ld = reinterpret_cast<double *>(lds);
-    const bool has_addend = EPI && a.epi_mode == NTT_EPI_SUB_MUL_ADD;
+    const bool fma_mode = EPI && a.epi_mode == NTT_EPI_FMA_SUB_MUL;   // ((a * pro_w + b) - v) * w
+    const bool has_addend = EPI && (a.epi_mode == NTT_EPI_SUB_MUL_ADD || fma_mode);
 
     Job job = decode_job(a, g.unit.j0);
     const FpCtx fc = fp_ctx(a, job.table);
@@ -431,11 +451,21 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_fp_kernel(NttArgs a) {
             if (EPI) {
                 const double wd = fp_from_u64(a.w[2 * job.limb]);
                 const FpTw w{wd, wd * m.qinv};
+                if (fma_mode) {
+                    const double pd = fp_from_u64(a.pro_w[2 * job.limb]);
+                    const FpTw pw{pd, pd * m.qinv};
 #pragma unroll
-                for (int i = 0; i < kPer; i++) {
-                    double r = fp_mulmod(fp_from_u64(pre_a[EPI ? i : 0]) - v[i], w, m);
-                    if (has_addend) r += fp_from_u64(pre_b[EPI ? i : 0]);
-                    v[i] = fp_canonical(r, m);
+                    for (int i = 0; i < kPer; i++) {
+                        const double lhs = fp_mulmod(fp_from_u64(pre_a[EPI ? i : 0]), pw, m) + fp_from_u64(pre_b[EPI ? i : 0]);
+                        v[i] = fp_canonical(fp_mulmod(lhs - v[i], w, m), m);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < kPer; i++) {
+                        double r = fp_mulmod(fp_from_u64(pre_a[EPI ? i : 0]) - v[i], w, m);
+                        if (has_addend) r += fp_from_u64(pre_b[EPI ? i : 0]);
+                        v[i] = fp_canonical(r, m);
+                    }
                 }
             }
 #pragma unroll
@@ -576,8 +606,9 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_int_kernel(NttArgs a) {
     const BlocksGeom g = blocks_geom(a);
     const size_t off = g.off;
     const size_t n = (size_t)1 << a.log_n;
-    const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD);
-    const bool has_addend = FWD && a.epi_mode == NTT_EPI_SUB_MUL_ADD;
+    const bool fma_mode = FWD && a.epi_mode == NTT_EPI_FMA_SUB_MUL;
+    const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD || fma_mode);
+    const bool has_addend = FWD && (a.epi_mode == NTT_EPI_SUB_MUL_ADD || fma_mode);
 
     for (uint32_t b = 0; b < g.unit.count; b++) {
         const Job job = decode_job(a, g.unit.j0 + b * g.unit.jstride);
@@ -598,12 +629,18 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_int_kernel(NttArgs a) {
                 const uint64_t *addend = has_addend ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
                 uint64_t *dst = a.epi_dst + (size_t)job.poly * a.epi_dst_poly_stride * n + epi_off;
                 const Shoup w = load_shoup(a.w, job.limb);
+                const Shoup pw = fma_mode ? load_shoup(a.pro_w, job.limb) : w;
 #pragma unroll
                 for (int i = 0; i < kPer; i++) {
                     const uint32_t e = threadIdx.x + i * nthreads;
                     const uint64_t c = reduce_4q(lds[skew(e)], q);
-                    uint64_t r = mul_shoup(sub_mod(minuend[e], c, q), w, q);
-                    if (has_addend) r = add_mod(r, addend[e], q);
+                    uint64_t r;
+                    if (fma_mode) {
+                        r = mul_shoup(sub_mod(add_mod(mul_shoup(minuend[e], pw, q), addend[e], q), c, q), w, q);
+                    } else {
+                        r = mul_shoup(sub_mod(minuend[e], c, q), w, q);
+                        if (has_addend) r = add_mod(r, addend[e], q);
+                    }
                     dst[e] = r;
                 }
             } else {
@@ -691,7 +728,8 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
     const BlocksPlan p = plan_blocks(a, n_polys);
     a.batch = p.batch;
     a.n_polys = n_polys;
-    const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD);
+    const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD ||
+                             a.epi_mode == NTT_EPI_FMA_SUB_MUL);
     if (!FP)
         hipLaunchKernelGGL((ntt_blocks_int_kernel<FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
     else if (epi)

@@ -125,8 +125,7 @@ def pair_distance(state: KrumState, cts_i, cts_j):
             tmp = c.ciphertext(ctx)
         else:
             c.add_inplace(ctx, acc, tmp)
-    c.relinearize_inplace(ctx, acc, state.rlk)
-    c.rescale_to_next_inplace(ctx, acc)
+    c.relinearize_rescale_inplace(ctx, acc, state.rlk)     # = relinearize_inplace + rescale_to_next_inplace
     acc.set_scale(cfg.scale)
     log_slots = int(math.log2(state.slots))
     rot = c.ciphertext(ctx)

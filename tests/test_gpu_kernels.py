@@ -158,6 +158,30 @@ def test_fused_and_separate_key_switch_agree(oracle, capi, monkeypatch, logn, bi
             assert (dct.numpy() == want).all(), (no_fuse, elt)
 
 
+@pytest.mark.parametrize("logn,bits,size_p,L", [(13, [50, 50, 49, 50, 50, 50], 2, 4), (13, [50, 50, 49, 50, 50, 50], 2, 3),
+                                                 (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 6), (11, [45, 40, 40, 50], 1, 3),
+                                                 (11, [45, 40, 40, 50], 1, 2), (9, [40, 40, 45, 45], 2, 2)])
+def test_keyswitch_rescale_equals_the_two_steps(oracle, capi, logn, bits, size_p, L):
+    """he_keyswitch_rescale (ModDown's and the rescale's forward transforms merged) against the oracle's key switch
+    followed by its rescale, on both arithmetic back ends, with and without a Galois element."""
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(13)
+    lib, h = capi.lib(), ctx.he_handle()
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    for elt in (0, 2 * p.n - 1):
+        c = rand_limbs(p, rng, range(L))
+        ct = rand_limbs(p, rng, range(L), n_polys=2)
+        dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
+        dout = DeviceArray(capi, shape=(2, L - 1, p.n))
+        capi.check(lib.he_keyswitch_rescale(h, L, dc.ptr, ptrs, dct.ptr, dout.ptr, elt, ws.ptr, None))
+        ks = p.key_switch(p.galois_ntt(c, elt) if elt else c, host_evk)
+        want = p.rescale(np.stack([p.add(ct[b], ks[b]) for b in range(2)]))
+        assert (dout.numpy() == want).all(), elt
+        assert (dct.numpy() == ct).all()                 # the input ciphertext is only read
+    assert lib.he_keyswitch_rescale(h, 1, dc.ptr, ptrs, dct.ptr, dout.ptr, 0, ws.ptr, None) == -1
+
+
 def test_ntt_rejects_bad_arguments(small, capi):
     cahel, parms, ctx, p = small
     d = DeviceArray(capi, shape=(1, p.n))
@@ -300,7 +324,7 @@ def test_keyswitch(small, capi, L, elt):
     host_evk, dev_evk, ptrs = _evk(p, rng, capi)
     words = lib.he_keyswitch_workspace_words(h, L)
     beta = -(-L // p.size_p)
-    assert words == (beta + 2) * (L + p.size_p) * p.n + 2 * L * p.n
+    assert words == (beta + 2) * (L + p.size_p) * p.n + 2 * L * p.n + 2 * p.n
     dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
     ws = DeviceArray(capi, shape=(words,))
     capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, elt, ws.ptr, None))

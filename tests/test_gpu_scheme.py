@@ -126,6 +126,12 @@ def test_encrypt_multiply_relin_rescale_bit_exact(world):
     want = w["o_enc"].decode(o_pt, prod.scale()).real
     assert rel_err(got, want) < REL
     assert np.max(np.abs(got - x * y)) < 1e-5          # cahel-main/unittest/evaluator.cu:419-472 bound
+    # relinearise + rescale in one call: the same limbs
+    both = c.ciphertext(ctx)
+    c.multiply(ctx, cx, cy, both)
+    c.relinearize_rescale_inplace(ctx, both, w["rlk"])
+    assert both.size() == 2 and both.chain_index() == 2 and both.scale() == prod.scale()
+    assert (both.to_numpy() == o_s).all()
     # square, multiply_and_relin_inplace
     sq = c.ciphertext(ctx)
     c.square(ctx, cx, sq)
