@@ -187,7 +187,7 @@ int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uin
                  uint32_t galois_elt, uint64_t *workspace, he_stream stream);
 
 /* out [2][L-1][N] = rescale(ct + KeySwitch(c)): he_keyswitch followed by he_rescale with the same limbs, in one
- * pass less over the data (ModDown's and the rescale's forward transforms are merged: the NTT is linear).
+ * pass less over the data (ModDown and the rescale share one inverse and one forward transform: the NTT is linear).
  * ct [2][L][N] is only read.  workspace as for he_keyswitch.
  * Replaces the sequence switch_key_inplace (src/eval_key_switch.cu:80-216) + rescale_to_next
  * (src/evaluate.cu:2058-2085) that relinearize_inplace + rescale_to_next_inplace run back to back. */

@@ -30,6 +30,7 @@ struct Level {
     uint64_t *d_part_hat_inv = nullptr;  // [L][2]
     uint64_t *d_mats = nullptr;
     uint64_t *d_qlast_inv = nullptr;     // [L-1][2]
+    uint64_t *d_mdr_w = nullptr;         // [1+K][2]: 1 mod q_{L-1}, then (P/p_k)^-1 mod p_k (merged ModDown + rescale)
     std::vector<Digit> digits;
     LimbJob *d_modup_jobs = nullptr;     // NTT jobs over the converted limbs of all digits
     uint32_t n_modup_jobs = 0;
@@ -51,6 +52,7 @@ struct he_context {
     uint64_t *d_moduli = nullptr, *d_barrett = nullptr, *d_psi = nullptr, *d_ipsi = nullptr;
     uint64_t *d_p_mod_q = nullptr, *d_pinv_mod_q = nullptr, *d_phat_inv = nullptr, *d_phat_mod_q = nullptr;
     uint32_t *d_iota = nullptr;  // 0, 1, 2, ...: row -> limb/table map of the P -> Ql conversion
+    std::vector<uint64_t> h_phat_inv;    // host copy of d_phat_inv
     double *d_psi_fp = nullptr, *d_ipsi_fp = nullptr, *d_fp_consts = nullptr;  // FP64 back end tables
     double *d_phat_mod_q_fp = nullptr;   // (M, M/q_j) pairs of the P -> Ql matrix
     uint32_t *d_rot_group = nullptr;     // encoder: 5^j mod 2N
@@ -270,6 +272,7 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         rc = upload(ctx, &ctx->d_p_mod_q, d->p_mod_q, 2 * (size_t)d->size_q);
         if (!rc) rc = upload(ctx, &ctx->d_pinv_mod_q, d->pinv_mod_q, 2 * (size_t)d->size_q);
         if (!rc) rc = upload(ctx, &ctx->d_phat_inv, d->phat_inv_mod_p, 2 * (size_t)d->size_p);
+        ctx->h_phat_inv.assign(d->phat_inv_mod_p, d->phat_inv_mod_p + 2 * (size_t)d->size_p);
         if (!rc) rc = upload(ctx, &ctx->d_phat_mod_q, d->phat_mod_q, (size_t)d->size_q * d->size_p);
     }
     if (!rc) {
@@ -366,6 +369,13 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
     if (L > 1) {
         if (!d->qlast_inv) return HE_E_INVALID_ARGUMENT;
         rc = upload(ctx, &lv.d_qlast_inv, d->qlast_inv, 2 * (size_t)(L - 1));
+        if (!rc && K) {
+            std::vector<uint64_t> w(2 * (size_t)(K + 1));
+            w[0] = 1;
+            w[1] = (uint64_t)((((unsigned __int128)1) << 64) / ctx->h_moduli[L - 1]);
+            std::copy(ctx->h_phat_inv.begin(), ctx->h_phat_inv.end(), w.begin() + 2);
+            rc = upload(ctx, &lv.d_mdr_w, w.data(), w.size());
+        }
         if (rc) return rc;
     }
     if (K) {
@@ -651,7 +661,7 @@ int he_ks_inner_product(const he_context *ctx, uint32_t L, const uint64_t *y, co
         ptrs.p[d] = evk[d];
     }
     HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, out, L, ctx->size_p, ctx->size_q, beta, galois_elt,
-                                accumulate != 0, S(s)));
+                                accumulate != 0, nullptr, nullptr, S(s)));
     return HE_OK;
 }
 
@@ -710,8 +720,10 @@ size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L) {
 namespace {
 
 // ModUp and inner product of a key switch: ws -> cx [2][L+K][N] (the layout of he_keyswitch_workspace_words)
+// fold_ct != nullptr: limb L-1 of cx becomes cx * P^-1 + fold_ct (see KsFuseArgs)
 int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint64_t *c, const uint64_t *const *evk,
-                  uint32_t galois_elt, uint64_t *ws, he_stream s) {
+                  uint32_t galois_elt, const uint64_t *fold_ct, uint64_t *ws, he_stream s) {
+    const uint64_t *fold_w = fold_ct ? ctx->d_pinv_mod_q + 2 * (size_t)(L - 1) : nullptr;
     const size_t n = ctx->n(), LK = L + ctx->size_p;
     uint64_t *y = ws;
     uint64_t *cx = y + (size_t)lv->beta * LK * n;
@@ -758,10 +770,19 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         x.size_q = ctx->size_q;
         x.size_qp = ctx->size_qp;
         x.beta = lv->beta;
+        x.fold_ct = fold_ct;
+        x.fold_w = fold_w;
         HE_HIP(launch_ntt_forward_inner(fwd, x, S(s)));
     } else {
         if (int rc = he_modup(ctx, L, src, y, tmp, s)) return rc;
-        if (int rc = he_ks_inner_product(ctx, L, y, evk, cx, 0, 0, s)) return rc;
+        EvkPtrs ptrs;
+        memset(&ptrs, 0, sizeof(ptrs));
+        for (uint32_t d = 0; d < lv->beta; d++) {
+            if (!evk[d]) return HE_E_INVALID_ARGUMENT;
+            ptrs.p[d] = evk[d];
+        }
+        HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, cx, L, ctx->size_p, ctx->size_q, lv->beta, 0, false,
+                                    fold_ct, fold_w, S(s)));
     }
     return HE_OK;
 }
@@ -778,7 +799,7 @@ int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uin
     const size_t n = ctx->n(), LK = L + ctx->size_p;
     uint64_t *cx = ws + (size_t)lv->beta * LK * n;
     uint64_t *tmp = cx + 2 * LK * n;
-    if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, ws, s)) return rc;
+    if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, nullptr, ws, s)) return rc;
     return he_moddown(ctx, L, cx, ct, 2, 1, tmp, s);
 }
 
@@ -791,17 +812,23 @@ int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, c
     const uint32_t K = ctx->size_p, LK = L + K;
     uint64_t *cx = ws + (size_t)lv->beta * LK * n;
     uint64_t *delta = cx + 2 * LK * n;             // [2][L][N]
-    uint64_t *last = delta + 2 * (size_t)L * n;    // [2][N]
-    if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, ws, s)) return rc;
-    // ModDown up to the base conversion: delta = P -> Ql conversion of the special limbs, coefficient form
+    // With c' = (cx - NTT(delta)) P^-1 + ct the ModDown result and t = INTT(cx_{L-1} P^-1 + ct_{L-1}), linearity of
+    // the transform gives INTT(c'_{L-1}) = t - delta_{L-1} P^-1 and
+    //   rescale(c')_j = ((cx_j P^-1 + ct_j) - NTT_j(delta_j P^-1 + [INTT(c'_{L-1})]_{q_j})) q_last^-1,
+    // so ModDown and rescale share one inverse and one forward transform.  Every step is exact modular arithmetic:
+    // the limbs equal he_keyswitch followed by he_rescale.
+    // (1) inner product; limb L-1 of cx leaves as cx_{L-1} P^-1 + ct_{L-1}
+    if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, ct, ws, s)) return rc;
+    // (2) limb L-1 and the special limbs -> coefficient form, the latter scaled by (P / p_k)^-1
     NttArgs inv = base_args(ctx, false);
-    inv.in = cx + (size_t)L * n;
-    inv.out = cx + (size_t)L * n;
+    inv.in = cx + (size_t)(L - 1) * n;
+    inv.out = cx + (size_t)(L - 1) * n;
     inv.in_poly_stride = inv.out_poly_stride = LK;
-    inv.map = plain_map(K, ctx->size_q);
+    inv.map = LimbMap{K + 1, L - 1, 1, ctx->size_q};
     inv.epi_mode = NTT_EPI_MUL;
-    inv.w = ctx->d_phat_inv;
+    inv.w = lv->d_mdr_w;
     HE_HIP(launch_ntt_inverse(inv, 2, fp_for(ctx, inv.map), S(s)));
+    // (3) delta = P -> Ql conversion of the special limbs
     if (lv->batched) {
         BconvBatch b{cx, delta, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
                      fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts};
@@ -813,37 +840,18 @@ int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, c
             HE_HIP(launch_bconv(ctx->tables(), b, S(s)));
         }
     }
-    const bool fp = fp_for(ctx, plain_map(L, 0));
-    // the last limb of the switched ciphertext, c'_{L-1} = (cx - NTT(delta)) P^-1 + ct, then its coefficients
-    NttArgs one = base_args(ctx, true);
-    one.in = one.out = delta + (size_t)(L - 1) * n;
-    one.in_poly_stride = one.out_poly_stride = L;
-    one.map = plain_map(1, L - 1);
-    one.epi_mode = NTT_EPI_SUB_MUL_ADD;
-    one.epi_a = cx + (size_t)(L - 1) * n;
-    one.epi_a_poly_stride = LK;
-    one.epi_b = ct + (size_t)(L - 1) * n;
-    one.epi_b_poly_stride = L;
-    one.w = ctx->d_pinv_mod_q + 2 * (size_t)(L - 1);
-    one.epi_dst = last;
-    one.epi_dst_poly_stride = 1;
-    HE_HIP(launch_ntt_forward(one, 2, fp, S(s)));
-    NttArgs linv = base_args(ctx, false);
-    linv.in = linv.out = last;
-    linv.in_poly_stride = linv.out_poly_stride = 1;
-    linv.map = plain_map(1, L - 1);
-    HE_HIP(launch_ntt_inverse(linv, 2, fp, S(s)));
-    // every other limb j: rescale(c')_j = ((cx_j P^-1 + ct_j) - NTT_j(delta_j P^-1 + [last]_{q_j})) q_last^-1.
-    // One transform serves ModDown and rescale because the NTT is linear; every step is exact modular
-    // arithmetic, so the limbs equal he_keyswitch followed by he_rescale.
+    // (4) the merged forward transform over the limbs that stay
     NttArgs fwd = base_args(ctx, true);
     fwd.in = fwd.out = delta;
     fwd.in_poly_stride = fwd.out_poly_stride = L;
     fwd.map = plain_map(L - 1, 0);
-    fwd.pro_mode = NTT_PRO_SCALE_ADD_BROADCAST;
-    fwd.pro_src = last;
-    fwd.pro_poly_stride = 1;
+    fwd.pro_mode = NTT_PRO_MODDOWN_RESCALE;
+    fwd.pro_src = cx + (size_t)(L - 1) * n;
+    fwd.pro_poly_stride = LK;
+    fwd.pro_src2 = delta + (size_t)(L - 1) * n;
+    fwd.pro2_poly_stride = L;
     fwd.pro_w = ctx->d_pinv_mod_q;
+    fwd.pro_last = L - 1;
     fwd.epi_mode = NTT_EPI_FMA_SUB_MUL;
     fwd.epi_a = cx;
     fwd.epi_a_poly_stride = LK;
@@ -852,7 +860,7 @@ int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, c
     fwd.w = lv->d_qlast_inv;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L - 1;
-    HE_HIP(launch_ntt_forward(fwd, 2, fp, S(s)));
+    HE_HIP(launch_ntt_forward(fwd, 2, fp_for(ctx, plain_map(L, 0)), S(s)));
     return HE_OK;
 }
 

@@ -47,11 +47,11 @@ enum : int {
     NTT_EPI_SUB_MUL_ADD = 3,
     // inverse epilogue: out = v * w mod q
     NTT_EPI_MUL = 4,
-    // forward prologue: input value = in * pro_w + (pro_src mod q)  (ModDown's delta * P^-1 plus the broadcast
-    // last limb of a rescale: one transform serves both, because the NTT is linear)
-    NTT_PRO_SCALE_ADD_BROADCAST = 5,
     // forward epilogue: dst = ((epi_a * pro_w + epi_b) - v) * w mod q
     NTT_EPI_FMA_SUB_MUL = 6,
+    // forward prologue of the merged ModDown + rescale: with r = pro_src - pro_src2 * pro_w[pro_last] mod q_last
+    // (the coefficients of the last limb of the ModDown result), input value = in * pro_w + (r mod q)
+    NTT_PRO_MODDOWN_RESCALE = 7,
 };
 
 struct NttArgs {
@@ -80,6 +80,9 @@ struct NttArgs {
     const uint64_t *epi_b;
     uint32_t epi_b_poly_stride;
     const uint64_t *pro_w;    // [limbs][2] Shoup constants of the scaling prologue / epilogue, indexed like w
+    const uint64_t *pro_src2; // NTT_PRO_MODDOWN_RESCALE: second source, limb (poly) at pro_src2 + poly * pro2_poly_stride * N
+    uint32_t pro2_poly_stride;
+    uint32_t pro_last;        // NTT_PRO_MODDOWN_RESCALE: table (and index into pro_w) of the limb that is dropped
     const uint64_t *w;        // [limbs][2] Shoup constants indexed by limb i of the map
     uint64_t *epi_dst;        // destination of the forward epilogues
     uint32_t epi_dst_poly_stride;
@@ -156,9 +159,10 @@ struct EvkPtrs {
     const uint64_t *p[kMaxDigits];
 };
 // (2, L+K, N) <- sum_d y_d * evk_d ; galois_elt != 0 applies the NTT-domain automorphism to y on load.
+// fold_ct / fold_w as in KsFuseArgs (nullptr: plain inner product).
 hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
-                                hipStream_t s);
+                                const uint64_t *fold_ct, const uint64_t *fold_w, hipStream_t s);
 
 // Forward NTT of ModUp's converted limbs fused with the key-switch inner product (FP64 back end only).
 // `a` describes the converted limbs as launch_ntt_forward's job list does (a.out = the beta x (L+K) x N digit
@@ -170,6 +174,10 @@ struct KsFuseArgs {
     const uint64_t *own;  // the key-switch input c, [L][N], NTT form
     uint64_t *out;        // [2][L+K][N]
     uint32_t L, K, size_q, size_qp, beta;
+    // optional: limb L-1 of the result becomes out * fold_w + fold_ct[k][L-1] (what the merged ModDown + rescale
+    // transforms back to coefficients); fold_ct = nullptr leaves the inner product as it is
+    const uint64_t *fold_ct;  // [2][L][N]
+    const uint64_t *fold_w;   // Shoup pair of P^-1 mod q_{L-1}
 };
 hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s);
 

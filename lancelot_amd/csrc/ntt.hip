@@ -187,13 +187,17 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
             // input: canonical residues (or one broadcast source limb); output: lazy signed doubles
             const uint64_t *bsrc = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
             const uint64_t *src = a.pro_mode == NTT_PRO_BROADCAST_REDUCE ? bsrc : job.in;
-            if (a.pro_mode == NTT_PRO_SCALE_ADD_BROADCAST) {
-                const double wd = fp_from_u64(a.pro_w[2 * job.limb]);
-                const FpTw w{wd, wd * c.m.qinv};
+            if (a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
+                const uint64_t *dsrc = a.pro_src2 + ((size_t)job.poly * a.pro2_poly_stride << a.log_n);
+                const FpMod ml = fp_ctx(a, a.pro_last).m;
+                const double wd = fp_from_u64(a.pro_w[2 * job.limb]), wl = fp_from_u64(a.pro_w[2 * a.pro_last]);
+                const FpTw w{wd, wd * c.m.qinv}, wlast{wl, wl * ml.qinv};
                 for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                     uint32_t row = e >> LOGC, col = e & (C - 1);
                     const size_t g = (size_t)row * 256 + col0 + col;
-                    ld[skew(e)] = fp_mulmod(fp_from_u64(src[g]), w, c.m) + fp_reduce(fp_from_u64(bsrc[g]), c.m);
+                    // coefficient of the dropped limb of the ModDown result, canonical mod q_last
+                    const double r = fp_canonical(fp_from_u64(bsrc[g]) - fp_mulmod(fp_from_u64(dsrc[g]), wlast, ml), ml);
+                    ld[skew(e)] = fp_mulmod(fp_from_u64(src[g]), w, c.m) + fp_reduce(r, c.m);
                 }
             } else {
                 for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
@@ -247,14 +251,17 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
             uint32_t row = e >> LOGC, col = e & (C - 1);
             lds[skew(e)] = barrett64(src[(size_t)row * 256 + col0 + col], q, r1);
         }
-    } else if (FWD && a.pro_mode == NTT_PRO_SCALE_ADD_BROADCAST) {
+    } else if (FWD && a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
         const uint64_t r1 = a.barrett[2 * job.table + 1];
-        const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
-        const Shoup w = load_shoup(a.pro_w, job.limb);
+        const uint64_t *tsrc = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+        const uint64_t *dsrc = a.pro_src2 + ((size_t)job.poly * a.pro2_poly_stride << a.log_n);
+        const uint64_t ql = a.moduli[a.pro_last];
+        const Shoup w = load_shoup(a.pro_w, job.limb), wlast = load_shoup(a.pro_w, a.pro_last);
         for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
             uint32_t row = e >> LOGC, col = e & (C - 1);
             const size_t g = (size_t)row * 256 + col0 + col;
-            lds[skew(e)] = add_mod(mul_shoup(job.in[g], w, q), barrett64(src[g], q, r1), q);
+            const uint64_t r = sub_mod(tsrc[g], mul_shoup(dsrc[g], wlast, ql), ql);
+            lds[skew(e)] = add_mod(mul_shoup(job.in[g], w, q), barrett64(r, q, r1), q);
         }
     } else {
         for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
@@ -593,6 +600,14 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
         lds_barrier();  // every read of this tile is done before the next one overwrites it
     }
     uint64_t *o = x.out + ((size_t)role * LK + t) * n + off;
+    if (x.fold_ct && t == x.L - 1) {
+        const uint64_t *cl = x.fold_ct + ((size_t)role * x.L + t) * n + off;
+        const double wd = fp_from_u64(x.fold_w[0]);
+        const FpTw w{wd, wd * m.qinv};
+#pragma unroll
+        for (int i = 0; i < kPer; i++)
+            acc[i] = fp_mulmod(fp_canonical(acc[i], m), w, m) + fp_from_u64(cl[tid + i * half]);
+    }
 #pragma unroll
     for (int i = 0; i < kPer; i++) o[tid + i * half] = fp_to_u64(fp_canonical(acc[i], m));
 }

@@ -239,6 +239,7 @@ struct InnerArgs {
     EvkPtrs evk;
     uint32_t L, K, size_q, beta, log_n, galois_elt;
     int accumulate;
+    const uint64_t *fold_ct, *fold_w;
 };
 
 // grid: (N / 256, L + K).  Streams beta digit limbs of y and 2 beta key limbs, writes (or accumulates) the
@@ -267,6 +268,12 @@ __global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
     if (p.accumulate) {
         o0 = add_mod(o0, p.out[o], q);
         o1 = add_mod(o1, p.out[o + opoly], q);
+    }
+    if (p.fold_ct && t == p.L - 1) {
+        const Shoup w = load_shoup(p.fold_w, 0);
+        const size_t cpoly = (size_t)p.L << p.log_n;
+        o0 = add_mod(mul_shoup(o0, w, q), p.fold_ct[o], q);
+        o1 = add_mod(mul_shoup(o1, w, q), p.fold_ct[o + cpoly], q);
     }
     p.out[o] = o0;
     p.out[o + opoly] = o1;
@@ -433,8 +440,9 @@ hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_
 
 hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
-                                hipStream_t s) {
-    InnerArgs p{y, out, t.moduli, t.barrett, evk, L, K, size_q, beta, t.log_n, galois_elt, accumulate ? 1 : 0};
+                                const uint64_t *fold_ct, const uint64_t *fold_w, hipStream_t s) {
+    InnerArgs p{y, out, t.moduli, t.barrett, evk, L, K, size_q, beta, t.log_n, galois_elt, accumulate ? 1 : 0,
+                fold_ct, fold_w};
     hipLaunchKernelGGL(inner_product_kernel, dim3((1u << t.log_n) / kThreads, L + K), dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
