@@ -186,6 +186,13 @@ size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L);
 int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk, uint64_t *ct,
                  uint32_t galois_elt, uint64_t *workspace, he_stream stream);
 
+/* ct_out [2][L][N] = (sigma(c0), 0) + KeySwitch(sigma(c1)) for ct_in = (c0, c1) and sigma = X -> X^galois_elt: one
+ * keyed rotation.  ct_in and ct_out must not overlap.  workspace as for he_keyswitch.
+ * Replaces apply_galois_inplace (src/evaluate.cu:2631-2702): two apply_galois_ntt gathers, a memset and
+ * switch_key_inplace. */
+int he_rotate(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const uint64_t *const *evk, uint64_t *ct_out,
+              uint32_t galois_elt, uint64_t *workspace, he_stream stream);
+
 /* out [2][L-1][N] = rescale(ct + KeySwitch(c)): he_keyswitch followed by he_rescale with the same limbs, in one
  * pass less over the data (ModDown and the rescale share one inverse and one forward transform: the NTT is linear).
  * ct [2][L][N] is only read.  workspace as for he_keyswitch.

@@ -109,6 +109,7 @@ NttArgs base_args(const he_context *ctx, bool forward) {
     a.moduli = ctx->d_moduli;
     a.barrett = ctx->d_barrett;
     a.log_n = ctx->log_n;
+    a.epi_b_mask = 0xffffffffu;
     return a;
 }
 
@@ -665,9 +666,15 @@ int he_ks_inner_product(const he_context *ctx, uint32_t L, const uint64_t *y, co
     return HE_OK;
 }
 
-int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, uint32_t n_polys, int accumulate,
-               uint64_t *ws, he_stream s) {
+}  // extern "C"
+
+namespace {
+
+// add_mask: which polynomials of `out` are added onto (bit p set) instead of overwritten
+int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, uint32_t n_polys, uint32_t add_mask,
+                 uint64_t *ws, he_stream s) {
     if (!ctx || !cx || !out || !ws || ctx->size_p == 0 || L == 0 || L > ctx->size_q) return HE_E_INVALID_ARGUMENT;
+    const int accumulate = add_mask != 0;
     const size_t n = ctx->n();
     const uint32_t K = ctx->size_p, LK = L + K;
     // special limbs -> coefficient form, scaled by (P / p_k)^-1, in place
@@ -700,11 +707,21 @@ int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, u
     fwd.epi_a_poly_stride = LK;
     fwd.epi_b = out;
     fwd.epi_b_poly_stride = L;
+    fwd.epi_b_mask = add_mask;
     fwd.w = ctx->d_pinv_mod_q;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L;
     HE_HIP(launch_ntt_forward(fwd, n_polys, fp_for(ctx, fwd.map), S(s)));
     return HE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int he_moddown(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out, uint32_t n_polys, int accumulate,
+               uint64_t *ws, he_stream s) {
+    return moddown_impl(ctx, L, cx, out, n_polys, accumulate ? 0xffffffffu : 0u, ws, s);
 }
 
 size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L) {
@@ -801,6 +818,21 @@ int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uin
     uint64_t *tmp = cx + 2 * LK * n;
     if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, nullptr, ws, s)) return rc;
     return he_moddown(ctx, L, cx, ct, 2, 1, tmp, s);
+}
+
+int he_rotate(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const uint64_t *const *evk, uint64_t *ct_out,
+              uint32_t galois_elt, uint64_t *ws, he_stream s) {
+    if (!ctx || !ct_in || !evk || !ct_out || !ws || ctx->size_p == 0 || ct_in == ct_out) return HE_E_INVALID_ARGUMENT;
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    const size_t n = ctx->n(), LK = L + ctx->size_p;
+    uint64_t *cx = ws + (size_t)lv->beta * LK * n;
+    uint64_t *tmp = cx + 2 * LK * n;
+    // (sigma(c0), sigma(c1)) in one pass; sigma(c1) is the key-switch input and is overwritten at the end
+    if (int rc = he_galois_ntt(ctx, ct_in, ct_out, 2 * L, galois_elt, s)) return rc;
+    if (int rc = ks_accumulate(ctx, lv, L, ct_out + (size_t)L * n, evk, 0, nullptr, ws, s)) return rc;
+    // out0 = sigma(c0) + ks0, out1 = ks1
+    return moddown_impl(ctx, L, cx, ct_out, 2, 1u, tmp, s);
 }
 
 int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk,

@@ -384,8 +384,12 @@ void rescale_to_next_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext 
 }
 
 // ---- rotations ----
-void apply_galois_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, std::size_t galois_elt_index,
-                          const CAHELGPUGaloisKey &galois_keys) {
+// destination = rotation of encrypted by the element at galois_elt_index; the two may be the same object.
+// (sigma(c0), 0) + KeySwitch(sigma(c1)) is one device call that writes a fresh buffer, so a distinct destination
+// costs no copy of the input.
+static void apply_galois_into(const CAHELGPUContext &context, const CAHELGPUCiphertext &encrypted,
+                              std::size_t galois_elt_index, const CAHELGPUGaloisKey &galois_keys,
+                              CAHELGPUCiphertext &destination) {
     if (galois_keys.parms_id() != context.key_parms_id())
         throw std::invalid_argument("galois_keys is not valid for encryption parameters");
     if (encrypted.size() > 2) throw std::invalid_argument("encrypted size must be 2");
@@ -395,46 +399,76 @@ void apply_galois_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &en
     const std::size_t n = context.poly_degree();
     const uint32_t L = (uint32_t)encrypted.coeff_modulus_size();
     const std::size_t poly = (std::size_t)L * n;
-    // (sigma(c0), 0) + KeySwitch(sigma(c1)); the automorphism of c1 is applied inside the key switch
-    DeviceBuffer rotated(2 * poly);
-    check_status(he_galois_ntt(context.handle(), encrypted.data(), rotated.get(), L, elt, context.stream()), "he_galois_ntt");
-    check_status(he_memset_zero(rotated.get() + poly, poly * sizeof(uint64_t), context.stream()), "memset");
-    std::swap(encrypted.data_, rotated);  // `rotated` now holds the input ciphertext; its c1 feeds the key switch
-    switch_key_inplace(context, encrypted, rotated.get() + poly, galois_keys.relin_keys_[galois_elt_index], false, elt);
+    const CAHELGPURelinKey &key = galois_keys.relin_keys_[galois_elt_index];
+    if (key.parms_id() != context.key_parms_id())
+        throw std::invalid_argument("relin_keys is not valid for encryption parameters");
+    if (!context.using_keyswitching()) throw std::logic_error("keyswitching is not supported by the context");
+    if (encrypted.chain_index() == 0) throw std::invalid_argument("key switching needs a data-level ciphertext");
+    auto ptrs = key.key_ptrs();
+    const std::size_t beta = (L + context.size_p() - 1) / context.size_p();
+    if (ptrs.size() < beta) throw std::invalid_argument("key_poly_num != 2");
+    DeviceBuffer rotated(2 * poly), ws(he_keyswitch_workspace_words(context.handle(), L));
+    check_status(he_rotate(context.handle(), L, encrypted.data(), ptrs.data(), rotated.get(), elt, ws.get(),
+                           context.stream()),
+                 "he_rotate");
+    if (&encrypted != &destination) {
+        destination.size_ = encrypted.size_;
+        destination.coeff_modulus_size_ = encrypted.coeff_modulus_size_;
+        destination.poly_modulus_degree_ = encrypted.poly_modulus_degree_;
+        destination.chain_index_ = encrypted.chain_index_;
+        destination.parms_id_ = encrypted.parms_id_;
+        destination.scale_ = encrypted.scale_;
+        destination.is_ntt_form_ = encrypted.is_ntt_form_;
+        destination.is_asymmetric_ = encrypted.is_asymmetric_;
+    }
+    destination.data_ = std::move(rotated);
+}
+
+void apply_galois_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, std::size_t galois_elt_index,
+                          const CAHELGPUGaloisKey &galois_keys) {
+    apply_galois_into(context, encrypted, galois_elt_index, galois_keys, encrypted);
 }
 
 void apply_galois(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, std::size_t galois_elt_index,
                   const CAHELGPUGaloisKey &galois_keys, CAHELGPUCiphertext &destination) {
-    if (&encrypted != &destination) destination = encrypted;
-    apply_galois_inplace(context, destination, galois_elt_index, galois_keys);
+    apply_galois_into(context, encrypted, galois_elt_index, galois_keys, destination);
 }
 
-static void rotate_internal(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, int step,
-                            const CAHELGPUGaloisKey &galois_key) {
+// destination = encrypted rotated by `step`
+static void rotate_internal(const CAHELGPUContext &context, const CAHELGPUCiphertext &encrypted, int step,
+                            const CAHELGPUGaloisKey &galois_key, CAHELGPUCiphertext &destination) {
     if (galois_key.parms_id() != context.key_parms_id())
         throw std::invalid_argument("galois_keys is not valid for encryption parameters");
-    if (step == 0) return;
+    if (step == 0) {
+        if (&encrypted != &destination) destination = encrypted;
+        return;
+    }
     const std::size_t coeff_count = context.poly_degree();
     const long idx = context.find_galois_elt(context.get_elt_from_step(step));
     if (idx >= 0) {
-        apply_galois_inplace(context, encrypted, (std::size_t)idx, galois_key);
+        apply_galois_into(context, encrypted, (std::size_t)idx, galois_key, destination);
         return;
     }
     // no key for this step: split it into signed powers of two (src/evaluate.cu:2395-2408)
     const std::vector<int> parts = naf(step);
     if (parts.size() == 1) throw std::invalid_argument("Galois key not present");
-    for (int part : parts)
-        if (static_cast<std::size_t>(std::abs(part)) != (coeff_count >> 1)) rotate_internal(context, encrypted, part, galois_key);
+    const CAHELGPUCiphertext *src = &encrypted;
+    for (int part : parts) {
+        if (static_cast<std::size_t>(std::abs(part)) == (coeff_count >> 1)) continue;
+        rotate_internal(context, *src, part, galois_key, destination);
+        src = &destination;
+    }
+    if (src == &encrypted && &encrypted != &destination) destination = encrypted;
 }
 
-static void conjugate_internal(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted,
-                               const CAHELGPUGaloisKey &galois_key) {
+static void conjugate_internal(const CAHELGPUContext &context, const CAHELGPUCiphertext &encrypted,
+                               const CAHELGPUGaloisKey &galois_key, CAHELGPUCiphertext &destination) {
     if (galois_key.parms_id() != context.key_parms_id())
         throw std::invalid_argument("galois_keys is not valid for encryption parameters");
     // the reference uses element index 0, which holds 2N-1 in the default element list (src/evaluate.cu:2690-2702)
     const long idx = context.find_galois_elt((uint32_t)(2 * context.poly_degree() - 1));
     if (idx < 0) throw std::invalid_argument("Galois key not present");
-    apply_galois_inplace(context, encrypted, (std::size_t)idx, galois_key);
+    apply_galois_into(context, encrypted, (std::size_t)idx, galois_key, destination);
 }
 
 void rotate_rows_inplace(const CAHELGPUContext &, CAHELGPUCiphertext &, int, const CAHELGPUGaloisKey &) {
@@ -458,25 +492,25 @@ void rotate_columns(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypte
 void rotate_vector_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, int step,
                            const CAHELGPUGaloisKey &galois_key) {
     require_ckks(context);
-    rotate_internal(context, encrypted, step, galois_key);
+    rotate_internal(context, encrypted, step, galois_key, encrypted);
 }
 
 void rotate_vector(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, int step,
                    const CAHELGPUGaloisKey &galois_key, CAHELGPUCiphertext &destination) {
-    if (&encrypted != &destination) destination = encrypted;
-    rotate_vector_inplace(context, destination, step, galois_key);
+    require_ckks(context);
+    rotate_internal(context, encrypted, step, galois_key, destination);
 }
 
 void complex_conjugate_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted,
                                const CAHELGPUGaloisKey &galois_key) {
     require_ckks(context);
-    conjugate_internal(context, encrypted, galois_key);
+    conjugate_internal(context, encrypted, galois_key, encrypted);
 }
 
 void complex_conjugate(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, const CAHELGPUGaloisKey &galois_key,
                        CAHELGPUCiphertext &destination) {
-    if (&encrypted != &destination) destination = encrypted;
-    complex_conjugate_inplace(context, destination, galois_key);
+    require_ckks(context);
+    conjugate_internal(context, encrypted, galois_key, destination);
 }
 
 // sum over steps of rot(ct, step) with one ModUp of c1 and one ModDown pair (src/evaluate.cu:2412-2629)

@@ -79,6 +79,7 @@ struct NttArgs {
     uint32_t epi_a_poly_stride;
     const uint64_t *epi_b;
     uint32_t epi_b_poly_stride;
+    uint32_t epi_b_mask;      // NTT_EPI_SUB_MUL_ADD: bit (poly mod 32) set = that polynomial has an addend
     const uint64_t *pro_w;    // [limbs][2] Shoup constants of the scaling prologue / epilogue, indexed like w
     const uint64_t *pro_src2; // NTT_PRO_MODDOWN_RESCALE: second source, limb (poly) at pro_src2 + poly * pro2_poly_stride * N
     uint32_t pro2_poly_stride;

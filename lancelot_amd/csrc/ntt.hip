@@ -427,11 +427,13 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_fp_kernel(NttArgs a) {
             for (int i = 0; i < kPer; i++) nx[i] = src[threadIdx.x + i * nthreads];
         }
         const size_t epi_off = off + (size_t)job.limb * n;
+        // SUB_MUL_ADD adds onto the polynomials named by epi_b_mask only (a rotation adds onto c0, not c1)
+        const bool add_b = has_addend && (fma_mode || ((a.epi_b_mask >> (job.poly & 31)) & 1));
         uint64_t *dst = (FWD && EPI) ? a.epi_dst + (size_t)job.poly * a.epi_dst_poly_stride * n + epi_off : job.out + off;
         uint64_t pre_a[EPI ? kPer : 1], pre_b[EPI ? kPer : 1];
         if (FWD && EPI) {
             const uint64_t *minuend = a.epi_a + (size_t)job.poly * a.epi_a_poly_stride * n + epi_off;
-            const uint64_t *addend = has_addend ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
+            const uint64_t *addend = add_b ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
 #pragma unroll
             for (int i = 0; i < kPer; i++) {
                 pre_a[EPI ? i : 0] = minuend[threadIdx.x + i * nthreads];
@@ -470,7 +472,7 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_fp_kernel(NttArgs a) {
 #pragma unroll
                     for (int i = 0; i < kPer; i++) {
                         double r = fp_mulmod(fp_from_u64(pre_a[EPI ? i : 0]) - v[i], w, m);
-                        if (has_addend) r += fp_from_u64(pre_b[EPI ? i : 0]);
+                        if (add_b) r += fp_from_u64(pre_b[EPI ? i : 0]);
                         v[i] = fp_canonical(r, m);
                     }
                 }
@@ -641,7 +643,8 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_int_kernel(NttArgs a) {
             __syncthreads();
             if (epi) {
                 const uint64_t *minuend = a.epi_a + (size_t)job.poly * a.epi_a_poly_stride * n + epi_off;
-                const uint64_t *addend = has_addend ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
+                const bool add_b = has_addend && (fma_mode || ((a.epi_b_mask >> (job.poly & 31)) & 1));
+                const uint64_t *addend = add_b ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
                 uint64_t *dst = a.epi_dst + (size_t)job.poly * a.epi_dst_poly_stride * n + epi_off;
                 const Shoup w = load_shoup(a.w, job.limb);
                 const Shoup pw = fma_mode ? load_shoup(a.pro_w, job.limb) : w;
@@ -654,7 +657,7 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_int_kernel(NttArgs a) {
                         r = mul_shoup(sub_mod(add_mod(mul_shoup(minuend[e], pw, q), addend[e], q), c, q), w, q);
                     } else {
                         r = mul_shoup(sub_mod(minuend[e], c, q), w, q);
-                        if (has_addend) r = add_mod(r, addend[e], q);
+                        if (add_b) r = add_mod(r, addend[e], q);
                     }
                     dst[e] = r;
                 }

@@ -182,6 +182,26 @@ def test_keyswitch_rescale_equals_the_two_steps(oracle, capi, logn, bits, size_p
     assert lib.he_keyswitch_rescale(h, 1, dc.ptr, ptrs, dct.ptr, dout.ptr, 0, ws.ptr, None) == -1
 
 
+@pytest.mark.parametrize("logn,bits,size_p,L", [(13, [50, 50, 49, 50, 50, 50], 2, 4), (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5),
+                                                 (11, [45, 40, 40, 50], 1, 2)])
+def test_rotate_entry_point(oracle, capi, logn, bits, size_p, L):
+    """he_rotate = (sigma(c0), 0) + KeySwitch(sigma(c1)) against the oracle, both back ends."""
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(14)
+    lib, h = capi.lib(), ctx.he_handle()
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    for elt in (5, 2 * p.n - 1):
+        ct = rand_limbs(p, rng, range(L), n_polys=2)
+        din, dout = DeviceArray(capi, host=ct), DeviceArray(capi, shape=(2, L, p.n))
+        capi.check(lib.he_rotate(h, L, din.ptr, ptrs, dout.ptr, elt, ws.ptr, None))
+        ks = p.key_switch(p.galois_ntt(ct[1], elt), host_evk)
+        want = np.stack([p.add(p.galois_ntt(ct[0], elt), ks[0]), ks[1]])
+        assert (dout.numpy() == want).all(), elt
+        assert (din.numpy() == ct).all()
+    assert lib.he_rotate(h, L, din.ptr, ptrs, din.ptr, 5, ws.ptr, None) == -1      # in place
+
+
 def test_ntt_rejects_bad_arguments(small, capi):
     cahel, parms, ctx, p = small
     d = DeviceArray(capi, shape=(1, p.n))
