@@ -193,6 +193,17 @@ int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uin
 int he_rotate(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const uint64_t *const *evk, uint64_t *ct_out,
               uint32_t galois_elt, uint64_t *workspace, he_stream stream);
 
+/* ct_out [2][L][N] = sum over the n_steps Galois elements of the rotation of ct_in = (c0, c1), with ONE ModUp of c1
+ * and ONE ModDown pair (hoisting): ct_out = (sum_s sigma_s(c0), 0) + ModDown(sum_s <sigma_s(ModUp(c1)), evk_s>).
+ * evk: HOST array of n_steps * beta device pointers, step-major (evk[s * beta + d] = digit d of the key of
+ * galois_elts[s], each as in he_ks_inner_product); galois_elts: HOST array of n_steps odd elements below 2N.
+ * All steps of up to 64 / beta keys run in one launch.  ct_in and ct_out must not overlap; workspace as for
+ * he_keyswitch.  Replaces hoisting_inplace (src/evaluate.cu:2412-2629: per step 1 + beta gathers, an inner product
+ * and three additions). */
+int he_hoisted_rotations(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const uint64_t *const *evk,
+                         const uint32_t *galois_elts, uint32_t n_steps, uint64_t *ct_out, uint64_t *workspace,
+                         he_stream stream);
+
 /* out [2][L-1][N] = rescale(ct + KeySwitch(c)): he_keyswitch followed by he_rescale with the same limbs, in one
  * pass less over the data (ModDown and the rescale share one inverse and one forward transform: the NTT is linear).
  * ct [2][L][N] is only read.  workspace as for he_keyswitch.

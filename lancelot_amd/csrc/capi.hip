@@ -835,6 +835,34 @@ int he_rotate(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const ui
     return moddown_impl(ctx, L, cx, ct_out, 2, 1u, tmp, s);
 }
 
+int he_hoisted_rotations(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const uint64_t *const *evk,
+                         const uint32_t *galois_elts, uint32_t n_steps, uint64_t *ct_out, uint64_t *ws, he_stream s) {
+    if (!ctx || !ct_in || !evk || !galois_elts || !ct_out || !ws || ctx->size_p == 0 || n_steps == 0 || ct_in == ct_out)
+        return HE_E_INVALID_ARGUMENT;
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    if (lv->beta > (uint32_t)kMaxDigits) return HE_E_UNSUPPORTED;
+    for (uint32_t i = 0; i < n_steps; i++) {
+        if (!(galois_elts[i] & 1) || galois_elts[i] >= (2u << ctx->log_n)) return HE_E_INVALID_ARGUMENT;
+        for (uint32_t d = 0; d < lv->beta; d++)
+            if (!evk[(size_t)i * lv->beta + d]) return HE_E_INVALID_ARGUMENT;
+    }
+    const size_t n = ctx->n(), LK = L + ctx->size_p;
+    uint64_t *y = ws;
+    uint64_t *cx = y + (size_t)lv->beta * LK * n;
+    uint64_t *tmp = cx + 2 * LK * n;
+    if (int rc = he_modup(ctx, L, ct_in + (size_t)L * n, y, tmp, s)) return rc;
+    // as many steps per launch as the 128-bit accumulator and the pointer table allow
+    const uint32_t per_launch = (uint32_t)kMaxDigits / lv->beta;
+    for (uint32_t first = 0; first < n_steps; first += per_launch) {
+        const uint32_t count = n_steps - first < per_launch ? n_steps - first : per_launch;
+        HE_HIP(launch_hoist_inner(ctx->tables(), y, ct_in, evk + (size_t)first * lv->beta, galois_elts + first, count, cx,
+                                  ct_out, L, ctx->size_p, ctx->size_q, lv->beta, first != 0, S(s)));
+    }
+    // out0 = sum sigma(c0) + ModDown(cx0), out1 = ModDown(cx1)
+    return moddown_impl(ctx, L, cx, ct_out, 2, 1u, tmp, s);
+}
+
 int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk,
                          const uint64_t *ct, uint64_t *out, uint32_t galois_elt, uint64_t *ws, he_stream s) {
     if (!ctx || !c || !evk || !ct || !out || !ws || ctx->size_p == 0 || L < 2) return HE_E_INVALID_ARGUMENT;

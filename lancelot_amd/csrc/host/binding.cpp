@@ -104,7 +104,8 @@ PYBIND11_MODULE(pyCAHEL, m) {
         .def("encrypt_symmetric",
              py::overload_cast<const CAHELGPUContext &, const CAHELGPUPlaintext &, bool>(&CAHELGPUSecretKey::encrypt_symmetric,
                                                                                          py::const_))
-        .def("decrypt", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &>(&CAHELGPUSecretKey::decrypt))
+        .def("decrypt", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &>(&CAHELGPUSecretKey::decrypt),
+             py::call_guard<py::gil_scoped_release>())
         .def("set_noise_flooding", &CAHELGPUSecretKey::set_noise_flooding)
         .def("to_numpy", [](const CAHELGPUSecretKey &s, const CAHELGPUContext &c) {
             return to_host(s.secret_key_array(), {(py::ssize_t)c.size_qp(), (py::ssize_t)c.poly_degree()});
@@ -115,7 +116,7 @@ PYBIND11_MODULE(pyCAHEL, m) {
         .def("encrypt_asymmetric",
              py::overload_cast<const CAHELGPUContext &, const CAHELGPUPlaintext &, bool>(&CAHELGPUPublicKey::encrypt_asymmetric,
                                                                                          py::const_),
-             py::arg("context"), py::arg("plaintext"), py::arg("save_seed") = false)
+             py::arg("context"), py::arg("plaintext"), py::arg("save_seed") = false, py::call_guard<py::gil_scoped_release>())
         .def("to_numpy", [](const CAHELGPUPublicKey &k) {
             return to_host(k.pk_.data(), {(py::ssize_t)k.pk_.size(), (py::ssize_t)k.pk_.coeff_modulus_size(),
                                           (py::ssize_t)k.pk_.poly_modulus_degree()});
@@ -149,7 +150,10 @@ PYBIND11_MODULE(pyCAHEL, m) {
         .def("encode",
              [](CAHELGPUCKKSEncoder &e, const CAHELGPUContext &c, py::array_t<double, py::array::c_style> v, double scale) {
                  CAHELGPUPlaintext p(c);
-                 e.encode_complex(c, v.data(), nullptr, (std::size_t)v.size(), e.first_chain_index(), scale, p);
+                 const double *values = v.data();
+                 const std::size_t count = (std::size_t)v.size();
+                 py::gil_scoped_release release;
+                 e.encode_complex(c, values, nullptr, count, e.first_chain_index(), scale, p);
                  return p;
              },
              py::arg("context"), py::arg("values").noconvert(), py::arg("scale"))
@@ -162,11 +166,15 @@ PYBIND11_MODULE(pyCAHEL, m) {
              },
              py::arg("context"), py::arg("values").noconvert(), py::arg("chain_index"), py::arg("scale"))
         .def("decode_array",
-             [](CAHELGPUCKKSEncoder &e, const CAHELGPUContext &c, const CAHELGPUPlaintext &p) {
+             [](CAHELGPUCKKSEncoder &e, const CAHELGPUContext &c, const CAHELGPUPlaintext &p, std::size_t count) {
                  std::vector<double> out;
-                 e.decode(c, p, out);
+                 {
+                     py::gil_scoped_release release;
+                     e.decode_prefix(c, p, count, out);
+                 }
                  return py::array_t<double>((py::ssize_t)out.size(), out.data());
-             })
+             },
+             py::arg("context"), py::arg("plain"), py::arg("count") = 0)
         .def("encode", py::overload_cast<const CAHELGPUContext &, const std::vector<double> &, double>(
                            &CAHELGPUCKKSEncoder::encode))
         .def("encode_to", py::overload_cast<const CAHELGPUContext &, const std::vector<double> &, std::size_t, double>(

@@ -7,6 +7,7 @@
 // names) and throw std::logic_error("unsupported scheme") the way the reference does for the scheme it
 // is not running (src/evaluate.cu:305-306, include/evaluate.h:501-535).
 #pragma once
+#include <atomic>
 #include <cstddef>
 #include <cstdint>
 #include <memory>
@@ -135,7 +136,7 @@ public:
     // The default key comes from /dev/urandom (include/prng.cuh:12-23); set_seed makes runs reproducible.
     void set_seed(uint64_t seed);
     const uint32_t *prng_key() const { return prng_key_; }
-    uint64_t next_stream() const { return prng_stream_++; }
+    uint64_t next_stream() const { return prng_stream_.fetch_add(1, std::memory_order_relaxed); }
     const uint64_t *gauss_cdt() const { return gauss_cdt_.get(); }
     uint32_t gauss_cdt_len() const { return gauss_cdt_len_; }
 
@@ -158,7 +159,7 @@ private:
     std::vector<uint32_t> galois_elts_;
     he_context *he_ = nullptr;
     uint32_t prng_key_[8];
-    mutable uint64_t prng_stream_ = 0;
+    mutable std::atomic<uint64_t> prng_stream_{0};
     cahel::DeviceBuffer gauss_cdt_;
     uint32_t gauss_cdt_len_ = 0;
     std::vector<LevelHost> level_host_;
@@ -326,6 +327,11 @@ public:
         return destination;
     }
     void decode(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain, std::vector<double> &destination);
+    // real parts of the first `count` slots only (0: all): the transform runs in full, the download is `count` values
+    void decode_values(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain, std::size_t count,
+                       std::vector<double> &interleaved);
+    void decode_prefix(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain, std::size_t count,
+                       std::vector<double> &destination);
     void decode_complex(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain, std::vector<double> &re,
                         std::vector<double> &im);
     std::vector<double> decode(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain) {

@@ -67,16 +67,18 @@ void CAHELGPUCKKSEncoder::encode(const CAHELGPUContext &context, const std::vect
     encode_complex(context, values.data(), nullptr, values.size(), chain_index, scale, destination);
 }
 
-void CAHELGPUCKKSEncoder::decode_complex(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain,
-                                         std::vector<double> &re, std::vector<double> &im) {
+// the first `count` complex values of the decoding, interleaved (re, im), into v
+void CAHELGPUCKKSEncoder::decode_values(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain,
+                                        std::size_t count, std::vector<double> &v) {
     if (!plain.is_ntt_form()) throw std::invalid_argument("plain is not in NTT form");
     const uint32_t limbs = (uint32_t)plain.coeff_modulus_size();
     if (limbs == 0 || !plain.data()) throw std::invalid_argument("plain is empty");
     const int total_bits = context.total_coeff_modulus_bit_count(plain.chain_index());
     if (plain.scale() <= 0 || (static_cast<int>(std::log2(plain.scale())) >= total_bits))
         throw std::invalid_argument("scale out of bounds");
-    if (sparse_slots_ == 0) sparse_slots_ = slots_;
+    if (sparse_slots_ == 0) sparse_slots_ = slots_;   // as the reference: decoding first fixes the full slot count
     const std::size_t ss = sparse_slots_;
+    if (count == 0 || count > ss) count = ss;
 
     he_context *h = context.handle();
     DeviceBuffer ws(he_ckks_workspace_words(h, limbs));
@@ -84,14 +86,29 @@ void CAHELGPUCKKSEncoder::decode_complex(const CAHELGPUContext &context, const C
     check_status(he_ckks_decode(h, plain.data(), limbs, (uint32_t)ss, plain.scale(),
                                 reinterpret_cast<double *>(out.get()), ws.get(), context.stream()),
                  "he_ckks_decode");
-    std::vector<double> v(2 * ss);
+    v.resize(2 * count);
     check_status(he_memcpy_d2h(v.data(), out.get(), v.size() * sizeof(double), context.stream()), "download");
+}
+
+void CAHELGPUCKKSEncoder::decode_complex(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain,
+                                         std::vector<double> &re, std::vector<double> &im) {
+    std::vector<double> v;
+    decode_values(context, plain, 0, v);
+    const std::size_t ss = v.size() / 2;
     re.resize(ss);
     im.resize(ss);
     for (std::size_t i = 0; i < ss; i++) {
         re[i] = v[2 * i];
         im[i] = v[2 * i + 1];
     }
+}
+
+void CAHELGPUCKKSEncoder::decode_prefix(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain,
+                                        std::size_t count, std::vector<double> &destination) {
+    std::vector<double> v;
+    decode_values(context, plain, count, v);
+    destination.resize(v.size() / 2);
+    for (std::size_t i = 0; i < destination.size(); i++) destination[i] = v[2 * i];
 }
 
 void CAHELGPUCKKSEncoder::decode(const CAHELGPUContext &context, const CAHELGPUPlaintext &plain,

@@ -514,8 +514,8 @@ void complex_conjugate(const CAHELGPUContext &context, CAHELGPUCiphertext &encry
 }
 
 // sum over steps of rot(ct, step) with one ModUp of c1 and one ModDown pair (src/evaluate.cu:2412-2629)
-void hoisting_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &ct, const CAHELGPUGaloisKey &glk,
-                      const std::vector<int> &steps) {
+static void hoisting_into(const CAHELGPUContext &context, const CAHELGPUCiphertext &ct, const CAHELGPUGaloisKey &glk,
+                          const std::vector<int> &steps, CAHELGPUCiphertext &destination) {
     if (ct.size() > 2) throw std::invalid_argument("ciphertext size must be 2");
     if (steps.empty()) throw std::invalid_argument("steps cannot be empty");
     if (glk.parms_id() != context.key_parms_id())
@@ -525,7 +525,7 @@ void hoisting_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &ct, co
     he_context *h = context.handle();
     he_stream st = context.stream();
     const std::size_t n = context.poly_degree(), K = context.size_p();
-    const uint32_t L = (uint32_t)ct.coeff_modulus_size(), LK = L + (uint32_t)K;
+    const uint32_t L = (uint32_t)ct.coeff_modulus_size();
     const std::size_t poly = (std::size_t)L * n, beta = (L + K - 1) / K;
     std::vector<std::size_t> idxs;
     for (int s : steps) {
@@ -533,30 +533,41 @@ void hoisting_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &ct, co
         if (idx < 0 || (std::size_t)idx >= glk.relin_keys_.size()) throw std::logic_error("Galois key not present in hoisting");
         idxs.push_back((std::size_t)idx);
     }
-    DeviceBuffer y(beta * LK * n), acc(2 * (std::size_t)LK * n), acc_c0(poly), tmp(2 * poly);
-    check_status(he_modup(h, L, ct.data() + poly, y.get(), tmp.get(), st), "he_modup");
-    for (std::size_t i = 0; i < idxs.size(); i++) {
-        const uint32_t elt = context.galois_elts()[idxs[i]];
-        // sigma(c0) accumulates in Ql, the inner products accumulate in Ql u P
-        if (i == 0) {
-            check_status(he_galois_ntt(h, ct.data(), acc_c0.get(), L, elt, st), "he_galois_ntt");
-        } else {
-            check_status(he_galois_ntt(h, ct.data(), tmp.get(), L, elt, st), "he_galois_ntt");
-            check_status(he_add(h, acc_c0.get(), tmp.get(), acc_c0.get(), 1, L, 0, st), "he_add");
-        }
-        auto ptrs = glk.relin_keys_[idxs[i]].key_ptrs();
-        if (ptrs.size() < beta) throw std::invalid_argument("key_poly_num must be 2 in hoisting");
-        check_status(he_ks_inner_product(h, L, y.get(), ptrs.data(), acc.get(), elt, i != 0, st), "he_ks_inner_product");
+    // every step's key pointers, step-major, and its Galois element
+    std::vector<const uint64_t *> ptrs;
+    std::vector<uint32_t> elts;
+    for (std::size_t idx : idxs) {
+        auto key = glk.relin_keys_[idx].key_ptrs();
+        if (key.size() < beta) throw std::invalid_argument("key_poly_num must be 2 in hoisting");
+        ptrs.insert(ptrs.end(), key.begin(), key.begin() + beta);
+        elts.push_back(context.galois_elts()[idx]);
     }
-    // new c0 = sum sigma(c0) + ModDown(acc_0), new c1 = ModDown(acc_1)
-    check_status(he_memcpy_d2d(ct.data(), acc_c0.get(), poly * sizeof(uint64_t), st), "copy");
-    check_status(he_memset_zero(ct.data() + poly, poly * sizeof(uint64_t), st), "memset");
-    check_status(he_moddown(h, L, acc.get(), ct.data(), 2, 1, tmp.get(), st), "he_moddown");
+    // new c0 = sum sigma(c0) + ModDown(acc_0), new c1 = ModDown(acc_1): one device call into a fresh buffer
+    DeviceBuffer sum(2 * poly), ws(he_keyswitch_workspace_words(h, L));
+    check_status(he_hoisted_rotations(h, L, ct.data(), ptrs.data(), elts.data(), (uint32_t)elts.size(), sum.get(),
+                                      ws.get(), st),
+                 "he_hoisted_rotations");
+    if (&ct != &destination) {
+        destination.size_ = ct.size_;
+        destination.coeff_modulus_size_ = ct.coeff_modulus_size_;
+        destination.poly_modulus_degree_ = ct.poly_modulus_degree_;
+        destination.chain_index_ = ct.chain_index_;
+        destination.parms_id_ = ct.parms_id_;
+        destination.scale_ = ct.scale_;
+        destination.is_ntt_form_ = ct.is_ntt_form_;
+        destination.is_asymmetric_ = ct.is_asymmetric_;
+    }
+    destination.data_ = std::move(sum);
+}
+
+void hoisting_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &ct, const CAHELGPUGaloisKey &glk,
+                      const std::vector<int> &steps) {
+    hoisting_into(context, ct, glk, steps, ct);
 }
 
 CAHELGPUCiphertext hoisting(const CAHELGPUContext &context, const CAHELGPUCiphertext &encrypted,
                             const CAHELGPUGaloisKey &glk, const std::vector<int> &steps) {
-    CAHELGPUCiphertext destination = encrypted;
-    hoisting_inplace(context, destination, glk, steps);
+    CAHELGPUCiphertext destination;
+    hoisting_into(context, encrypted, glk, steps, destination);
     return destination;
 }

@@ -210,10 +210,10 @@ void CAHELGPUSecretKey::decrypt(const CAHELGPUContext &context, const CAHELGPUCi
     he_context *h = context.handle();
     he_stream st = context.stream();
     plain.resize(limbs, n);
-    check_status(he_memcpy_d2d(plain.data(), cipher.data(), poly * sizeof(uint64_t), st), "copy");
+    // c0 + c1 s (+ c2 s^2 ...): the first product reads c0 directly
     for (std::size_t i = 1; i <= needed; i++)
-        check_status(he_multiply_add(h, cipher.data() + i * poly, sk_powers_.get() + (i - 1) * sk_poly, plain.data(),
-                                     plain.data(), 1, limbs, 0, 0, st),
+        check_status(he_multiply_add(h, cipher.data() + i * poly, sk_powers_.get() + (i - 1) * sk_poly,
+                                     i == 1 ? cipher.data() : plain.data(), plain.data(), 1, limbs, 0, 0, st),
                      "he_multiply_add");
     if (noise_flooding_) {
         DeviceBuffer noise(poly);

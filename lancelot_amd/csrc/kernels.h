@@ -165,6 +165,13 @@ hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtr
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
                                 const uint64_t *fold_ct, const uint64_t *fold_w, hipStream_t s);
 
+// Hoisted rotations: out (2, L+K, N) (+)= sum over steps of the inner product of sigma_s(y) with the step's key, and
+// c0_out (L, N) (+)= sum_s sigma_s(c0).  evk: n_steps * beta HOST-side device pointers, step-major; n_steps * beta <=
+// kMaxDigits per launch.
+hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
+                              const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
+                              uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, hipStream_t s);
+
 // Forward NTT of ModUp's converted limbs fused with the key-switch inner product (FP64 back end only).
 // `a` describes the converted limbs as launch_ntt_forward's job list does (a.out = the beta x (L+K) x N digit
 // buffer, whose own-digit limbs are never touched); the blocks pass multiplies every transformed tile by the

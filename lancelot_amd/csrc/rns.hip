@@ -9,6 +9,7 @@
 // (base conversion, uncorrected sum, one reduction), src/eval_key_switch.cu:13-76 (inner product) and
 // src/prng.cu:143-242 (distributions of the samplers).
 #include <cstdlib>
+#include <cstring>
 
 #include "kernels.h"
 #include "modarith.cuh"
@@ -279,6 +280,60 @@ __global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
     p.out[o + opoly] = o1;
 }
 
+struct HoistArgs {
+    const uint64_t *y, *c0;
+    uint64_t *out, *c0_out;
+    const uint64_t *moduli, *barrett;
+    EvkPtrs evk;                    // [step * beta + digit]
+    uint32_t elts[kMaxDigits];      // Galois element of every step
+    uint32_t n_steps, L, K, size_q, beta, log_n;
+    int accumulate;
+};
+
+// Hoisted rotations in one launch: grid (N / 256, (L + K) + L).
+// rows t < L + K:  out[p][t] = sum_s sum_d sigma_s(y_d)[t] * evk_{s,d}[p][t]  (n_steps * beta <= 64 products, summed in
+//                  128 bits and reduced once); the automorphism is the gather index of the load of y.
+// rows L + K + t:  c0_out[t] = sum_s sigma_s(c0)[t]
+__global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
+    const uint32_t LK = p.L + p.K;
+    const uint32_t j = blockIdx.x * kThreads + threadIdx.x;
+    if (blockIdx.y >= LK) {
+        const uint32_t t = blockIdx.y - LK;
+        const uint64_t q = p.moduli[t];
+        const uint64_t *in = p.c0 + ((size_t)t << p.log_n);
+        const size_t o = ((size_t)t << p.log_n) + j;
+        uint64_t acc = p.accumulate ? p.c0_out[o] : 0;
+        for (uint32_t s = 0; s < p.n_steps; s++) acc = add_mod(acc, in[galois_index(j, p.elts[s], p.log_n)], q);
+        p.c0_out[o] = acc;
+        return;
+    }
+    const uint32_t t = blockIdx.y;
+    const uint32_t table = t < p.L ? t : p.size_q + (t - p.L);
+    const size_t key_off = ((size_t)table << p.log_n) + j;
+    const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
+    U128 a0{0, 0}, a1{0, 0};
+    for (uint32_t s = 0; s < p.n_steps; s++) {
+        const uint32_t src = galois_index(j, p.elts[s], p.log_n);
+        for (uint32_t d = 0; d < p.beta; d++) {
+            const uint64_t v = p.y[(((size_t)d * LK + t) << p.log_n) + src];
+            const uint64_t *k = p.evk.p[s * p.beta + d];
+            mac128(a0, v, k[key_off]);
+            mac128(a1, v, k[key_off + key_poly]);
+        }
+    }
+    const uint64_t q = p.moduli[table], r0 = p.barrett[2 * table], r1 = p.barrett[2 * table + 1];
+    uint64_t o0 = barrett128(a0.lo, a0.hi, q, r0, r1);
+    uint64_t o1 = barrett128(a1.lo, a1.hi, q, r0, r1);
+    const size_t o = ((size_t)t << p.log_n) + j;
+    const size_t opoly = (size_t)LK << p.log_n;
+    if (p.accumulate) {
+        o0 = add_mod(o0, p.out[o], q);
+        o1 = add_mod(o1, p.out[o + opoly], q);
+    }
+    p.out[o] = o0;
+    p.out[o + opoly] = o1;
+}
+
 // ---------------------------------------------------------------------------------------------------
 // samplers: ChaCha20 block function (RFC 8439 section 2.3), 64-bit block counter in words 12-13,
 // 64-bit stream id in words 14-15
@@ -444,6 +499,31 @@ hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtr
     InnerArgs p{y, out, t.moduli, t.barrett, evk, L, K, size_q, beta, t.log_n, galois_elt, accumulate ? 1 : 0,
                 fold_ct, fold_w};
     hipLaunchKernelGGL(inner_product_kernel, dim3((1u << t.log_n) / kThreads, L + K), dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
+                              const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
+                              uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, hipStream_t s) {
+    if (n_steps == 0 || n_steps * beta > (uint32_t)kMaxDigits) return hipErrorInvalidValue;
+    HoistArgs p;
+    memset(&p, 0, sizeof(p));
+    p.y = y;
+    p.c0 = c0;
+    p.out = out;
+    p.c0_out = c0_out;
+    p.moduli = t.moduli;
+    p.barrett = t.barrett;
+    for (uint32_t i = 0; i < n_steps * beta; i++) p.evk.p[i] = evk[i];
+    for (uint32_t i = 0; i < n_steps; i++) p.elts[i] = elts[i];
+    p.n_steps = n_steps;
+    p.L = L;
+    p.K = K;
+    p.size_q = size_q;
+    p.beta = beta;
+    p.log_n = t.log_n;
+    p.accumulate = accumulate ? 1 : 0;
+    hipLaunchKernelGGL(hoist_inner_kernel, dim3((1u << t.log_n) / kThreads, (L + K) + L), dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
 

@@ -27,10 +27,14 @@ class KrumConfig:
     special_modulus_size: int = 1            # GPU_init: size_P = 1
     scale: float = 2.0 ** 40
     hoisting: bool = True                    # byzantine_fl.py: Hoisting_flag = 1
+    hoisting_radix: int = 16                 # every round of the slot sum is a hoisted sum of radix - 1 rotations;
+                                             # 0: the reference's split, hoisting(1..15) then one rotation per doubling
     lanes: int = 3                           # host threads / streams that the pairs are dealt to (0: null stream);
                                              # three streams and the null stream fill the four hardware queues
     sec_level: str = "tc128"
     seed: int | None = None
+    reproducible: bool = False               # with a seed: encrypt on the calling thread, so that every ciphertext
+                                             # draws the same randomness in every run
 
 
 @dataclass
@@ -58,11 +62,7 @@ def gpu_init(config: KrumConfig | None = None) -> KrumState:
     config = config or KrumConfig()
     n = 1 << config.log_n
     log_slots = config.log_n - 1
-    if config.hoisting:
-        steps = list(range(1, 16)) + [2 ** i for i in range(4, log_slots)]
-    else:
-        steps = [2 ** i for i in range(0, log_slots)]
-    steps = [s for s in steps if s < n // 2]
+    steps = sorted({s for rnd in rotate_sum_plan(log_slots, config) for s in rnd if s < n // 2})
     params = cahel.params(cahel.scheme_type.ckks)
     params.set_poly_modulus_degree(n)
     params.set_coeff_modulus(cahel.coeff_modulus_create(n, list(config.modulus_bits)))
@@ -83,6 +83,23 @@ def gpu_init(config: KrumConfig | None = None) -> KrumState:
     return KrumState(cahel, config, context, pk, sk, glk, rlk, encoder, encoder.slot_count())
 
 
+def rotate_sum_plan(log_slots: int, config: KrumConfig):
+    """Rounds of the slot sum: after round r every slot holds the sum of a block of prod(len(round) + 1) slots.
+    A round [s1, s2, ...] is acc += sum_k rot(acc, s_k): hoisted when it has several steps, one rotation otherwise.
+    The reference (byzantine_fl.py:252-300) hoists the first four doublings, steps 1..15, and rotates for the rest."""
+    if not config.hoisting:
+        return [[2 ** k] for k in range(log_slots)]
+    if config.hoisting_radix < 2 or log_slots <= 4:
+        head = [list(range(1, 16))] if log_slots > 4 else []
+        return head + [[2 ** k] for k in range(4 if head else 0, log_slots)]
+    rounds, block, slots = [], 1, 1 << log_slots
+    while block < slots:
+        radix = min(config.hoisting_radix, slots // block)
+        rounds.append([block * s for s in range(1, radix)])
+        block *= radix
+    return rounds
+
+
 def split_updates(vectors, slots: int):
     """Zero-pad every flattened update to a multiple of `slots` and split it (byzantine_fl.py:474-490)."""
     vectors = [np.asarray(v, dtype=np.float64).reshape(-1) for v in vectors]
@@ -94,22 +111,34 @@ def split_updates(vectors, slots: int):
 
 
 def encrypt_updates(state: KrumState, chunks):
-    """One ciphertext per (client, chunk)."""
-    c, ctx = state.cahel, state.context
-    out = []
-    for client in chunks:
-        row = []
-        for chunk in client:
-            t0 = time.perf_counter()
-            pt = state.encoder.encode(ctx, np.ascontiguousarray(chunk, dtype=np.float64), state.config.scale)
-            t1 = time.perf_counter()
-            row.append(state.pk.encrypt_asymmetric(ctx, pt))
-            _sync(c)
-            t2 = time.perf_counter()
-            state.timings["encode"] += t1 - t0
-            state.timings["encrypt"] += t2 - t1
-        out.append(row)
-    return out
+    """One ciphertext per (client, chunk); the chunks are independent and go over the lanes (unless the run is to
+    be reproducible).  The first one is encoded on the calling thread because the first message fixes the encoder's slot
+    count."""
+    ctx = state.context
+    spent = {"encode": 0.0, "encrypt": 0.0}
+
+    def one(item):
+        t0 = time.perf_counter()
+        pt = state.encoder.encode(ctx, np.ascontiguousarray(item, dtype=np.float64), state.config.scale)
+        t1 = time.perf_counter()
+        ct = state.pk.encrypt_asymmetric(ctx, pt)
+        t2 = time.perf_counter()
+        spent["encode"] += t1 - t0          # summed over the threads; scaled to the wall time below
+        spent["encrypt"] += t2 - t1
+        return ct
+
+    t0 = time.perf_counter()
+    flat = [chunk for client in chunks for chunk in client]
+    if state.config.reproducible:
+        cts = [one(item) for item in flat]      # the encryption randomness is drawn in a fixed order
+    else:
+        cts = [one(flat[0])] + _map_lanes(state, flat[1:], one)
+    wall = time.perf_counter() - t0
+    busy = max(spent["encode"] + spent["encrypt"], 1e-12)
+    for k in spent:
+        state.timings[k] += wall * spent[k] / busy
+    it = iter(cts)
+    return [[next(it) for _ in client] for client in chunks]
 
 
 def pair_distance(state: KrumState, cts_i, cts_j):
@@ -127,46 +156,49 @@ def pair_distance(state: KrumState, cts_i, cts_j):
             c.add_inplace(ctx, acc, tmp)
     c.relinearize_rescale_inplace(ctx, acc, state.rlk)     # = relinearize_inplace + rescale_to_next_inplace
     acc.set_scale(cfg.scale)
-    log_slots = int(math.log2(state.slots))
     rot = c.ciphertext(ctx)
-    if cfg.hoisting and log_slots > 4:
-        hoisted = c.hoisting(ctx, acc, state.glk, list(range(1, 16)))
-        c.add_inplace(ctx, acc, hoisted)
-        first = 4
-    else:
-        first = 0
-    for k in range(first, log_slots):
-        c.rotate_vector(ctx, acc, 2 ** k, state.glk, rot)
-        c.add_inplace(ctx, acc, rot)
+    for steps in rotate_sum_plan(int(math.log2(state.slots)), cfg):
+        if len(steps) > 1:
+            c.add_inplace(ctx, acc, c.hoisting(ctx, acc, state.glk, steps))
+        else:
+            c.rotate_vector(ctx, acc, steps[0], state.glk, rot)
+            c.add_inplace(ctx, acc, rot)
     return acc
+
+
+def _map_lanes(state: KrumState, items, fn):
+    """[fn(item) for item in items], the items dealt round-robin to `lanes` host threads, each issuing on its own
+    lane (stream) of the host layer (the evaluator, decrypt and decode calls release the interpreter lock);
+    everything is synchronised before and after."""
+    c = state.cahel
+    lanes = min(state.config.lanes, c._lane_count(), max(len(items), 1))
+    _sync(c)
+    if lanes <= 0:
+        out = [fn(item) for item in items]
+        _sync(c)
+        return out
+
+    def worker(w):
+        c._set_lane(1 + w)          # the current lane is per host thread
+        return [fn(item) for item in items[w::lanes]]
+
+    from concurrent.futures import ThreadPoolExecutor
+    out = [None] * len(items)
+    with ThreadPoolExecutor(max_workers=lanes) as pool:
+        for w, part in enumerate(pool.map(worker, range(lanes))):
+            out[w::lanes] = part
+    _sync(c)
+    return out
 
 
 def all_pair_distances(state: KrumState, cts, enc):
     """enc[i][j] = enc[j][i] = pair_distance(i, j) for every i < j.  The pairs are independent, and at Lancelot's
     sizes (three or four limbs) one of them neither fills the GPU nor keeps one host thread's launch rate busy, so
-    they are dealt round-robin to `lanes` host threads, each issuing on its own lane (stream) of the host layer
-    (the evaluator calls release the interpreter lock); everything is synchronised before returning."""
-    c = state.cahel
+    they are spread over the lanes."""
     n_clients = len(cts)
     pairs = [(i, j) for i in range(n_clients) for j in range(i + 1, n_clients)]
-    lanes = min(state.config.lanes, c._lane_count(), max(len(pairs), 1))
-    _sync(c)
-    if lanes <= 0:
-        for i, j in pairs:
-            enc[i][j] = enc[j][i] = pair_distance(state, cts[i], cts[j])
-        _sync(c)
-        return
-
-    def worker(w):
-        c._set_lane(1 + w)          # the current lane is per host thread
-        return [(i, j, pair_distance(state, cts[i], cts[j])) for i, j in pairs[w::lanes]]
-
-    from concurrent.futures import ThreadPoolExecutor
-    with ThreadPoolExecutor(max_workers=lanes) as pool:
-        for part in pool.map(worker, range(lanes)):
-            for i, j, ct in part:
-                enc[i][j] = enc[j][i] = ct
-    _sync(c)
+    for (i, j), ct in zip(pairs, _map_lanes(state, pairs, lambda ij: pair_distance(state, cts[ij[0]], cts[ij[1]]))):
+        enc[i][j] = enc[j][i] = ct
 
 
 def distance_matrix(state: KrumState, updates):
@@ -181,10 +213,12 @@ def distance_matrix(state: KrumState, updates):
     state.timings["evaluate"] += time.perf_counter() - t0
     t0 = time.perf_counter()
     dist = np.zeros((n_clients, n_clients))
-    for i in range(n_clients):
-        for j in range(i + 1, n_clients):
-            value = state.encoder.decode_array(state.context, state.sk.decrypt(state.context, enc[i][j]))[0]
-            dist[i, j] = dist[j, i] = value
+    pairs = [(i, j) for i in range(n_clients) for j in range(i + 1, n_clients)]
+    # every slot holds the distance: slot 0 is downloaded
+    values = _map_lanes(state, pairs, lambda ij: state.encoder.decode_array(
+        state.context, state.sk.decrypt(state.context, enc[ij[0]][ij[1]]), 1)[0])
+    for (i, j), value in zip(pairs, values):
+        dist[i, j] = dist[j, i] = value
     state.timings["decrypt"] += time.perf_counter() - t0
     return dist, enc
 
@@ -201,16 +235,20 @@ def decrypt_sort_mask(state: KrumState, enc):
     Returns (mask, order, scores)."""
     c, ctx = state.cahel, state.context
     n_clients = len(enc)
-    level = enc[0][1].chain_index()
-    scores = []
     t0 = time.perf_counter()
-    for i in range(n_clients):
-        total = _encrypt_constant(state, 0.0)
-        c.mod_switch_to_inplace(ctx, total, level)
-        for j in range(n_clients):
-            if enc[i][j] is not None:          # the i == j distance is zero and was never evaluated
-                c.add_inplace(ctx, total, enc[i][j])
-        scores.append(state.encoder.decode_array(ctx, state.sk.decrypt(ctx, total))[0])
+
+    def score(i):
+        # the i == j distance is zero and was never evaluated; the reference starts from an encryption of zero
+        row = [ct for ct in enc[i] if ct is not None]
+        total = row[0]
+        if len(row) > 1:
+            total = c.ciphertext(ctx)
+            c.add(ctx, row[0], row[1], total)
+            for ct in row[2:]:
+                c.add_inplace(ctx, total, ct)
+        return state.encoder.decode_array(ctx, state.sk.decrypt(ctx, total), 1)[0]
+
+    scores = _map_lanes(state, list(range(n_clients)), score)
     order = np.argsort(np.asarray(scores), kind="stable")
     zero, one = _encrypt_constant(state, 0.0), _encrypt_constant(state, 1.0)
     mask = [[one if order[r] == k else zero for k in range(n_clients)] for r in range(n_clients)]

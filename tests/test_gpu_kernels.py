@@ -202,6 +202,32 @@ def test_rotate_entry_point(oracle, capi, logn, bits, size_p, L):
     assert lib.he_rotate(h, L, din.ptr, ptrs, din.ptr, 5, ws.ptr, None) == -1      # in place
 
 
+@pytest.mark.parametrize("logn,bits,size_p,L,n_steps", [(11, [45, 40, 40, 50], 1, 3, 25), (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5, 4),
+                                                         (11, [50, 50, 49, 50, 50, 50], 2, 4, 3), (9, [40, 40, 45, 45], 2, 2, 1)])
+def test_hoisted_rotations_entry_point(oracle, capi, logn, bits, size_p, L, n_steps):
+    """he_hoisted_rotations (every step in one launch, or in several when steps * digits exceeds 64) against the
+    oracle's hoisting; two random keys alternate between the steps."""
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(15)
+    lib, h = capi.lib(), ctx.he_handle()
+    beta = -(-L // size_p)
+    keys = [_evk(p, rng, capi) for _ in range(2)]
+    elts = [pow(5, k + 1, 2 * p.n) for k in range(n_steps - 1)] + [2 * p.n - 1]
+    flat = capi.evk_array([keys[i % 2][1][d].ptr for i in range(n_steps) for d in range(beta)])
+    d_elts = (C.c_uint32 * n_steps)(*elts)
+    ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    ct = rand_limbs(p, rng, range(L), n_polys=2)
+    din, dout = DeviceArray(capi, host=ct), DeviceArray(capi, shape=(2, L, p.n))
+    capi.check(lib.he_hoisted_rotations(h, L, din.ptr, flat, d_elts, n_steps, dout.ptr, ws.ptr, None))
+    want = p.hoisting(ct, elts, [keys[i % 2][0] for i in range(n_steps)])
+    assert (dout.numpy() == want).all()
+    assert (din.numpy() == ct).all()
+    assert lib.he_hoisted_rotations(h, L, din.ptr, flat, d_elts, n_steps, din.ptr, ws.ptr, None) == -1   # in place
+    assert lib.he_hoisted_rotations(h, L, din.ptr, flat, d_elts, 0, dout.ptr, ws.ptr, None) == -1
+    d_elts[0] = 4
+    assert lib.he_hoisted_rotations(h, L, din.ptr, flat, d_elts, n_steps, dout.ptr, ws.ptr, None) == -1   # even element
+
+
 def test_ntt_rejects_bad_arguments(small, capi):
     cahel, parms, ctx, p = small
     d = DeviceArray(capi, shape=(1, p.n))

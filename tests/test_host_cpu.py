@@ -3,6 +3,7 @@ number theory agrees with the reference's known answers and with the oracle.  No
 import os
 import re
 
+import numpy as np
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -121,3 +122,20 @@ def test_krum_host_logic():
     assert krum.krum_select(d) != 4
     with pytest.raises(ValueError):
         krum.split_updates([np.zeros(3), np.zeros(4)], 2)
+
+
+@pytest.mark.parametrize("log_slots", [1, 3, 4, 5, 8, 12, 15])
+def test_rotate_sum_plan_adds_every_slot_once(log_slots):
+    """Whatever the split into hoisted rounds and single rotations, acc += sum_k rot(acc, s_k) over the rounds must
+    leave every slot holding each input slot exactly once."""
+    from lancelot_amd import krum
+    n = 1 << log_slots
+    for cfg in (krum.KrumConfig(), krum.KrumConfig(hoisting_radix=0), krum.KrumConfig(hoisting=False),
+                krum.KrumConfig(hoisting_radix=4), krum.KrumConfig(hoisting_radix=32)):
+        cover = np.zeros(n, dtype=np.int64)
+        cover[0] = 1
+        for steps in krum.rotate_sum_plan(log_slots, cfg):
+            assert all(0 < s < n for s in steps)
+            cover = cover + sum(np.roll(cover, s) for s in steps)
+        assert (cover == 1).all(), (log_slots, cfg)
+    assert krum.rotate_sum_plan(15, krum.KrumConfig(hoisting_radix=0))[0] == list(range(1, 16))   # the reference's split
