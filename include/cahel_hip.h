@@ -204,6 +204,34 @@ int he_hoisted_rotations(const he_context *ctx, uint32_t L, const uint64_t *ct_i
                          const uint32_t *galois_elts, uint32_t n_steps, uint64_t *ct_out, uint64_t *workspace,
                          he_stream stream);
 
+/* The batched forms below run the same kernels over `items` independent inputs in one launch each; Lancelot's
+ * ciphertexts have three or four limbs, and one of them neither fills the GPU nor amortises a launch.  They have
+ * no counterpart in the reference, which evaluates one ciphertext per call; the limbs they produce are those of
+ * `items` separate calls.  workspace: he_keyswitch_batch_workspace_words(ctx, L, items) words. */
+size_t he_keyswitch_batch_workspace_words(const he_context *ctx, uint32_t L, uint32_t items);
+
+/* he_hoisted_rotations over ct_in [items][2][L][N] -> ct_out [items][2][L][N]; add_input != 0 adds the input
+ * ciphertext as well: ct_out = ct_in + sum_s rot_s(ct_in), one round of a rotate-and-sum
+ * (lancelot-main-GPU/utils/byzantine_fl.py:252-300 does it as hoisting + add_inplace). */
+int he_hoisted_rotations_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *ct_in,
+                               const uint64_t *const *evk, const uint32_t *galois_elts, uint32_t n_steps, int add_input,
+                               uint64_t *ct_out, uint64_t *workspace, he_stream stream);
+
+/* he_keyswitch_rescale over `items` inputs: item k switches c + k * c_item_stride * N (stride in limbs, so that the
+ * third polynomial of dense size-3 ciphertexts is c = base + 2 L N, stride 3 L), adds onto ct [items][2][L][N] and
+ * writes out [items][2][L-1][N].  galois_elt must be 0 when items > 1. */
+int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *c,
+                               uint32_t c_item_stride, const uint64_t *const *evk, const uint64_t *ct, uint64_t *out,
+                               uint32_t galois_elt, uint64_t *workspace, he_stream stream);
+
+/* (out01 [items][2][L][N], out2 [items][L][N]) = sum over chunks of (a - b)^2 (size-3 tensor square: d0, d1 and d2)
+ * for the ciphertext pairs named by the DEVICE pointer table d_pairs [items][chunks][2] (each entry a [2][L][N]
+ * ciphertext): the sub, square_inplace and add_inplace loop of GPU_compute_pair_distance
+ * (byzantine_fl.py:201-246, lazy relinearisation) in one pass.  d2 is the input of he_keyswitch_rescale_batch
+ * (c = out2, c_item_stride = L) and (d0, d1) its ct. */
+int he_pair_square_sum(const he_context *ctx, uint32_t L, uint32_t items, uint32_t chunks,
+                       const uint64_t *const *d_pairs, uint64_t *out01, uint64_t *out2, he_stream stream);
+
 /* out [2][L-1][N] = rescale(ct + KeySwitch(c)): he_keyswitch followed by he_rescale with the same limbs, in one
  * pass less over the data (ModDown and the rescale share one inverse and one forward transform: the NTT is linear).
  * ct [2][L][N] is only read.  workspace as for he_keyswitch.

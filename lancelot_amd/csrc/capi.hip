@@ -569,6 +569,14 @@ int he_tensor_square(const he_context *ctx, const uint64_t *ct, uint64_t *out, u
     return HE_OK;
 }
 
+int he_pair_square_sum(const he_context *ctx, uint32_t L, uint32_t items, uint32_t chunks,
+                       const uint64_t *const *d_pairs, uint64_t *out01, uint64_t *out2, he_stream s) {
+    if (!ctx || !d_pairs || !out01 || !out2 || L == 0 || L > ctx->size_q || items == 0 || items > 16384 || chunks == 0)
+        return HE_E_INVALID_ARGUMENT;
+    HE_HIP(launch_pair_square_sum(ctx->tables(), d_pairs, out01, out2, L, items, chunks, S(s)));
+    return HE_OK;
+}
+
 int he_galois_ntt(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_t total_limbs, uint32_t elt,
                   he_stream s) {
     if (!ctx || !in || !out || in == out || !(elt & 1) || elt >= (2u << ctx->log_n)) return HE_E_INVALID_ARGUMENT;
@@ -609,24 +617,34 @@ int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_
     return HE_OK;
 }
 
-int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out, uint64_t *ws, he_stream s) {
-    if (!ctx || !c || !out || !ws || ctx->size_p == 0) return HE_E_INVALID_ARGUMENT;
+}  // extern "C"
+
+namespace {
+
+// ModUp of `items` polynomials: item k reads c + k * c_item_stride * N (stride in limbs), writes out [k][beta][L+K][N];
+// ws holds items * L limbs
+int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_item_stride, uint32_t items,
+               uint64_t *out, uint64_t *ws, he_stream s) {
+    if (!ctx || !c || !out || !ws || ctx->size_p == 0 || items == 0 || c_item_stride < L) return HE_E_INVALID_ARGUMENT;
     const Level *lv = level_of(ctx, L);
     if (!lv) return HE_E_LEVEL_NOT_SET;
+    if (items > 1 && !lv->batched) return HE_E_UNSUPPORTED;
     const size_t n = ctx->n();
     const uint32_t LK = L + ctx->size_p;
     // coefficient form scaled by (Q_d / q_i)^-1, out of place into the workspace
     NttArgs inv = base_args(ctx, false);
     inv.in = c;
     inv.out = ws;
-    inv.in_poly_stride = inv.out_poly_stride = L;
+    inv.in_poly_stride = c_item_stride;
+    inv.out_poly_stride = L;
     inv.map = plain_map(L, 0);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_part_hat_inv;
-    HE_HIP(launch_ntt_inverse(inv, 1, fp_for(ctx, inv.map), S(s)));
+    HE_HIP(launch_ntt_inverse(inv, items, fp_for(ctx, inv.map), S(s)));
     if (lv->batched) {
         BconvBatch b{ws, out, c, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                     lv->beta, lv->modup_max_rows, lv->modup_max_copy, lv->d_mats_fp, ctx->d_fp_consts};
+                     lv->beta, lv->modup_max_rows, lv->modup_max_copy, lv->d_mats_fp, ctx->d_fp_consts,
+                     items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n};
         HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
     }
     for (uint32_t d = 0; d < lv->beta && !lv->batched; d++) {
@@ -645,8 +663,18 @@ int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out
     fwd.n_jobs = lv->n_modup_jobs;
     fwd.groups = lv->d_modup_groups;
     fwd.n_groups = lv->n_modup_groups;
+    fwd.items = items;
+    fwd.item_stride = (size_t)lv->beta * LK * n;
     HE_HIP(launch_ntt_forward(fwd, 1, fp_for_level(ctx, L), S(s)));
     return HE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int he_modup(const he_context *ctx, uint32_t L, const uint64_t *c, uint64_t *out, uint64_t *ws, he_stream s) {
+    return modup_impl(ctx, L, c, L, 1, out, ws, s);
 }
 
 int he_ks_inner_product(const he_context *ctx, uint32_t L, const uint64_t *y, const uint64_t *const *evk,
@@ -662,7 +690,7 @@ int he_ks_inner_product(const he_context *ctx, uint32_t L, const uint64_t *y, co
         ptrs.p[d] = evk[d];
     }
     HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, out, L, ctx->size_p, ctx->size_q, beta, galois_elt,
-                                accumulate != 0, nullptr, nullptr, S(s)));
+                                accumulate != 0, nullptr, nullptr, 1, 0, S(s)));
     return HE_OK;
 }
 
@@ -687,10 +715,13 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     inv.w = ctx->d_phat_inv;
     HE_HIP(launch_ntt_inverse(inv, n_polys, fp_for(ctx, inv.map), S(s)));
     const Level *lv = level_of(ctx, L);
-    const bool batched = lv && lv->batched && n_polys <= 4;
+    // the conversion tables describe up to 4 polynomials; more of them go as items of 2 (ciphertexts)
+    const bool batched = lv && lv->batched && (n_polys <= 4 || n_polys % 2 == 0);
     if (batched) {
-        BconvBatch b{cx, ws, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, n_polys, L, 0,
-                     fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts};
+        const uint32_t units = n_polys <= 4 ? n_polys : 2, items = n_polys / units;
+        BconvBatch b{cx, ws, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, units, L, 0,
+                     fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts,
+                     items, (size_t)units * LK * n, (size_t)units * L * n, 0};
         HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
     }
     for (uint32_t p = 0; p < n_polys && !batched; p++) {
@@ -732,19 +763,38 @@ size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L) {
     return beta * LK * n + 2 * LK * n + 2 * (size_t)L * n + 2 * n;
 }
 
+size_t he_keyswitch_batch_workspace_words(const he_context *ctx, uint32_t L, uint32_t items) {
+    return (size_t)items * he_keyswitch_workspace_words(ctx, L);
+}
+
 }  // extern "C"
 
 namespace {
 
-// ModUp and inner product of a key switch: ws -> cx [2][L+K][N] (the layout of he_keyswitch_workspace_words)
-// fold_ct != nullptr: limb L-1 of cx becomes cx * P^-1 + fold_ct (see KsFuseArgs)
-int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint64_t *c, const uint64_t *const *evk,
-                  uint32_t galois_elt, const uint64_t *fold_ct, uint64_t *ws, he_stream s) {
-    const uint64_t *fold_w = fold_ct ? ctx->d_pinv_mod_q + 2 * (size_t)(L - 1) : nullptr;
+// Workspace of a key switch over `items` inputs: y [items][beta][L+K][N] | cx [items][2][L+K][N] | tmp [items][2][L][N]
+struct KsWorkspace {
+    uint64_t *y, *cx, *tmp;
+};
+
+KsWorkspace ks_workspace(const he_context *ctx, const Level *lv, uint32_t L, uint32_t items, uint64_t *ws) {
     const size_t n = ctx->n(), LK = L + ctx->size_p;
-    uint64_t *y = ws;
-    uint64_t *cx = y + (size_t)lv->beta * LK * n;
-    uint64_t *tmp = cx + 2 * LK * n;
+    KsWorkspace w;
+    w.y = ws;
+    w.cx = w.y + (size_t)items * lv->beta * LK * n;
+    w.tmp = w.cx + (size_t)items * 2 * LK * n;
+    return w;
+}
+
+// ModUp and inner product of a key switch over `items` inputs (item k at c + k * c_item_stride * N): ws -> cx.
+// fold_ct != nullptr: limb L-1 of cx becomes cx * P^-1 + fold_ct (see KsFuseArgs); fold_ct holds [items][2][L][N].
+int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint64_t *c, uint32_t c_item_stride,
+                  uint32_t items, const uint64_t *const *evk, uint32_t galois_elt, const uint64_t *fold_ct, uint64_t *ws,
+                  he_stream s) {
+    if (items == 0 || (items > 1 && galois_elt)) return HE_E_INVALID_ARGUMENT;
+    const uint64_t *fold_w = fold_ct ? ctx->d_pinv_mod_q + 2 * (size_t)(L - 1) : nullptr;
+    const size_t n = ctx->n();
+    const KsWorkspace w = ks_workspace(ctx, lv, L, items, ws);
+    uint64_t *y = w.y, *cx = w.cx, *tmp = w.tmp;
     const uint64_t *src = c;
     if (galois_elt) {
         // sigma(c) is staged in the second half of the ModDown workspace, which ModUp leaves alone and ModDown
@@ -753,7 +803,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         if (int rc = he_galois_ntt(ctx, c, staged, L, galois_elt, s)) return rc;
         src = staged;
     }
-    if (ctx->fuse_inner && lv->batched && fp_for_level(ctx, L)) {
+    if (items == 1 && ctx->fuse_inner && lv->batched && fp_for_level(ctx, L)) {
         // ModUp without the copy of a digit's own limbs, then the forward NTT fused with the inner product: the
         // transformed digits are never written (216 limb transfers less at L = 24, K = 8)
         NttArgs inv = base_args(ctx, false);
@@ -765,7 +815,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         inv.w = lv->d_part_hat_inv;
         HE_HIP(launch_ntt_inverse(inv, 1, true, S(s)));
         BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                     lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts};
+                     lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts, 1, 0, 0, 0};
         HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
         NttArgs fwd = base_args(ctx, true);
         fwd.in = y;
@@ -791,7 +841,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         x.fold_w = fold_w;
         HE_HIP(launch_ntt_forward_inner(fwd, x, S(s)));
     } else {
-        if (int rc = he_modup(ctx, L, src, y, tmp, s)) return rc;
+        if (int rc = modup_impl(ctx, L, src, galois_elt ? L : c_item_stride, items, y, tmp, s)) return rc;
         EvkPtrs ptrs;
         memset(&ptrs, 0, sizeof(ptrs));
         for (uint32_t d = 0; d < lv->beta; d++) {
@@ -799,7 +849,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
             ptrs.p[d] = evk[d];
         }
         HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, cx, L, ctx->size_p, ctx->size_q, lv->beta, 0, false,
-                                    fold_ct, fold_w, S(s)));
+                                    fold_ct, fold_w, items, 2 * (size_t)L * n, S(s)));
     }
     return HE_OK;
 }
@@ -813,11 +863,9 @@ int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uin
     if (!ctx || !c || !evk || !ct || !ws || ctx->size_p == 0) return HE_E_INVALID_ARGUMENT;
     const Level *lv = level_of(ctx, L);
     if (!lv) return HE_E_LEVEL_NOT_SET;
-    const size_t n = ctx->n(), LK = L + ctx->size_p;
-    uint64_t *cx = ws + (size_t)lv->beta * LK * n;
-    uint64_t *tmp = cx + 2 * LK * n;
-    if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, nullptr, ws, s)) return rc;
-    return he_moddown(ctx, L, cx, ct, 2, 1, tmp, s);
+    const KsWorkspace w = ks_workspace(ctx, lv, L, 1, ws);
+    if (int rc = ks_accumulate(ctx, lv, L, c, L, 1, evk, galois_elt, nullptr, ws, s)) return rc;
+    return he_moddown(ctx, L, w.cx, ct, 2, 1, w.tmp, s);
 }
 
 int he_rotate(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const uint64_t *const *evk, uint64_t *ct_out,
@@ -825,19 +873,20 @@ int he_rotate(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const ui
     if (!ctx || !ct_in || !evk || !ct_out || !ws || ctx->size_p == 0 || ct_in == ct_out) return HE_E_INVALID_ARGUMENT;
     const Level *lv = level_of(ctx, L);
     if (!lv) return HE_E_LEVEL_NOT_SET;
-    const size_t n = ctx->n(), LK = L + ctx->size_p;
-    uint64_t *cx = ws + (size_t)lv->beta * LK * n;
-    uint64_t *tmp = cx + 2 * LK * n;
+    const size_t n = ctx->n();
+    const KsWorkspace w = ks_workspace(ctx, lv, L, 1, ws);
     // (sigma(c0), sigma(c1)) in one pass; sigma(c1) is the key-switch input and is overwritten at the end
     if (int rc = he_galois_ntt(ctx, ct_in, ct_out, 2 * L, galois_elt, s)) return rc;
-    if (int rc = ks_accumulate(ctx, lv, L, ct_out + (size_t)L * n, evk, 0, nullptr, ws, s)) return rc;
+    if (int rc = ks_accumulate(ctx, lv, L, ct_out + (size_t)L * n, L, 1, evk, 0, nullptr, ws, s)) return rc;
     // out0 = sigma(c0) + ks0, out1 = ks1
-    return moddown_impl(ctx, L, cx, ct_out, 2, 1u, tmp, s);
+    return moddown_impl(ctx, L, w.cx, ct_out, 2, 1u, w.tmp, s);
 }
 
-int he_hoisted_rotations(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const uint64_t *const *evk,
-                         const uint32_t *galois_elts, uint32_t n_steps, uint64_t *ct_out, uint64_t *ws, he_stream s) {
-    if (!ctx || !ct_in || !evk || !galois_elts || !ct_out || !ws || ctx->size_p == 0 || n_steps == 0 || ct_in == ct_out)
+int he_hoisted_rotations_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *ct_in,
+                               const uint64_t *const *evk, const uint32_t *galois_elts, uint32_t n_steps, int add_input,
+                               uint64_t *ct_out, uint64_t *ws, he_stream s) {
+    if (!ctx || !ct_in || !evk || !galois_elts || !ct_out || !ws || ctx->size_p == 0 || n_steps == 0 || items == 0 ||
+        items > 16384 || ct_in == ct_out)
         return HE_E_INVALID_ARGUMENT;
     const Level *lv = level_of(ctx, L);
     if (!lv) return HE_E_LEVEL_NOT_SET;
@@ -847,38 +896,46 @@ int he_hoisted_rotations(const he_context *ctx, uint32_t L, const uint64_t *ct_i
         for (uint32_t d = 0; d < lv->beta; d++)
             if (!evk[(size_t)i * lv->beta + d]) return HE_E_INVALID_ARGUMENT;
     }
-    const size_t n = ctx->n(), LK = L + ctx->size_p;
-    uint64_t *y = ws;
-    uint64_t *cx = y + (size_t)lv->beta * LK * n;
-    uint64_t *tmp = cx + 2 * LK * n;
-    if (int rc = he_modup(ctx, L, ct_in + (size_t)L * n, y, tmp, s)) return rc;
+    const size_t n = ctx->n();
+    const KsWorkspace w = ks_workspace(ctx, lv, L, items, ws);
+    if (int rc = modup_impl(ctx, L, ct_in + (size_t)L * n, 2 * L, items, w.y, w.tmp, s)) return rc;
     // as many steps per launch as the 128-bit accumulator and the pointer table allow
     const uint32_t per_launch = (uint32_t)kMaxDigits / lv->beta;
     for (uint32_t first = 0; first < n_steps; first += per_launch) {
         const uint32_t count = n_steps - first < per_launch ? n_steps - first : per_launch;
-        HE_HIP(launch_hoist_inner(ctx->tables(), y, ct_in, evk + (size_t)first * lv->beta, galois_elts + first, count, cx,
-                                  ct_out, L, ctx->size_p, ctx->size_q, lv->beta, first != 0, S(s)));
+        HE_HIP(launch_hoist_inner(ctx->tables(), w.y, ct_in, evk + (size_t)first * lv->beta, galois_elts + first, count,
+                                  w.cx, ct_out, L, ctx->size_p, ctx->size_q, lv->beta, first != 0, add_input != 0, items,
+                                  2 * (size_t)L * n, S(s)));
     }
-    // out0 = sum sigma(c0) + ModDown(cx0), out1 = ModDown(cx1)
-    return moddown_impl(ctx, L, cx, ct_out, 2, 1u, tmp, s);
+    // out0 = [c0 +] sum sigma(c0) + ModDown(cx0), out1 = [c1 +] ModDown(cx1)
+    return moddown_impl(ctx, L, w.cx, ct_out, 2 * items, add_input ? 0xffffffffu : 0x55555555u, w.tmp, s);
 }
 
-int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk,
-                         const uint64_t *ct, uint64_t *out, uint32_t galois_elt, uint64_t *ws, he_stream s) {
-    if (!ctx || !c || !evk || !ct || !out || !ws || ctx->size_p == 0 || L < 2) return HE_E_INVALID_ARGUMENT;
+int he_hoisted_rotations(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const uint64_t *const *evk,
+                         const uint32_t *galois_elts, uint32_t n_steps, uint64_t *ct_out, uint64_t *ws, he_stream s) {
+    return he_hoisted_rotations_batch(ctx, L, 1, ct_in, evk, galois_elts, n_steps, 0, ct_out, ws, s);
+}
+
+int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *c,
+                               uint32_t c_item_stride, const uint64_t *const *evk, const uint64_t *ct, uint64_t *out,
+                               uint32_t galois_elt, uint64_t *ws, he_stream s) {
+    if (!ctx || !c || !evk || !ct || !out || !ws || ctx->size_p == 0 || L < 2 || items == 0 || items > 16384 ||
+        c_item_stride < L)
+        return HE_E_INVALID_ARGUMENT;
     const Level *lv = level_of(ctx, L);
     if (!lv) return HE_E_LEVEL_NOT_SET;
+    if (items > 1 && !lv->batched) return HE_E_UNSUPPORTED;
     const size_t n = ctx->n();
-    const uint32_t K = ctx->size_p, LK = L + K;
-    uint64_t *cx = ws + (size_t)lv->beta * LK * n;
-    uint64_t *delta = cx + 2 * LK * n;             // [2][L][N]
+    const uint32_t K = ctx->size_p, LK = L + K, polys = 2 * items;
+    const KsWorkspace w = ks_workspace(ctx, lv, L, items, ws);
+    uint64_t *cx = w.cx, *delta = w.tmp;           // [items][2][L+K][N], [items][2][L][N]
     // With c' = (cx - NTT(delta)) P^-1 + ct the ModDown result and t = INTT(cx_{L-1} P^-1 + ct_{L-1}), linearity of
     // the transform gives INTT(c'_{L-1}) = t - delta_{L-1} P^-1 and
     //   rescale(c')_j = ((cx_j P^-1 + ct_j) - NTT_j(delta_j P^-1 + [INTT(c'_{L-1})]_{q_j})) q_last^-1,
     // so ModDown and rescale share one inverse and one forward transform.  Every step is exact modular arithmetic:
     // the limbs equal he_keyswitch followed by he_rescale.
     // (1) inner product; limb L-1 of cx leaves as cx_{L-1} P^-1 + ct_{L-1}
-    if (int rc = ks_accumulate(ctx, lv, L, c, evk, galois_elt, ct, ws, s)) return rc;
+    if (int rc = ks_accumulate(ctx, lv, L, c, c_item_stride, items, evk, galois_elt, ct, ws, s)) return rc;
     // (2) limb L-1 and the special limbs -> coefficient form, the latter scaled by (P / p_k)^-1
     NttArgs inv = base_args(ctx, false);
     inv.in = cx + (size_t)(L - 1) * n;
@@ -887,11 +944,12 @@ int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, c
     inv.map = LimbMap{K + 1, L - 1, 1, ctx->size_q};
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_mdr_w;
-    HE_HIP(launch_ntt_inverse(inv, 2, fp_for(ctx, inv.map), S(s)));
+    HE_HIP(launch_ntt_inverse(inv, polys, fp_for(ctx, inv.map), S(s)));
     // (3) delta = P -> Ql conversion of the special limbs
     if (lv->batched) {
         BconvBatch b{cx, delta, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
-                     fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts};
+                     fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts,
+                     items, 2 * (size_t)LK * n, 2 * (size_t)L * n, 0};
         HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
     } else {
         for (uint32_t p = 0; p < 2; p++) {
@@ -920,8 +978,13 @@ int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, c
     fwd.w = lv->d_qlast_inv;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L - 1;
-    HE_HIP(launch_ntt_forward(fwd, 2, fp_for(ctx, plain_map(L, 0)), S(s)));
+    HE_HIP(launch_ntt_forward(fwd, polys, fp_for(ctx, plain_map(L, 0)), S(s)));
     return HE_OK;
+}
+
+int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk,
+                         const uint64_t *ct, uint64_t *out, uint32_t galois_elt, uint64_t *ws, he_stream s) {
+    return he_keyswitch_rescale_batch(ctx, L, 1, c, L, evk, ct, out, galois_elt, ws, s);
 }
 
 int he_decompose_real(const he_context *ctx, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,

@@ -12,6 +12,7 @@
 #include <cstdint>
 #include <memory>
 #include <stdexcept>
+#include <utility>
 #include <vector>
 
 #include "cahel_hip.h"
@@ -380,6 +381,11 @@ void exponentiate_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &en
 void exponentiate(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, uint64_t exponent,
                   CAHELGPUCiphertext &destination, CAHELGPURelinKey &relin_key);
 void relinearize_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, const CAHELGPURelinKey &relin_keys);
+// Batched squared distances of ciphertext pairs (batch.cpp); not in the reference
+std::vector<CAHELGPUCiphertext> pair_square_distances(
+    const CAHELGPUContext &context, const std::vector<std::vector<const CAHELGPUCiphertext *>> &clients,
+    const std::vector<std::pair<std::size_t, std::size_t>> &pairs, const CAHELGPURelinKey &rlk,
+    const CAHELGPUGaloisKey &glk, const std::vector<std::vector<int>> &rounds, double scale);
 void relinearize_rescale_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted,
                                  const CAHELGPURelinKey &relin_keys);  // this build's addition
 void relinearize(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, CAHELGPUCiphertext &destination,

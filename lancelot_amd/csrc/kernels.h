@@ -68,6 +68,8 @@ struct NttArgs {
     uint32_t n_jobs;
     const LimbGroup *groups;  // partition of `jobs` into runs with one table each (required with `jobs`)
     uint32_t n_groups;
+    uint32_t items;           // list mode: the whole list is applied to `items` buffers (0 = 1) ...
+    size_t item_stride;       // ... that lie item_stride words apart
     uint32_t batch, n_polys;  // filled in by the launcher
     uint32_t log_n;
     LimbMap map;
@@ -112,6 +114,10 @@ hipError_t launch_scalar_mul_add(const Tables &t, const uint64_t *a, const uint6
                                  const uint64_t *w, uint32_t first, uint32_t limbs, hipStream_t s);
 hipError_t launch_tensor(const Tables &t, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
                          bool square, hipStream_t s);
+// (out01 [items][2][L][N], out2 [items][L][N]) = sum over chunks of (a - b)^2 for the pairs of ciphertexts in the
+// device pointer table pairs [items][chunks][2]
+hipError_t launch_pair_square_sum(const Tables &t, const uint64_t *const *pairs, uint64_t *out01, uint64_t *out2,
+                                  uint32_t L, uint32_t items, uint32_t chunks, hipStream_t s);
 hipError_t launch_galois(const Tables &t, const uint64_t *in, uint64_t *out, uint32_t total_limbs, uint32_t elt,
                          hipStream_t s);
 
@@ -148,10 +154,14 @@ struct BconvBatch {
     const uint32_t *out_table;
     const BconvDesc *descs;  // device memory
     uint32_t n_units, max_rows, max_copy;
+    // the same units applied to `items` inputs (0 = 1): item k reads x_base + k * x_item_stride (and copy_base + k *
+    // copy_item_stride) and writes out_base + k * out_item_stride (strides in words)
     // FP64 back end (all primes involved below 2^50): the matrix as (M, M/m) pairs at the same offsets * 2,
     // per-table constants as in NttArgs::fp_consts; null selects the integer kernel
     const double *mat_fp;
     const double *fp_consts;
+    uint32_t items;
+    size_t x_item_stride, out_item_stride, copy_item_stride;
 };
 hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s);
 
@@ -160,17 +170,22 @@ struct EvkPtrs {
     const uint64_t *p[kMaxDigits];
 };
 // (2, L+K, N) <- sum_d y_d * evk_d ; galois_elt != 0 applies the NTT-domain automorphism to y on load.
+// items inputs (y and out dense, fold_ct fold_item_stride words apart) in one launch.
 // fold_ct / fold_w as in KsFuseArgs (nullptr: plain inner product).
 hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
-                                const uint64_t *fold_ct, const uint64_t *fold_w, hipStream_t s);
+                                const uint64_t *fold_ct, const uint64_t *fold_w, uint32_t items, size_t fold_item_stride,
+                                hipStream_t s);
 
 // Hoisted rotations: out (2, L+K, N) (+)= sum over steps of the inner product of sigma_s(y) with the step's key, and
-// c0_out (L, N) (+)= sum_s sigma_s(c0).  evk: n_steps * beta HOST-side device pointers, step-major; n_steps * beta <=
+// c0_out (L, N) (+)= sum_s sigma_s(c0).  with_self: c0_out also receives c0 itself and the L limbs after it a copy
+// of the L limbs after c0 (c1), so that ModDown can add onto the input ciphertext.  items: that many inputs,
+// y and out dense, the ciphertexts ct_item_stride words apart.  evk: n_steps * beta HOST-side device pointers, step-major; n_steps * beta <=
 // kMaxDigits per launch.
 hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
                               const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
-                              uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, hipStream_t s);
+                              uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, bool with_self, uint32_t items,
+                              size_t ct_item_stride, hipStream_t s);
 
 // Forward NTT of ModUp's converted limbs fused with the key-switch inner product (FP64 back end only).
 // `a` describes the converted limbs as launch_ntt_forward's job list does (a.out = the beta x (L+K) x N digit

@@ -61,9 +61,11 @@ __device__ __forceinline__ Job decode_job(const NttArgs &a, uint32_t job) {
     Job j;
     const size_t n = (size_t)1 << a.log_n;
     if (a.jobs) {
-        LimbJob lj = a.jobs[job];
-        j.in = a.in + (size_t)lj.data_limb * n;
-        j.out = a.out + (size_t)lj.data_limb * n;
+        // job = item * n_jobs + entry of the list
+        const uint32_t item = job / a.n_jobs;
+        LimbJob lj = a.jobs[job - item * a.n_jobs];
+        j.in = a.in + item * a.item_stride + (size_t)lj.data_limb * n;
+        j.out = a.out + item * a.item_stride + (size_t)lj.data_limb * n;
         j.table = lj.table;
         j.poly = 0;
         j.limb = 0;
@@ -320,8 +322,9 @@ struct Unit {
 // map mode: unit = (limb i, group of `batch` polynomials); list mode: unit = group of consecutive jobs
 __device__ __forceinline__ Unit decode_unit(const NttArgs &a, uint32_t u) {
     if (a.jobs) {
-        const LimbGroup g = a.groups[u];
-        return Unit{g.first, 1u, g.count};
+        const uint32_t item = u / a.n_groups;
+        const LimbGroup g = a.groups[u - item * a.n_groups];
+        return Unit{item * a.n_jobs + g.first, 1u, g.count};
     }
     const uint32_t limb = u % a.map.limbs, pg = u / a.map.limbs;
     const uint32_t p0 = pg * a.batch;
@@ -383,14 +386,17 @@ __global__ __launch_bounds__(kThreads) void ntt_blocks_fp_kernel(NttArgs a) {
 
     // list mode: the unit's jobs are read before the first store, so that they stay scalar loads
     LimbJob pre[kMaxGroup];
+    const uint32_t item = a.jobs ? g.unit.j0 / a.n_jobs : 0;
+    const uint32_t first = g.unit.j0 - item * (a.jobs ? a.n_jobs : 0);
 #pragma unroll
-    for (int i = 0; i < kMaxGroup; i++) pre[i] = (a.jobs && (uint32_t)i < g.unit.count) ? a.jobs[g.unit.j0 + i] : LimbJob{0, 0};
+    for (int i = 0; i < kMaxGroup; i++) pre[i] = (a.jobs && (uint32_t)i < g.unit.count) ? a.jobs[first + i] : LimbJob{0, 0};
+    const size_t item_off = a.jobs ? item * a.item_stride : 0;
     auto entry = [&](uint32_t b) {
         if (!a.jobs) return decode_job(a, g.unit.j0 + b * g.unit.jstride);
         LimbJob lj = pre[0];
 #pragma unroll
         for (int i = 1; i < kMaxGroup; i++) lj = b == (uint32_t)i ? pre[i] : lj;
-        return Job{a.in + (size_t)lj.data_limb * n, a.out + (size_t)lj.data_limb * n, lj.table, 0, 0};
+        return Job{a.in + item_off + (size_t)lj.data_limb * n, a.out + item_off + (size_t)lj.data_limb * n, lj.table, 0, 0};
     };
 
     uint64_t nx[kPer];
@@ -729,7 +735,7 @@ BlocksPlan plan_blocks(const NttArgs &a, uint32_t n_polys) {
     uint32_t units;
     if (a.jobs) {
         p.batch = 1;
-        units = a.n_groups;
+        units = a.n_groups * (a.items ? a.items : 1);
     } else {
         // batching pays once the launch has enough workgroups without splitting the polynomials
         p.batch = (n_polys > 1 && a.map.limbs * tiles(2048) >= 512) ? n_polys : 1;
@@ -761,7 +767,7 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
 
 hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s) {
     if (a.log_n < 9 || a.log_n > 16) return hipErrorInvalidValue;
-    const uint32_t n_jobs = a.jobs ? a.n_jobs : n_polys * a.map.limbs;
+    const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
     hipError_t e = fp ? launch_rows<true, true>(a, n_jobs, s) : launch_rows<true, false>(a, n_jobs, s);
     if (e != hipSuccess) return e;
@@ -788,7 +794,7 @@ hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipSt
 
 hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s) {
     if (a.log_n < 9 || a.log_n > 16) return hipErrorInvalidValue;
-    const uint32_t n_jobs = a.jobs ? a.n_jobs : n_polys * a.map.limbs;
+    const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
     hipError_t e = fp ? launch_blocks<false, true>(a, n_polys, s) : launch_blocks<false, false>(a, n_polys, s);
     if (e != hipSuccess) return e;

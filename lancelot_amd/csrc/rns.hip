@@ -106,6 +106,38 @@ __global__ __launch_bounds__(kThreads) void tensor_kernel(TensorArgs p) {
     p.out[idx + 2 * poly] = d2;
 }
 
+struct PairSquareArgs {
+    const uint64_t *const *pairs;   // device array [items][chunks][2] of ciphertext pointers, each [2][L][N]
+    uint64_t *out01, *out2;         // [items][2][L][N] (d0, d1) and [items][L][N] (d2)
+    const uint64_t *moduli, *barrett;
+    uint32_t L, log_n, chunks;
+};
+
+// grid: (N / 256, L, items).  (d0, d1 | d2)[item] = sum over chunks of (a - b)^2 as a size-3 ciphertext, for the pair
+// (a, b) of every chunk: the subtraction, the tensor square and the accumulation of the lazily relinearised
+// squared distance in one pass over the inputs.  d2, the key-switch input, goes to a buffer of its own so that
+// (d0, d1) is a dense batch of size-2 ciphertexts.
+__global__ __launch_bounds__(kThreads) void pair_square_sum_kernel(PairSquareArgs p) {
+    const uint32_t limb = blockIdx.y;
+    const uint64_t q = p.moduli[limb], r0 = p.barrett[2 * limb], r1 = p.barrett[2 * limb + 1];
+    const size_t poly = (size_t)p.L << p.log_n;
+    const size_t idx = ((size_t)limb << p.log_n) + blockIdx.x * kThreads + threadIdx.x;
+    const uint64_t *const *pair = p.pairs + (size_t)blockIdx.z * p.chunks * 2;
+    uint64_t d0 = 0, d1 = 0, d2 = 0;
+    for (uint32_t c = 0; c < p.chunks; c++) {
+        const uint64_t *a = pair[2 * c], *b = pair[2 * c + 1];
+        const uint64_t x0 = sub_mod(a[idx], b[idx], q), x1 = sub_mod(a[idx + poly], b[idx + poly], q);
+        d0 = add_mod(d0, mul_mod(x0, x0, q, r0, r1), q);
+        d2 = add_mod(d2, mul_mod(x1, x1, q, r0, r1), q);
+        const uint64_t m = mul_mod(x0, x1, q, r0, r1);
+        d1 = add_mod(d1, add_mod(m, m, q), q);
+    }
+    uint64_t *out = p.out01 + (size_t)blockIdx.z * 2 * poly;
+    out[idx] = d0;
+    out[idx + poly] = d1;
+    p.out2[(size_t)blockIdx.z * poly + idx] = d2;
+}
+
 // NTT-domain automorphism X -> X^elt as a gather: out[i] = in[pi(i)],
 // pi(i) = bitrev(((elt * (2 bitrev(i) + 1)) >> 1) mod N)
 __device__ __forceinline__ uint32_t galois_index(uint32_t i, uint32_t elt, uint32_t log_n) {
@@ -169,21 +201,23 @@ struct BconvBatchK {
 
 // grid: (N / 256, compute groups + copy groups, units); thread = one coefficient x kBatchRows output limbs
 __global__ __launch_bounds__(kThreads) void bconv_batched_kernel(BconvBatchK p) {
-    const BconvDesc d = p.b.descs[blockIdx.z];
+    const uint32_t item = blockIdx.z / p.b.n_units;
+    const BconvDesc d = p.b.descs[blockIdx.z - item * p.b.n_units];
     const size_t j = (size_t)blockIdx.x * kThreads + threadIdx.x;
-    uint64_t *out = p.b.out_base + d.out_off;
+    uint64_t *out = p.b.out_base + item * p.b.out_item_stride + d.out_off;
     if (blockIdx.y >= p.compute_groups) {
         // limbs that pass through unchanged
+        const uint64_t *from = p.b.copy_base + item * p.b.copy_item_stride;
         const uint32_t first = (blockIdx.y - p.compute_groups) * p.rows_per;
         for (uint32_t r = first; r < first + p.rows_per && r < d.copy_count; r++) {
             const size_t idx = ((size_t)(d.copy_first + r) << p.log_n) + j;
-            out[idx] = p.b.copy_base[idx];
+            out[idx] = from[idx];
         }
         return;
     }
     const uint32_t row0 = blockIdx.y * p.rows_per;
     if (row0 >= d.n_out) return;
-    const uint64_t *x = p.b.x_base + d.x_off;
+    const uint64_t *x = p.b.x_base + item * p.b.x_item_stride + d.x_off;
     uint64_t xv[kBatchIn];
 #pragma unroll
     for (int i = 0; i < kBatchIn; i++) xv[i] = (uint32_t)i < d.n_in ? x[((size_t)i << p.log_n) + j] : 0;
@@ -203,20 +237,22 @@ __global__ __launch_bounds__(kThreads) void bconv_batched_kernel(BconvBatchK p) 
 // FP64 variant: every product is reduced on the fly to |r| <= 0.75 m, so the sum of up to 8 terms stays an
 // exact integer below 6 m < 2^53; one canonicalisation per output.
 __global__ __launch_bounds__(kThreads) void bconv_batched_fp_kernel(BconvBatchK p) {
-    const BconvDesc d = p.b.descs[blockIdx.z];
+    const uint32_t item = blockIdx.z / p.b.n_units;
+    const BconvDesc d = p.b.descs[blockIdx.z - item * p.b.n_units];
     const size_t j = (size_t)blockIdx.x * kThreads + threadIdx.x;
-    uint64_t *out = p.b.out_base + d.out_off;
+    uint64_t *out = p.b.out_base + item * p.b.out_item_stride + d.out_off;
     if (blockIdx.y >= p.compute_groups) {
+        const uint64_t *from = p.b.copy_base + item * p.b.copy_item_stride;
         const uint32_t first = (blockIdx.y - p.compute_groups) * p.rows_per;
         for (uint32_t r = first; r < first + p.rows_per && r < d.copy_count; r++) {
             const size_t idx = ((size_t)(d.copy_first + r) << p.log_n) + j;
-            out[idx] = p.b.copy_base[idx];
+            out[idx] = from[idx];
         }
         return;
     }
     const uint32_t row0 = blockIdx.y * p.rows_per;
     if (row0 >= d.n_out) return;
-    const uint64_t *x = p.b.x_base + d.x_off;
+    const uint64_t *x = p.b.x_base + item * p.b.x_item_stride + d.x_off;
     double xv[kBatchIn];
 #pragma unroll
     for (int i = 0; i < kBatchIn; i++) xv[i] = (uint32_t)i < d.n_in ? fp_from_u64(x[((size_t)i << p.log_n) + j]) : 0.0;
@@ -241,9 +277,10 @@ struct InnerArgs {
     uint32_t L, K, size_q, beta, log_n, galois_elt;
     int accumulate;
     const uint64_t *fold_ct, *fold_w;
+    size_t y_item_stride, out_item_stride, fold_item_stride;   // blockIdx.z = item (words between items)
 };
 
-// grid: (N / 256, L + K).  Streams beta digit limbs of y and 2 beta key limbs, writes (or accumulates) the
+// grid: (N / 256, L + K, items).  Streams beta digit limbs of y and 2 beta key limbs, writes (or accumulates) the
 // two output limbs.  The products are summed in 128 bits and reduced once (beta <= 64 products of
 // 61-bit factors cannot overflow).
 __global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
@@ -254,9 +291,12 @@ __global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
     const uint32_t src = p.galois_elt ? galois_index(j, p.galois_elt, p.log_n) : j;
     const size_t key_off = ((size_t)table << p.log_n) + j;
     const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
+    // (the argument struct stays untouched: a modified copy would move its pointer table to scratch memory)
+    const uint64_t *y = p.y + blockIdx.z * p.y_item_stride;
+    uint64_t *out = p.out + blockIdx.z * p.out_item_stride;
     U128 a0{0, 0}, a1{0, 0};
     for (uint32_t d = 0; d < p.beta; d++) {
-        const uint64_t v = p.y[(((size_t)d * LK + t) << p.log_n) + src];
+        const uint64_t v = y[(((size_t)d * LK + t) << p.log_n) + src];
         const uint64_t *k = p.evk.p[d];
         mac128(a0, v, k[key_off]);
         mac128(a1, v, k[key_off + key_poly]);
@@ -267,17 +307,18 @@ __global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
     const size_t o = ((size_t)t << p.log_n) + j;
     const size_t opoly = (size_t)LK << p.log_n;
     if (p.accumulate) {
-        o0 = add_mod(o0, p.out[o], q);
-        o1 = add_mod(o1, p.out[o + opoly], q);
+        o0 = add_mod(o0, out[o], q);
+        o1 = add_mod(o1, out[o + opoly], q);
     }
     if (p.fold_ct && t == p.L - 1) {
         const Shoup w = load_shoup(p.fold_w, 0);
         const size_t cpoly = (size_t)p.L << p.log_n;
-        o0 = add_mod(mul_shoup(o0, w, q), p.fold_ct[o], q);
-        o1 = add_mod(mul_shoup(o1, w, q), p.fold_ct[o + cpoly], q);
+        const uint64_t *fold = p.fold_ct + blockIdx.z * p.fold_item_stride;
+        o0 = add_mod(mul_shoup(o0, w, q), fold[o], q);
+        o1 = add_mod(mul_shoup(o1, w, q), fold[o + cpoly], q);
     }
-    p.out[o] = o0;
-    p.out[o + opoly] = o1;
+    out[o] = o0;
+    out[o + opoly] = o1;
 }
 
 struct HoistArgs {
@@ -287,35 +328,51 @@ struct HoistArgs {
     EvkPtrs evk;                    // [step * beta + digit]
     uint32_t elts[kMaxDigits];      // Galois element of every step
     uint32_t n_steps, L, K, size_q, beta, log_n;
-    int accumulate;
+    int accumulate, with_self;
+    size_t ct_item_stride;          // words between the ciphertexts of consecutive items (blockIdx.z), in and out
 };
 
-// Hoisted rotations in one launch: grid (N / 256, (L + K) + L).
+// Hoisted rotations in one launch: grid (N / 256, (L + K) + L [+ L], items).
 // rows t < L + K:  out[p][t] = sum_s sum_d sigma_s(y_d)[t] * evk_{s,d}[p][t]  (n_steps * beta <= 64 products, summed in
 //                  128 bits and reduced once); the automorphism is the gather index of the load of y.
-// rows L + K + t:  c0_out[t] = sum_s sigma_s(c0)[t]
+// rows L + K + t:  c0_out[t] = sum_s sigma_s(c0)[t]  (+ c0[t] with_self)
+// rows L + K + L + t (with_self only): c1 is copied to the output, so that the ModDown that follows adds onto
+//                  the input ciphertext: ct_out = ct_in + sum_s rot_s(ct_in)
 __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     const uint32_t LK = p.L + p.K;
     const uint32_t j = blockIdx.x * kThreads + threadIdx.x;
+    // (the argument struct stays untouched: a modified copy would move its tables to scratch memory)
+    const uint64_t *c0 = p.c0 + blockIdx.z * p.ct_item_stride;
+    uint64_t *c0_out = p.c0_out + blockIdx.z * p.ct_item_stride;
+    if (blockIdx.y >= LK + p.L) {
+        const size_t o = ((size_t)(blockIdx.y - LK) << p.log_n) + j;
+        if (!p.accumulate) c0_out[o] = c0[o];
+        return;
+    }
     if (blockIdx.y >= LK) {
         const uint32_t t = blockIdx.y - LK;
         const uint64_t q = p.moduli[t];
-        const uint64_t *in = p.c0 + ((size_t)t << p.log_n);
+        const uint64_t *in = c0 + ((size_t)t << p.log_n);
         const size_t o = ((size_t)t << p.log_n) + j;
-        uint64_t acc = p.accumulate ? p.c0_out[o] : 0;
+        uint64_t acc = p.accumulate ? c0_out[o] : (p.with_self ? in[j] : 0);
         for (uint32_t s = 0; s < p.n_steps; s++) acc = add_mod(acc, in[galois_index(j, p.elts[s], p.log_n)], q);
-        p.c0_out[o] = acc;
+        c0_out[o] = acc;
         return;
     }
     const uint32_t t = blockIdx.y;
+    const uint64_t *y = p.y + blockIdx.z * ((size_t)p.beta * LK << p.log_n) + ((size_t)t << p.log_n);
+    uint64_t *out = p.out + blockIdx.z * ((size_t)2 * LK << p.log_n);
     const uint32_t table = t < p.L ? t : p.size_q + (t - p.L);
     const size_t key_off = ((size_t)table << p.log_n) + j;
     const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
+    const size_t digit = (size_t)LK << p.log_n;
     U128 a0{0, 0}, a1{0, 0};
     for (uint32_t s = 0; s < p.n_steps; s++) {
         const uint32_t src = galois_index(j, p.elts[s], p.log_n);
+        // the loads of a step's digits are issued together
+#pragma unroll 4
         for (uint32_t d = 0; d < p.beta; d++) {
-            const uint64_t v = p.y[(((size_t)d * LK + t) << p.log_n) + src];
+            const uint64_t v = y[d * digit + src];
             const uint64_t *k = p.evk.p[s * p.beta + d];
             mac128(a0, v, k[key_off]);
             mac128(a1, v, k[key_off + key_poly]);
@@ -327,11 +384,11 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     const size_t o = ((size_t)t << p.log_n) + j;
     const size_t opoly = (size_t)LK << p.log_n;
     if (p.accumulate) {
-        o0 = add_mod(o0, p.out[o], q);
-        o1 = add_mod(o1, p.out[o + opoly], q);
+        o0 = add_mod(o0, out[o], q);
+        o1 = add_mod(o1, out[o + opoly], q);
     }
-    p.out[o] = o0;
-    p.out[o + opoly] = o1;
+    out[o] = o0;
+    out[o + opoly] = o1;
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -453,6 +510,14 @@ hipError_t launch_tensor(const Tables &t, const uint64_t *ct1, const uint64_t *c
     return hipGetLastError();
 }
 
+hipError_t launch_pair_square_sum(const Tables &t, const uint64_t *const *pairs, uint64_t *out01, uint64_t *out2,
+                                  uint32_t L, uint32_t items, uint32_t chunks, hipStream_t s) {
+    if (items == 0 || items > 65535 || chunks == 0 || L == 0) return hipErrorInvalidValue;
+    PairSquareArgs p{pairs, out01, out2, t.moduli, t.barrett, L, t.log_n, chunks};
+    hipLaunchKernelGGL(pair_square_sum_kernel, dim3((1u << t.log_n) / kThreads, L, items), dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_galois(const Tables &t, const uint64_t *in, uint64_t *out, uint32_t total_limbs, uint32_t elt,
                          hipStream_t s) {
     if (total_limbs == 0) return hipSuccess;
@@ -485,7 +550,9 @@ hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_
     const uint32_t rows_per = (b.max_rows + cg - 1) / cg;
     const uint32_t kg = (b.max_copy + rows_per - 1) / rows_per;
     BconvBatchK p{b, t.moduli, t.barrett, t.log_n, cg, rows_per};
-    const dim3 grid((1u << t.log_n) / kThreads, cg + kg, b.n_units);
+    const uint32_t items = b.items ? b.items : 1;
+    if ((uint64_t)b.n_units * items > 65535) return hipErrorInvalidValue;
+    const dim3 grid((1u << t.log_n) / kThreads, cg + kg, b.n_units * items);
     if (b.mat_fp)
         hipLaunchKernelGGL(bconv_batched_fp_kernel, grid, dim3(kThreads), 0, s, p);
     else
@@ -495,17 +562,21 @@ hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_
 
 hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
-                                const uint64_t *fold_ct, const uint64_t *fold_w, hipStream_t s) {
+                                const uint64_t *fold_ct, const uint64_t *fold_w, uint32_t items, size_t fold_item_stride,
+                                hipStream_t s) {
+    const size_t n = (size_t)1 << t.log_n;
     InnerArgs p{y, out, t.moduli, t.barrett, evk, L, K, size_q, beta, t.log_n, galois_elt, accumulate ? 1 : 0,
-                fold_ct, fold_w};
-    hipLaunchKernelGGL(inner_product_kernel, dim3((1u << t.log_n) / kThreads, L + K), dim3(kThreads), 0, s, p);
+                fold_ct, fold_w, (size_t)beta * (L + K) * n, 2 * (size_t)(L + K) * n, fold_item_stride};
+    if (items == 0 || items > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(inner_product_kernel, dim3((1u << t.log_n) / kThreads, L + K, items), dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
 
 hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
                               const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
-                              uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, hipStream_t s) {
-    if (n_steps == 0 || n_steps * beta > (uint32_t)kMaxDigits) return hipErrorInvalidValue;
+                              uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, bool with_self, uint32_t items,
+                              size_t ct_item_stride, hipStream_t s) {
+    if (n_steps == 0 || n_steps * beta > (uint32_t)kMaxDigits || items == 0 || items > 65535) return hipErrorInvalidValue;
     HoistArgs p;
     memset(&p, 0, sizeof(p));
     p.y = y;
@@ -523,7 +594,10 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
     p.beta = beta;
     p.log_n = t.log_n;
     p.accumulate = accumulate ? 1 : 0;
-    hipLaunchKernelGGL(hoist_inner_kernel, dim3((1u << t.log_n) / kThreads, (L + K) + L), dim3(kThreads), 0, s, p);
+    p.with_self = with_self ? 1 : 0;
+    p.ct_item_stride = ct_item_stride;
+    hipLaunchKernelGGL(hoist_inner_kernel, dim3((1u << t.log_n) / kThreads, (L + K) + (with_self ? 2 : 1) * L, items),
+                       dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
 

@@ -29,6 +29,8 @@ class KrumConfig:
     hoisting: bool = True                    # byzantine_fl.py: Hoisting_flag = 1
     hoisting_radix: int = 16                 # every round of the slot sum is a hoisted sum of radix - 1 rotations;
                                              # 0: the reference's split, hoisting(1..15) then one rotation per doubling
+    batched: bool = True                     # all pairs go through every stage together, one launch per stage
+                                             # (pair_square_distances); False: pair by pair over the lanes
     lanes: int = 3                           # host threads / streams that the pairs are dealt to (0: null stream);
                                              # three streams and the null stream fill the four hardware queues
     sec_level: str = "tc128"
@@ -194,10 +196,17 @@ def _map_lanes(state: KrumState, items, fn):
 def all_pair_distances(state: KrumState, cts, enc):
     """enc[i][j] = enc[j][i] = pair_distance(i, j) for every i < j.  The pairs are independent, and at Lancelot's
     sizes (three or four limbs) one of them neither fills the GPU nor keeps one host thread's launch rate busy, so
-    they are spread over the lanes."""
+    they go through every stage together (one launch per stage for all pairs) or, pair by pair, over the lanes."""
     n_clients = len(cts)
     pairs = [(i, j) for i in range(n_clients) for j in range(i + 1, n_clients)]
-    for (i, j), ct in zip(pairs, _map_lanes(state, pairs, lambda ij: pair_distance(state, cts[ij[0]], cts[ij[1]]))):
+    if state.config.batched:
+        c = state.cahel
+        rounds = rotate_sum_plan(int(math.log2(state.slots)), state.config)
+        out = c.pair_square_distances(state.context, cts, pairs, state.rlk, state.glk, rounds, state.config.scale)
+        _sync(c)
+    else:
+        out = _map_lanes(state, pairs, lambda ij: pair_distance(state, cts[ij[0]], cts[ij[1]]))
+    for (i, j), ct in zip(pairs, out):
         enc[i][j] = enc[j][i] = ct
 
 

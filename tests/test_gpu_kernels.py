@@ -228,6 +228,77 @@ def test_hoisted_rotations_entry_point(oracle, capi, logn, bits, size_p, L, n_st
     assert lib.he_hoisted_rotations(h, L, din.ptr, flat, d_elts, n_steps, dout.ptr, ws.ptr, None) == -1   # even element
 
 
+@pytest.mark.parametrize("logn,bits,size_p,L,items", [(11, [45, 40, 40, 50], 1, 3, 5), (11, [60, 40, 40, 60], 1, 2, 3),
+                                                       (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5, 2),
+                                                       (11, [50, 50, 49, 50, 50, 50], 2, 4, 3)])
+def test_batched_entry_points_equal_separate_calls(oracle, capi, logn, bits, size_p, L, items):
+    """he_keyswitch_rescale_batch, he_hoisted_rotations_batch and he_pair_square_sum over several inputs against
+    one call per input (which the other tests pin to the oracle), on both arithmetic back ends."""
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(16)
+    lib, h = capi.lib(), ctx.he_handle()
+    beta = -(-L // size_p)
+    keys = [_evk(p, rng, capi) for _ in range(2)]
+    ws1 = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    wsb = DeviceArray(capi, shape=(lib.he_keyswitch_batch_workspace_words(h, L, items),))
+    assert wsb.numpy().size == items * ws1.numpy().size
+
+    # relinearise + rescale of dense size-3 ciphertexts: c = third polynomial, stride 3 L limbs
+    ct3 = np.stack([rand_limbs(p, rng, range(L), n_polys=3) for _ in range(items)])
+    ct2 = np.ascontiguousarray(ct3[:, :2])
+    d3, d2 = DeviceArray(capi, host=ct3), DeviceArray(capi, host=ct2)
+    dout = DeviceArray(capi, shape=(items, 2, L - 1, p.n))
+    c_ptr = d3.ptr + 2 * L * p.n * 8
+    capi.check(lib.he_keyswitch_rescale_batch(h, L, items, c_ptr, 3 * L, keys[0][2], d2.ptr, dout.ptr, 0, wsb.ptr, None))
+    got = dout.numpy()
+    for k in range(items):
+        dc, dct = DeviceArray(capi, host=ct3[k, 2]), DeviceArray(capi, host=ct2[k])
+        one = DeviceArray(capi, shape=(2, L - 1, p.n))
+        capi.check(lib.he_keyswitch_rescale(h, L, dc.ptr, keys[0][2], dct.ptr, one.ptr, 0, ws1.ptr, None))
+        assert (got[k] == one.numpy()).all(), k
+    assert lib.he_keyswitch_rescale_batch(h, L, 2, c_ptr, 3 * L, keys[0][2], d2.ptr, dout.ptr, 5, wsb.ptr, None) == -1
+    assert lib.he_keyswitch_rescale_batch(h, L, items, c_ptr, L - 1, keys[0][2], d2.ptr, dout.ptr, 0, wsb.ptr, None) == -1
+
+    # hoisted rotations, with and without the input added
+    n_steps = 3
+    elts = [5, 25, 2 * p.n - 1]
+    flat = capi.evk_array([keys[i % 2][1][d].ptr for i in range(n_steps) for d in range(beta)])
+    d_elts = (C.c_uint32 * n_steps)(*elts)
+    hout = DeviceArray(capi, shape=(items, 2, L, p.n))
+    for add_input in (0, 1):
+        capi.check(lib.he_hoisted_rotations_batch(h, L, items, d2.ptr, flat, d_elts, n_steps, add_input, hout.ptr,
+                                                  wsb.ptr, None))
+        got = hout.numpy()
+        for k in range(items):
+            din, one = DeviceArray(capi, host=ct2[k]), DeviceArray(capi, shape=(2, L, p.n))
+            capi.check(lib.he_hoisted_rotations(h, L, din.ptr, flat, d_elts, n_steps, one.ptr, ws1.ptr, None))
+            want = one.numpy()
+            if add_input:
+                want = np.stack([p.add(want[b], ct2[k, b]) for b in range(2)])
+            assert (got[k] == want).all(), (add_input, k)
+    assert (d2.numpy() == ct2).all()
+
+    # sum over chunks of (a - b)^2 from a device table of ciphertext pointers
+    chunks = 2
+    cts = [DeviceArray(capi, host=rand_limbs(p, rng, range(L), n_polys=2)) for _ in range(4)]
+    pairs = [(0, 1), (2, 3), (1, 3), (3, 0), (2, 2)][:items]
+    table = np.array([[cts[a].ptr, cts[b].ptr] * chunks for a, b in pairs], dtype=np.uint64)     # both chunks the same pair
+    table[0, 2:] = [cts[2].ptr, cts[0].ptr]                                                         # but for item 0
+    dtab = DeviceArray(capi, host=table)
+    sq01, sq2 = DeviceArray(capi, shape=(len(pairs), 2, L, p.n)), DeviceArray(capi, shape=(len(pairs), 1, L, p.n))
+    capi.check(lib.he_pair_square_sum(h, L, len(pairs), chunks, dtab.ptr, sq01.ptr, sq2.ptr, None))
+    got = np.concatenate([sq01.numpy(), sq2.numpy()], axis=1)
+    host = [c.numpy() for c in cts]
+    def square(a, b):
+        d = np.stack([p.sub(host[a][i], host[b][i]) for i in range(2)])
+        return p.tensor(d, d)
+    for k, (a, b) in enumerate(pairs):
+        second = square(2, 0) if k == 0 else square(a, b)
+        want = np.stack([p.add(x, y) for x, y in zip(square(a, b), second)])
+        assert (got[k] == want).all(), k
+    assert lib.he_pair_square_sum(h, L, 0, chunks, dtab.ptr, sq01.ptr, sq2.ptr, None) == -1
+
+
 def test_ntt_rejects_bad_arguments(small, capi):
     cahel, parms, ctx, p = small
     d = DeviceArray(capi, shape=(1, p.n))

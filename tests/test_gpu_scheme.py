@@ -341,17 +341,51 @@ def test_encrypted_krum_small(oracle):
     want = krum.plain_distance_matrix(updates)
     assert rel_err(dist, want) < 1e-3
     assert chosen == krum.krum_select(want) and chosen != 3
+    # pair by pair over the lanes instead of all pairs at once: the same ciphertexts, so the same values up to the
+    # flooding noise of the decryptions
+    cfg_pairs = krum.KrumConfig(log_n=13, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=11,
+                                reproducible=True, batched=False)
+    chosen1, dist1, _ = krum.gpu_krum(updates, cfg_pairs)
+    assert chosen1 == chosen and rel_err(dist1, dist) < 1e-6
     # the slot sum as doublings only, and as the reference's split (hoisting(1..15), then doublings)
-    for variant in (dict(hoisting=False), dict(hoisting_radix=0)):
+    for variant in (dict(hoisting=False), dict(hoisting_radix=0), dict(hoisting=False, batched=False)):
         plain = krum.KrumConfig(log_n=13, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=11, **variant)
         chosen2, dist2, _ = krum.gpu_krum(updates, plain)
         assert chosen2 == chosen and rel_err(dist2, want) < 1e-3
     assert {"encode", "encrypt", "evaluate", "decrypt", "total"} <= set(timings)
     # the pairs are spread over streams by default; on the null stream alone the ciphertexts are the same, and the
     # decryptions differ only by which flooding-noise sample each of them drew (the threads share one counter)
-    serial = krum.KrumConfig(log_n=13, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=11, lanes=0, reproducible=True)
+    serial = krum.KrumConfig(log_n=13, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=11, lanes=0, reproducible=True, batched=False)
     chosen3, dist3, _ = krum.gpu_krum(updates, serial)
-    assert chosen3 == chosen and rel_err(dist3, dist) < 1e-6
+    assert chosen3 == chosen and rel_err(dist3, dist1) < 1e-6
+
+
+def test_batched_pair_distances_equal_the_pairwise_ciphertexts(oracle):
+    """pair_square_distances (every stage one launch for all pairs) against sub / square / add / relinearise +
+    rescale / hoisting per pair: the same limbs."""
+    from lancelot_amd import krum
+    rng = np.random.default_rng(9)
+    updates = [rng.normal(0, 0.01, 3000).astype(np.float32) for _ in range(3)]
+    cfg = krum.KrumConfig(log_n=12, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=13, reproducible=True,
+                          hoisting_radix=8, lanes=0, sec_level="none")
+    state = krum.gpu_init(cfg)
+    cts = krum.encrypt_updates(state, krum.split_updates(updates, state.slots))
+    assert len(cts[0]) == 2
+    pairs = [(0, 1), (0, 2), (1, 2), (2, 0)]
+    rounds = krum.rotate_sum_plan(11, cfg)
+    assert [len(r) for r in rounds] == [7, 7, 7, 3]
+    c = state.cahel
+    batch = c.pair_square_distances(state.context, cts, pairs, state.rlk, state.glk, rounds, cfg.scale)
+    c._synchronize()
+    for (i, j), got in zip(pairs, batch):
+        want = krum.pair_distance(state, cts[i], cts[j])
+        assert got.chain_index() == want.chain_index() and got.scale() == want.scale()
+        assert (got.to_numpy() == want.to_numpy()).all(), (i, j)
+    assert c.pair_square_distances(state.context, cts, [], state.rlk, state.glk, rounds, 0.0) == []
+    with pytest.raises(ValueError, match="pair out of range"):
+        c.pair_square_distances(state.context, cts, [(0, 3)], state.rlk, state.glk, rounds, 0.0)
+    with pytest.raises(RuntimeError, match="Galois key not present"):
+        c.pair_square_distances(state.context, cts, pairs, state.rlk, state.glk, [[9]], 0.0)
 
 
 def test_encrypted_krum_aggregate_small(oracle):
