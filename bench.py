@@ -141,6 +141,7 @@ def main():
                          "hardware queues of a process; four measured slower than three or six)")
     ap.add_argument("--separate-rescale", action="store_true",
                     help="he_keyswitch then he_rescale instead of the merged he_keyswitch_rescale")
+    ap.add_argument("--no-krum", action="store_true", help="skip the encrypted Krum round (BASELINE.json configs[4])")
     ap.add_argument("--only", choices=["all", "roofline", "krum"], default="all",
                     help="roofline: run just the kernel the roofline object describes (for rocprofv3)")
     args = ap.parse_args()
@@ -333,6 +334,8 @@ def main():
                      "traffic": NTT72_TRAFFIC_BYTES, "ms_per_launch": fwd72, "algorithmic_bytes_per_launch": ntt_bytes},
         "ntt": ntt, "rotate": rotate,
     }
+    if not args.no_krum:
+        line["krum"] = krum_round()
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

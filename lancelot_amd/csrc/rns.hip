@@ -329,66 +329,83 @@ struct HoistArgs {
     uint32_t elts[kMaxDigits];      // Galois element of every step
     uint32_t n_steps, L, K, size_q, beta, log_n;
     int accumulate, with_self;
+    uint32_t items;
     size_t ct_item_stride;          // words between the ciphertexts of consecutive items (blockIdx.z), in and out
 };
 
-// Hoisted rotations in one launch: grid (N / 256, (L + K) + L [+ L], items).
+// Hoisted rotations in one launch: grid (N / 256, (L + K) + L [+ L], ceil(items / I)); a thread serves the same
+// coefficient of I consecutive items, so that a key word is loaded once for all of them.
 // rows t < L + K:  out[p][t] = sum_s sum_d sigma_s(y_d)[t] * evk_{s,d}[p][t]  (n_steps * beta <= 64 products, summed in
 //                  128 bits and reduced once); the automorphism is the gather index of the load of y.
 // rows L + K + t:  c0_out[t] = sum_s sigma_s(c0)[t]  (+ c0[t] with_self)
 // rows L + K + L + t (with_self only): c1 is copied to the output, so that the ModDown that follows adds onto
 //                  the input ciphertext: ct_out = ct_in + sum_s rot_s(ct_in)
+template <int I>
 __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     const uint32_t LK = p.L + p.K;
     const uint32_t j = blockIdx.x * kThreads + threadIdx.x;
+    const uint32_t item0 = blockIdx.z * I;
+    const uint32_t count = p.items - item0 < (uint32_t)I ? p.items - item0 : (uint32_t)I;
     // (the argument struct stays untouched: a modified copy would move its tables to scratch memory)
-    const uint64_t *c0 = p.c0 + blockIdx.z * p.ct_item_stride;
-    uint64_t *c0_out = p.c0_out + blockIdx.z * p.ct_item_stride;
-    if (blockIdx.y >= LK + p.L) {
-        const size_t o = ((size_t)(blockIdx.y - LK) << p.log_n) + j;
-        if (!p.accumulate) c0_out[o] = c0[o];
-        return;
-    }
     if (blockIdx.y >= LK) {
-        const uint32_t t = blockIdx.y - LK;
-        const uint64_t q = p.moduli[t];
-        const uint64_t *in = c0 + ((size_t)t << p.log_n);
-        const size_t o = ((size_t)t << p.log_n) + j;
-        uint64_t acc = p.accumulate ? c0_out[o] : (p.with_self ? in[j] : 0);
-        for (uint32_t s = 0; s < p.n_steps; s++) acc = add_mod(acc, in[galois_index(j, p.elts[s], p.log_n)], q);
-        c0_out[o] = acc;
+        for (uint32_t it = 0; it < count; it++) {
+            const uint64_t *c0 = p.c0 + (item0 + it) * p.ct_item_stride;
+            uint64_t *c0_out = p.c0_out + (item0 + it) * p.ct_item_stride;
+            const size_t o = ((size_t)(blockIdx.y - LK) << p.log_n) + j;
+            if (blockIdx.y >= LK + p.L) {
+                if (!p.accumulate) c0_out[o] = c0[o];
+                continue;
+            }
+            const uint32_t t = blockIdx.y - LK;
+            const uint64_t q = p.moduli[t];
+            const uint64_t *in = c0 + ((size_t)t << p.log_n);
+            uint64_t acc = p.accumulate ? c0_out[o] : (p.with_self ? in[j] : 0);
+            for (uint32_t s = 0; s < p.n_steps; s++) acc = add_mod(acc, in[galois_index(j, p.elts[s], p.log_n)], q);
+            c0_out[o] = acc;
+        }
         return;
     }
     const uint32_t t = blockIdx.y;
-    const uint64_t *y = p.y + blockIdx.z * ((size_t)p.beta * LK << p.log_n) + ((size_t)t << p.log_n);
-    uint64_t *out = p.out + blockIdx.z * ((size_t)2 * LK << p.log_n);
+    const size_t y_item = (size_t)p.beta * LK << p.log_n;
+    const uint64_t *y = p.y + item0 * y_item + ((size_t)t << p.log_n);
     const uint32_t table = t < p.L ? t : p.size_q + (t - p.L);
     const size_t key_off = ((size_t)table << p.log_n) + j;
     const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
     const size_t digit = (size_t)LK << p.log_n;
-    U128 a0{0, 0}, a1{0, 0};
+    U128 a0[I], a1[I];
+#pragma unroll
+    for (int it = 0; it < I; it++) a0[it] = a1[it] = U128{0, 0};
     for (uint32_t s = 0; s < p.n_steps; s++) {
         const uint32_t src = galois_index(j, p.elts[s], p.log_n);
-        // the loads of a step's digits are issued together
-#pragma unroll 4
         for (uint32_t d = 0; d < p.beta; d++) {
-            const uint64_t v = y[d * digit + src];
             const uint64_t *k = p.evk.p[s * p.beta + d];
-            mac128(a0, v, k[key_off]);
-            mac128(a1, v, k[key_off + key_poly]);
+            const uint64_t k0 = k[key_off], k1 = k[key_off + key_poly];
+            uint64_t v[I];
+#pragma unroll
+            for (int it = 0; it < I; it++) v[it] = (uint32_t)it < count ? y[it * y_item + d * digit + src] : 0;
+#pragma unroll
+            for (int it = 0; it < I; it++) {
+                mac128(a0[it], v[it], k0);
+                mac128(a1[it], v[it], k1);
+            }
         }
     }
     const uint64_t q = p.moduli[table], r0 = p.barrett[2 * table], r1 = p.barrett[2 * table + 1];
-    uint64_t o0 = barrett128(a0.lo, a0.hi, q, r0, r1);
-    uint64_t o1 = barrett128(a1.lo, a1.hi, q, r0, r1);
     const size_t o = ((size_t)t << p.log_n) + j;
     const size_t opoly = (size_t)LK << p.log_n;
-    if (p.accumulate) {
-        o0 = add_mod(o0, out[o], q);
-        o1 = add_mod(o1, out[o + opoly], q);
+#pragma unroll
+    for (int it = 0; it < I; it++) {
+        if ((uint32_t)it >= count) break;
+        uint64_t *out = p.out + (item0 + it) * ((size_t)2 * LK << p.log_n);
+        uint64_t o0 = barrett128(a0[it].lo, a0[it].hi, q, r0, r1);
+        uint64_t o1 = barrett128(a1[it].lo, a1[it].hi, q, r0, r1);
+        if (p.accumulate) {
+            o0 = add_mod(o0, out[o], q);
+            o1 = add_mod(o1, out[o + opoly], q);
+        }
+        out[o] = o0;
+        out[o + opoly] = o1;
     }
-    out[o] = o0;
-    out[o + opoly] = o1;
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -596,8 +613,17 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
     p.accumulate = accumulate ? 1 : 0;
     p.with_self = with_self ? 1 : 0;
     p.ct_item_stride = ct_item_stride;
-    hipLaunchKernelGGL(hoist_inner_kernel, dim3((1u << t.log_n) / kThreads, (L + K) + (with_self ? 2 : 1) * L, items),
-                       dim3(kThreads), 0, s, p);
+    p.items = items;
+    const uint32_t rows = (L + K) + (with_self ? 2 : 1) * L;
+    auto grid = [&](uint32_t per) { return dim3((1u << t.log_n) / kThreads, rows, (items + per - 1) / per); };
+    if (items >= 8)
+        hipLaunchKernelGGL(hoist_inner_kernel<8>, grid(8), dim3(kThreads), 0, s, p);
+    else if (items >= 4)
+        hipLaunchKernelGGL(hoist_inner_kernel<4>, grid(4), dim3(kThreads), 0, s, p);
+    else if (items >= 2)
+        hipLaunchKernelGGL(hoist_inner_kernel<2>, grid(2), dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL(hoist_inner_kernel<1>, grid(1), dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
 
