@@ -62,6 +62,8 @@ struct he_context {
     std::vector<uint8_t> fp_ok;  // per table: prime below 2^50
     bool use_fp = true;          // environment CAHEL_HIP_NO_FP64=1 forces the integer back end
     bool fuse_inner = true;      // environment CAHEL_HIP_NO_FUSED_KS=1: separate NTT and inner-product kernels
+    bool fuse_modup_rows = true; // environment CAHEL_HIP_NO_FUSED_MODUP=1: base conversion and rows pass as two kernels
+    uint32_t modup_group = 6;    // output limbs per workgroup of the fused kernel (CAHEL_HIP_MODUP_GROUP)
     std::vector<Level> levels;   // indexed by L
     std::vector<void *> owned;
 
@@ -314,6 +316,12 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->use_fp = !(env && env[0] == '1');
         const char *nf = getenv("CAHEL_HIP_NO_FUSED_KS");
         ctx->fuse_inner = !(nf && nf[0] == '1');
+        const char *nm = getenv("CAHEL_HIP_NO_FUSED_MODUP");
+        ctx->fuse_modup_rows = !(nm && nm[0] == '1');
+        if (const char *g = getenv("CAHEL_HIP_MODUP_GROUP")) {
+            const int v = atoi(g);
+            if (v >= 1 && v <= 64) ctx->modup_group = (uint32_t)v;
+        }
         ctx->fp_ok.assign(qp, 0);
         std::vector<double> psi_fp(qp * n, 0.0), ipsi_fp(qp * n, 0.0), consts(4 * qp, 0.0);
         for (size_t t = 0; t < qp; t++) {
@@ -814,9 +822,6 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         inv.epi_mode = NTT_EPI_MUL;
         inv.w = lv->d_part_hat_inv;
         HE_HIP(launch_ntt_inverse(inv, 1, true, S(s)));
-        BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                     lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts, 1, 0, 0, 0};
-        HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
         NttArgs fwd = base_args(ctx, true);
         fwd.in = y;
         fwd.out = y;
@@ -824,6 +829,18 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         fwd.n_jobs = lv->n_modup_jobs;
         fwd.groups = lv->d_modup_groups;
         fwd.n_groups = lv->n_modup_groups;
+        const bool fused_rows = ctx->fuse_modup_rows && modup_rows_supported(ctx->log_n);
+        if (fused_rows) {
+            // base conversion and the rows pass of the forward transform in one kernel
+            const uint32_t group = ctx->modup_group;
+            ModupRowsArgs m{tmp, y, lv->d_modup_descs, lv->d_modup_limb, lv->d_modup_table, lv->d_mats_fp,
+                            group, (lv->modup_max_rows + group - 1) / group};
+            HE_HIP(launch_modup_rows(fwd, m, lv->beta, S(s)));
+        } else {
+            BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
+                         lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts, 1, 0, 0, 0};
+            HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+        }
         KsFuseArgs x;
         memset(&x, 0, sizeof(x));
         for (uint32_t d = 0; d < lv->beta; d++) {
@@ -839,7 +856,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         x.beta = lv->beta;
         x.fold_ct = fold_ct;
         x.fold_w = fold_w;
-        HE_HIP(launch_ntt_forward_inner(fwd, x, S(s)));
+        HE_HIP(launch_ntt_forward_inner(fwd, x, fused_rows, S(s)));
     } else {
         if (int rc = modup_impl(ctx, L, src, galois_elt ? L : c_item_stride, items, y, tmp, s)) return rc;
         EvkPtrs ptrs;

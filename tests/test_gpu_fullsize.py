@@ -121,6 +121,43 @@ def test_c3_hmult_properties(bench_world):
     assert (fused.to_numpy() == xy.to_numpy()).all()
 
 
+def test_c3_fused_and_separate_kernels_agree(monkeypatch):
+    """At N = 2^16, L = 24, K = 8 the key switch with its fused kernels (base conversion inside the rows pass, inner
+    product inside the blocks pass) and with the separate ones must give the same limbs (the separate kernels are
+    the ones that the small-size tests pin to the oracle)."""
+    from lancelot_amd import capi
+    outs = []
+    for no_fuse, no_modup in (("0", "0"), ("0", "1"), ("1", "1")):
+        monkeypatch.setenv("CAHEL_HIP_NO_FUSED_KS", no_fuse)
+        monkeypatch.setenv("CAHEL_HIP_NO_FUSED_MODUP", no_modup)
+        cahel, parms, ctx, mods = _context(16, [50] * 32, 8)
+        lib, h = capi.lib(), ctx.he_handle()
+        n, L, qp = 1 << 16, 24, 32
+        rng = np.random.default_rng(77)
+        q = np.array([m.value() for m in mods], dtype=np.uint64)
+        rand = lambda limbs, polys: (rng.integers(0, 1 << 62, (polys, len(limbs), n), dtype=np.uint64)
+                                     % q[list(limbs)][None, :, None])
+        evk = [rand(range(qp), 2) for _ in range(3)]
+        c, ct = rand(range(L), 1)[0], rand(range(L), 2)
+        import ctypes as C
+        def dev(a):
+            ptr = C.c_void_p()
+            capi.check(lib.he_malloc(C.byref(ptr), a.nbytes))
+            capi.check(lib.he_memcpy_h2d(ptr.value, np.ascontiguousarray(a).ctypes.data, a.nbytes, None))
+            return ptr.value
+        d_evk = [dev(k) for k in evk]
+        d_c, d_ct = dev(c), dev(ct)
+        ws = C.c_void_p()
+        capi.check(lib.he_malloc(C.byref(ws), 8 * lib.he_keyswitch_workspace_words(h, L)))
+        capi.check(lib.he_keyswitch(h, L, d_c, capi.evk_array(d_evk), d_ct, 0, ws.value, None))
+        out = np.empty_like(ct)
+        capi.check(lib.he_memcpy_d2h(out.ctypes.data, d_ct, out.nbytes, None))
+        for ptr in d_evk + [d_c, d_ct, ws.value]:
+            lib.he_free(ptr)
+        outs.append(out)
+    assert (outs[0] == outs[2]).all() and (outs[1] == outs[2]).all()
+
+
 def test_c4_rotations(bench_world):
     w = bench_world
     c, ctx = w["cahel"], w["ctx"]
