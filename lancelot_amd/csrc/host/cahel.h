@@ -86,7 +86,8 @@ private:
 // Lanes (not in the reference, which runs everything on the legacy default stream): lane 0 is the null stream,
 // lanes 1 .. lane_count() are non-blocking streams.  Every evaluator, encoder and key function enqueues on the
 // current lane, and temporaries are recycled per lane, so independent ciphertext pipelines given different lanes
-// overlap on the GPU.  An object produced on one lane may be used on another only after synchronize_lanes().
+// overlap on the GPU.  An object produced on one lane may be used on another only after synchronize_lanes(); it
+// may be dropped there (its storage returns to the producing lane after the dropping lane has drained).
 he_stream current_stream();
 int current_lane();
 int lane_count();

@@ -114,6 +114,9 @@ void DeviceBuffer::allocate(std::size_t words) {
 }
 
 void DeviceBuffer::release() {
+    // A block goes back to the lane that took it.  Dropped from another lane, it may still be read by work that
+    // the dropping thread has enqueued there: wait for that lane before the owner's lane can reuse the block.
+    if (ptr_ && g_lane != lane_) (void)he_stream_synchronize(g_lane_streams[g_lane]);
     if (ptr_) pool().give(ptr_, words_ * sizeof(uint64_t), lane_);
     ptr_ = nullptr;
     words_ = 0;
