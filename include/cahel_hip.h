@@ -268,6 +268,17 @@ int he_ckks_decode(const he_context *ctx, const uint64_t *plain, uint32_t limbs,
 
 size_t he_ckks_workspace_words(const he_context *ctx, uint32_t limbs);
 
+/* Decryption and decoding of `items` size-2 ciphertexts in one launch per stage: for the ciphertexts [2][limbs][N]
+ * named by the DEVICE pointer table d_cts, m = c0 + c1 s (+ noise [items][limbs][N] in NTT form, or NULL), inverse
+ * NTT, CRT composition and the special FFT; the first `count` complex slots of every item are written to
+ * out [items][count] (re, im).  sk: the secret key in NTT form (its first `limbs` limbs are read).
+ * Replaces, per item, ckks_decrypt (src/secretkey.cu:594-654) followed by decode_internal (src/ckks.cu:292-465).
+ * workspace: he_decrypt_decode_batch_workspace_words words. */
+size_t he_decrypt_decode_batch_workspace_words(const he_context *ctx, uint32_t limbs, uint32_t slots, uint32_t items);
+int he_decrypt_decode_batch(const he_context *ctx, const uint64_t *const *d_cts, uint32_t items, uint32_t limbs,
+                            const uint64_t *sk, const uint64_t *noise, uint32_t slots, double scale, uint32_t count,
+                            double *out, uint64_t *workspace, he_stream stream);
+
 /* ---- samplers (replace sample_ternary_poly / sample_error_poly / sample_uniform_poly, src/prng.cu:143-242,
  *      and the OpenFHE Gaussian of src/secretkey.cu:632-649) ----
  * ChaCha20 block function keyed by key[8]; `stream_id` selects an independent stream.  out: [limbs][N],
@@ -277,6 +288,12 @@ size_t he_ckks_workspace_words(const he_context *ctx, uint32_t limbs);
 int he_sample(const he_context *ctx, int kind, const uint32_t key[8], uint64_t stream_id, uint64_t *out,
               uint32_t limbs, uint32_t first_table, uint32_t split, uint32_t tail_table, const uint64_t *cdt,
               uint32_t cdt_len, he_stream stream);
+
+/* `items` polynomials in one launch: item k draws from stream_id + k (what `items` calls with consecutive stream ids
+ * would give) and is written limbs * N words after item k - 1.  No counterpart in the reference. */
+int he_sample_batch(const he_context *ctx, int kind, const uint32_t key[8], uint64_t stream_id, uint64_t *out,
+                    uint32_t limbs, uint32_t first_table, uint32_t split, uint32_t tail_table, const uint64_t *cdt,
+                    uint32_t cdt_len, uint32_t items, he_stream stream);
 
 #ifdef __cplusplus
 }

@@ -1043,20 +1043,58 @@ int he_ckks_decode(const he_context *ctx, const uint64_t *plain, uint32_t limbs,
     if (int rc = he_ntt_inverse(ctx, ws, 1, limbs, limbs, 0, limbs, 0, s)) return rc;
     const FftTables ft{ctx->d_rot_group, ctx->d_ksi, ctx->log_n};
     HE_HIP(launch_ckks_decode(ft, ctx->tables(), ws, limbs, slots, scale, ctx->d_garner_inv, ctx->size_q,
-                              reinterpret_cast<double2 *>(out), S(s)));
+                              reinterpret_cast<double2 *>(out), 1, S(s)));
+    return HE_OK;
+}
+
+size_t he_decrypt_decode_batch_workspace_words(const he_context *ctx, uint32_t limbs, uint32_t slots, uint32_t items) {
+    if (!ctx) return 0;
+    // [items][limbs][N] plaintexts | [items][slots] complex values
+    return (size_t)items * limbs * ctx->n() + 2 * (size_t)items * slots;
+}
+
+int he_decrypt_decode_batch(const he_context *ctx, const uint64_t *const *d_cts, uint32_t items, uint32_t limbs,
+                            const uint64_t *sk, const uint64_t *noise, uint32_t slots, double scale, uint32_t count,
+                            double *out, uint64_t *ws, he_stream s) {
+    if (!ctx || !d_cts || !sk || !out || !ws || items == 0 || items > 16384 || limbs == 0 || limbs > ctx->size_q)
+        return HE_E_INVALID_ARGUMENT;
+    if (slots < 2 || (slots & (slots - 1)) || slots > ctx->n() / 2 || !(scale > 0) || count == 0 || count > slots)
+        return HE_E_INVALID_ARGUMENT;
+    const size_t n = ctx->n();
+    uint64_t *plain = ws;
+    double2 *v = reinterpret_cast<double2 *>(ws + (size_t)items * limbs * n);
+    HE_HIP(launch_decrypt_gather(ctx->tables(), d_cts, sk, noise, plain, limbs, items, S(s)));
+    if (int rc = he_ntt_inverse(ctx, plain, items, limbs, limbs, 0, limbs, 0, s)) return rc;
+    const FftTables ft{ctx->d_rot_group, ctx->d_ksi, ctx->log_n};
+    HE_HIP(launch_ckks_decode(ft, ctx->tables(), plain, limbs, slots, scale, ctx->d_garner_inv, ctx->size_q, v, items, S(s)));
+    HE_HIP(launch_take_slots(v, slots, items, count, reinterpret_cast<double2 *>(out), S(s)));
+    return HE_OK;
+}
+
+static int sample_impl(const he_context *ctx, int kind, const uint32_t key[8], uint64_t stream_id, uint64_t *out,
+                       uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail, const uint64_t *cdt,
+                       uint32_t cdt_len, uint32_t items, he_stream s) {
+    if (!ctx || !key || !out || kind < 0 || kind > 3 || (kind == SAMPLE_GAUSS && (!cdt || !cdt_len)) || items == 0 ||
+        items > 16384)
+        return HE_E_INVALID_ARGUMENT;
+    if (int rc = check_map(ctx, limbs, first, split, tail)) return rc;
+    ChaChaKey k;
+    memcpy(k.k, key, sizeof(k.k));
+    HE_HIP(launch_sample(ctx->tables(), kind, k, stream_id, out, LimbMap{limbs, first, split, tail}, cdt, cdt_len, items,
+                         S(s)));
     return HE_OK;
 }
 
 int he_sample(const he_context *ctx, int kind, const uint32_t key[8], uint64_t stream_id, uint64_t *out,
               uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail, const uint64_t *cdt, uint32_t cdt_len,
               he_stream s) {
-    if (!ctx || !key || !out || kind < 0 || kind > 3 || (kind == SAMPLE_GAUSS && (!cdt || !cdt_len)))
-        return HE_E_INVALID_ARGUMENT;
-    if (int rc = check_map(ctx, limbs, first, split, tail)) return rc;
-    ChaChaKey k;
-    memcpy(k.k, key, sizeof(k.k));
-    HE_HIP(launch_sample(ctx->tables(), kind, k, stream_id, out, LimbMap{limbs, first, split, tail}, cdt, cdt_len, S(s)));
-    return HE_OK;
+    return sample_impl(ctx, kind, key, stream_id, out, limbs, first, split, tail, cdt, cdt_len, 1, s);
+}
+
+int he_sample_batch(const he_context *ctx, int kind, const uint32_t key[8], uint64_t stream_id, uint64_t *out,
+                    uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail, const uint64_t *cdt, uint32_t cdt_len,
+                    uint32_t items, he_stream s) {
+    return sample_impl(ctx, kind, key, stream_id, out, limbs, first, split, tail, cdt, cdt_len, items, s);
 }
 
 }  // extern "C"

@@ -47,9 +47,10 @@ __device__ __forceinline__ void butterfly(double2 &a, double2 &b, double2 w) {
     }
 }
 
-// one stage over global memory; thread = one butterfly
+// one stage over global memory; thread = one butterfly; blockIdx.y = item (vectors `slots` apart)
 template <bool INVERSE>
-__global__ __launch_bounds__(kThreads) void cfft_stage_kernel(double2 *v, uint32_t len, FftTables t) {
+__global__ __launch_bounds__(kThreads) void cfft_stage_kernel(double2 *v, uint32_t len, FftTables t, uint32_t slots) {
+    v += (size_t)blockIdx.y * slots;
     const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
     const uint32_t lenh = len >> 1;
     const uint32_t j = b & (lenh - 1), pos = ((b / lenh) * len) + j;
@@ -61,9 +62,9 @@ __global__ __launch_bounds__(kThreads) void cfft_stage_kernel(double2 *v, uint32
 
 // every stage of span <= tile inside LDS; tile = min(slots, kFftTile) values per workgroup
 template <bool INVERSE>
-__global__ __launch_bounds__(kThreads) void cfft_lds_kernel(double2 *v, uint32_t tile, FftTables t) {
+__global__ __launch_bounds__(kThreads) void cfft_lds_kernel(double2 *v, uint32_t tile, FftTables t, uint32_t slots) {
     __shared__ double2 s[kFftTile];
-    double2 *g = v + (size_t)blockIdx.x * tile;
+    double2 *g = v + (size_t)blockIdx.y * slots + (size_t)blockIdx.x * tile;
     for (uint32_t i = threadIdx.x; i < tile; i += kThreads) s[i] = g[i];
     __syncthreads();
     for (uint32_t k = 2; k <= tile; k <<= 1) {
@@ -120,6 +121,8 @@ __global__ __launch_bounds__(kThreads) void decode_compose_kernel(const uint64_t
     const uint32_t s = blockIdx.x * kThreads + threadIdx.x;
     const uint32_t slots = 1u << log_slots, half = 1u << (log_n - 1);
     if (s >= 2 * slots) return;
+    res += ((size_t)blockIdx.y * limbs) << log_n;   // blockIdx.y = item: dense plaintexts, dense slot vectors
+    v += (size_t)blockIdx.y * slots;
     const bool imag = s >= slots;
     const uint32_t i0 = imag ? s - slots : s;
     const size_t coeff = (imag ? half : 0) + (size_t)i0 * gap;
@@ -158,18 +161,25 @@ __global__ __launch_bounds__(kThreads) void decode_compose_kernel(const uint64_t
 }
 
 template <bool INVERSE>
-hipError_t run_fft(double2 *v, uint32_t slots, const FftTables &t, hipStream_t s) {
+hipError_t run_fft(double2 *v, uint32_t slots, uint32_t items, const FftTables &t, hipStream_t s) {
     const uint32_t tile = slots < kFftTile ? slots : kFftTile;
+    const dim3 stage_grid(slots / 2 / kThreads, items), lds_grid(slots / tile, items);
     if (INVERSE) {
         for (uint32_t len = slots; len > tile; len >>= 1)
-            hipLaunchKernelGGL(cfft_stage_kernel<true>, dim3(slots / 2 / kThreads), dim3(kThreads), 0, s, v, len, t);
-        hipLaunchKernelGGL(cfft_lds_kernel<true>, dim3(slots / tile), dim3(kThreads), 0, s, v, tile, t);
+            hipLaunchKernelGGL(cfft_stage_kernel<true>, stage_grid, dim3(kThreads), 0, s, v, len, t, slots);
+        hipLaunchKernelGGL(cfft_lds_kernel<true>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots);
     } else {
-        hipLaunchKernelGGL(cfft_lds_kernel<false>, dim3(slots / tile), dim3(kThreads), 0, s, v, tile, t);
+        hipLaunchKernelGGL(cfft_lds_kernel<false>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots);
         for (uint32_t len = tile << 1; len <= slots; len <<= 1)
-            hipLaunchKernelGGL(cfft_stage_kernel<false>, dim3(slots / 2 / kThreads), dim3(kThreads), 0, s, v, len, t);
+            hipLaunchKernelGGL(cfft_stage_kernel<false>, stage_grid, dim3(kThreads), 0, s, v, len, t, slots);
     }
     return hipGetLastError();
+}
+
+// out[item][i] = v[item][i] for i < count: the leading slots of every item, packed
+__global__ __launch_bounds__(kThreads) void take_slots_kernel(const double2 *v, uint32_t slots, uint32_t count, double2 *out) {
+    const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+    if (i < count) out[(size_t)blockIdx.y * count + i] = v[(size_t)blockIdx.y * slots + i];
 }
 
 }  // namespace
@@ -180,7 +190,7 @@ hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double
     auto blocks = [](uint32_t items) { return dim3((items + kThreads - 1) / kThreads); };
     hipLaunchKernelGGL(encode_load_kernel, blocks(slots), dim3(kThreads), 0, s, re, im, count, slots, v,
                        reinterpret_cast<unsigned long long *>(max_bits));
-    hipError_t e = run_fft<true>(v, slots, t, s);
+    hipError_t e = run_fft<true>(v, slots, 1, t, s);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(encode_round_kernel, blocks(n), dim3(kThreads), 0, s, v, log_slots, (n / 2) / slots, n / 2,
                        scale / (double)slots, coeffs, reinterpret_cast<unsigned long long *>(max_bits));
@@ -189,12 +199,20 @@ hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double
 
 hipError_t launch_ckks_decode(const FftTables &t, const Tables &tab, const uint64_t *res, uint32_t limbs,
                               uint32_t slots, double scale, const uint64_t *garner_inv, uint32_t garner_stride,
-                              double2 *v, hipStream_t s) {
+                              double2 *v, uint32_t items, hipStream_t s) {
     const uint32_t n = 1u << t.log_n, log_slots = 31 - __builtin_clz(slots);
-    if (limbs == 0 || limbs > (uint32_t)kMaxComposeLimbs) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(decode_compose_kernel, dim3((2 * slots + kThreads - 1) / kThreads), dim3(kThreads), 0, s, res, limbs, t.log_n,
-                       log_slots, (n / 2) / slots, 1.0 / scale, tab.moduli, tab.barrett, garner_inv, garner_stride, v);
-    return run_fft<false>(v, slots, t, s);
+    if (limbs == 0 || limbs > (uint32_t)kMaxComposeLimbs || items == 0 || items > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(decode_compose_kernel, dim3((2 * slots + kThreads - 1) / kThreads, items), dim3(kThreads), 0, s, res,
+                       limbs, t.log_n, log_slots, (n / 2) / slots, 1.0 / scale, tab.moduli, tab.barrett, garner_inv,
+                       garner_stride, v);
+    return run_fft<false>(v, slots, items, t, s);
+}
+
+hipError_t launch_take_slots(const double2 *v, uint32_t slots, uint32_t items, uint32_t count, double2 *out, hipStream_t s) {
+    if (count == 0 || count > slots || items == 0 || items > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(take_slots_kernel, dim3((count + kThreads - 1) / kThreads, items), dim3(kThreads), 0, s, v, slots,
+                       count, out);
+    return hipGetLastError();
 }
 
 }  // namespace he

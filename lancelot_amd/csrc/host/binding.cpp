@@ -107,6 +107,19 @@ PYBIND11_MODULE(pyCAHEL, m) {
         .def("decrypt", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &>(&CAHELGPUSecretKey::decrypt),
              py::call_guard<py::gil_scoped_release>())
         .def("set_noise_flooding", &CAHELGPUSecretKey::set_noise_flooding)
+        .def("decrypt_decode_many",
+             [](CAHELGPUSecretKey &k, const CAHELGPUContext &c, const std::vector<const CAHELGPUCiphertext *> &cts,
+                std::size_t slots, std::size_t count) {
+                 std::vector<double> out;
+                 {
+                     py::gil_scoped_release release;
+                     out = k.decrypt_decode_many(c, cts, slots, count);
+                 }
+                 py::array_t<double> a({(py::ssize_t)cts.size(), (py::ssize_t)count});
+                 std::copy(out.begin(), out.end(), a.mutable_data());
+                 return a;
+             },
+             py::arg("context"), py::arg("ciphertexts"), py::arg("slots"), py::arg("count") = 1)
         .def("to_numpy", [](const CAHELGPUSecretKey &s, const CAHELGPUContext &c) {
             return to_host(s.secret_key_array(), {(py::ssize_t)c.size_qp(), (py::ssize_t)c.poly_degree()});
         });

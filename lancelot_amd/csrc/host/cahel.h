@@ -138,7 +138,7 @@ public:
     // The default key comes from /dev/urandom (include/prng.cuh:12-23); set_seed makes runs reproducible.
     void set_seed(uint64_t seed);
     const uint32_t *prng_key() const { return prng_key_; }
-    uint64_t next_stream() const { return prng_stream_.fetch_add(1, std::memory_order_relaxed); }
+    uint64_t next_stream(uint64_t count = 1) const { return prng_stream_.fetch_add(count, std::memory_order_relaxed); }
     const uint64_t *gauss_cdt() const { return gauss_cdt_.get(); }
     uint32_t gauss_cdt_len() const { return gauss_cdt_len_; }
 
@@ -289,6 +289,12 @@ public:
     // Decryption adds discrete-Gaussian noise (sigma = 5.574611952644673) as the reference does
     // (src/secretkey.cu:632-649); tests that compare limbs switch it off.
     void set_noise_flooding(bool on) { noise_flooding_ = on; }
+    // Real parts of the first `count` slots of every ciphertext, [items][count] row-major: decrypt + decode of all of
+    // them with one launch per stage (not in the reference).  All ciphertexts: size 2, one level, one scale;
+    // `slots` = the encoder's slot count.
+    std::vector<double> decrypt_decode_many(const CAHELGPUContext &context,
+                                            const std::vector<const CAHELGPUCiphertext *> &ciphers, std::size_t slots,
+                                            std::size_t count);
     const uint64_t *secret_key_array() const { return sk_powers_.get(); }
 
 private:

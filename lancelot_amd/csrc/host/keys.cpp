@@ -3,6 +3,7 @@
 // :374-396, create_galois_keys :398-442, encrypt_zero_asymmetric :47-117 and its ModDown :126-170,
 // ckks_decrypt :594-654).  Randomness comes from the context's seeded ChaCha20 streams, one stream id per
 // sampled polynomial, handed out in the order the polynomials are drawn.
+#include <cmath>
 #include <string>
 
 #include "cahel.h"
@@ -225,4 +226,51 @@ void CAHELGPUSecretKey::decrypt(const CAHELGPUContext &context, const CAHELGPUCi
     plain.scale() = cipher.scale();
     plain.parms_id() = cipher.parms_id();
     plain.is_ntt_form_ = true;
+}
+
+std::vector<double> CAHELGPUSecretKey::decrypt_decode_many(const CAHELGPUContext &context,
+                                                           const std::vector<const CAHELGPUCiphertext *> &ciphers,
+                                                           std::size_t slots, std::size_t count) {
+    if (!gen_flag_) throw std::logic_error("secret key has not been generated");
+    if (ciphers.empty()) return {};
+    if (ciphers.size() > 16384) throw std::invalid_argument("too many ciphertexts");
+    const CAHELGPUCiphertext &first = *ciphers[0];
+    for (const CAHELGPUCiphertext *ct : ciphers) {
+        if (!ct || ct->size() != 2 || !ct->is_ntt_form()) throw std::invalid_argument("encrypted is not valid");
+        if (ct->parms_id() != first.parms_id() || ct->chain_index() != first.chain_index() || ct->scale() != first.scale())
+            throw std::invalid_argument("encrypted parameter mismatch");
+    }
+    const std::size_t n = context.poly_degree();
+    const uint32_t limbs = (uint32_t)first.coeff_modulus_size(), items = (uint32_t)ciphers.size();
+    if (slots < 2 || (slots & (slots - 1)) || slots > n / 2 || count == 0 || count > slots)
+        throw std::invalid_argument("slot count out of range");
+    const int total_bits = context.total_coeff_modulus_bit_count(first.chain_index());
+    if (first.scale() <= 0 || (static_cast<int>(std::log2(first.scale())) >= total_bits))
+        throw std::invalid_argument("scale out of bounds");
+    he_context *h = context.handle();
+    he_stream st = context.stream();
+    std::vector<const uint64_t *> table;
+    for (const CAHELGPUCiphertext *ct : ciphers) table.push_back(ct->data());
+    DeviceBuffer d_table(items);
+    check_status(he_memcpy_h2d(d_table.get(), table.data(), table.size() * sizeof(uint64_t), st), "upload");
+    DeviceBuffer noise;
+    if (noise_flooding_) {
+        // one flooding-noise polynomial per ciphertext, the stream ids that `items` calls of decrypt would draw
+        noise.allocate((std::size_t)items * limbs * n);
+        check_status(he_sample_batch(h, 3, context.prng_key(), context.next_stream(items), noise.get(), limbs, 0, limbs, 0,
+                                     context.gauss_cdt(), context.gauss_cdt_len(), items, st),
+                     "he_sample_batch");
+        check_status(he_ntt_forward(h, noise.get(), items, limbs, limbs, 0, limbs, 0, st), "he_ntt_forward");
+    }
+    DeviceBuffer ws(he_decrypt_decode_batch_workspace_words(h, limbs, (uint32_t)slots, items));
+    DeviceBuffer out(2 * (std::size_t)items * count);
+    check_status(he_decrypt_decode_batch(h, reinterpret_cast<const uint64_t *const *>(d_table.get()), items, limbs,
+                                         sk_powers_.get(), noise.get(), (uint32_t)slots, first.scale(), (uint32_t)count,
+                                         reinterpret_cast<double *>(out.get()), ws.get(), st),
+                 "he_decrypt_decode_batch");
+    std::vector<double> v(2 * (std::size_t)items * count);
+    check_status(he_memcpy_d2h(v.data(), out.get(), v.size() * sizeof(double), st), "download");
+    std::vector<double> re((std::size_t)items * count);
+    for (std::size_t i = 0; i < re.size(); i++) re[i] = v[2 * i];
+    return re;
 }

@@ -226,8 +226,9 @@ enum : int { SAMPLE_TERNARY = 0, SAMPLE_ERROR = 1, SAMPLE_UNIFORM = 2, SAMPLE_GA
 struct ChaChaKey {
     uint32_t k[8];
 };
+// items polynomials in one launch: item k draws from stream_id + k and lands map.limbs * N words after item k - 1
 hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
-                         const uint64_t *cdt, uint32_t cdt_len, hipStream_t s);
+                         const uint64_t *cdt, uint32_t cdt_len, uint32_t items, hipStream_t s);
 
 // CKKS encoder tables: 5^j mod 2N for j < N/2 and e^{2 pi i k / 2N} for k <= 2N.
 struct FftTables {
@@ -241,8 +242,15 @@ hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double
                               double scale, double2 *v, double *coeffs, uint64_t *max_bits, hipStream_t s);
 // res: [limbs][N] coefficient-form residues of the first `limbs` primes -> v: `slots` complex values.
 // garner_inv[i * stride + j] = q_j^-1 mod q_i for j < i.
+// items: that many dense plaintexts res [items][limbs][N] -> v [items][slots].
 hipError_t launch_ckks_decode(const FftTables &t, const Tables &tab, const uint64_t *res, uint32_t limbs,
                               uint32_t slots, double scale, const uint64_t *garner_inv, uint32_t garner_stride,
-                              double2 *v, hipStream_t s);
+                              double2 *v, uint32_t items, hipStream_t s);
+// out [items][count] = the first `count` values of every v [items][slots]
+hipError_t launch_take_slots(const double2 *v, uint32_t slots, uint32_t items, uint32_t count, double2 *out, hipStream_t s);
+// out [items][limbs][N] = c0 + c1 * s (+ noise [items][limbs][N]) for the size-2 ciphertexts [2][limbs][N] named by the
+// device pointer table cts [items]; s holds the secret key's first `limbs` limbs
+hipError_t launch_decrypt_gather(const Tables &t, const uint64_t *const *cts, const uint64_t *sk, const uint64_t *noise,
+                                 uint64_t *out, uint32_t limbs, uint32_t items, hipStream_t s);
 
 }  // namespace he

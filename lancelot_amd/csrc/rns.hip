@@ -106,6 +106,22 @@ __global__ __launch_bounds__(kThreads) void tensor_kernel(TensorArgs p) {
     p.out[idx + 2 * poly] = d2;
 }
 
+// grid: (N / 256, limbs, items).  out[item][limb] = c0 + c1 * s (+ noise[item][limb]) for the ciphertext cts[item]
+__global__ __launch_bounds__(kThreads) void decrypt_gather_kernel(const uint64_t *const *cts, const uint64_t *sk,
+                                                                  const uint64_t *noise, uint64_t *out,
+                                                                  const uint64_t *moduli, const uint64_t *barrett,
+                                                                  uint32_t limbs, uint32_t log_n) {
+    const uint32_t limb = blockIdx.y;
+    const uint64_t q = moduli[limb], r0 = barrett[2 * limb], r1 = barrett[2 * limb + 1];
+    const size_t idx = ((size_t)limb << log_n) + blockIdx.x * kThreads + threadIdx.x;
+    const size_t poly = (size_t)limbs << log_n;
+    const uint64_t *ct = cts[blockIdx.z];
+    uint64_t v = add_mod(ct[idx], mul_mod(ct[idx + poly], sk[idx], q, r0, r1), q);
+    const size_t o = (size_t)blockIdx.z * poly + idx;
+    if (noise) v = add_mod(v, noise[o], q);
+    out[o] = v;
+}
+
 struct PairSquareArgs {
     const uint64_t *const *pairs;   // device array [items][chunks][2] of ciphertext pointers, each [2][L][N]
     uint64_t *out01, *out2;         // [items][2][L][N] (d0, d1) and [items][L][N] (d2)
@@ -451,6 +467,9 @@ struct SampleArgs {
 __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
     const uint32_t n = 1u << p.log_n;
     const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
+    // blockIdx.y = item: the next stream id, the next polynomial
+    const uint64_t stream = p.stream + blockIdx.y;
+    uint64_t *out = p.out + (((size_t)blockIdx.y * p.map.limbs) << p.log_n);
     uint32_t w[16];
     if (p.kind == SAMPLE_UNIFORM) {
         const uint32_t per_limb = n / 4;
@@ -458,17 +477,17 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
         const uint32_t limb = b / per_limb, blk = b % per_limb;
         const uint32_t table = map_table(p.map, limb);
         const uint64_t q = p.moduli[table], r0 = p.barrett[2 * table], r1 = p.barrett[2 * table + 1];
-        chacha20_block(p.key, b, p.stream, w);
+        chacha20_block(p.key, b, stream, w);
         for (int e = 0; e < 4; e++) {
             uint64_t lo = ((uint64_t)w[4 * e + 1] << 32) | w[4 * e];
             uint64_t hi = ((uint64_t)w[4 * e + 3] << 32) | w[4 * e + 2];
-            p.out[((size_t)limb << p.log_n) + 4 * blk + e] = barrett128(lo, hi, q, r0, r1);
+            out[((size_t)limb << p.log_n) + 4 * blk + e] = barrett128(lo, hi, q, r0, r1);
         }
         return;
     }
     const uint32_t per_block = p.kind == SAMPLE_TERNARY ? 16 : 8;
     if (b >= n / per_block) return;
-    chacha20_block(p.key, b, p.stream, w);
+    chacha20_block(p.key, b, stream, w);
     for (uint32_t e = 0; e < per_block; e++) {
         int v;
         if (p.kind == SAMPLE_TERNARY) {
@@ -485,7 +504,7 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
         }
         for (uint32_t limb = 0; limb < p.map.limbs; limb++) {
             const uint64_t q = p.moduli[map_table(p.map, limb)];
-            p.out[((size_t)limb << p.log_n) + per_block * b + e] = v < 0 ? q - (uint64_t)(-v) : (uint64_t)v;
+            out[((size_t)limb << p.log_n) + per_block * b + e] = v < 0 ? q - (uint64_t)(-v) : (uint64_t)v;
         }
     }
 }
@@ -532,6 +551,14 @@ hipError_t launch_pair_square_sum(const Tables &t, const uint64_t *const *pairs,
     if (items == 0 || items > 65535 || chunks == 0 || L == 0) return hipErrorInvalidValue;
     PairSquareArgs p{pairs, out01, out2, t.moduli, t.barrett, L, t.log_n, chunks};
     hipLaunchKernelGGL(pair_square_sum_kernel, dim3((1u << t.log_n) / kThreads, L, items), dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_decrypt_gather(const Tables &t, const uint64_t *const *cts, const uint64_t *sk, const uint64_t *noise,
+                                 uint64_t *out, uint32_t limbs, uint32_t items, hipStream_t s) {
+    if (items == 0 || items > 65535 || limbs == 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(decrypt_gather_kernel, dim3((1u << t.log_n) / kThreads, limbs, items), dim3(kThreads), 0, s, cts, sk,
+                       noise, out, t.moduli, t.barrett, limbs, t.log_n);
     return hipGetLastError();
 }
 
@@ -628,11 +655,12 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
 }
 
 hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
-                         const uint64_t *cdt, uint32_t cdt_len, hipStream_t s) {
+                         const uint64_t *cdt, uint32_t cdt_len, uint32_t items, hipStream_t s) {
+    if (items == 0 || items > 65535) return hipErrorInvalidValue;
     const uint32_t n = 1u << t.log_n;
     uint32_t blocks = kind == SAMPLE_UNIFORM ? (n / 4) * map.limbs : (kind == SAMPLE_TERNARY ? n / 16 : n / 8);
     SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind};
-    hipLaunchKernelGGL(sample_kernel, dim3((blocks + kThreads - 1) / kThreads), dim3(kThreads), 0, s, p);
+    hipLaunchKernelGGL(sample_kernel, dim3((blocks + kThreads - 1) / kThreads, items), dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
 

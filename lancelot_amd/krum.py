@@ -224,8 +224,11 @@ def distance_matrix(state: KrumState, updates):
     dist = np.zeros((n_clients, n_clients))
     pairs = [(i, j) for i in range(n_clients) for j in range(i + 1, n_clients)]
     # every slot holds the distance: slot 0 is downloaded
-    values = _map_lanes(state, pairs, lambda ij: state.encoder.decode_array(
-        state.context, state.sk.decrypt(state.context, enc[ij[0]][ij[1]]), 1)[0])
+    if state.config.batched:
+        values = state.sk.decrypt_decode_many(state.context, [enc[i][j] for i, j in pairs], state.slots, 1)[:, 0]
+    else:
+        values = _map_lanes(state, pairs, lambda ij: state.encoder.decode_array(
+            state.context, state.sk.decrypt(state.context, enc[ij[0]][ij[1]]), 1)[0])
     for (i, j), value in zip(pairs, values):
         dist[i, j] = dist[j, i] = value
     state.timings["decrypt"] += time.perf_counter() - t0
@@ -246,7 +249,7 @@ def decrypt_sort_mask(state: KrumState, enc):
     n_clients = len(enc)
     t0 = time.perf_counter()
 
-    def score(i):
+    def row_sum(i):
         # the i == j distance is zero and was never evaluated; the reference starts from an encryption of zero
         row = [ct for ct in enc[i] if ct is not None]
         total = row[0]
@@ -255,9 +258,14 @@ def decrypt_sort_mask(state: KrumState, enc):
             c.add(ctx, row[0], row[1], total)
             for ct in row[2:]:
                 c.add_inplace(ctx, total, ct)
-        return state.encoder.decode_array(ctx, state.sk.decrypt(ctx, total), 1)[0]
+        return total
 
-    scores = _map_lanes(state, list(range(n_clients)), score)
+    if state.config.batched:
+        totals = [row_sum(i) for i in range(n_clients)]
+        scores = list(state.sk.decrypt_decode_many(ctx, totals, state.slots, 1)[:, 0])
+    else:
+        scores = _map_lanes(state, list(range(n_clients)), lambda i: state.encoder.decode_array(
+            ctx, state.sk.decrypt(ctx, row_sum(i)), 1)[0])
     order = np.argsort(np.asarray(scores), kind="stable")
     zero, one = _encrypt_constant(state, 0.0), _encrypt_constant(state, 1.0)
     mask = [[one if order[r] == k else zero for k in range(n_clients)] for r in range(n_clients)]

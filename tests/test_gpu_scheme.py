@@ -388,6 +388,31 @@ def test_batched_pair_distances_equal_the_pairwise_ciphertexts(oracle):
         c.pair_square_distances(state.context, cts, pairs, state.rlk, state.glk, [[9]], 0.0)
 
 
+def test_decrypt_decode_many_equals_one_by_one(world):
+    """secret_key.decrypt_decode_many against decrypt + decode_array per ciphertext: identical without the flooding
+    noise, within its size with it (the batch draws the stream ids that the single calls would)."""
+    w = world
+    c, ctx = w["cahel"], w["ctx"]
+    rng = np.random.default_rng(21)
+    slots = w["p"].n // 2
+    cts = [_encrypt_both(w, rng.uniform(-1, 1, slots))[2] for _ in range(5)]
+    c.rotate_vector_inplace(ctx, cts[3], 1, w["glk"])
+    w["sk"].set_noise_flooding(False)
+    one = np.stack([w["enc"].decode_array(ctx, w["sk"].decrypt(ctx, ct), 7) for ct in cts])
+    many = w["sk"].decrypt_decode_many(ctx, cts, slots, 7)
+    assert many.shape == (5, 7) and (many == one).all()
+    w["sk"].set_noise_flooding(True)
+    noisy = w["sk"].decrypt_decode_many(ctx, cts, slots, 7)
+    assert 0 < np.max(np.abs(noisy - one)) < 1e-6
+    assert w["sk"].decrypt_decode_many(ctx, [], slots, 1).shape == (0, 1)
+    with pytest.raises(ValueError, match="slot count out of range"):
+        w["sk"].decrypt_decode_many(ctx, cts, slots, slots + 1)
+    other = c.ciphertext(ctx)
+    c.multiply(ctx, cts[0], cts[1], other)          # size 3
+    with pytest.raises(ValueError, match="encrypted is not valid"):
+        w["sk"].decrypt_decode_many(ctx, [cts[0], other], slots, 1)
+
+
 def test_encrypted_krum_aggregate_small(oracle):
     """Distances, decrypt-sort-mask and the masked sum: the aggregate is the chosen client's update."""
     from lancelot_amd import krum
