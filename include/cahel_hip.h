@@ -268,6 +268,25 @@ int he_ckks_decode(const he_context *ctx, const uint64_t *plain, uint32_t limbs,
 
 size_t he_ckks_workspace_words(const he_context *ctx, uint32_t limbs);
 
+/* he_ckks_encode over `items` messages with one launch per stage: message k is re + k * value_stride (and im likewise,
+ * or NULL), plaintext k is written to out + k * out_poly_stride * N ([limbs][N], NTT form; a stride of 2 * limbs puts
+ * it into polynomial 0 of a dense batch of ciphertexts).  The largest |coefficient| of message k is left as a double
+ * in workspace[k].  workspace: he_ckks_encode_batch_workspace_words words.  No counterpart in the reference. */
+size_t he_ckks_encode_batch_workspace_words(const he_context *ctx, uint32_t items);
+int he_ckks_encode_batch(const he_context *ctx, const double *re, const double *im, uint32_t count, uint32_t slots,
+                         double scale, uint32_t limbs, uint32_t items, size_t value_stride, uint64_t *out,
+                         uint32_t out_poly_stride, uint64_t *workspace, he_stream stream);
+
+/* Public-key encryption of `items` plaintexts with one launch per stage: cts [items][2][L][N] holds plaintext k in
+ * polynomial 0 of ciphertext k on entry and ciphertext k on return: (u pk_0 + e_0, u pk_1 + e_1) over Ql u P, divided
+ * by P, plus the plaintext.  pk: [2][size_q + size_p][N] at the key level.  Item k draws u, e_0, e_1 from the
+ * ChaCha20 streams stream_id + 3 k, + 1, + 2 (what `items` encryptions in a row draw).  Replaces, per item,
+ * encrypt_asymmetric (src/secretkey.cu:179-246: encrypt_zero_asymmetric at the key level, DRNSTool::moddown, add).
+ * workspace: he_encrypt_batch_workspace_words words. */
+size_t he_encrypt_batch_workspace_words(const he_context *ctx, uint32_t L, uint32_t items);
+int he_encrypt_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *pk, const uint32_t key[8],
+                     uint64_t stream_id, uint64_t *cts, uint64_t *workspace, he_stream stream);
+
 /* Decryption and decoding of `items` size-2 ciphertexts in one launch per stage: for the ciphertexts [2][limbs][N]
  * named by the DEVICE pointer table d_cts, m = c0 + c1 s (+ noise [items][limbs][N] in NTT form, or NULL), inverse
  * NTT, CRT composition and the special FFT; the first `count` complex slots of every item are written to

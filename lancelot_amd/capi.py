@@ -66,6 +66,10 @@ SIGNATURES = {
     "he_ckks_decode": (C.c_int, [vp, vp, u32, u32, C.c_double, vp, vp, vp]),
     "he_ckks_workspace_words": (C.c_size_t, [vp, u32]),
     "he_sample": (C.c_int, [vp, C.c_int, C.POINTER(u32), u64, vp, u32, u32, u32, u32, vp, u32, vp]),
+    "he_ckks_encode_batch_workspace_words": (C.c_size_t, [vp, u32]),
+    "he_ckks_encode_batch": (C.c_int, [vp, vp, vp, u32, u32, C.c_double, u32, u32, C.c_size_t, vp, u32, vp, vp]),
+    "he_encrypt_batch_workspace_words": (C.c_size_t, [vp, u32, u32]),
+    "he_encrypt_batch": (C.c_int, [vp, u32, u32, vp, C.POINTER(u32), u64, vp, vp, vp]),
     "he_sample_batch": (C.c_int, [vp, C.c_int, C.POINTER(u32), u64, vp, u32, u32, u32, u32, vp, u32, u32, vp]),
     "he_decrypt_decode_batch_workspace_words": (C.c_size_t, [vp, u32, u32, u32]),
     "he_decrypt_decode_batch": (C.c_int, [vp, vp, u32, u32, vp, vp, u32, C.c_double, u32, vp, vp, vp]),

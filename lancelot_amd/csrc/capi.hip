@@ -1007,7 +1007,7 @@ int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, c
 int he_decompose_real(const he_context *ctx, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,
                       he_stream s) {
     if (!ctx || !coeffs || !out || first + limbs > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
-    HE_HIP(launch_decompose_real(ctx->tables(), coeffs, out, limbs, first, S(s)));
+    HE_HIP(launch_decompose_real(ctx->tables(), coeffs, out, limbs, first, 1, 0, S(s)));
     return HE_OK;
 }
 
@@ -1020,18 +1020,65 @@ size_t he_ckks_workspace_words(const he_context *ctx, uint32_t limbs) {
     return enc > dec ? enc : dec;
 }
 
-int he_ckks_encode(const he_context *ctx, const double *re, const double *im, uint32_t count, uint32_t slots,
-                   double scale, uint32_t limbs, uint64_t *out, uint64_t *ws, he_stream s) {
-    if (!ctx || !re || !out || !ws || limbs == 0 || limbs > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
-    if (slots < 2 || (slots & (slots - 1)) || slots > ctx->n() / 2 || count > slots || !(scale > 0))
+size_t he_ckks_encode_batch_workspace_words(const he_context *ctx, uint32_t items) {
+    if (!ctx) return 0;
+    // [items words rounded up to 8: the maxima] [items][N words: complex scratch] [items][N words: coefficients]
+    return (((size_t)items + 7) & ~(size_t)7) + 2 * (size_t)items * ctx->n();
+}
+
+int he_ckks_encode_batch(const he_context *ctx, const double *re, const double *im, uint32_t count, uint32_t slots,
+                         double scale, uint32_t limbs, uint32_t items, size_t value_stride, uint64_t *out,
+                         uint32_t out_poly_stride, uint64_t *ws, he_stream s) {
+    if (!ctx || !re || !out || !ws || limbs == 0 || limbs > ctx->size_qp || items == 0 || items > 16384 ||
+        out_poly_stride < limbs)
+        return HE_E_INVALID_ARGUMENT;
+    if (slots < 2 || (slots & (slots - 1)) || slots > ctx->n() / 2 || count > slots || !(scale > 0) ||
+        (items > 1 && value_stride < count))
         return HE_E_INVALID_ARGUMENT;
     const size_t n = ctx->n();
-    double2 *v = reinterpret_cast<double2 *>(ws + 8);
-    double *coeffs = reinterpret_cast<double *>(ws + 8 + n);
+    const size_t head = ((size_t)items + 7) & ~(size_t)7;
+    double2 *v = reinterpret_cast<double2 *>(ws + head);
+    double *coeffs = reinterpret_cast<double *>(ws + head + (size_t)items * n);
     const FftTables ft{ctx->d_rot_group, ctx->d_ksi, ctx->log_n};
-    HE_HIP(launch_ckks_encode(ft, re, im, count, slots, scale, v, coeffs, ws, S(s)));
-    HE_HIP(launch_decompose_real(ctx->tables(), coeffs, out, limbs, 0, S(s)));
-    return he_ntt_forward(ctx, out, 1, limbs, limbs, 0, limbs, 0, s);
+    // (the complex scratch of an item is `slots` values = at most N words: the items are packed `slots` apart)
+    HE_HIP(launch_ckks_encode(ft, re, im, count, slots, scale, v, coeffs, ws, items, value_stride, S(s)));
+    HE_HIP(launch_decompose_real(ctx->tables(), coeffs, out, limbs, 0, items, (size_t)out_poly_stride * n, S(s)));
+    return he_ntt_forward(ctx, out, items, out_poly_stride, limbs, 0, limbs, 0, s);
+}
+
+int he_ckks_encode(const he_context *ctx, const double *re, const double *im, uint32_t count, uint32_t slots,
+                   double scale, uint32_t limbs, uint64_t *out, uint64_t *ws, he_stream s) {
+    // one item: the maximum in ws[0], then the scratch (the layout of he_ckks_workspace_words)
+    return he_ckks_encode_batch(ctx, re, im, count, slots, scale, limbs, 1, 0, out, limbs, ws, s);
+}
+
+size_t he_encrypt_batch_workspace_words(const he_context *ctx, uint32_t L, uint32_t items) {
+    if (!ctx || L == 0 || L > ctx->size_q) return 0;
+    const size_t n = ctx->n(), LK = L + ctx->size_p;
+    // u [items][L+K][N] | wide [items][2][L+K][N] | ModDown scratch [items][2][L][N]
+    return (size_t)items * (3 * LK + 2 * L) * n;
+}
+
+int he_encrypt_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *pk, const uint32_t key[8],
+                     uint64_t stream_id, uint64_t *cts, uint64_t *ws, he_stream s) {
+    if (!ctx || !pk || !key || !cts || !ws || ctx->size_p == 0 || L == 0 || L > ctx->size_q || items == 0 || items > 8192)
+        return HE_E_INVALID_ARGUMENT;
+    const size_t n = ctx->n();
+    const uint32_t K = ctx->size_p, Q = ctx->size_q, LK = L + K;
+    uint64_t *u = ws, *wide = u + (size_t)items * LK * n, *tmp = wide + (size_t)items * 2 * LK * n;
+    ChaChaKey k;
+    memcpy(k.k, key, sizeof(k.k));
+    const LimbMap map{LK, 0, L, Q};
+    // item k draws u, e0, e1 from the stream ids stream_id + 3 k, + 1, + 2: what `items` encryptions in a row draw
+    HE_HIP(launch_sample(ctx->tables(), SAMPLE_TERNARY, k, stream_id, u, map, nullptr, 0, items, 3, (size_t)LK * n, S(s)));
+    for (uint32_t i = 0; i < 2; i++)
+        HE_HIP(launch_sample(ctx->tables(), SAMPLE_ERROR, k, stream_id + 1 + i, wide + (size_t)i * LK * n, map, nullptr, 0,
+                             items, 3, 2 * (size_t)LK * n, S(s)));
+    if (int rc = he_ntt_forward(ctx, u, items, LK, LK, 0, L, Q, s)) return rc;
+    if (int rc = he_ntt_forward(ctx, wide, 2 * items, LK, LK, 0, L, Q, s)) return rc;
+    HE_HIP(launch_encrypt_fma(ctx->tables(), u, pk, wide, L, K, Q, items, S(s)));
+    // divide by P; polynomial 0 of every ciphertext already holds the plaintext and is added onto
+    return moddown_impl(ctx, L, wide, cts, 2 * items, 0x55555555u, tmp, s);
 }
 
 int he_ckks_decode(const he_context *ctx, const uint64_t *plain, uint32_t limbs, uint32_t slots, double scale,
@@ -1081,7 +1128,7 @@ static int sample_impl(const he_context *ctx, int kind, const uint32_t key[8], u
     ChaChaKey k;
     memcpy(k.k, key, sizeof(k.k));
     HE_HIP(launch_sample(ctx->tables(), kind, k, stream_id, out, LimbMap{limbs, first, split, tail}, cdt, cdt_len, items,
-                         S(s)));
+                         1, (size_t)limbs * ctx->n(), S(s)));
     return HE_OK;
 }
 

@@ -85,8 +85,13 @@ __global__ __launch_bounds__(kThreads) void cfft_lds_kernel(double2 *v, uint32_t
 // values -> complex vector, zero padded; also clears the maximum that the rounding kernel accumulates
 __global__ __launch_bounds__(kThreads) void encode_load_kernel(const double *re, const double *im, uint32_t count,
                                                                uint32_t slots, double2 *v,
-                                                               unsigned long long *max_bits) {
+                                                               unsigned long long *max_bits, size_t value_stride) {
     const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
+    // blockIdx.y = item: its values value_stride doubles on, its vector `slots` on, its own maximum
+    re += blockIdx.y * value_stride;
+    if (im) im += blockIdx.y * value_stride;
+    v += (size_t)blockIdx.y * slots;
+    max_bits += blockIdx.y;
     if (i == 0) *max_bits = 0;
     if (i < slots) v[i] = i < count ? double2{re[i], im ? im[i] : 0.0} : double2{0.0, 0.0};
 }
@@ -97,6 +102,9 @@ __global__ __launch_bounds__(kThreads) void encode_round_kernel(const double2 *v
                                                                 uint32_t half, double fix, double *coeffs,
                                                                 unsigned long long *max_bits) {
     const uint32_t c = blockIdx.x * kThreads + threadIdx.x;
+    v += (size_t)blockIdx.y << log_slots;
+    coeffs += (size_t)blockIdx.y * 2 * half;
+    max_bits += blockIdx.y;
     const bool imag = c >= half;
     const uint32_t k = imag ? c - half : c;
     double val = 0.0;
@@ -185,12 +193,14 @@ __global__ __launch_bounds__(kThreads) void take_slots_kernel(const double2 *v, 
 }  // namespace
 
 hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double *im, uint32_t count, uint32_t slots,
-                              double scale, double2 *v, double *coeffs, uint64_t *max_bits, hipStream_t s) {
+                              double scale, double2 *v, double *coeffs, uint64_t *max_bits, uint32_t items,
+                              size_t value_stride, hipStream_t s) {
     const uint32_t n = 1u << t.log_n, log_slots = 31 - __builtin_clz(slots);
-    auto blocks = [](uint32_t items) { return dim3((items + kThreads - 1) / kThreads); };
+    if (items == 0 || items > 65535) return hipErrorInvalidValue;
+    auto blocks = [&](uint32_t work) { return dim3((work + kThreads - 1) / kThreads, items); };
     hipLaunchKernelGGL(encode_load_kernel, blocks(slots), dim3(kThreads), 0, s, re, im, count, slots, v,
-                       reinterpret_cast<unsigned long long *>(max_bits));
-    hipError_t e = run_fft<true>(v, slots, 1, t, s);
+                       reinterpret_cast<unsigned long long *>(max_bits), value_stride);
+    hipError_t e = run_fft<true>(v, slots, items, t, s);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(encode_round_kernel, blocks(n), dim3(kThreads), 0, s, v, log_slots, (n / 2) / slots, n / 2,
                        scale / (double)slots, coeffs, reinterpret_cast<unsigned long long *>(max_bits));

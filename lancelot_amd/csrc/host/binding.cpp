@@ -178,6 +178,16 @@ PYBIND11_MODULE(pyCAHEL, m) {
                  return p;
              },
              py::arg("context"), py::arg("values").noconvert(), py::arg("chain_index"), py::arg("scale"))
+        .def("encode_encrypt_many",
+             [](CAHELGPUCKKSEncoder &e, const CAHELGPUContext &c, const CAHELGPUPublicKey &pk,
+                py::array_t<double, py::array::c_style> v, double scale) {
+                 if (v.ndim() != 2) throw std::invalid_argument("values must be a two-dimensional array");
+                 const double *values = v.data();
+                 const std::size_t items = (std::size_t)v.shape(0), count = (std::size_t)v.shape(1);
+                 py::gil_scoped_release release;
+                 return e.encode_encrypt_many(c, pk, values, items, count, count, scale);
+             },
+             py::arg("context"), py::arg("public_key"), py::arg("values").noconvert(), py::arg("scale"))
         .def("decode_array",
              [](CAHELGPUCKKSEncoder &e, const CAHELGPUContext &c, const CAHELGPUPlaintext &p, std::size_t count) {
                  std::vector<double> out;

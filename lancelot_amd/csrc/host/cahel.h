@@ -315,6 +315,15 @@ public:
     std::size_t slot_count() const { return slots_; }
     void reset_sparse_slots() { sparse_slots_ = 0; }
     std::size_t first_chain_index() const { return first_chain_index_; }
+    // slot count of a message of `count` values: the first message fixes it for the lifetime of the encoder
+    // (src/ckks.cu:131-142)
+    std::size_t message_slots(std::size_t count);
+    // Encode and encrypt `items` real vectors (row k at values + k * value_stride, `count` values each) at the
+    // encoder's first chain index with one launch per stage; the ciphertexts equal those of encode +
+    // encrypt_asymmetric called item by item (same randomness).  Not in the reference.
+    std::vector<CAHELGPUCiphertext> encode_encrypt_many(const CAHELGPUContext &context, const CAHELGPUPublicKey &pk,
+                                                        const double *values, std::size_t items, std::size_t count,
+                                                        std::size_t value_stride, double scale);
     void encode(const CAHELGPUContext &context, const std::vector<double> &values, std::size_t chain_index, double scale,
                 CAHELGPUPlaintext &destination);
     void encode(const CAHELGPUContext &context, const std::vector<double> &values, double scale,

@@ -18,14 +18,7 @@ CAHELGPUCKKSEncoder::CAHELGPUCKKSEncoder(const CAHELGPUContext &context) {
     first_chain_index_ = context.get_first_index();
 }
 
-void CAHELGPUCKKSEncoder::encode_complex(const CAHELGPUContext &context, const double *re, const double *im,
-                                         std::size_t count, std::size_t chain_index, double scale,
-                                         CAHELGPUPlaintext &destination) {
-    const std::size_t n = context.poly_degree();
-    if (count > slots_) throw std::invalid_argument("values_size is too large");
-    const int total_bits = context.total_coeff_modulus_bit_count(chain_index);
-    if (scale <= 0 || (static_cast<int>(std::log2(scale)) + 1 >= total_bits))
-        throw std::invalid_argument("scale out of bounds");
+std::size_t CAHELGPUCKKSEncoder::message_slots(std::size_t count) {
     if (sparse_slots_ == 0) {
         // the first message fixes the slot count for the lifetime of the encoder (src/ckks.cu:131-142)
         std::size_t s = 1;
@@ -35,7 +28,82 @@ void CAHELGPUCKKSEncoder::encode_complex(const CAHELGPUContext &context, const d
         throw std::invalid_argument("values_size exceeds previous message length");
     }
     if (sparse_slots_ < 2) throw std::invalid_argument("single value encoding is not available");
-    const std::size_t ss = sparse_slots_;
+    return sparse_slots_;
+}
+
+std::vector<CAHELGPUCiphertext> CAHELGPUCKKSEncoder::encode_encrypt_many(const CAHELGPUContext &context,
+                                                                         const CAHELGPUPublicKey &pk, const double *values,
+                                                                         std::size_t items, std::size_t count,
+                                                                         std::size_t value_stride, double scale) {
+    if (items == 0) return {};
+    if (items > 8192) throw std::invalid_argument("too many messages");
+    if (!pk.gen_flag_) throw std::logic_error("public key has not been generated");
+    if (count > slots_ || value_stride < count) throw std::invalid_argument("values_size is too large");
+    const std::size_t chain = first_chain_index_;
+    if (chain == 0 || context.size_p() == 0) throw std::logic_error("batched encryption needs a data level and special primes");
+    const int total_bits = context.total_coeff_modulus_bit_count(chain);
+    if (scale <= 0 || (static_cast<int>(std::log2(scale)) + 1 >= total_bits))
+        throw std::invalid_argument("scale out of bounds");
+    const std::size_t ss = message_slots(count);
+    const std::size_t n = context.poly_degree();
+    const uint32_t L = (uint32_t)context.limbs_at(chain);
+    he_context *h = context.handle();
+    he_stream st = context.stream();
+
+    // values -> device, packed
+    DeviceBuffer staging(items * count);
+    double *d_values = reinterpret_cast<double *>(staging.get());
+    if (count) {
+        if (value_stride == count) {
+            check_status(he_memcpy_h2d(d_values, values, items * count * sizeof(double), st), "upload");
+        } else {
+            for (std::size_t k = 0; k < items; k++)
+                check_status(he_memcpy_h2d(d_values + k * count, values + k * value_stride, count * sizeof(double), st), "upload");
+        }
+    }
+    // plaintexts straight into polynomial 0 of the ciphertexts
+    const std::size_t words = 2 * (std::size_t)L * n;
+    DeviceBuffer batch(items * words), ws(he_ckks_encode_batch_workspace_words(h, (uint32_t)items));
+    check_status(he_ckks_encode_batch(h, d_values, nullptr, (uint32_t)count, (uint32_t)ss, scale, L, (uint32_t)items, count,
+                                      batch.get(), 2 * L, ws.get(), st),
+                 "he_ckks_encode_batch");
+    std::vector<double> maxima(items);
+    check_status(he_memcpy_d2h(maxima.data(), ws.get(), items * sizeof(double), st), "download");
+    for (double max_coeff : maxima) {
+        const int max_coeff_bit_count = static_cast<int>(std::ceil(std::log2(std::max(max_coeff, 1.0)))) + 1;
+        if (max_coeff_bit_count >= total_bits || max_coeff_bit_count > 63)
+            throw std::invalid_argument("encoded values are too large");
+    }
+    DeviceBuffer ews(he_encrypt_batch_workspace_words(h, L, (uint32_t)items));
+    check_status(he_encrypt_batch(h, L, (uint32_t)items, pk.pk_.data(), context.prng_key(), context.next_stream(3 * items),
+                                  batch.get(), ews.get(), st),
+                 "he_encrypt_batch");
+    std::vector<CAHELGPUCiphertext> out(items);
+    for (std::size_t k = 0; k < items; k++) {
+        CAHELGPUCiphertext &ct = out[k];
+        ct.data_.allocate(words);
+        check_status(he_memcpy_d2d(ct.data(), batch.get() + k * words, words * sizeof(uint64_t), st), "copy");
+        ct.size_ = 2;
+        ct.coeff_modulus_size_ = L;
+        ct.poly_modulus_degree_ = n;
+        ct.chain_index_ = chain;
+        ct.parms_id_ = context.parms_id_at(chain);
+        ct.scale_ = scale;
+        ct.is_ntt_form_ = true;
+        ct.is_asymmetric_ = true;
+    }
+    return out;
+}
+
+void CAHELGPUCKKSEncoder::encode_complex(const CAHELGPUContext &context, const double *re, const double *im,
+                                         std::size_t count, std::size_t chain_index, double scale,
+                                         CAHELGPUPlaintext &destination) {
+    const std::size_t n = context.poly_degree();
+    if (count > slots_) throw std::invalid_argument("values_size is too large");
+    const int total_bits = context.total_coeff_modulus_bit_count(chain_index);
+    if (scale <= 0 || (static_cast<int>(std::log2(scale)) + 1 >= total_bits))
+        throw std::invalid_argument("scale out of bounds");
+    const std::size_t ss = message_slots(count);
     const uint32_t limbs = (uint32_t)context.limbs_at(chain_index);
     destination.resize(limbs, n);
     he_context *h = context.handle();

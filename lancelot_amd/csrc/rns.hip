@@ -60,15 +60,34 @@ __global__ __launch_bounds__(kThreads) void scalar_mul_add_kernel(const uint64_t
 }
 
 // grid: (N / 256, limbs): residue of a rounded real coefficient
+// blockIdx.z = item: coefficient vectors N apart, outputs out_item_stride words apart
 __global__ __launch_bounds__(kThreads) void decompose_real_kernel(const double *coeffs, uint64_t *out,
                                                                   const uint64_t *moduli, const uint64_t *barrett,
-                                                                  uint32_t first, uint32_t log_n) {
+                                                                  uint32_t first, uint32_t log_n, size_t out_item_stride) {
     const uint32_t table = first + blockIdx.y;
     const uint64_t q = moduli[table];
     const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
-    const double c = coeffs[i];
+    const double c = coeffs[((size_t)blockIdx.z << log_n) + i];
     const uint64_t r = barrett64((uint64_t)fabs(c), q, barrett[2 * table + 1]);
-    out[((size_t)blockIdx.y << log_n) + i] = c < 0 ? neg_mod(r, q) : r;
+    out[blockIdx.z * out_item_stride + ((size_t)blockIdx.y << log_n) + i] = c < 0 ? neg_mod(r, q) : r;
+}
+
+// grid: (N / 256, L + K, items).  wide[item][i][t] += u[item][t] * pk[i][table(t)] for both polynomials of the public
+// key: the products of an encryption over Ql u P
+__global__ __launch_bounds__(kThreads) void encrypt_fma_kernel(const uint64_t *u, const uint64_t *pk, uint64_t *wide,
+                                                               const uint64_t *moduli, const uint64_t *barrett,
+                                                               uint32_t L, uint32_t K, uint32_t size_q, uint32_t log_n) {
+    const uint32_t t = blockIdx.y, LK = L + K;
+    const uint32_t table = t < L ? t : size_q + (t - L);
+    const uint64_t q = moduli[table], r0 = barrett[2 * table], r1 = barrett[2 * table + 1];
+    const uint32_t j = blockIdx.x * kThreads + threadIdx.x;
+    const uint64_t uv = u[(((size_t)blockIdx.z * LK + t) << log_n) + j];
+    const size_t key_poly = (size_t)(size_q + K) << log_n;
+    const uint64_t *k = pk + ((size_t)table << log_n) + j;
+    uint64_t *w = wide + (((size_t)blockIdx.z * 2 * LK + t) << log_n) + j;
+    const size_t wpoly = (size_t)LK << log_n;
+    w[0] = add_mod(w[0], mul_mod(uv, k[0], q, r0, r1), q);
+    w[wpoly] = add_mod(w[wpoly], mul_mod(uv, k[key_poly], q, r0, r1), q);
 }
 
 struct TensorArgs {
@@ -460,6 +479,8 @@ struct SampleArgs {
     LimbMap map;
     uint32_t log_n, cdt_len;
     int kind;
+    uint32_t stream_stride;
+    size_t out_item_stride;
 };
 
 // ternary / error / gauss: one thread = one ChaCha block = 16 (ternary) or 8 coefficients, the same
@@ -467,9 +488,9 @@ struct SampleArgs {
 __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
     const uint32_t n = 1u << p.log_n;
     const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
-    // blockIdx.y = item: the next stream id, the next polynomial
-    const uint64_t stream = p.stream + blockIdx.y;
-    uint64_t *out = p.out + (((size_t)blockIdx.y * p.map.limbs) << p.log_n);
+    // blockIdx.y = item: its own stream id, its own polynomial
+    const uint64_t stream = p.stream + (uint64_t)blockIdx.y * p.stream_stride;
+    uint64_t *out = p.out + blockIdx.y * p.out_item_stride;
     uint32_t w[16];
     if (p.kind == SAMPLE_UNIFORM) {
         const uint32_t per_limb = n / 4;
@@ -528,10 +549,19 @@ hipError_t launch_scalar_mul_add(const Tables &t, const uint64_t *a, const uint6
 }
 
 hipError_t launch_decompose_real(const Tables &t, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,
-                                 hipStream_t s) {
-    if (limbs == 0) return hipSuccess;
-    hipLaunchKernelGGL(decompose_real_kernel, dim3((1u << t.log_n) / kThreads, limbs), dim3(kThreads), 0, s, coeffs, out,
-                       t.moduli, t.barrett, first, t.log_n);
+                                 uint32_t items, size_t out_item_stride, hipStream_t s) {
+    if (limbs == 0 || items == 0) return hipSuccess;
+    if (items > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(decompose_real_kernel, dim3((1u << t.log_n) / kThreads, limbs, items), dim3(kThreads), 0, s, coeffs,
+                       out, t.moduli, t.barrett, first, t.log_n, out_item_stride);
+    return hipGetLastError();
+}
+
+hipError_t launch_encrypt_fma(const Tables &t, const uint64_t *u, const uint64_t *pk, uint64_t *wide, uint32_t L,
+                              uint32_t K, uint32_t size_q, uint32_t items, hipStream_t s) {
+    if (items == 0 || items > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(encrypt_fma_kernel, dim3((1u << t.log_n) / kThreads, L + K, items), dim3(kThreads), 0, s, u, pk, wide,
+                       t.moduli, t.barrett, L, K, size_q, t.log_n);
     return hipGetLastError();
 }
 
@@ -655,11 +685,12 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
 }
 
 hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
-                         const uint64_t *cdt, uint32_t cdt_len, uint32_t items, hipStream_t s) {
+                         const uint64_t *cdt, uint32_t cdt_len, uint32_t items, uint32_t stream_stride,
+                         size_t out_item_stride, hipStream_t s) {
     if (items == 0 || items > 65535) return hipErrorInvalidValue;
     const uint32_t n = 1u << t.log_n;
     uint32_t blocks = kind == SAMPLE_UNIFORM ? (n / 4) * map.limbs : (kind == SAMPLE_TERNARY ? n / 16 : n / 8);
-    SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind};
+    SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind, stream_stride, out_item_stride};
     hipLaunchKernelGGL(sample_kernel, dim3((blocks + kThreads - 1) / kThreads, items), dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }

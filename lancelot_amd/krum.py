@@ -103,13 +103,16 @@ def rotate_sum_plan(log_slots: int, config: KrumConfig):
 
 
 def split_updates(vectors, slots: int):
-    """Zero-pad every flattened update to a multiple of `slots` and split it (byzantine_fl.py:474-490)."""
-    vectors = [np.asarray(v, dtype=np.float64).reshape(-1) for v in vectors]
-    length = len(vectors[0])
-    if any(len(v) != length for v in vectors):
+    """Zero-pad every flattened update to a multiple of `slots` and split it (byzantine_fl.py:474-490): one float64
+    matrix [client][padded length], the chunks are views of its rows."""
+    length = int(np.asarray(vectors[0]).size)
+    if any(int(np.asarray(v).size) != length for v in vectors):
         raise ValueError("all client updates must have the same length")
     whole = length if length % slots == 0 else (length // slots + 1) * slots
-    return [np.array_split(np.pad(v, (0, whole - length)), whole // slots) for v in vectors]
+    padded = np.zeros((len(vectors), whole), dtype=np.float64)
+    for row, v in zip(padded, vectors):
+        row[:length] = np.asarray(v).reshape(-1)
+    return [[row[k:k + slots] for k in range(0, whole, slots)] for row in padded]
 
 
 def encrypt_updates(state: KrumState, chunks):
@@ -131,6 +134,21 @@ def encrypt_updates(state: KrumState, chunks):
 
     t0 = time.perf_counter()
     flat = [chunk for client in chunks for chunk in client]
+    if state.config.batched:
+        # all chunks through encode and encrypt together, one launch per stage; the chunks of split_updates are the
+        # rows of one matrix already
+        base = flat[0].base
+        if base is not None and base.ndim == 2 and base.size == len(flat) * state.slots and base.flags.c_contiguous \
+                and all(c.base is base for c in flat):
+            matrix = base.reshape(len(flat), state.slots)
+        else:
+            matrix = np.ascontiguousarray(np.stack([np.asarray(c, dtype=np.float64) for c in flat]))
+        cts = state.encoder.encode_encrypt_many(ctx, state.pk, matrix, state.config.scale)
+        _sync(state.cahel)
+        wall = time.perf_counter() - t0
+        state.timings["encode"] += wall        # encode and encrypt are one pipeline here
+        it = iter(cts)
+        return [[next(it) for _ in client] for client in chunks]
     if state.config.reproducible:
         cts = [one(item) for item in flat]      # the encryption randomness is drawn in a fixed order
     else:

@@ -388,6 +388,33 @@ def test_batched_pair_distances_equal_the_pairwise_ciphertexts(oracle):
         c.pair_square_distances(state.context, cts, pairs, state.rlk, state.glk, [[9]], 0.0)
 
 
+def test_encode_encrypt_many_equals_one_by_one(oracle):
+    """ckks_encoder.encode_encrypt_many against encode + encrypt_asymmetric item by item on a context with the same
+    seed: the same ciphertexts (item k draws the stream ids that the k-th single encryption draws)."""
+    from lancelot_amd import krum
+    rng = np.random.default_rng(22)
+    updates = [rng.normal(0, 0.01, 9000).astype(np.float32) for _ in range(3)]     # 3 chunks of 4096 slots, the last ragged
+    base = dict(log_n=13, modulus_bits=(60, 40, 40, 60), special_modulus_size=1, seed=14)
+    many = krum.gpu_init(krum.KrumConfig(batched=True, **base))
+    single = krum.gpu_init(krum.KrumConfig(batched=False, reproducible=True, **base))
+    cts_many = krum.encrypt_updates(many, krum.split_updates(updates, many.slots))
+    cts_single = krum.encrypt_updates(single, krum.split_updates(updates, single.slots))
+    assert len(cts_many) == 3 and len(cts_many[0]) == 3
+    for a_row, b_row in zip(cts_many, cts_single):
+        for a, b in zip(a_row, b_row):
+            assert a.chain_index() == b.chain_index() and a.scale() == b.scale()
+            assert (a.to_numpy() == b.to_numpy()).all()
+    # a matrix that is not the one of split_updates, and the argument checks
+    c, ctx = many.cahel, many.context
+    cts = many.encoder.encode_encrypt_many(ctx, many.pk, np.ones((2, 100)), 2.0 ** 40)
+    got = many.sk.decrypt_decode_many(ctx, cts, many.slots, 101)
+    assert np.max(np.abs(got[:, :100] - 1.0)) < 1e-6 and np.max(np.abs(got[:, 100])) < 1e-6
+    with pytest.raises(ValueError, match="two-dimensional"):
+        many.encoder.encode_encrypt_many(ctx, many.pk, np.ones(8), 2.0 ** 40)
+    with pytest.raises(ValueError, match="too large"):
+        many.encoder.encode_encrypt_many(ctx, many.pk, np.full((1, 8), 1e30), 2.0 ** 40)
+
+
 def test_decrypt_decode_many_equals_one_by_one(world):
     """secret_key.decrypt_decode_many against decrypt + decode_array per ciphertext: identical without the flooding
     noise, within its size with it (the batch draws the stream ids that the single calls would)."""
