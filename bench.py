@@ -292,6 +292,15 @@ def main():
     ntt = {"forward_ms": f, "inverse_ms": i, "bytes_fwd_plus_inv": 4 * 2 * L * limb_bytes,
            "GBps": 4 * 2 * L * limb_bytes / ((f + i) * 1e-3) / 1e9}
     ntt["frac_of_hbm_peak"] = ntt["GBps"] / HBM_PEAK_GBS
+    # the same kernels over 6 ciphertexts in one call (288 limbs): a launch that spans several rounds of resident
+    # workgroups overlaps the load, butterfly and store phases that a single round runs one after the other
+    six = Buf(capi, 12 * L * n)
+    capi.check(lib.he_memset_zero(six.ptr, 8 * 12 * L * n, None))
+    f6 = timer.time(lambda: capi.check(lib.he_ntt_forward(h, six.ptr, 12, L, L, 0, L, 0, None)), 30)
+    i6 = timer.time(lambda: capi.check(lib.he_ntt_inverse(h, six.ptr, 12, L, L, 0, L, 0, None)), 30)
+    ntt["six_ciphertexts_per_call"] = {"forward_ms": f6, "inverse_ms": i6,
+                                       "GBps": 4 * 12 * L * limb_bytes / ((f6 + i6) * 1e-3) / 1e9}
+    ntt["six_ciphertexts_per_call"]["frac_of_hbm_peak"] = ntt["six_ciphertexts_per_call"]["GBps"] / HBM_PEAK_GBS
 
     # rotations (config "rotate-and-sum"): one keyed rotation; 15 dependent rotations + adds; hoisted form
     rot_in = ct1.copy()

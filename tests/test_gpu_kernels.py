@@ -235,7 +235,9 @@ def test_hoisted_rotations_entry_point(oracle, capi, logn, bits, size_p, L, n_st
 
 @pytest.mark.parametrize("logn,bits,size_p,L,items", [(11, [45, 40, 40, 50], 1, 3, 5), (11, [60, 40, 40, 60], 1, 2, 3),
                                                        (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5, 2),
-                                                       (11, [50, 50, 49, 50, 50, 50], 2, 4, 3)])
+                                                       (11, [50, 50, 49, 50, 50, 50], 2, 4, 3),
+                                                       (13, [50, 50, 49, 50, 50, 50], 2, 4, 3),
+                                                       (13, [50, 50, 49, 50, 50, 50], 2, 3, 2)])
 def test_batched_entry_points_equal_separate_calls(oracle, capi, logn, bits, size_p, L, items):
     """he_keyswitch_rescale_batch, he_hoisted_rotations_batch and he_pair_square_sum over several inputs against
     one call per input (which the other tests pin to the oracle), on both arithmetic back ends."""
