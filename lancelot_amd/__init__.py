@@ -27,5 +27,14 @@ def _load():
     return mod
 
 
-pyCAHEL = _load()
-from . import capi  # noqa: E402,F401
+def _building() -> bool:
+    """True while the package is imported only to reach its build module (`python -m lancelot_amd.build`, or a
+    caller that set LANCELOT_AMD_BUILD=1 around the import): the native module cannot exist yet."""
+    argv = list(getattr(sys, "orig_argv", []))
+    return os.environ.get("LANCELOT_AMD_BUILD") == "1" or any(
+        a == "-m" and b == __name__ + ".build" for a, b in zip(argv, argv[1:]))
+
+
+if not _building():
+    pyCAHEL = _load()
+    from . import capi  # noqa: E402,F401

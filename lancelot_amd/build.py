@@ -75,4 +75,7 @@ def build_all(verbose: bool = False):
 
 
 if __name__ == "__main__":
-    build_all(verbose=True)
+    if "--help" in sys.argv[1:] or "-h" in sys.argv[1:]:
+        print(__doc__)
+    else:
+        build_all(verbose=True)

@@ -139,3 +139,26 @@ def test_rotate_sum_plan_adds_every_slot_once(log_slots):
             cover = cover + sum(np.roll(cover, s) for s in steps)
         assert (cover == 1).all(), (log_slots, cfg)
     assert krum.rotate_sum_plan(15, krum.KrumConfig(hoisting_radix=0))[0] == list(range(1, 16))   # the reference's split
+
+
+def test_package_without_native_module_only_imports_for_the_build(tmp_path):
+    """A tree that has not been built yet: `import lancelot_amd` must fail loudly, but the build module must still
+    be reachable (python -m lancelot_amd.build, and the LANCELOT_AMD_BUILD=1 import that build() does)."""
+    import shutil
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    pkg = tmp_path / "lancelot_amd"
+    pkg.mkdir()
+    for name in ("__init__.py", "build.py", "capi.py", "krum.py"):
+        shutil.copy(os.path.join(root, "lancelot_amd", name), pkg / name)
+    env = dict(os.environ, PYTHONPATH=str(tmp_path))
+    run = lambda code, **extra: subprocess.run([sys.executable, "-c", code], cwd=tmp_path, env=dict(env, **extra),
+                                               capture_output=True, text=True)
+    plain = run("import lancelot_amd")
+    assert plain.returncode != 0 and "native module is missing" in plain.stderr
+    building = run("from lancelot_amd import build; print(build.LIB)", LANCELOT_AMD_BUILD="1")
+    assert building.returncode == 0 and "libcahel_hip.so" in building.stdout
+    as_module = subprocess.run([sys.executable, "-m", "lancelot_amd.build", "--help"], cwd=tmp_path, env=env,
+                               capture_output=True, text=True)
+    assert as_module.returncode == 0 and "libcahel_hip.so" in as_module.stdout
