@@ -10,6 +10,11 @@ Per pair (i, j): for every chunk  d = ct_j - ct_i ; d = d^2 (size 3) ; acc += d 
 then one relinearise + rescale, then rotate-and-sum so that every slot holds sum_k (u_i[k] - u_j[k])^2.
 The score of a client is the plain row sum of its distances (no nearest-neighbour truncation), as in
 byzantine_fl.py:344-353 and :531-533; the chosen client is the argmin.
+
+Two ways through the same arithmetic (KrumConfig.batched): all chunks / pairs / results through every stage together,
+one launch per stage (encode_encrypt_many, pair_square_distances, decrypt_decode_many: three- and four-limb
+ciphertexts are too small to fill the GPU one at a time), or call by call as the reference does, spread over the
+lanes of the host layer.
 """
 from __future__ import annotations
 
@@ -116,11 +121,13 @@ def split_updates(vectors, slots: int):
 
 
 def encrypt_updates(state: KrumState, chunks):
-    """One ciphertext per (client, chunk); the chunks are independent and go over the lanes (unless the run is to
-    be reproducible).  The first one is encoded on the calling thread because the first message fixes the encoder's slot
-    count."""
+    """One ciphertext per (client, chunk).  Batched: all chunks through encode and encrypt together.  Otherwise the
+    chunks go over the lanes (unless the run is to be reproducible); the first one is then encoded on the calling
+    thread because the first message fixes the encoder's slot count."""
+    import threading
     ctx = state.context
     spent = {"encode": 0.0, "encrypt": 0.0}
+    spent_lock = threading.Lock()
 
     def one(item):
         t0 = time.perf_counter()
@@ -128,8 +135,9 @@ def encrypt_updates(state: KrumState, chunks):
         t1 = time.perf_counter()
         ct = state.pk.encrypt_asymmetric(ctx, pt)
         t2 = time.perf_counter()
-        spent["encode"] += t1 - t0          # summed over the threads; scaled to the wall time below
-        spent["encrypt"] += t2 - t1
+        with spent_lock:                    # summed over the threads; scaled to the wall time below
+            spent["encode"] += t1 - t0
+            spent["encrypt"] += t2 - t1
         return ct
 
     t0 = time.perf_counter()
