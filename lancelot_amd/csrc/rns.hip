@@ -259,13 +259,19 @@ __global__ __launch_bounds__(kThreads) void bconv_batched_kernel(BconvBatchK p) 
     const uint64_t *mat = p.b.mat_base + d.mat_off;
     for (uint32_t row = row0; row < row0 + p.rows_per && row < d.n_out; row++) {
         const uint64_t *m = mat + (size_t)row * d.n_in;
-        U128 acc{0, 0};
-#pragma unroll
-        for (int i = 0; i < kBatchIn; i++)
-            if ((uint32_t)i < d.n_in) mac128(acc, xv[i], m[i]);
         const uint32_t t = p.b.out_table[d.map_off + row];
-        out[((size_t)p.b.out_limb[d.map_off + row] << p.log_n) + j] =
-            barrett128(acc.lo, acc.hi, p.moduli[t], p.barrett[2 * t], p.barrett[2 * t + 1]);
+        uint64_t r;
+        if (d.n_in == 1 && m[0] == 1) {
+            // a digit of one limb (one special prime): Q_d / q_i = 1, the conversion is a plain reduction
+            r = barrett64(xv[0], p.moduli[t], p.barrett[2 * t + 1]);
+        } else {
+            U128 acc{0, 0};
+#pragma unroll
+            for (int i = 0; i < kBatchIn; i++)
+                if ((uint32_t)i < d.n_in) mac128(acc, xv[i], m[i]);
+            r = barrett128(acc.lo, acc.hi, p.moduli[t], p.barrett[2 * t], p.barrett[2 * t + 1]);
+        }
+        out[((size_t)p.b.out_limb[d.map_off + row] << p.log_n) + j] = r;
     }
 }
 

@@ -306,6 +306,56 @@ def test_batched_entry_points_equal_separate_calls(oracle, capi, logn, bits, siz
     assert lib.he_pair_square_sum(h, L, 0, chunks, dtab.ptr, sq01.ptr, sq2.ptr, None) == -1
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_random_parameter_sets(oracle, capi, seed):
+    """Seeded random shapes: degree, number and size of the primes (which decides the arithmetic back end per
+    launch), special primes, digits, level, Galois elements.  Key switch, key switch + rescale, rotation and
+    hoisted rotations against the oracle, limb for limb."""
+    rng = np.random.default_rng(1000 + seed)
+    logn = int(rng.integers(9, 14))
+    size_p = int(rng.integers(1, 4))
+    dnum = int(rng.integers(1, 5))
+    size_q = size_p * dnum
+    style = int(rng.integers(0, 3))          # all below 2^50, all above, mixed
+    lo, hi = ((30, 50), (51, 60), (30, 60))[style]
+    bits = [int(b) for b in rng.integers(lo, hi + 1, size_q + size_p)]
+    for b in set(bits):                      # at most four primes per bit size keeps the prime search short
+        while bits.count(b) > 4:
+            bits[bits.index(b)] = b - 1 if b > 31 else b + 1
+    L = int(rng.integers(1, size_q + 1))
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    lib, h = capi.lib(), ctx.he_handle()
+    beta = -(-L // size_p)
+    keys = [_evk(p, rng, capi) for _ in range(2)]
+    ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    elt = int(2 * rng.integers(0, p.n) + 1)
+    tag = (logn, bits, size_p, L, elt)
+
+    c, ct = rand_limbs(p, rng, range(L)), rand_limbs(p, rng, range(L), n_polys=2)
+    dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
+    capi.check(lib.he_keyswitch(h, L, dc.ptr, keys[0][2], dct.ptr, elt, ws.ptr, None))
+    ks = p.key_switch(p.galois_ntt(c, elt), keys[0][0])
+    summed = np.stack([p.add(ct[b], ks[b]) for b in range(2)])
+    assert (dct.numpy() == summed).all(), tag
+
+    if L >= 2:
+        dct = DeviceArray(capi, host=ct)
+        dout = DeviceArray(capi, shape=(2, L - 1, p.n))
+        capi.check(lib.he_keyswitch_rescale(h, L, dc.ptr, keys[0][2], dct.ptr, dout.ptr, elt, ws.ptr, None))
+        assert (dout.numpy() == p.rescale(summed)).all(), tag
+
+    dout = DeviceArray(capi, shape=(2, L, p.n))
+    dct = DeviceArray(capi, host=ct)
+    capi.check(lib.he_rotate(h, L, dct.ptr, keys[1][2], dout.ptr, elt, ws.ptr, None))
+    ks = p.key_switch(p.galois_ntt(ct[1], elt), keys[1][0])
+    assert (dout.numpy() == np.stack([p.add(p.galois_ntt(ct[0], elt), ks[0]), ks[1]])).all(), tag
+
+    elts = [elt, int(2 * rng.integers(0, p.n) + 1), 2 * p.n - 1]
+    flat = capi.evk_array([keys[i % 2][1][d].ptr for i in range(3) for d in range(beta)])
+    capi.check(lib.he_hoisted_rotations(h, L, dct.ptr, flat, (C.c_uint32 * 3)(*elts), 3, dout.ptr, ws.ptr, None))
+    assert (dout.numpy() == p.hoisting(ct, elts, [keys[i % 2][0] for i in range(3)])).all(), tag
+
+
 def test_ntt_rejects_bad_arguments(small, capi):
     cahel, parms, ctx, p = small
     d = DeviceArray(capi, shape=(1, p.n))
