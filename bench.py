@@ -107,7 +107,7 @@ def cpu_baseline(seconds_budget=12.0):
             "ms_per_op": dt * 1e3}
 
 
-def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60)):
+def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60), sum_drop_levels=0):
     """One encrypted Krum round at its real shape (10 clients x 62,006 parameters, N = 2^16, moduli
     [60, 40, 40, 60], one special prime): seconds per phase and the error against the float64 closed form."""
     from lancelot_amd import krum
@@ -116,7 +116,7 @@ def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60)):
     for k in (8, 9):
         updates[k] = updates[k] * 10
     t0 = time.perf_counter()
-    state = krum.gpu_init(krum.KrumConfig(seed=seed, modulus_bits=tuple(modulus_bits)))
+    state = krum.gpu_init(krum.KrumConfig(seed=seed, modulus_bits=tuple(modulus_bits), sum_drop_levels=sum_drop_levels))
     setup = time.perf_counter() - t0
     krum.gpu_krum_aggregate(updates, state=state)  # warm-up round (pool growth, first-touch of the keys)
     # the fastest of three rounds each (a round is about 12 ms of host-driven work: one scheduling hiccup of the host
@@ -350,10 +350,15 @@ def main():
     }
     if not args.no_krum:
         line["krum"] = krum_round()
-        # the same round on primes below 2^50 (exact FP64 butterflies instead of 64-bit integer ones); Lancelot's own
-        # chain is the one above
-        fp = krum_round(modulus_bits=(50, 40, 40, 50))
-        line["krum_50bit_chain"] = {k: fp[k] for k in ("workload", "round_s", "chosen", "max_rel_err_vs_float64")}
+        # The same round with two settings that Lancelot's driver does not use (its own are the ones above): primes
+        # below 2^50 (exact FP64 butterflies instead of 64-bit integer ones), and the slot sum one level further down
+        # (mod_switch_to_next after the rescale: its key switches run over one limb instead of two).
+        keep = ("round_s", "chosen", "max_rel_err_vs_float64")
+        variants = {"primes_of_50_40_40_50_bits": dict(modulus_bits=(50, 40, 40, 50)),
+                    "slot_sum_one_level_down": dict(sum_drop_levels=1),
+                    "both": dict(modulus_bits=(50, 40, 40, 50), sum_drop_levels=1)}
+        line["krum_variants"] = {name: {k: v for k, v in krum_round(**kw).items() if k in keep}
+                                 for name, kw in variants.items()}
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline()
     print(json.dumps(line))

@@ -48,6 +48,11 @@ int he_free(void *dev_ptr);
 int he_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, he_stream stream);
 int he_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, he_stream stream);
 int he_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes, he_stream stream);
+/* `rows` runs of `width` bytes, the runs src_pitch bytes apart in the source and dst_pitch bytes apart in the
+ * destination (the leading limbs of every polynomial of a batch: a modulus switch that drops limbs without scaling,
+ * mod_switch_drop_to_next, src/evaluate.cu:2253-2305, for many polynomials at once). */
+int he_memcpy2d_d2d(void *dst_dev, size_t dst_pitch, const void *src_dev, size_t src_pitch, size_t width, size_t rows,
+                    he_stream stream);
 int he_memset_zero(void *dst_dev, size_t bytes, he_stream stream);
 int he_stream_create(he_stream *stream);
 int he_stream_destroy(he_stream stream);

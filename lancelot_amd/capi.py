@@ -24,6 +24,7 @@ SIGNATURES = {
     "he_memcpy_h2d": (C.c_int, [vp, vp, C.c_size_t, vp]),
     "he_memcpy_d2h": (C.c_int, [vp, vp, C.c_size_t, vp]),
     "he_memcpy_d2d": (C.c_int, [vp, vp, C.c_size_t, vp]),
+    "he_memcpy2d_d2d": (C.c_int, [vp, C.c_size_t, vp, C.c_size_t, C.c_size_t, C.c_size_t, vp]),
     "he_memset_zero": (C.c_int, [vp, C.c_size_t, vp]),
     "he_stream_create": (C.c_int, [C.POINTER(vp)]),
     "he_stream_destroy": (C.c_int, [vp]),

@@ -191,6 +191,14 @@ int he_memcpy_d2d(void *dst, const void *src, size_t bytes, he_stream s) {
     return HE_OK;
 }
 
+int he_memcpy2d_d2d(void *dst, size_t dst_pitch, const void *src, size_t src_pitch, size_t width, size_t rows,
+                    he_stream s) {
+    if (width == 0 || rows == 0) return HE_OK;
+    if (!dst || !src || dst_pitch < width || src_pitch < width) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(hipMemcpy2DAsync(dst, dst_pitch, src, src_pitch, width, rows, hipMemcpyDeviceToDevice, S(s)));
+    return HE_OK;
+}
+
 int he_memset_zero(void *dst, size_t bytes, he_stream s) {
     if (bytes == 0) return HE_OK;
     HE_HIP(hipMemsetAsync(dst, 0, bytes, S(s)));

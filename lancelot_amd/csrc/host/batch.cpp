@@ -14,10 +14,12 @@ using cahel::DeviceBuffer;
 // then for every round acc += sum over the round's steps of rot(acc, step) (hoisted), as
 // GPU_compute_pair_distance does per pair (lancelot-main-GPU/utils/byzantine_fl.py:173-321) -- here with one
 // launch per stage for all pairs.  scale > 0 overrides the scale after the rescale (the reference's set_scale).
+// drop_levels > 0 switches the rescaled ciphertexts down by that many further limbs without scaling
+// (mod_switch_to_next) before the slot sum, whose key switches then run over fewer limbs.
 std::vector<CAHELGPUCiphertext> pair_square_distances(
     const CAHELGPUContext &context, const std::vector<std::vector<const CAHELGPUCiphertext *>> &clients,
     const std::vector<std::pair<std::size_t, std::size_t>> &pairs, const CAHELGPURelinKey &rlk,
-    const CAHELGPUGaloisKey &glk, const std::vector<std::vector<int>> &rounds, double scale) {
+    const CAHELGPUGaloisKey &glk, const std::vector<std::vector<int>> &rounds, double scale, std::size_t drop_levels) {
     if (context.scheme() != cahel::scheme_type::ckks) throw std::logic_error("unsupported scheme");
     if (clients.empty() || clients[0].empty()) throw std::invalid_argument("no ciphertexts");
     if (pairs.empty()) return {};
@@ -66,12 +68,27 @@ std::vector<CAHELGPUCiphertext> pair_square_distances(
     auto rl = rlk.key_ptrs();
     if (rl.size() < (L + K - 1) / K) throw std::invalid_argument("key_poly_num != 2");
     DeviceBuffer ws(he_keyswitch_batch_workspace_words(h, L, items));
-    const uint32_t L1 = L - 1;
-    DeviceBuffer acc((std::size_t)items * 2 * L1 * n);
+    DeviceBuffer acc((std::size_t)items * 2 * (L - 1) * n);
     check_status(he_keyswitch_rescale_batch(h, L, items, d2.get(), L, rl.data(), d01.get(), acc.get(), 0, ws.get(), st),
                  "he_keyswitch_rescale_batch");
     double out_scale = first.scale() * first.scale() / static_cast<double>(context.key_modulus()[L - 1].value());
     if (scale > 0) out_scale = scale;
+
+    // (2b) optional: drop limbs without scaling, the leading limbs of every polynomial move to a denser batch
+    uint32_t L1 = L - 1;
+    std::size_t out_chain = chain + 1;
+    if (drop_levels) {
+        if (drop_levels >= L1) throw std::invalid_argument("end of modulus switching chain reached");
+        const uint32_t L2 = L1 - (uint32_t)drop_levels;
+        DeviceBuffer dense((std::size_t)items * 2 * L2 * n);
+        check_status(he_memcpy2d_d2d(dense.get(), (std::size_t)L2 * n * sizeof(uint64_t), acc.get(),
+                                     (std::size_t)L1 * n * sizeof(uint64_t), (std::size_t)L2 * n * sizeof(uint64_t),
+                                     (std::size_t)items * 2, st),
+                     "he_memcpy2d_d2d");
+        acc = std::move(dense);
+        L1 = L2;
+        out_chain += drop_levels;
+    }
 
     // (3) the slot sum, one hoisted round at a time: acc += sum_s rot(acc, s)
     const std::size_t beta = (L1 + K - 1) / K;
@@ -105,8 +122,8 @@ std::vector<CAHELGPUCiphertext> pair_square_distances(
         ct.size_ = 2;
         ct.coeff_modulus_size_ = L1;
         ct.poly_modulus_degree_ = n;
-        ct.chain_index_ = chain + 1;
-        ct.parms_id_ = context.parms_id_at(chain + 1);
+        ct.chain_index_ = out_chain;
+        ct.parms_id_ = context.parms_id_at(out_chain);
         ct.scale_ = out_scale;
         ct.is_ntt_form_ = true;
         ct.is_asymmetric_ = first.is_asymmetric_;

@@ -278,7 +278,8 @@ PYBIND11_MODULE(pyCAHEL, m) {
     m.def("relinearize_inplace", &relinearize_inplace, nogil);
     m.def("relinearize_rescale_inplace", &relinearize_rescale_inplace, nogil);
     m.def("pair_square_distances", &pair_square_distances, py::arg("context"), py::arg("clients"), py::arg("pairs"),
-          py::arg("relin_key"), py::arg("galois_key"), py::arg("rounds"), py::arg("scale") = 0.0, nogil);
+          py::arg("relin_key"), py::arg("galois_key"), py::arg("rounds"), py::arg("scale") = 0.0, py::arg("drop_levels") = 0,
+          nogil);
     m.def("mod_switch_to", py::overload_cast<const CAHELGPUContext &, const CAHELGPUPlaintext &, CAHELGPUPlaintext &, std::size_t>(&mod_switch_to), nogil);
     m.def("mod_switch_to", py::overload_cast<const CAHELGPUContext &, const CAHELGPUCiphertext &, CAHELGPUCiphertext &, std::size_t>(&mod_switch_to), nogil);
     m.def("mod_switch_to_inplace", py::overload_cast<const CAHELGPUContext &, CAHELGPUPlaintext &, std::size_t>(&mod_switch_to_inplace), nogil);

@@ -401,7 +401,7 @@ void relinearize_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &enc
 std::vector<CAHELGPUCiphertext> pair_square_distances(
     const CAHELGPUContext &context, const std::vector<std::vector<const CAHELGPUCiphertext *>> &clients,
     const std::vector<std::pair<std::size_t, std::size_t>> &pairs, const CAHELGPURelinKey &rlk,
-    const CAHELGPUGaloisKey &glk, const std::vector<std::vector<int>> &rounds, double scale);
+    const CAHELGPUGaloisKey &glk, const std::vector<std::vector<int>> &rounds, double scale, std::size_t drop_levels = 0);
 void relinearize_rescale_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted,
                                  const CAHELGPURelinKey &relin_keys);  // this build's addition
 void relinearize(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, CAHELGPUCiphertext &destination,

@@ -34,6 +34,9 @@ class KrumConfig:
     hoisting: bool = True                    # byzantine_fl.py: Hoisting_flag = 1
     hoisting_radix: int = 16                 # every round of the slot sum is a hoisted sum of radix - 1 rotations;
                                              # 0: the reference's split, hoisting(1..15) then one rotation per doubling
+    sum_drop_levels: int = 0                 # limbs dropped without scaling (mod_switch_to_next) after the rescale:
+                                             # the slot sum's key switches then run over fewer limbs; 0 = as the
+                                             # reference, which rotates at the level the rescale leaves
     batched: bool = True                     # all pairs go through every stage together, one launch per stage
                                              # (pair_square_distances); False: pair by pair over the lanes
     lanes: int = 3                           # host threads / streams that the pairs are dealt to (0: null stream);
@@ -184,6 +187,8 @@ def pair_distance(state: KrumState, cts_i, cts_j):
             c.add_inplace(ctx, acc, tmp)
     c.relinearize_rescale_inplace(ctx, acc, state.rlk)     # = relinearize_inplace + rescale_to_next_inplace
     acc.set_scale(cfg.scale)
+    for _ in range(cfg.sum_drop_levels):
+        c.mod_switch_to_next_inplace(ctx, acc)
     rot = c.ciphertext(ctx)
     for steps in rotate_sum_plan(int(math.log2(state.slots)), cfg):
         if len(steps) > 1:
@@ -228,7 +233,8 @@ def all_pair_distances(state: KrumState, cts, enc):
     if state.config.batched:
         c = state.cahel
         rounds = rotate_sum_plan(int(math.log2(state.slots)), state.config)
-        out = c.pair_square_distances(state.context, cts, pairs, state.rlk, state.glk, rounds, state.config.scale)
+        out = c.pair_square_distances(state.context, cts, pairs, state.rlk, state.glk, rounds, state.config.scale,
+                                      state.config.sum_drop_levels)
         _sync(c)
     else:
         out = _map_lanes(state, pairs, lambda ij: pair_distance(state, cts[ij[0]], cts[ij[1]]))

@@ -381,6 +381,19 @@ def test_batched_pair_distances_equal_the_pairwise_ciphertexts(oracle):
         want = krum.pair_distance(state, cts[i], cts[j])
         assert got.chain_index() == want.chain_index() and got.scale() == want.scale()
         assert (got.to_numpy() == want.to_numpy()).all(), (i, j)
+    # the slot sum one level further down
+    state.config.sum_drop_levels = 1
+    low = c.pair_square_distances(state.context, cts, pairs[:2], state.rlk, state.glk, rounds, cfg.scale, 1)
+    for (i, j), got in zip(pairs, low):
+        want = krum.pair_distance(state, cts[i], cts[j])
+        assert got.chain_index() == want.chain_index() == batch[0].chain_index() + 1
+        assert (got.to_numpy() == want.to_numpy()).all(), (i, j)
+    decoded = state.sk.decrypt_decode_many(state.context, low, state.slots, 1)[:, 0]
+    plain = krum.plain_distance_matrix(updates)
+    assert abs(decoded[0] - plain[0, 1]) < 1e-3 * plain[0, 1] and abs(decoded[1] - plain[0, 2]) < 1e-3 * plain[0, 2]
+    with pytest.raises(ValueError, match="end of modulus switching chain"):
+        c.pair_square_distances(state.context, cts, pairs[:1], state.rlk, state.glk, rounds, cfg.scale, 2)
+    state.config.sum_drop_levels = 0
     assert c.pair_square_distances(state.context, cts, [], state.rlk, state.glk, rounds, 0.0) == []
     with pytest.raises(ValueError, match="pair out of range"):
         c.pair_square_distances(state.context, cts, [(0, 3)], state.rlk, state.glk, rounds, 0.0)
