@@ -718,9 +718,11 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
     for (int i = 0; i < kPer; i++) o[tid + i * half] = fp_to_u64(fp_canonical(acc[i], m));
 }
 
-// Integer back end (twiddles stay in the table: 30 Shoup pairs per thread do not fit in registers).
+// Integer back end (twiddles stay in the table: 30 Shoup pairs per thread do not fit in registers).  Three waves
+// per SIMD (168 registers, 24 bytes of spill in the forward kernel) hide the latency of the epilogue's operand loads
+// better than the two waves that 196 registers allow.
 template <bool FWD>
-__global__ __launch_bounds__(kThreads) void ntt_blocks_int_kernel(NttArgs a) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void ntt_blocks_int_kernel(NttArgs a) {
     __shared__ uint64_t lds[kLdsWords];
     const uint32_t nthreads = blockDim.x;
     const uint32_t tile_elems = nthreads << 4;
