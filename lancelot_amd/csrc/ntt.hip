@@ -458,9 +458,11 @@ __device__ __forceinline__ BlocksGeom blocks_geom(const NttArgs &a) {
 constexpr int kPer = 16;  // words per thread in the blocks pass
 constexpr int kMaxGroup = 4;  // most jobs in one LimbGroup
 
-// FP64 back end.  EPI compiles the fused forward epilogues in (they cost 64 registers).
+// FP64 back end.  EPI compiles the fused forward epilogues in (they cost 64 registers).  Two waves per SIMD: with
+// the epilogues the kernel needs 254 registers; left to itself the compiler spreads into the accumulation registers
+// and a single wave, which costs a third more time (three waves would spill, and measure slower).
 template <bool FWD, bool EPI>
-__global__ __launch_bounds__(kThreads) void ntt_blocks_fp_kernel(NttArgs a) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void ntt_blocks_fp_kernel(NttArgs a) {
     __shared__ uint64_t lds[kLdsWords];
     const uint32_t nthreads = blockDim.x;
     const BlocksGeom g = blocks_geom(a);
