@@ -62,6 +62,8 @@ struct he_context {
     std::vector<uint8_t> fp_ok;  // per table: prime below 2^50
     bool use_fp = true;          // environment CAHEL_HIP_NO_FP64=1 forces the integer back end
     bool fuse_inner = true;      // environment CAHEL_HIP_NO_FUSED_KS=1: separate NTT and inner-product kernels
+    uint64_t fp_mask = 0;        // bit t: table t has a prime below 2^50
+    bool mixed_ok = false;       // mixed launches allowed (at most 64 tables; CAHEL_HIP_NO_MIXED=1 switches them off)
     bool fuse_modup_rows = true; // environment CAHEL_HIP_NO_FUSED_MODUP=1: base conversion and rows pass as two kernels
     uint32_t modup_group = 6;    // output limbs per workgroup of the fused kernel (CAHEL_HIP_MODUP_GROUP)
     std::vector<Level> levels;   // indexed by L
@@ -112,7 +114,29 @@ NttArgs base_args(const he_context *ctx, bool forward) {
     a.barrett = ctx->d_barrett;
     a.log_n = ctx->log_n;
     a.epi_b_mask = 0xffffffffu;
+    a.fp_mask = ctx->fp_mask;
     return a;
+}
+
+// Back end of a launch over the tables of a map: FP64 when every prime is below 2^50, integer when none is (or the
+// FP64 back end is switched off), else the mixed kernels, in which every workgroup follows its own limb's prime.
+// `also`: a further table whose residues the launch reads (the source limb of a prologue); when its prime is not
+// below 2^50 the FP64 code cannot take it in and the whole launch stays on the integer back end.
+int backend_for(const he_context *ctx, const LimbMap &m, int also = -1) {
+    if (!ctx->use_fp || (also >= 0 && !ctx->fp_ok[(size_t)also])) return NTT_BACKEND_INT;
+    uint32_t capable = 0;
+    for (uint32_t i = 0; i < m.limbs; i++) capable += ctx->fp_ok[map_table(m, i)] != 0;
+    if (capable == m.limbs) return NTT_BACKEND_FP;
+    return capable && ctx->mixed_ok ? NTT_BACKEND_MIXED : NTT_BACKEND_INT;
+}
+
+// the same over the converted limbs of a ModUp at level L (every table of Ql u P takes part)
+int backend_for_level(const he_context *ctx, uint32_t L) {
+    if (!ctx->use_fp) return NTT_BACKEND_INT;
+    uint32_t capable = 0;
+    for (uint32_t t = 0; t < L + ctx->size_p; t++) capable += ctx->fp_ok[table_of(ctx, L, t)] != 0;
+    if (capable == L + ctx->size_p) return NTT_BACKEND_FP;
+    return capable && ctx->mixed_ok ? NTT_BACKEND_MIXED : NTT_BACKEND_INT;
 }
 
 // the FP64 back end applies when every table of the launch has a prime below 2^50
@@ -324,6 +348,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->use_fp = !(env && env[0] == '1');
         const char *nf = getenv("CAHEL_HIP_NO_FUSED_KS");
         ctx->fuse_inner = !(nf && nf[0] == '1');
+        const char *nx = getenv("CAHEL_HIP_NO_MIXED");
+        ctx->mixed_ok = qp <= 64 && !(nx && nx[0] == '1');
         const char *nm = getenv("CAHEL_HIP_NO_FUSED_MODUP");
         ctx->fuse_modup_rows = !(nm && nm[0] == '1');
         if (const char *g = getenv("CAHEL_HIP_MODUP_GROUP")) {
@@ -336,6 +362,7 @@ int he_context_create(const he_context_desc *d, he_context **out) {
             const uint64_t q = d->moduli[t];
             if (q >> 50) continue;
             ctx->fp_ok[t] = 1;
+            if (t < 64) ctx->fp_mask |= 1ull << t;
             const double qd = (double)q;
             for (size_t i = 0; i < n; i++) {
                 const uint64_t w = d->psi[2 * (t * n + i)];
@@ -514,7 +541,7 @@ int he_ntt_forward(const he_context *ctx, uint64_t *data, uint32_t n_polys, uint
     a.out = data;
     a.in_poly_stride = a.out_poly_stride = poly_stride;
     a.map = LimbMap{limbs, first, split, tail};
-    HE_HIP(launch_ntt_forward(a, n_polys, fp_for(ctx, a.map), S(s)));
+    HE_HIP(launch_ntt_forward(a, n_polys, backend_for(ctx, a.map), S(s)));
     return HE_OK;
 }
 
@@ -527,7 +554,7 @@ int he_ntt_inverse(const he_context *ctx, uint64_t *data, uint32_t n_polys, uint
     a.out = data;
     a.in_poly_stride = a.out_poly_stride = poly_stride;
     a.map = LimbMap{limbs, first, split, tail};
-    HE_HIP(launch_ntt_inverse(a, n_polys, fp_for(ctx, a.map), S(s)));
+    HE_HIP(launch_ntt_inverse(a, n_polys, backend_for(ctx, a.map), S(s)));
     return HE_OK;
 }
 
@@ -613,7 +640,7 @@ int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_
     inv.out = ws;
     inv.out_poly_stride = 1;
     inv.map = plain_map(1, L - 1);
-    HE_HIP(launch_ntt_inverse(inv, n_polys, fp_for(ctx, inv.map), S(s)));
+    HE_HIP(launch_ntt_inverse(inv, n_polys, backend_for(ctx, inv.map), S(s)));
     // every remaining limb: NTT_j(ws mod q_j), then (in_j - that) / q_last
     NttArgs fwd = base_args(ctx, true);
     fwd.pro_mode = NTT_PRO_BROADCAST_REDUCE;
@@ -629,7 +656,7 @@ int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L - 1;
     // the broadcast source is a residue of q_{L-1}: the FP64 back end needs it below 2^50 as well
-    HE_HIP(launch_ntt_forward(fwd, n_polys, fp_for(ctx, plain_map(L, 0)), S(s)));
+    HE_HIP(launch_ntt_forward(fwd, n_polys, backend_for(ctx, fwd.map, (int)L - 1), S(s)));
     return HE_OK;
 }
 
@@ -656,7 +683,7 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     inv.map = plain_map(L, 0);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_part_hat_inv;
-    HE_HIP(launch_ntt_inverse(inv, items, fp_for(ctx, inv.map), S(s)));
+    HE_HIP(launch_ntt_inverse(inv, items, backend_for(ctx, inv.map), S(s)));
     if (lv->batched) {
         BconvBatch b{ws, out, c, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                      lv->beta, lv->modup_max_rows, lv->modup_max_copy, lv->d_mats_fp, ctx->d_fp_consts,
@@ -681,7 +708,7 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     fwd.n_groups = lv->n_modup_groups;
     fwd.items = items;
     fwd.item_stride = (size_t)lv->beta * LK * n;
-    HE_HIP(launch_ntt_forward(fwd, 1, fp_for_level(ctx, L), S(s)));
+    HE_HIP(launch_ntt_forward(fwd, 1, backend_for_level(ctx, L), S(s)));
     return HE_OK;
 }
 
@@ -729,7 +756,7 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     inv.map = plain_map(K, ctx->size_q);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = ctx->d_phat_inv;
-    HE_HIP(launch_ntt_inverse(inv, n_polys, fp_for(ctx, inv.map), S(s)));
+    HE_HIP(launch_ntt_inverse(inv, n_polys, backend_for(ctx, inv.map), S(s)));
     const Level *lv = level_of(ctx, L);
     // the conversion tables describe up to 4 polynomials; more of them go as items of 2 (ciphertexts)
     const bool batched = lv && lv->batched && (n_polys <= 4 || n_polys % 2 == 0);
@@ -758,7 +785,7 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     fwd.w = ctx->d_pinv_mod_q;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L;
-    HE_HIP(launch_ntt_forward(fwd, n_polys, fp_for(ctx, fwd.map), S(s)));
+    HE_HIP(launch_ntt_forward(fwd, n_polys, backend_for(ctx, fwd.map), S(s)));
     return HE_OK;
 }
 
@@ -969,7 +996,7 @@ int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items
     inv.map = LimbMap{K + 1, L - 1, 1, ctx->size_q};
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_mdr_w;
-    HE_HIP(launch_ntt_inverse(inv, polys, fp_for(ctx, inv.map), S(s)));
+    HE_HIP(launch_ntt_inverse(inv, polys, backend_for(ctx, inv.map), S(s)));
     // (3) delta = P -> Ql conversion of the special limbs
     if (lv->batched) {
         BconvBatch b{cx, delta, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
@@ -1003,7 +1030,7 @@ int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items
     fwd.w = lv->d_qlast_inv;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L - 1;
-    HE_HIP(launch_ntt_forward(fwd, polys, fp_for(ctx, plain_map(L, 0)), S(s)));
+    HE_HIP(launch_ntt_forward(fwd, polys, backend_for(ctx, fwd.map, (int)L - 1), S(s)));
     return HE_OK;
 }
 

@@ -62,6 +62,7 @@ struct NttArgs {
     const uint64_t *tw;       // [tables][N][2] (operand, Shoup quotient)
     const double *tw_fp;      // [tables][N] twiddles as exact doubles for the FP64 back end (primes below 2^50)
     const double *fp_consts;  // [tables][4]: q, 1/q, N^-1 mod q, (N^-1 mod q)/q
+    uint64_t fp_mask;         // bit t: table t has a prime below 2^50 (read by the mixed back end only)
     const uint64_t *moduli;   // [tables]
     const uint64_t *barrett;  // [tables][2]
     const LimbJob *jobs;      // explicit list (then in/out limbs are absolute, no prologue/epilogue)
@@ -93,11 +94,14 @@ struct NttArgs {
 
 // Forward transform: phase 1 (strided rows) then phase 2 (contiguous 256-blocks).  `a.in`/`a.out` and the
 // prologue describe phase 1's input; phase 2 runs in place on a.out unless an epilogue redirects it.
-// fp selects the FP64 back end; every table the launch touches must then hold a prime below 2^50.
-hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s);
+// backend: NTT_BACKEND_INT, NTT_BACKEND_FP (every table the launch touches must then hold a prime below 2^50) or
+// NTT_BACKEND_MIXED (every workgroup picks the FP64 back end when its limb's bit of fp_mask is set, the integer
+// one otherwise: for chains that mix primes below and above 2^50, tables below 64 only).
+enum : int { NTT_BACKEND_INT = 0, NTT_BACKEND_FP = 1, NTT_BACKEND_MIXED = 2 };
+hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s);
 // Inverse transform: phase A (contiguous blocks, reads a.in writes a.out) then phase B (rows, in place on
 // a.out, epilogue NTT_EPI_MUL optional).
-hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s);
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s);
 
 struct Tables {
     const uint64_t *moduli;

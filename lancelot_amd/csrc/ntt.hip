@@ -168,7 +168,7 @@ __device__ __forceinline__ FpTw inverse_scale(const NttArgs &a, const Job &job, 
 // ---------------------------------------------------------------------------------------------------
 // rows pass: stages 0 .. LD-1 (forward) over an R = 2^LD rows x 256 matrix
 // ---------------------------------------------------------------------------------------------------
-template <int LD, bool FWD, bool FP, int TL>
+template <int LD, bool FWD, int BE, int TL>
 __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     __shared__ uint64_t lds[(1 << TL) + (1 << (TL - 4))];
     constexpr uint32_t kRowThreads = (1u << TL) / 16;
@@ -183,7 +183,9 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     const uint32_t col0 = (lb % tiles_per_limb) << LOGC;
     double *ld = reinterpret_cast<double *>(lds);
 
-    if (FP) {
+    // the back end of this workgroup's limb: fixed by the launch, or (mixed) by the limb's prime
+    const bool fp = BE == NTT_BACKEND_FP || (BE == NTT_BACKEND_MIXED && ((a.fp_mask >> job.table) & 1));
+    if (BE != NTT_BACKEND_INT && fp) {
         const FpCtx c = fp_ctx(a, job.table);
         if (FWD) {
             // input: canonical residues (or one broadcast source limb); output: lazy signed doubles
@@ -462,8 +464,7 @@ constexpr int kMaxGroup = 4;  // most jobs in one LimbGroup
 // the epilogues the kernel needs 254 registers; left to itself the compiler spreads into the accumulation registers
 // and a single wave, which costs a third more time (three waves would spill, and measure slower).
 template <bool FWD, bool EPI>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void ntt_blocks_fp_kernel(NttArgs a) {
-    __shared__ uint64_t lds[kLdsWords];
+__device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *lds) {
     const uint32_t nthreads = blockDim.x;
     const BlocksGeom g = blocks_geom(a);
     const size_t off = g.off;
@@ -617,6 +618,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     }
 }
 
+template <bool FWD, bool EPI>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void ntt_blocks_fp_kernel(NttArgs a) {
+    __shared__ uint64_t lds[kLdsWords];
+    ntt_blocks_fp_body<FWD, EPI>(a, lds);
+}
+
 // Forward blocks pass of ModUp fused with the key-switch inner product.  Workgroup = (limb t of Ql u P, tile of
 // 16 T words): its first T threads transform that tile of every digit in turn; all 2 T threads then multiply
 // it by a key polynomial (threads below T by the first, the others by the second) and accumulate in registers.
@@ -724,8 +731,7 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
 // per SIMD (168 registers, 24 bytes of spill in the forward kernel) hide the latency of the epilogue's operand loads
 // better than the two waves that 196 registers allow.
 template <bool FWD>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void ntt_blocks_int_kernel(NttArgs a) {
-    __shared__ uint64_t lds[kLdsWords];
+__device__ __forceinline__ void ntt_blocks_int_body(const NttArgs &a, uint64_t *lds) {
     const uint32_t nthreads = blockDim.x;
     const uint32_t tile_elems = nthreads << 4;
     const BlocksGeom g = blocks_geom(a);
@@ -792,7 +798,26 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))
     }
 }
 
-template <bool FWD, bool FP>
+template <bool FWD>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void ntt_blocks_int_kernel(NttArgs a) {
+    __shared__ uint64_t lds[kLdsWords];
+    ntt_blocks_int_body<FWD>(a, lds);
+}
+
+// Mixed back end: the limbs of a unit share a modulus, so the whole workgroup takes one branch.  EPI as in
+// ntt_blocks_fp_kernel: the FP64 body compiled with the fused epilogues addresses their operands unconditionally,
+// so it is only launched when the launch has an epilogue.
+template <bool FWD, bool EPI>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void ntt_blocks_mixed_kernel(NttArgs a) {
+    __shared__ uint64_t lds[kLdsWords];
+    const Job first = decode_job(a, blocks_geom(a).unit.j0);
+    if ((a.fp_mask >> first.table) & 1)
+        ntt_blocks_fp_body<FWD, EPI>(a, lds);
+    else
+        ntt_blocks_int_body<FWD>(a, lds);
+}
+
+template <bool FWD, int FP>
 hipError_t launch_rows(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
     const int ld = (int)a.log_n - 8;
     auto grid = [&](int ldv, int tl) {
@@ -849,14 +874,18 @@ BlocksPlan plan_blocks(const NttArgs &a, uint32_t n_polys) {
     return p;
 }
 
-template <bool FWD, bool FP>
+template <bool FWD, int FP>
 hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
     const BlocksPlan p = plan_blocks(a, n_polys);
     a.batch = p.batch;
     a.n_polys = n_polys;
     const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD ||
                              a.epi_mode == NTT_EPI_FMA_SUB_MUL);
-    if (!FP)
+    if (FP == NTT_BACKEND_MIXED && epi)
+        hipLaunchKernelGGL((ntt_blocks_mixed_kernel<FWD, FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
+    else if (FP == NTT_BACKEND_MIXED)
+        hipLaunchKernelGGL((ntt_blocks_mixed_kernel<FWD, false>), dim3(p.grid), dim3(p.threads), 0, s, a);
+    else if (!FP)
         hipLaunchKernelGGL((ntt_blocks_int_kernel<FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
     else if (epi)
         hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
@@ -867,13 +896,17 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
 
 }  // namespace
 
-hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s) {
-    if (a.log_n < 9 || a.log_n > 16) return hipErrorInvalidValue;
+hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s) {
+    if (a.log_n < 9 || a.log_n > 16 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
-    hipError_t e = fp ? launch_rows<true, true>(a, n_jobs, s) : launch_rows<true, false>(a, n_jobs, s);
+    hipError_t e = backend == NTT_BACKEND_MIXED ? launch_rows<true, NTT_BACKEND_MIXED>(a, n_jobs, s)
+                   : backend                    ? launch_rows<true, NTT_BACKEND_FP>(a, n_jobs, s)
+                                                : launch_rows<true, NTT_BACKEND_INT>(a, n_jobs, s);
     if (e != hipSuccess) return e;
-    return fp ? launch_blocks<true, true>(a, n_polys, s) : launch_blocks<true, false>(a, n_polys, s);
+    return backend == NTT_BACKEND_MIXED ? launch_blocks<true, NTT_BACKEND_MIXED>(a, n_polys, s)
+           : backend                    ? launch_blocks<true, NTT_BACKEND_FP>(a, n_polys, s)
+                                        : launch_blocks<true, NTT_BACKEND_INT>(a, n_polys, s);
 }
 
 bool modup_rows_supported(uint32_t log_n) { return log_n >= 13 && log_n <= 16; }
@@ -896,7 +929,7 @@ hipError_t launch_modup_rows(const NttArgs &a, const ModupRowsArgs &m, uint32_t 
 hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, bool rows_done, hipStream_t s) {
     if (a.log_n < 9 || a.log_n > 16 || !a.jobs) return hipErrorInvalidValue;
     if (a.n_jobs && !rows_done) {
-        hipError_t e = launch_rows<true, true>(a, a.n_jobs, s);
+        hipError_t e = launch_rows<true, NTT_BACKEND_FP>(a, a.n_jobs, s);
         if (e != hipSuccess) return e;
     }
     const uint32_t n = 1u << a.log_n;
@@ -911,16 +944,20 @@ hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, bool 
     return hipGetLastError();
 }
 
-hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, bool fp, hipStream_t s) {
-    if (a.log_n < 9 || a.log_n > 16) return hipErrorInvalidValue;
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s) {
+    if (a.log_n < 9 || a.log_n > 16 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
-    hipError_t e = fp ? launch_blocks<false, true>(a, n_polys, s) : launch_blocks<false, false>(a, n_polys, s);
+    hipError_t e = backend == NTT_BACKEND_MIXED ? launch_blocks<false, NTT_BACKEND_MIXED>(a, n_polys, s)
+                   : backend                    ? launch_blocks<false, NTT_BACKEND_FP>(a, n_polys, s)
+                                                : launch_blocks<false, NTT_BACKEND_INT>(a, n_polys, s);
     if (e != hipSuccess) return e;
     NttArgs rows = a;
     rows.in = a.out;  // the rows pass continues in place on the output buffer
     rows.in_poly_stride = a.out_poly_stride;
-    return fp ? launch_rows<false, true>(rows, n_jobs, s) : launch_rows<false, false>(rows, n_jobs, s);
+    return backend == NTT_BACKEND_MIXED ? launch_rows<false, NTT_BACKEND_MIXED>(rows, n_jobs, s)
+           : backend                    ? launch_rows<false, NTT_BACKEND_FP>(rows, n_jobs, s)
+                                        : launch_rows<false, NTT_BACKEND_INT>(rows, n_jobs, s);
 }
 
 }  // namespace he
