@@ -135,6 +135,44 @@ def test_integer_and_fp64_back_ends_agree(oracle, capi, monkeypatch):
     assert (results[0] == results[1]).all()
 
 
+@pytest.mark.parametrize("logn,bits,size_p,L", [(13, [60, 40, 40, 60], 1, 3), (13, [60, 40, 40, 60], 1, 2),
+                                                 (12, [60, 45, 50, 52, 44, 60, 49, 58], 2, 5)])
+def test_mixed_back_end_agrees_with_the_integer_one(oracle, capi, monkeypatch, logn, bits, size_p, L):
+    """Chains that mix primes below and above 2^50 (Lancelot's [60, 40, 40, 60]): by default every workgroup follows
+    its own limb's prime, with CAHEL_HIP_NO_MIXED=1 the whole launch takes the integer kernels.  Key switch, key
+    switch + rescale, plain rescale and the public transforms (with the limb maps of the key level) against the
+    oracle, both ways."""
+    for no_mixed in ("0", "1"):
+        monkeypatch.setenv("CAHEL_HIP_NO_MIXED", no_mixed)
+        cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+        rng = np.random.default_rng(17)
+        lib, h = capi.lib(), ctx.he_handle()
+        host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+        ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+        c, ct = rand_limbs(p, rng, range(L)), rand_limbs(p, rng, range(L), n_polys=2)
+        dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
+        capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, 5, ws.ptr, None))
+        ks = p.key_switch(p.galois_ntt(c, 5), host_evk)
+        want = np.stack([p.add(ct[b], ks[b]) for b in range(2)])
+        assert (dct.numpy() == want).all(), no_mixed
+        if L >= 2:
+            dres = DeviceArray(capi, shape=(2, L - 1, p.n))
+            rws = DeviceArray(capi, shape=(2, p.n))
+            capi.check(lib.he_rescale(h, dct.ptr, dres.ptr, 2, L, rws.ptr, None))
+            assert (dres.numpy() == p.rescale(want)).all(), no_mixed
+            dct2 = DeviceArray(capi, host=ct)
+            capi.check(lib.he_keyswitch_rescale(h, L, dc.ptr, ptrs, dct2.ptr, dres.ptr, 0, ws.ptr, None))
+            ks0 = p.key_switch(c, host_evk)
+            assert (dres.numpy() == p.rescale(np.stack([p.add(ct[b], ks0[b]) for b in range(2)]))).all(), no_mixed
+        # forward and inverse transforms over all of Q u P (two polynomials), in place
+        full = rand_limbs(p, rng, range(p.size_qp), n_polys=2)
+        dfull = DeviceArray(capi, host=full)
+        capi.check(lib.he_ntt_forward(h, dfull.ptr, 2, p.size_qp, p.size_qp, 0, p.size_qp, 0, None))
+        assert (dfull.numpy() == np.stack([p.ntt_fwd(full[b].copy(), list(range(p.size_qp))) for b in range(2)])).all(), no_mixed
+        capi.check(lib.he_ntt_inverse(h, dfull.ptr, 2, p.size_qp, p.size_qp, 0, p.size_qp, 0, None))
+        assert (dfull.numpy() == full).all(), no_mixed
+
+
 @pytest.mark.parametrize("logn,bits,size_p,L", [(13, [50, 50, 49, 50, 50, 50], 2, 4), (13, [50, 50, 49, 50, 50, 50], 2, 3),
                                                  (14, [50, 49, 48, 50, 47, 50, 50, 50, 50], 3, 5),
                                                  (11, [45, 40, 40, 50], 1, 3), (9, [40, 40, 45, 45], 2, 2)])
