@@ -624,7 +624,8 @@ hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_
     if (b.n_units == 0) return hipSuccess;
     static const uint32_t target = [] {
         const char *e = getenv("CAHEL_HIP_BCONV_ROWS");
-        return e ? (uint32_t)atoi(e) : 6u;
+        const int v = e ? atoi(e) : 6;
+        return (uint32_t)(v >= 1 && v <= 64 ? v : 6);
     }();
     const uint32_t cg = (b.max_rows + target - 1) / target;
     const uint32_t rows_per = (b.max_rows + cg - 1) / cg;
