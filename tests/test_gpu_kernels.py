@@ -226,6 +226,29 @@ def test_keyswitch_rescale_equals_the_two_steps(oracle, capi, logn, bits, size_p
 
 
 @pytest.mark.parametrize("logn,bits,size_p,L", [(13, [50, 50, 49, 50, 50, 50], 2, 4), (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5),
+                                                 (14, [50, 49, 48, 50, 47, 50, 50, 50, 50], 3, 5)])
+def test_moddown_on_one_to_six_polynomials(oracle, capi, logn, bits, size_p, L):
+    """he_moddown on 1 to 4 polynomials (one conversion launch) and on 6 (three ciphertexts as items of two),
+    overwriting and adding, against the oracle on both arithmetic back ends."""
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(31)
+    lib, h = capi.lib(), ctx.he_handle()
+    K, n = p.size_p, p.n
+    tables = [p.table_index(L, t) for t in range(L + K)]
+    for n_polys in (1, 2, 3, 4, 6):
+        ws = DeviceArray(capi, shape=(n_polys, L, n))
+        cx = np.stack([rand_limbs(p, rng, tables) for _ in range(n_polys)])
+        md = np.stack([p.moddown(cx[b]) for b in range(n_polys)])
+        dcx, dout = DeviceArray(capi, host=cx), DeviceArray(capi, shape=(n_polys, L, n))
+        capi.check(lib.he_moddown(h, L, dcx.ptr, dout.ptr, n_polys, 0, ws.ptr, None))
+        assert (dout.numpy() == md).all(), n_polys
+        base = rand_limbs(p, rng, range(L), n_polys=n_polys)
+        dcx, dacc = DeviceArray(capi, host=cx), DeviceArray(capi, host=base)
+        capi.check(lib.he_moddown(h, L, dcx.ptr, dacc.ptr, n_polys, 1, ws.ptr, None))
+        assert (dacc.numpy() == np.stack([p.add(base[b], md[b]) for b in range(n_polys)])).all(), n_polys
+
+
+@pytest.mark.parametrize("logn,bits,size_p,L", [(13, [50, 50, 49, 50, 50, 50], 2, 4), (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5),
                                                  (11, [45, 40, 40, 50], 1, 2)])
 def test_rotate_entry_point(oracle, capi, logn, bits, size_p, L):
     """he_rotate = (sigma(c0), 0) + KeySwitch(sigma(c1)) against the oracle, both back ends."""
