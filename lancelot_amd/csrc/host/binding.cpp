@@ -3,6 +3,9 @@
 // with an underscore, and the accessor methods on context / plaintext / ciphertext / keys, are additions used
 // by the test-suite and the benchmark (seeding, raw device pointers, host copies); they do not exist in the
 // reference and nothing in Lancelot calls them.
+#include <fstream>
+#include <sstream>
+
 #include <pybind11/numpy.h>
 #include <pybind11/pybind11.h>
 #include <pybind11/stl.h>
@@ -21,6 +24,32 @@ py::array_t<uint64_t> to_host(const uint64_t *dev, std::vector<py::ssize_t> shap
     if (words) check_status(he_memcpy_d2h(out.mutable_data(), dev, words * sizeof(uint64_t), cahel::current_stream()), "download");
     return out;
 }
+
+// save / load / to_bytes / from_bytes on top of the C++ stream members (the reference binds none of them)
+template <typename T, typename C>
+void def_serialization(C &cls) {
+    cls.def("save", [](const T &self, const std::string &path) {
+           std::ofstream f(path, std::ios::binary | std::ios::trunc);
+           if (!f) throw std::runtime_error("I/O error");
+           self.save(f);
+       })
+        .def("load", [](T &self, const CAHELGPUContext &context, const std::string &path) {
+            std::ifstream f(path, std::ios::binary);
+            if (!f) throw std::runtime_error("I/O error");
+            self.load(context, f);
+        })
+        .def("to_bytes", [](const T &self) {
+            std::ostringstream s(std::ios::binary);
+            self.save(s);
+            return py::bytes(s.str());
+        })
+        .def("from_bytes", [](T &self, const CAHELGPUContext &context, const py::bytes &data) {
+            std::istringstream s(std::string(data), std::ios::binary);
+            self.load(context, s);
+        });
+}
+
+py::tuple id_tuple(const parms_id_type &id) { return py::make_tuple(id[0], id[1], id[2], id[3]); }
 
 }  // namespace
 
@@ -57,7 +86,14 @@ PYBIND11_MODULE(pyCAHEL, m) {
         .def("set_poly_modulus_degree", &EncryptionParameters::set_poly_modulus_degree)
         .def("set_special_modulus_size", &EncryptionParameters::set_special_modulus_size)
         .def("set_galois_elts", &EncryptionParameters::set_galois_elts)
-        .def("set_coeff_modulus", &EncryptionParameters::set_coeff_modulus);
+        .def("set_coeff_modulus", &EncryptionParameters::set_coeff_modulus)
+        .def("parms_id", [](const EncryptionParameters &p) { return id_tuple(p.parms_id()); });
+    m.def("_blake2b", [](const py::bytes &data, std::size_t digest_size) {
+        const std::string in(data);
+        std::string out(digest_size, '\0');
+        blake2b(out.data(), digest_size, in.data(), in.size());
+        return py::bytes(out);
+    });
 
     py::class_<CAHELGPUContext>(m, "context")
         .def(py::init<EncryptionParameters &, bool, sec_level_type>())
@@ -315,4 +351,22 @@ PYBIND11_MODULE(pyCAHEL, m) {
     m.def("_set_lane", &cahel::set_lane);
     m.def("_current_lane", &cahel::current_lane);
     m.def("_lane_count", &cahel::lane_count);
+
+    // serialization in the reference's byte layout, and the identifiers it carries
+    {
+        auto plain = py::reinterpret_borrow<py::class_<CAHELGPUPlaintext>>(m.attr("plaintext"));
+        auto cipher = py::reinterpret_borrow<py::class_<CAHELGPUCiphertext>>(m.attr("ciphertext"));
+        auto pk = py::reinterpret_borrow<py::class_<CAHELGPUPublicKey>>(m.attr("public_key"));
+        auto rlk = py::reinterpret_borrow<py::class_<CAHELGPURelinKey>>(m.attr("relin_key"));
+        auto glk = py::reinterpret_borrow<py::class_<CAHELGPUGaloisKey>>(m.attr("galois_key"));
+        def_serialization<CAHELGPUPlaintext>(plain);
+        def_serialization<CAHELGPUCiphertext>(cipher);
+        def_serialization<CAHELGPUPublicKey>(pk);
+        def_serialization<CAHELGPURelinKey>(rlk);
+        def_serialization<CAHELGPUGaloisKey>(glk);
+        plain.def("parms_id", [](const CAHELGPUPlaintext &p) { return id_tuple(p.parms_id()); });
+        cipher.def("parms_id", [](const CAHELGPUCiphertext &c) { return id_tuple(c.parms_id()); });
+        auto context = py::reinterpret_borrow<py::class_<CAHELGPUContext>>(m.attr("context"));
+        context.def("parms_id_at", [](const CAHELGPUContext &c, std::size_t i) { return id_tuple(c.parms_id_at(i)); });
+    }
 }

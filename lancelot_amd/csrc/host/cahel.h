@@ -7,9 +7,11 @@
 // names) and throw std::logic_error("unsupported scheme") the way the reference does for the scheme it
 // is not running (src/evaluate.cu:305-306, include/evaluate.h:501-535).
 #pragma once
+#include <array>
 #include <atomic>
 #include <cstddef>
 #include <cstdint>
+#include <iosfwd>
 #include <memory>
 #include <stdexcept>
 #include <utility>
@@ -24,8 +26,13 @@ enum class scheme_type : std::uint8_t { none = 0, bgv = 1, bfv = 2, ckks = 3 };
 enum class mul_tech_type : std::uint8_t { none = 0, behz = 1, hps = 2, hps_overq = 3, hps_overq_leveled = 4 };
 enum class sec_level_type : int { none = 0, tc128 = 128, tc192 = 192, tc256 = 256 };
 
-using parms_id_type = std::uint64_t;
-constexpr parms_id_type parms_id_zero = 0;
+// 256-bit BLAKE2b digest of the parameter words (include/util/hash.h:22-37)
+using parms_id_type = std::array<std::uint64_t, 4>;
+constexpr parms_id_type parms_id_zero{{0, 0, 0, 0}};
+// The words the reference hashes (include/util/encryptionparams.h:337-379): scheme, degree, special modulus
+// count, every key modulus, the first `limbs` coefficient moduli, the plain modulus (0 for CKKS).
+parms_id_type compute_parms_id(scheme_type scheme, std::size_t poly_modulus_degree, std::size_t special_modulus_size,
+                               const std::vector<std::uint64_t> &key_modulus, std::size_t limbs);
 
 // include/util/encryptionparams.h:40-149
 class EncryptionParameters {
@@ -44,6 +51,8 @@ public:
     const std::vector<Modulus> &coeff_modulus() const { return coeff_modulus_; }
     const std::vector<Modulus> &key_modulus() const { return coeff_modulus_; }
     const std::vector<uint32_t> &galois_elts() const { return galois_elts_; }
+    // identifier of the key level (all moduli), as include/util/encryptionparams.h:315-317 returns it
+    parms_id_type parms_id() const;
 
 private:
     scheme_type scheme_;
@@ -158,6 +167,7 @@ private:
     std::size_t n_ = 0, size_q_ = 0, size_p_ = 0;
     int log_n_ = 0;
     std::vector<std::size_t> chain_limbs_;
+    std::vector<cahel::parms_id_type> parms_ids_;
     std::vector<uint32_t> galois_elts_;
     he_context *he_ = nullptr;
     uint32_t prng_key_[8];
@@ -184,6 +194,9 @@ public:
     std::size_t poly_modulus_degree() const { return poly_modulus_degree_; }
     cahel::parms_id_type &parms_id() { return parms_id_; }
     cahel::parms_id_type parms_id() const { return parms_id_; }
+    // the reference's byte layout (include/plaintext.h:109-200); load checks the header against the context
+    void save(std::ostream &stream) const;
+    void load(const CAHELGPUContext &context, std::istream &stream);
 
     cahel::DeviceBuffer data_;
     std::size_t chain_index_ = 0, coeff_modulus_size_ = 0, poly_modulus_degree_ = 0;
@@ -214,12 +227,18 @@ public:
     std::size_t poly_modulus_degree() const { return poly_modulus_degree_; }
     cahel::parms_id_type &parms_id() { return parms_id_; }
     cahel::parms_id_type parms_id() const { return parms_id_; }
+    // the reference's byte layout (include/ciphertext.h:174-290); load checks the header against the context
+    void save(std::ostream &stream) const;
+    void load(const CAHELGPUContext &context, std::istream &stream);
 
     cahel::DeviceBuffer data_;
     std::size_t size_ = 0, chain_index_ = 0, coeff_modulus_size_ = 0, poly_modulus_degree_ = 0;
     double scale_ = 1.0;
     bool is_ntt_form_ = true, is_asymmetric_ = false;
     cahel::parms_id_type parms_id_ = cahel::parms_id_zero;
+    // the 64 seed bytes that close a ciphertext record (the reference keeps them on the device and fills them only
+    // when asked to save the seed, include/ciphertext.h:31, 205-213); kept here so that a record survives a round trip
+    std::array<std::uint8_t, 64> prng_seed_{};
 };
 
 // include/secretkey.h:20-108: a key-level ciphertext (-(a s + e), a)
@@ -235,6 +254,8 @@ public:
         encrypt_asymmetric(context, plain, cipher, save_seed);
         return cipher;
     }
+    void save(std::ostream &stream) const;  // include/secretkey.h:53-59: the pair as a ciphertext record
+    void load(const CAHELGPUContext &context, std::istream &stream);
     CAHELGPUCiphertext pk_;
     bool gen_flag_ = false;
 };
@@ -246,6 +267,8 @@ public:
     explicit CAHELGPURelinKey(const CAHELGPUContext &context);
     cahel::parms_id_type parms_id() const { return parms_id_; }
     std::vector<const uint64_t *> key_ptrs() const;
+    void save(std::ostream &stream) const;  // include/secretkey.h:212-256
+    void load(const CAHELGPUContext &context, std::istream &stream);
     std::vector<CAHELGPUPublicKey> public_keys_;
     std::size_t pk_num_ = 0;
     bool gen_flag_ = false;
@@ -258,6 +281,8 @@ public:
     CAHELGPUGaloisKey() = default;
     explicit CAHELGPUGaloisKey(const CAHELGPUContext &) {}
     cahel::parms_id_type parms_id() const { return parms_id_; }
+    void save(std::ostream &stream) const;  // include/secretkey.h:354-398
+    void load(const CAHELGPUContext &context, std::istream &stream);
     std::vector<CAHELGPURelinKey> relin_keys_;
     std::size_t relin_key_num_ = 0;
     bool gen_flag_ = false;

@@ -48,6 +48,25 @@ void EncryptionParameters::set_coeff_modulus(const std::vector<Modulus> &coeff_m
     coeff_modulus_ = coeff_modulus;
 }
 
+parms_id_type compute_parms_id(scheme_type scheme, std::size_t poly_modulus_degree, std::size_t special_modulus_size,
+                               const std::vector<uint64_t> &key_modulus, std::size_t limbs) {
+    if (limbs > key_modulus.size()) throw std::invalid_argument("more limbs than key moduli");
+    std::vector<uint64_t> words{(uint64_t)scheme, (uint64_t)poly_modulus_degree, (uint64_t)special_modulus_size};
+    words.insert(words.end(), key_modulus.begin(), key_modulus.end());
+    words.insert(words.end(), key_modulus.begin(), key_modulus.begin() + (std::ptrdiff_t)limbs);
+    words.push_back(0);  // plain modulus: one zero word outside BFV / BGV
+    parms_id_type id;
+    blake2b(id.data(), sizeof(id), words.data(), words.size() * sizeof(uint64_t));
+    if (id == parms_id_zero) throw std::logic_error("parms_id cannot be zero");
+    return id;
+}
+
+parms_id_type EncryptionParameters::parms_id() const {
+    std::vector<uint64_t> mods;
+    for (const auto &m : coeff_modulus_) mods.push_back(m.value());
+    return compute_parms_id(scheme_, poly_modulus_degree_, special_modulus_size_, mods, mods.size());
+}
+
 // ---------------------------------------------------------------------------------------------------
 // device memory pool
 // ---------------------------------------------------------------------------------------------------
@@ -297,6 +316,14 @@ CAHELGPUContext::CAHELGPUContext(const EncryptionParameters &params, bool expand
         const std::size_t levels = expand_mod_chain ? size_q_ : 1;
         for (std::size_t i = 0; i < levels; i++) chain_limbs_.push_back(size_q_ - i);
     }
+    {
+        // src/context.cu:352-401: the key level hashes all moduli, data level c the first size_q - c + 1 of them;
+        // a single-modulus chain has no special modulus
+        std::vector<uint64_t> vals;
+        for (auto &m : mods) vals.push_back(m.value());
+        for (std::size_t limbs : chain_limbs_)
+            parms_ids_.push_back(compute_parms_id(params.scheme(), n_, size_p_, vals, limbs));
+    }
     galois_elts_ = params.galois_elts();
     if (galois_elts_.empty()) {
         // include/galois.cuh / src/galois.cu:109-133: conjugation, then 5^(2^i) and 5^-(2^i)
@@ -331,20 +358,8 @@ std::size_t CAHELGPUContext::limbs_at(std::size_t chain_index) const {
 }
 
 parms_id_type CAHELGPUContext::parms_id_at(std::size_t chain_index) const {
-    uint64_t h = 0xcbf29ce484222325ull;
-    auto mix = [&h](uint64_t v) {
-        for (int i = 0; i < 8; i++) {
-            h ^= (v >> (8 * i)) & 0xff;
-            h *= 0x100000001b3ull;
-        }
-    };
-    mix((uint64_t)params_.scheme());
-    mix(n_);
-    const std::size_t limbs = limbs_at(chain_index);
-    mix(limbs);
-    const auto &mods = params_.coeff_modulus();
-    for (std::size_t i = 0; i < limbs; i++) mix(mods[i].value());
-    return h ? h : 1;
+    if (chain_index >= parms_ids_.size()) throw std::invalid_argument("chain index out of range");
+    return parms_ids_[chain_index];
 }
 
 int CAHELGPUContext::total_coeff_modulus_bit_count(std::size_t chain_index) const {

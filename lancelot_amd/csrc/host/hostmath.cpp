@@ -261,4 +261,82 @@ void BigUInt::reduce_small(const BigUInt &m) {
     while (compare(m) >= 0) sub(m);
 }
 
+// ---------------------------------------------------------------------------------------------------
+// BLAKE2b, RFC 7693 section 3: 12 rounds of the mixing function G over a 16-word working vector, message
+// words chosen by the SIGMA schedule, little-endian words throughout.
+// ---------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr uint64_t kBlakeIv[8] = {0x6a09e667f3bcc908ull, 0xbb67ae8584caa73bull, 0x3c6ef372fe94f82bull,
+                                  0xa54ff53a5f1d36f1ull, 0x510e527fade682d1ull, 0x9b05688c2b3e6c1full,
+                                  0x1f83d9abfb41bd6bull, 0x5be0cd19137e2179ull};
+
+constexpr uint8_t kBlakeSigma[10][16] = {
+    {0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15}, {14, 10, 4, 8, 9, 15, 13, 6, 1, 12, 0, 2, 11, 7, 5, 3},
+    {11, 8, 12, 0, 5, 2, 15, 13, 10, 14, 3, 6, 7, 1, 9, 4}, {7, 9, 3, 1, 13, 12, 11, 14, 2, 6, 5, 10, 4, 0, 15, 8},
+    {9, 0, 5, 7, 2, 4, 10, 15, 14, 1, 11, 12, 6, 8, 3, 13}, {2, 12, 6, 10, 0, 11, 8, 3, 4, 13, 7, 5, 15, 14, 1, 9},
+    {12, 5, 1, 15, 14, 13, 4, 10, 0, 7, 6, 3, 9, 2, 8, 11}, {13, 11, 7, 14, 12, 1, 3, 9, 5, 0, 15, 4, 8, 6, 2, 10},
+    {6, 15, 14, 9, 11, 3, 0, 8, 12, 2, 13, 7, 1, 4, 10, 5}, {10, 2, 8, 4, 7, 6, 1, 5, 15, 11, 9, 14, 3, 12, 13, 0}};
+
+inline uint64_t rotr64(uint64_t v, int r) { return (v >> r) | (v << (64 - r)); }
+
+// one 128-byte block; t = bytes hashed so far including this block (below 2^64 here), last = final block
+void blake_compress(uint64_t h[8], const uint8_t block[128], uint64_t t, bool last) {
+    uint64_t m[16], v[16];
+    for (int i = 0; i < 16; i++) {
+        uint64_t w = 0;
+        for (int b = 7; b >= 0; b--) w = (w << 8) | block[8 * i + b];
+        m[i] = w;
+    }
+    for (int i = 0; i < 8; i++) {
+        v[i] = h[i];
+        v[i + 8] = kBlakeIv[i];
+    }
+    v[12] ^= t;
+    if (last) v[14] = ~v[14];
+    auto g = [&](int a, int b, int c, int d, uint64_t x, uint64_t y) {
+        v[a] = v[a] + v[b] + x;
+        v[d] = rotr64(v[d] ^ v[a], 32);
+        v[c] = v[c] + v[d];
+        v[b] = rotr64(v[b] ^ v[c], 24);
+        v[a] = v[a] + v[b] + y;
+        v[d] = rotr64(v[d] ^ v[a], 16);
+        v[c] = v[c] + v[d];
+        v[b] = rotr64(v[b] ^ v[c], 63);
+    };
+    for (int r = 0; r < 12; r++) {
+        const uint8_t *s = kBlakeSigma[r % 10];
+        g(0, 4, 8, 12, m[s[0]], m[s[1]]);
+        g(1, 5, 9, 13, m[s[2]], m[s[3]]);
+        g(2, 6, 10, 14, m[s[4]], m[s[5]]);
+        g(3, 7, 11, 15, m[s[6]], m[s[7]]);
+        g(0, 5, 10, 15, m[s[8]], m[s[9]]);
+        g(1, 6, 11, 12, m[s[10]], m[s[11]]);
+        g(2, 7, 8, 13, m[s[12]], m[s[13]]);
+        g(3, 4, 9, 14, m[s[14]], m[s[15]]);
+    }
+    for (int i = 0; i < 8; i++) h[i] ^= v[i] ^ v[i + 8];
+}
+
+}  // namespace
+
+void blake2b(void *out, size_t out_len, const void *in, size_t in_len) {
+    if (!out || out_len == 0 || out_len > 64 || (!in && in_len)) throw std::invalid_argument("blake2b: invalid argument");
+    uint64_t h[8];
+    for (int i = 0; i < 8; i++) h[i] = kBlakeIv[i];
+    h[0] ^= 0x01010000ull ^ (uint64_t)out_len;  // parameter block: digest length, no key, fanout = depth = 1
+    const uint8_t *src = static_cast<const uint8_t *>(in);
+    uint64_t done = 0;
+    // every block but the last (the last one is padded with zeros and may be empty only for an empty message)
+    while (in_len - done > 128) {
+        done += 128;
+        blake_compress(h, src + done - 128, done, false);
+    }
+    uint8_t tail[128] = {0};
+    for (size_t i = 0; i < in_len - done; i++) tail[i] = src[done + i];
+    blake_compress(h, tail, in_len, true);
+    uint8_t *dst = static_cast<uint8_t *>(out);
+    for (size_t i = 0; i < out_len; i++) dst[i] = (uint8_t)(h[i / 8] >> (8 * (i % 8)));
+}
+
 }  // namespace cahel

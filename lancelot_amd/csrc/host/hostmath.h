@@ -34,6 +34,10 @@ bool try_minimal_primitive_root(uint64_t degree, uint64_t q, uint64_t &root);
 // non-adjacent form: signed powers of two summing to value, least significant first
 std::vector<int> naf(int value);
 
+// BLAKE2b (RFC 7693), unkeyed, digest of 1..64 bytes: the hash behind the parameter identifiers
+// (cahel-main/include/util/hash.h:30-37 calls blake2b with a 32-byte digest).
+void blake2b(void *out, size_t out_len, const void *in, size_t in_len);
+
 // A modulus below 2^61 with its 128-bit Barrett ratio floor(2^128 / value).
 class Modulus {
 public:

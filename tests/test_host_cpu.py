@@ -162,3 +162,42 @@ def test_package_without_native_module_only_imports_for_the_build(tmp_path):
     as_module = subprocess.run([sys.executable, "-m", "lancelot_amd.build", "--help"], cwd=tmp_path, env=env,
                                capture_output=True, text=True)
     assert as_module.returncode == 0 and "libcahel_hip.so" in as_module.stdout
+
+
+def test_blake2b_known_answers(cahel):
+    """The hash behind the parameter identifiers: RFC 7693 appendix A ("abc", 64-byte digest) and Python's own
+    BLAKE2b over lengths around the 128-byte block boundary, for several digest sizes."""
+    import hashlib
+    rfc = ("ba80a53f981c4d0d6a2797b69f12f6e94c212f14685ac4b74b12bb6fdbffa2d1"
+           "7d87c5392aab792dc252d5de4533cc9518d38aa8dbf1925ab92386edd4009923")
+    assert cahel._blake2b(b"abc", 64).hex() == rfc
+    for n in (0, 1, 3, 64, 127, 128, 129, 255, 256, 257, 1000):
+        data = bytes((7 * i + 3) & 255 for i in range(n))
+        for size in (1, 20, 32, 64):
+            assert cahel._blake2b(data, size) == hashlib.blake2b(data, digest_size=size).digest(), (n, size)
+    with pytest.raises(ValueError):
+        cahel._blake2b(b"", 65)
+
+
+def test_parms_id_hashes_the_reference_words(cahel):
+    """parms_id = BLAKE2b-256 over the 64-bit words (scheme, degree, special modulus count, key moduli, coefficient
+    moduli, plain modulus = 0), include/util/encryptionparams.h:337-379; it changes with every one of them."""
+    import hashlib
+    import struct
+
+    def make(n, bits, special, scheme=None):
+        p = cahel.params(scheme or cahel.scheme_type.ckks)
+        p.set_poly_modulus_degree(n)
+        mods = cahel.coeff_modulus_create(n, bits)
+        p.set_coeff_modulus(mods)
+        p.set_special_modulus_size(special)
+        return p, [m.value() for m in mods]
+
+    p, vals = make(8192, [60, 40, 40, 60], 1)
+    words = [3, 8192, 1] + vals + vals + [0]
+    digest = hashlib.blake2b(struct.pack("<%dQ" % len(words), *words), digest_size=32).digest()
+    assert p.parms_id() == struct.unpack("<4Q", digest)
+    others = [make(4096, [60, 40, 40, 60], 1)[0], make(8192, [60, 40, 40, 60], 2)[0], make(8192, [60, 40, 41, 60], 1)[0],
+              make(8192, [60, 40, 40, 60], 1, cahel.scheme_type.bfv)[0]]
+    ids = {p.parms_id()} | {o.parms_id() for o in others}
+    assert len(ids) == 5
