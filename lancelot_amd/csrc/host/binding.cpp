@@ -87,7 +87,22 @@ PYBIND11_MODULE(pyCAHEL, m) {
         .def("set_special_modulus_size", &EncryptionParameters::set_special_modulus_size)
         .def("set_galois_elts", &EncryptionParameters::set_galois_elts)
         .def("set_coeff_modulus", &EncryptionParameters::set_coeff_modulus)
-        .def("parms_id", [](const EncryptionParameters &p) { return id_tuple(p.parms_id()); });
+        .def("parms_id", [](const EncryptionParameters &p) { return id_tuple(p.parms_id()); })
+        .def("poly_modulus_degree", &EncryptionParameters::poly_modulus_degree)
+        .def("coeff_modulus", [](const EncryptionParameters &p) {
+            std::vector<uint64_t> v;
+            for (const auto &mod : p.coeff_modulus()) v.push_back(mod.value());
+            return v;
+        })
+        .def("to_bytes", [](const EncryptionParameters &p) {
+            std::ostringstream s(std::ios::binary);
+            p.save(s);
+            return py::bytes(s.str());
+        })
+        .def("from_bytes", [](EncryptionParameters &p, const py::bytes &data) {
+            std::istringstream s(std::string(data), std::ios::binary);
+            p.load(s);
+        });
     m.def("_blake2b", [](const py::bytes &data, std::size_t digest_size) {
         const std::string in(data);
         std::string out(digest_size, '\0');

@@ -53,6 +53,10 @@ public:
     const std::vector<uint32_t> &galois_elts() const { return galois_elts_; }
     // identifier of the key level (all moduli), as include/util/encryptionparams.h:315-317 returns it
     parms_id_type parms_id() const;
+    // include/util/encryptionparams.h:302-308, 381-474: scheme u8 | degree u64 | count u64 | moduli u64... | plain
+    // modulus u64 (0); the special modulus count and the Galois elements are not part of the record
+    void save(std::ostream &stream) const;
+    void load(std::istream &stream);
 
 private:
     scheme_type scheme_;

@@ -3,6 +3,8 @@
 // 212-256, 354-398), so that files written by either side can be read by the other.  Everything is little-endian
 // and unpadded:
 //
+//   parameters  scheme u8 | N u64 | count u64 | moduli[count] u64 | plain modulus u64 (include/util/
+//               encryptionparams.h:381-474, src/modulus.cu:134-178)
 //   plaintext   parms_id[32] | limbs u64 | chain u64 | N u64 | scale f64 | words u64 | data[words] u64
 //   ciphertext  parms_id[32] | ntt u8 | chain u64 | size u64 | N u64 | limbs u64 | scale f64 | words u64 |
 //               data[words] u64 | seed[64]
@@ -90,6 +92,37 @@ void check_header(const CAHELGPUContext &context, const parms_id_type &id, uint6
 }
 
 }  // namespace
+
+// ---------------------------------------------------------------------------------------------------
+// parameters
+// ---------------------------------------------------------------------------------------------------
+void EncryptionParameters::save(std::ostream &stream) const {
+    io_section(stream, [&] {
+        put<uint8_t>(stream, (uint8_t)scheme_);
+        put<uint64_t>(stream, poly_modulus_degree_);
+        put<uint64_t>(stream, coeff_modulus_.size());
+        for (const auto &m : coeff_modulus_) put<uint64_t>(stream, m.value());
+        put<uint64_t>(stream, 0);  // plain modulus: BFV / BGV only
+    });
+}
+
+void EncryptionParameters::load(std::istream &stream) {
+    io_section(stream, [&] {
+        const uint8_t scheme = get<uint8_t>(stream);
+        if (scheme > (uint8_t)scheme_type::ckks) throw std::invalid_argument("unsupported scheme");
+        EncryptionParameters fresh((scheme_type)scheme);
+        const uint64_t degree = get<uint64_t>(stream), count = get<uint64_t>(stream);
+        if (degree > 131072) throw std::logic_error("poly_modulus_degree is invalid");  // CAHEL_POLY_MOD_DEGREE_MAX
+        if (count > 64) throw std::logic_error("coeff_modulus is invalid");
+        std::vector<Modulus> moduli;
+        for (uint64_t i = 0; i < count; i++) moduli.emplace_back(get<uint64_t>(stream));
+        if (get<uint64_t>(stream) != 0 && (scheme_type)scheme == scheme_type::ckks)
+            throw std::logic_error("plain_modulus is not supported for this scheme");
+        fresh.set_poly_modulus_degree((std::size_t)degree);
+        fresh.set_coeff_modulus(moduli);
+        *this = std::move(fresh);
+    });
+}
 
 // ---------------------------------------------------------------------------------------------------
 // plaintext

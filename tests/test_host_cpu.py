@@ -201,3 +201,26 @@ def test_parms_id_hashes_the_reference_words(cahel):
               make(8192, [60, 40, 40, 60], 1, cahel.scheme_type.bfv)[0]]
     ids = {p.parms_id()} | {o.parms_id() for o in others}
     assert len(ids) == 5
+
+
+def test_params_record_layout_and_round_trip(cahel):
+    """EncryptionParameters.save: scheme u8 | degree u64 | count u64 | moduli | plain modulus 0
+    (include/util/encryptionparams.h:381-409, src/modulus.cu:134-155); load gives the same parameters and
+    identifier back, refuses a bad scheme byte or modulus, and reports truncation as an I/O error."""
+    import struct
+    p = cahel.params(cahel.scheme_type.ckks)
+    p.set_poly_modulus_degree(4096)
+    mods = [m.value() for m in cahel.coeff_modulus_create(4096, [50, 40, 50])]
+    p.set_coeff_modulus([cahel.modulus(v) for v in mods])
+    blob = p.to_bytes()
+    assert blob == struct.pack("<BQQ", 3, 4096, 3) + struct.pack("<3Q", *mods) + struct.pack("<Q", 0)
+    q = cahel.params(cahel.scheme_type.bfv)
+    q.from_bytes(blob)
+    assert (q.poly_modulus_degree(), q.coeff_modulus(), q.parms_id()) == (4096, mods, p.parms_id())
+    with pytest.raises(RuntimeError, match="I/O error"):
+        q.from_bytes(blob[:-3])
+    with pytest.raises(ValueError):
+        q.from_bytes(bytes([7]) + blob[1:])                                   # no such scheme
+    with pytest.raises(ValueError):
+        q.from_bytes(blob[:17] + struct.pack("<Q", 1) + blob[25:])            # modulus 1
+    assert (q.poly_modulus_degree(), q.coeff_modulus()) == (4096, mods)       # failed loads change nothing
