@@ -36,7 +36,10 @@ class KrumConfig:
                                              # 0: the reference's split, hoisting(1..15) then one rotation per doubling
     sum_drop_levels: int = 0                 # limbs dropped without scaling (mod_switch_to_next) after the rescale:
                                              # the slot sum's key switches then run over fewer limbs; 0 = as the
-                                             # reference, which rotates at the level the rescale leaves
+                                             # reference, which rotates at the level the rescale leaves.  The
+                                             # moduli that remain must still hold distance * scale (with one limb
+                                             # left that is the first prime alone: 60 bits are enough for the
+                                             # benchmark's distances at scale 2^40, 50 bits are not)
     batched: bool = True                     # all pairs go through every stage together, one launch per stage
                                              # (pair_square_distances); False: pair by pair over the lanes
     lanes: int = 3                           # host threads / streams that the pairs are dealt to (0: null stream);
