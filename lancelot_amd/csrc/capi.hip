@@ -64,6 +64,7 @@ struct he_context {
     bool fuse_inner = true;      // environment CAHEL_HIP_NO_FUSED_KS=1: separate NTT and inner-product kernels
     uint64_t fp_mask = 0;        // bit t: table t has a prime below 2^50
     bool mixed_ok = false;       // mixed launches allowed (at most 64 tables; CAHEL_HIP_NO_MIXED=1 switches them off)
+    int rows_direct = 1;         // environment CAHEL_HIP_ROWS_VIA_LDS=1: every half-pass of the rows pass through LDS
     bool fuse_modup_rows = true; // environment CAHEL_HIP_NO_FUSED_MODUP=1: base conversion and rows pass as two kernels
     uint32_t modup_group = 6;    // output limbs per workgroup of the fused kernel (CAHEL_HIP_MODUP_GROUP)
     std::vector<Level> levels;   // indexed by L
@@ -115,6 +116,7 @@ NttArgs base_args(const he_context *ctx, bool forward) {
     a.log_n = ctx->log_n;
     a.epi_b_mask = 0xffffffffu;
     a.fp_mask = ctx->fp_mask;
+    a.rows_direct = ctx->rows_direct;
     return a;
 }
 
@@ -350,6 +352,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->fuse_inner = !(nf && nf[0] == '1');
         const char *nx = getenv("CAHEL_HIP_NO_MIXED");
         ctx->mixed_ok = qp <= 64 && !(nx && nx[0] == '1');
+        const char *rv = getenv("CAHEL_HIP_ROWS_VIA_LDS");
+        ctx->rows_direct = !(rv && rv[0] == '1');
         const char *nm = getenv("CAHEL_HIP_NO_FUSED_MODUP");
         ctx->fuse_modup_rows = !(nm && nm[0] == '1');
         if (const char *g = getenv("CAHEL_HIP_MODUP_GROUP")) {

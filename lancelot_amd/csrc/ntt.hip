@@ -166,6 +166,141 @@ __device__ __forceinline__ FpTw inverse_scale(const NttArgs &a, const Job &job, 
 }
 
 // ---------------------------------------------------------------------------------------------------
+// rows pass at N = 2^16 with full tiles (256 rows x 16 columns, 256 threads): both half-passes are radix-16 with
+// exactly one group per thread, and the 16 words a thread needs for the outer half-pass (rows r, r + 16, ...) are
+// 16 coalesced accesses.  So the outer half-pass runs on registers straight from / to global memory and the tile
+// crosses LDS once, between the half-passes, instead of three times: the pass is bound by the latency of one
+// workgroup, and two of its three LDS round trips and barriers go away.  Same arithmetic, same words.
+//   far  (stages 0-3 forward): element j of thread t is row (t >> 4) + 16 j, column t & 15; twiddle index 1
+//   near (stages 4-7 forward): element j is row (t >> 4) * 16 + j, column t & 15; twiddle index 16 + (t >> 4)
+// ---------------------------------------------------------------------------------------------------
+template <bool FWD, int BE>
+__device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, uint32_t col0, uint64_t *lds) {
+    const uint32_t t = threadIdx.x, upper = t >> 4, col = t & 15;
+    double *ld = reinterpret_cast<double *>(lds);
+    size_t g_far[16], g_near[16];
+    uint32_t l_far[16], l_near[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) {
+        g_far[j] = (size_t)(upper + 16 * j) * 256 + col0 + col;
+        g_near[j] = (size_t)(upper * 16 + j) * 256 + col0 + col;
+        l_far[j] = skew(t + 256u * j);
+        l_near[j] = skew(upper * 256u + col + 16u * j);
+    }
+    const bool fp = BE == NTT_BACKEND_FP || (BE == NTT_BACKEND_MIXED && ((a.fp_mask >> job.table) & 1));
+    if (BE != NTT_BACKEND_INT && fp) {
+        const FpCtx c = fp_ctx(a, job.table);
+        double v[16];
+        if (FWD) {
+            if (a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
+                const uint64_t *tsrc = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+                const uint64_t *dsrc = a.pro_src2 + ((size_t)job.poly * a.pro2_poly_stride << a.log_n);
+                const FpMod ml = fp_ctx(a, a.pro_last).m;
+                const double wd = fp_from_u64(a.pro_w[2 * job.limb]), wl = fp_from_u64(a.pro_w[2 * a.pro_last]);
+                const FpTw w{wd, wd * c.m.qinv}, wlast{wl, wl * ml.qinv};
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    // coefficient of the dropped limb of the ModDown result, canonical mod q_last
+                    const double r = fp_canonical(
+                        fp_from_u64(tsrc[g_far[j]]) - fp_mulmod(fp_from_u64(dsrc[g_far[j]]), wlast, ml), ml);
+                    v[j] = fp_mulmod(fp_from_u64(job.in[g_far[j]]), w, c.m) + fp_reduce(r, c.m);
+                }
+                fp_ct_block<4, true>(v, c.tw, 1u, c.m);
+            } else if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE) {
+                // one source limb for every limb: it may exceed this limb's prime, so reduce first
+                const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = fp_from_u64(src[g_far[j]]);
+                fp_ct_block<4, true>(v, c.tw, 1u, c.m);
+            } else {
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = fp_from_u64(job.in[g_far[j]]);
+                fp_ct_block<4, false>(v, c.tw, 1u, c.m);
+            }
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[l_far[j]] = v[j];
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[l_near[j]];
+            fp_ct_block<4, true>(v, c.tw, 16u + upper, c.m);
+            // lazy signed doubles go to the blocks pass
+#pragma unroll
+            for (int j = 0; j < 16; j++) job.out[g_near[j]] = (uint64_t)__double_as_longlong(v[j]);
+        } else {
+            // input: lazy signed doubles from the blocks pass; output: canonical residues
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = __longlong_as_double((long long)job.in[g_near[j]]);
+            fp_gs_block<4, true>(v, c.tw, 16u + upper, c.m);
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[l_near[j]] = v[j];
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[l_far[j]];
+            fp_gs_block<4, true>(v, c.tw, 1u, c.m);
+            const FpTw scale = inverse_scale(a, job, c.m);
+#pragma unroll
+            for (int j = 0; j < 16; j++)
+                job.out[g_far[j]] = fp_to_u64(fp_canonical(fp_mulmod(v[j], scale, c.m), c.m));
+        }
+        return;
+    }
+
+    const IntCtx c = int_ctx(a, job.table);
+    const uint64_t q = c.q;
+    uint64_t v[16];
+    if (FWD) {
+        if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE) {
+            const uint64_t r1 = a.barrett[2 * job.table + 1];
+            const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = barrett64(src[g_far[j]], q, r1);
+        } else if (a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
+            const uint64_t r1 = a.barrett[2 * job.table + 1];
+            const uint64_t *tsrc = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+            const uint64_t *dsrc = a.pro_src2 + ((size_t)job.poly * a.pro2_poly_stride << a.log_n);
+            const uint64_t ql = a.moduli[a.pro_last];
+            const Shoup w = load_shoup(a.pro_w, job.limb), wlast = load_shoup(a.pro_w, a.pro_last);
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const uint64_t r = sub_mod(tsrc[g_far[j]], mul_shoup(dsrc[g_far[j]], wlast, ql), ql);
+                v[j] = add_mod(mul_shoup(job.in[g_far[j]], w, q), barrett64(r, q, r1), q);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = job.in[g_far[j]];
+        }
+        ct_block<4>(v, c.tw, 1u, q);
+#pragma unroll
+        for (int j = 0; j < 16; j++) lds[l_far[j]] = v[j];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = lds[l_near[j]];
+        ct_block<4>(v, c.tw, 16u + upper, q);
+        // lazy values in [0, 4q) go to the blocks pass
+#pragma unroll
+        for (int j = 0; j < 16; j++) job.out[g_near[j]] = v[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = job.in[g_near[j]];
+        gs_block<4>(v, c.tw, 16u + upper, q);
+#pragma unroll
+        for (int j = 0; j < 16; j++) lds[l_near[j]] = v[j];
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = lds[l_far[j]];
+        gs_block<4>(v, c.tw, 1u, q);
+        if (a.epi_mode == NTT_EPI_MUL) {
+            const Shoup w = load_shoup(a.w, job.limb);
+#pragma unroll
+            for (int j = 0; j < 16; j++) job.out[g_far[j]] = mul_shoup(v[j], w, q);
+        } else {
+#pragma unroll
+            for (int j = 0; j < 16; j++) job.out[g_far[j]] = reduce_2q(v[j], q);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // rows pass: stages 0 .. LD-1 (forward) over an R = 2^LD rows x 256 matrix
 // ---------------------------------------------------------------------------------------------------
 template <int LD, bool FWD, int BE, int TL>
@@ -181,6 +316,12 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     const uint32_t lb = logical_block();
     const Job job = decode_job(a, lb / tiles_per_limb);
     const uint32_t col0 = (lb % tiles_per_limb) << LOGC;
+    if constexpr (LD == 8 && TL == 12) {
+        if (a.rows_direct) {
+            rows_direct<FWD, BE>(a, job, col0, lds);
+            return;
+        }
+    }
     double *ld = reinterpret_cast<double *>(lds);
 
     // the back end of this workgroup's limb: fixed by the launch, or (mixed) by the limb's prime
