@@ -170,7 +170,7 @@ struct BconvBatch {
 };
 hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s);
 
-// ModUp base conversion fused with the rows pass of the forward transform (FP64 back end, N >= 2^13): reads the
+// ModUp base conversion fused with the rows pass of the forward transform (FP64 back end, 2^13 <= N <= 2^15): reads the
 // scaled coefficient-form limbs x [L][N], writes the rows-pass output of every converted limb into y
 // [beta][L+K][N] (the layout and tables of BconvBatch for ModUp).  `group` output limbs per workgroup.
 struct ModupRowsArgs {

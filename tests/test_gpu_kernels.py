@@ -178,7 +178,7 @@ def test_mixed_back_end_agrees_with_the_integer_one(oracle, capi, monkeypatch, l
                                                  (11, [45, 40, 40, 50], 1, 3), (9, [40, 40, 45, 45], 2, 2)])
 def test_fused_and_separate_key_switch_agree(oracle, capi, monkeypatch, logn, bits, size_p, L):
     """he_keyswitch with the inner product inside the forward NTT and the base conversion inside its rows pass
-    (defaults for primes below 2^50; the latter from N = 2^13), and, forced by the environment, with the separate
+    (defaults for primes below 2^50; the latter for N = 2^13 to 2^15), and, forced by the environment, with the separate
     kernels: all equal the oracle, with and without a Galois element, with a partial last digit (L = 3 over two
     special primes, L = 5 over three), with output groups that end inside a round of four, and at the smallest
     degree."""
@@ -583,6 +583,38 @@ def test_keyswitch_benchmark_shape(full, capi):
     capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, 0, ws.ptr, None))
     ks = p.key_switch(c, host_evk)
     assert (dct.numpy() == np.stack([p.add(ct[b], ks[b]) for b in range(2)])).all()
+
+
+@pytest.mark.parametrize("no_fp", ["0", "1"])
+def test_rows_pass_on_registers_at_benchmark_shape(oracle, capi, monkeypatch, no_fp):
+    """N = 2^16 with enough limbs for full tiles: the rows pass keeps its outer half on registers.  Both back ends
+    (FP64, and the integer one forced by the environment) against the oracle: plain forward and inverse transforms,
+    the rescale (prologue that broadcasts the last limb) and key switch + rescale (prologue of the merged ModDown +
+    rescale, inverse transform with a scaling epilogue)."""
+    monkeypatch.setenv("CAHEL_HIP_NO_FP64", no_fp)
+    cahel, parms, ctx, p = make_pair(oracle, 16, [50] * 32, 8)
+    rng = np.random.default_rng(33)
+    lib, h = capi.lib(), ctx.he_handle()
+    L = 24
+    x = rand_limbs(p, rng, range(L), n_polys=2)
+    x[0, 1, :] = p.moduli[1] - 1                               # a whole limb of q - 1: the largest lazy values
+    d = DeviceArray(capi, host=x)
+    capi.check(lib.he_ntt_forward(h, d.ptr, 2, L, L, 0, L, 0, None))
+    assert (d.numpy() == np.stack([p.ntt_fwd(x[i].copy()) for i in range(2)])).all()
+    d = DeviceArray(capi, host=x)
+    capi.check(lib.he_ntt_inverse(h, d.ptr, 2, L, L, 0, L, 0, None))
+    assert (d.numpy() == np.stack([p.ntt_inv(x[i].copy()) for i in range(2)])).all()
+    dres = DeviceArray(capi, shape=(2, L - 1, p.n))
+    rws = DeviceArray(capi, shape=(2, p.n))
+    capi.check(lib.he_rescale(h, DeviceArray(capi, host=x).ptr, dres.ptr, 2, L, rws.ptr, None))
+    assert (dres.numpy() == p.rescale(x)).all()
+    c = rand_limbs(p, rng, range(L))
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=x)
+    ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    capi.check(lib.he_keyswitch_rescale(h, L, dc.ptr, ptrs, dct.ptr, dres.ptr, 0, ws.ptr, None))
+    ks = p.key_switch(c, host_evk)
+    assert (dres.numpy() == p.rescale(np.stack([p.add(x[b], ks[b]) for b in range(2)]))).all()
 
 
 def test_samplers(small, capi, oracle):
