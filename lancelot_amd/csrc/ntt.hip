@@ -166,17 +166,19 @@ __device__ __forceinline__ FpTw inverse_scale(const NttArgs &a, const Job &job, 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// rows pass at N = 2^16 with full tiles (256 rows x 16 columns, 256 threads): both half-passes are radix-16 with
-// exactly one group per thread, and the 16 words a thread needs for the outer half-pass (rows r, r + 16, ...) are
-// 16 coalesced accesses.  So the outer half-pass runs on registers straight from / to global memory and the tile
-// crosses LDS once, between the half-passes, instead of three times: the pass is bound by the latency of one
-// workgroup, and two of its three LDS round trips and barriers go away.  Same arithmetic, same words.
-//   far  (stages 0-3 forward): element j of thread t is row (t >> 4) + 16 j, column t & 15; twiddle index 1
-//   near (stages 4-7 forward): element j is row (t >> 4) * 16 + j, column t & 15; twiddle index 16 + (t >> 4)
+// rows pass at N = 2^16 (256 rows x C columns per tile, C = 16 or 4, 16 C threads): both half-passes are radix-16
+// with exactly one group per thread, and the 16 words a thread needs for the outer half-pass (rows r, r + 16, ...)
+// are 16 accesses that neighbouring threads share lines of (C consecutive words per row).  So the outer half-pass
+// runs on registers straight from / to global memory and the tile crosses LDS once, between the half-passes,
+// instead of three times: the pass is bound by the latency of one workgroup, and two of its three LDS round trips
+// and barriers go away.  Same arithmetic, same words.  With u = t / C and c = t mod C:
+//   far  (stages 0-3 forward): element j of thread t is row u + 16 j, column c; twiddle index 1
+//   near (stages 4-7 forward): element j is row 16 u + j, column c; twiddle index 16 + u
 // ---------------------------------------------------------------------------------------------------
-template <bool FWD, int BE>
+template <bool FWD, int BE, int LOGC>
 __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, uint32_t col0, uint64_t *lds) {
-    const uint32_t t = threadIdx.x, upper = t >> 4, col = t & 15;
+    constexpr uint32_t C = 1u << LOGC, T = 16u << LOGC;
+    const uint32_t t = threadIdx.x, upper = t >> LOGC, col = t & (C - 1);
     double *ld = reinterpret_cast<double *>(lds);
     size_t g_far[16], g_near[16];
     uint32_t l_far[16], l_near[16];
@@ -184,8 +186,8 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
     for (int j = 0; j < 16; j++) {
         g_far[j] = (size_t)(upper + 16 * j) * 256 + col0 + col;
         g_near[j] = (size_t)(upper * 16 + j) * 256 + col0 + col;
-        l_far[j] = skew(t + 256u * j);
-        l_near[j] = skew(upper * 256u + col + 16u * j);
+        l_far[j] = skew(t + T * j);
+        l_near[j] = skew(upper * T + col + C * j);
     }
     const bool fp = BE == NTT_BACKEND_FP || (BE == NTT_BACKEND_MIXED && ((a.fp_mask >> job.table) & 1));
     if (BE != NTT_BACKEND_INT && fp) {
@@ -316,9 +318,9 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     const uint32_t lb = logical_block();
     const Job job = decode_job(a, lb / tiles_per_limb);
     const uint32_t col0 = (lb % tiles_per_limb) << LOGC;
-    if constexpr (LD == 8 && TL == 12) {
+    if constexpr (LD == 8 && (TL == 12 || TL == 10)) {
         if (a.rows_direct) {
-            rows_direct<FWD, BE>(a, job, col0, lds);
+            rows_direct<FWD, BE, LOGC>(a, job, col0, lds);
             return;
         }
     }

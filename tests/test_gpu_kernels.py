@@ -615,6 +615,24 @@ def test_rows_pass_on_registers_at_benchmark_shape(oracle, capi, monkeypatch, no
     capi.check(lib.he_keyswitch_rescale(h, L, dc.ptr, ptrs, dct.ptr, dres.ptr, 0, ws.ptr, None))
     ks = p.key_switch(c, host_evk)
     assert (dres.numpy() == p.rescale(np.stack([p.add(x[b], ks[b]) for b in range(2)]))).all()
+    # the same at L = 8: launches of fewer than 16 limbs take quarter tiles (256 rows x 4 columns, 64 threads)
+    L = 8
+    x = rand_limbs(p, rng, range(L), n_polys=2)
+    d = DeviceArray(capi, host=x)
+    capi.check(lib.he_ntt_forward(h, d.ptr, 2, L, L, 0, L, 0, None))
+    assert (d.numpy() == np.stack([p.ntt_fwd(x[i].copy(), list(range(L))) for i in range(2)])).all()
+    d = DeviceArray(capi, host=x)
+    capi.check(lib.he_ntt_inverse(h, d.ptr, 2, L, L, 0, L, 0, None))
+    assert (d.numpy() == np.stack([p.ntt_inv(x[i].copy(), list(range(L))) for i in range(2)])).all()
+    dres = DeviceArray(capi, shape=(2, L - 1, p.n))
+    capi.check(lib.he_rescale(h, DeviceArray(capi, host=x).ptr, dres.ptr, 2, L, rws.ptr, None))
+    assert (dres.numpy() == p.rescale(x)).all()
+    c = rand_limbs(p, rng, range(L))
+    dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=x)
+    ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    capi.check(lib.he_keyswitch_rescale(h, L, dc.ptr, ptrs, dct.ptr, dres.ptr, 0, ws.ptr, None))
+    ks = p.key_switch(c, host_evk)
+    assert (dres.numpy() == p.rescale(np.stack([p.add(x[b], ks[b]) for b in range(2)]))).all()
 
 
 def test_samplers(small, capi, oracle):
