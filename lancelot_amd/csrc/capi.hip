@@ -64,7 +64,8 @@ struct he_context {
     bool fuse_inner = true;      // environment CAHEL_HIP_NO_FUSED_KS=1: separate NTT and inner-product kernels
     uint64_t fp_mask = 0;        // bit t: table t has a prime below 2^50
     bool mixed_ok = false;       // mixed launches allowed (at most 64 tables; CAHEL_HIP_NO_MIXED=1 switches them off)
-    int rows_direct = 1;         // environment CAHEL_HIP_ROWS_VIA_LDS=1: every half-pass of the rows pass through LDS
+    int rows_direct = 1;         // environment CAHEL_HIP_ROWS_VIA_LDS=1: every register block of the rows pass (and of the
+                                 // fused inner-product kernel) takes its operands from LDS
     bool fuse_modup_rows = true; // environment CAHEL_HIP_NO_FUSED_MODUP=1: base conversion and rows pass as two kernels
     uint32_t modup_group = 6;    // output limbs per workgroup of the fused kernel (CAHEL_HIP_MODUP_GROUP)
     std::vector<Level> levels;   // indexed by L

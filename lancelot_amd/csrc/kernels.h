@@ -63,7 +63,8 @@ struct NttArgs {
     const double *tw_fp;      // [tables][N] twiddles as exact doubles for the FP64 back end (primes below 2^50)
     const double *fp_consts;  // [tables][4]: q, 1/q, N^-1 mod q, (N^-1 mod q)/q
     uint64_t fp_mask;         // bit t: table t has a prime below 2^50 (read by the mixed back end only)
-    int rows_direct;          // N = 2^16: rows pass with its outer half-pass on registers (one LDS exchange)
+    int rows_direct;          // N = 2^16: rows pass with its outer half-pass on registers (one LDS exchange); fused
+                              // inner-product kernel: first register block straight from global memory
     const uint64_t *moduli;   // [tables]
     const uint64_t *barrett;  // [tables][2]
     const LimbJob *jobs;      // explicit list (then in/out limbs are absolute, no prologue/epilogue)

@@ -820,19 +820,31 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
         uint64_t pk[kPer];
 #pragma unroll
         for (int i = 0; i < kPer; i++) pk[i] = key[tid + i * half];
-        if (!role) {
+        if (!role && a.rows_direct) {
+            // the 16 words of the first register block (stride 16 inside a 256-block) straight from global memory:
+            // 16 neighbouring threads read one 128-byte line per access
             const uint64_t *src = a.out + ((size_t)d * LK + t) * n + off;  // lazy values left by the rows pass
-#pragma unroll
-            for (int i = 0; i < kPer; i++) lds[skew(tid + i * half)] = src[tid + i * half];
-        }
-        lds_barrier();
-        if (!role) {
             double v[16];
 #pragma unroll
-            for (int j = 0; j < 16; j++) v[j] = ld[skew(base0 + (j << 4))];
+            for (int j = 0; j < 16; j++) v[j] = __longlong_as_double((long long)src[base0 + (j << 4)]);
             fp_ct_block<4, true>(v, fc.tw, idx0, m);
 #pragma unroll
             for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
+        } else if (!a.rows_direct) {
+            if (!role) {
+                const uint64_t *src = a.out + ((size_t)d * LK + t) * n + off;
+#pragma unroll
+                for (int i = 0; i < kPer; i++) lds[skew(tid + i * half)] = src[tid + i * half];
+            }
+            lds_barrier();
+            if (!role) {
+                double v[16];
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = ld[skew(base0 + (j << 4))];
+                fp_ct_block<4, true>(v, fc.tw, idx0, m);
+#pragma unroll
+                for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
+            }
         }
         lds_barrier();
         if (!role) {
