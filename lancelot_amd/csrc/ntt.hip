@@ -23,6 +23,8 @@
 //             butterfly, see modarith.cuh); values between the two passes are lazy signed doubles stored
 //             in the same 8-byte words; the factor 1/N is folded into the last multiplication
 // A launch uses the FP64 back end when every limb it touches has a prime below 2^50.
+#include <type_traits>
+
 #include "kernels.h"
 #include "modarith.cuh"
 
@@ -166,34 +168,56 @@ __device__ __forceinline__ FpTw inverse_scale(const NttArgs &a, const Job &job, 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// rows pass at N = 2^16 (256 rows x C columns per tile, C = 16 or 4, 16 C threads): both half-passes are radix-16
-// with exactly one group per thread, and the 16 words a thread needs for the outer half-pass (rows r, r + 16, ...)
-// are 16 accesses that neighbouring threads share lines of (C consecutive words per row).  So the outer half-pass
-// runs on registers straight from / to global memory and the tile crosses LDS once, between the half-passes,
-// instead of three times: the pass is bound by the latency of one workgroup, and two of its three LDS round trips
-// and barriers go away.  Same arithmetic, same words.  With u = t / C and c = t mod C:
-//   far  (stages 0-3 forward): element j of thread t is row u + 16 j, column c; twiddle index 1
-//   near (stages 4-7 forward): element j is row 16 u + j, column c; twiddle index 16 + u
+// rows pass with 16 words per thread (N >= 2^12: a tile of 2^LD rows x C columns is 16 T words for its T threads).
+// The stages split into an outer block of p0 and an inner block of p1 = LD - p0 stages.  The words of a thread's
+// outer groups are t, t + T, ..., t + 15 T in tile order, i.e. what a coalesced load of the tile hands to thread t
+// anyway, so the outer block runs on registers straight from (forward) or to (inverse) global memory and the
+// tile crosses LDS once, between the blocks, instead of three times (no LDS at all when p1 = 0): the pass is
+// bound by the latency of one workgroup, and two of its three LDS round trips and barriers go away.  Same
+// arithmetic, same words.
+//   outer: register i is tile word t + T i; group k of 16 >> p0 holds registers k + (16 >> p0) j; twiddle index 1
+//   inner: group k of 16 >> p1 is group g = t + T k of the tile: registers k 2^p1 + j are the tile words
+//          ((g / C) << (LOGC + p1)) + g mod C + j C; twiddle index 2^p0 + g / C
+// Tile word e lives at row e / C, column col0 + e mod C of the limb's (N / 256) x 256 view.
 // ---------------------------------------------------------------------------------------------------
-template <bool FWD, int BE, int LOGC>
+template <int LD, bool FWD, int BE, int LOGC>
 __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, uint32_t col0, uint64_t *lds) {
-    constexpr uint32_t C = 1u << LOGC, T = 16u << LOGC;
-    const uint32_t t = threadIdx.x, upper = t >> LOGC, col = t & (C - 1);
+    constexpr int p0 = Split<LD>::p0, p1 = Split<LD>::p1;
+    constexpr int R0 = 1 << p0, R1 = 1 << p1, NG0 = 16 >> p0, NG1 = 16 >> p1;
+    constexpr uint32_t C = 1u << LOGC, T = 1u << (LD + LOGC - 4);
+    const uint32_t t = threadIdx.x, col = t & (C - 1);
     double *ld = reinterpret_cast<double *>(lds);
-    size_t g_far[16], g_near[16];
-    uint32_t l_far[16], l_near[16];
+    // tile word, global offset and LDS slot of register i in the outer and in the inner layout (folded to a few
+    // shifts and adds where they are used; tables of them would have to stay live across both back ends)
+    auto e_far = [&](int i) { return t + T * (uint32_t)i; };
+    auto e_near = [&](int i) {
+        const uint32_t upper = (t + T * (uint32_t)(i >> p1)) >> LOGC;
+        return (upper << (LOGC + p1)) + col + ((uint32_t)(i & (R1 - 1)) << LOGC);
+    };
+    auto glob = [&](uint32_t e) { return (size_t)(e >> LOGC) * 256 + col0 + col; };
+    auto idx_near = [&](int k) { return (1u << p0) + ((t + T * (uint32_t)k) >> LOGC); };
+    // the outer / inner block on every group of the 16 registers
+    auto outer = [&](auto *v, auto block) {
 #pragma unroll
-    for (int j = 0; j < 16; j++) {
-        g_far[j] = (size_t)(upper + 16 * j) * 256 + col0 + col;
-        g_near[j] = (size_t)(upper * 16 + j) * 256 + col0 + col;
-        l_far[j] = skew(t + T * j);
-        l_near[j] = skew(upper * T + col + C * j);
-    }
+        for (int k = 0; k < NG0; k++) {
+            std::remove_reference_t<decltype(v[0])> w[R0];
+#pragma unroll
+            for (int j = 0; j < R0; j++) w[j] = v[k + NG0 * j];
+            block(w, 1u);
+#pragma unroll
+            for (int j = 0; j < R0; j++) v[k + NG0 * j] = w[j];
+        }
+    };
+    auto inner = [&](auto *v, auto block) {
+#pragma unroll
+        for (int k = 0; k < NG1; k++) block(v + k * R1, idx_near(k));
+    };
     const bool fp = BE == NTT_BACKEND_FP || (BE == NTT_BACKEND_MIXED && ((a.fp_mask >> job.table) & 1));
     if (BE != NTT_BACKEND_INT && fp) {
         const FpCtx c = fp_ctx(a, job.table);
         double v[16];
         if (FWD) {
+            bool reduce_first = true;
             if (a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
                 const uint64_t *tsrc = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
                 const uint64_t *dsrc = a.pro_src2 + ((size_t)job.poly * a.pro2_poly_stride << a.log_n);
@@ -204,45 +228,51 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
                 for (int j = 0; j < 16; j++) {
                     // coefficient of the dropped limb of the ModDown result, canonical mod q_last
                     const double r = fp_canonical(
-                        fp_from_u64(tsrc[g_far[j]]) - fp_mulmod(fp_from_u64(dsrc[g_far[j]]), wlast, ml), ml);
-                    v[j] = fp_mulmod(fp_from_u64(job.in[g_far[j]]), w, c.m) + fp_reduce(r, c.m);
+                        fp_from_u64(tsrc[glob(e_far(j))]) - fp_mulmod(fp_from_u64(dsrc[glob(e_far(j))]), wlast, ml), ml);
+                    v[j] = fp_mulmod(fp_from_u64(job.in[glob(e_far(j))]), w, c.m) + fp_reduce(r, c.m);
                 }
-                fp_ct_block<4, true>(v, c.tw, 1u, c.m);
             } else if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE) {
                 // one source limb for every limb: it may exceed this limb's prime, so reduce first
                 const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
 #pragma unroll
-                for (int j = 0; j < 16; j++) v[j] = fp_from_u64(src[g_far[j]]);
-                fp_ct_block<4, true>(v, c.tw, 1u, c.m);
+                for (int j = 0; j < 16; j++) v[j] = fp_from_u64(src[glob(e_far(j))]);
             } else {
 #pragma unroll
-                for (int j = 0; j < 16; j++) v[j] = fp_from_u64(job.in[g_far[j]]);
-                fp_ct_block<4, false>(v, c.tw, 1u, c.m);
+                for (int j = 0; j < 16; j++) v[j] = fp_from_u64(job.in[glob(e_far(j))]);
+                reduce_first = false;
             }
+            if (reduce_first)
+                outer(v, [&](double *w, uint32_t idx) { fp_ct_block<p0, true>(w, c.tw, idx, c.m); });
+            else
+                outer(v, [&](double *w, uint32_t idx) { fp_ct_block<p0, false>(w, c.tw, idx, c.m); });
+            if (p1 > 0) {
 #pragma unroll
-            for (int j = 0; j < 16; j++) ld[l_far[j]] = v[j];
-            __syncthreads();
+                for (int j = 0; j < 16; j++) ld[skew(e_far(j))] = v[j];
+                __syncthreads();
 #pragma unroll
-            for (int j = 0; j < 16; j++) v[j] = ld[l_near[j]];
-            fp_ct_block<4, true>(v, c.tw, 16u + upper, c.m);
+                for (int j = 0; j < 16; j++) v[j] = ld[skew(e_near(j))];
+                inner(v, [&](double *w, uint32_t idx) { fp_ct_block<(p1 > 0 ? p1 : 1), true>(w, c.tw, idx, c.m); });
+            }
             // lazy signed doubles go to the blocks pass
 #pragma unroll
-            for (int j = 0; j < 16; j++) job.out[g_near[j]] = (uint64_t)__double_as_longlong(v[j]);
+            for (int j = 0; j < 16; j++) job.out[p1 > 0 ? glob(e_near(j)) : glob(e_far(j))] = (uint64_t)__double_as_longlong(v[j]);
         } else {
             // input: lazy signed doubles from the blocks pass; output: canonical residues
 #pragma unroll
-            for (int j = 0; j < 16; j++) v[j] = __longlong_as_double((long long)job.in[g_near[j]]);
-            fp_gs_block<4, true>(v, c.tw, 16u + upper, c.m);
+            for (int j = 0; j < 16; j++) v[j] = __longlong_as_double((long long)job.in[p1 > 0 ? glob(e_near(j)) : glob(e_far(j))]);
+            if (p1 > 0) {
+                inner(v, [&](double *w, uint32_t idx) { fp_gs_block<(p1 > 0 ? p1 : 1), true>(w, c.tw, idx, c.m); });
 #pragma unroll
-            for (int j = 0; j < 16; j++) ld[l_near[j]] = v[j];
-            __syncthreads();
+                for (int j = 0; j < 16; j++) ld[skew(e_near(j))] = v[j];
+                __syncthreads();
 #pragma unroll
-            for (int j = 0; j < 16; j++) v[j] = ld[l_far[j]];
-            fp_gs_block<4, true>(v, c.tw, 1u, c.m);
+                for (int j = 0; j < 16; j++) v[j] = ld[skew(e_far(j))];
+            }
+            outer(v, [&](double *w, uint32_t idx) { fp_gs_block<p0, true>(w, c.tw, idx, c.m); });
             const FpTw scale = inverse_scale(a, job, c.m);
 #pragma unroll
             for (int j = 0; j < 16; j++)
-                job.out[g_far[j]] = fp_to_u64(fp_canonical(fp_mulmod(v[j], scale, c.m), c.m));
+                job.out[glob(e_far(j))] = fp_to_u64(fp_canonical(fp_mulmod(v[j], scale, c.m), c.m));
         }
         return;
     }
@@ -255,7 +285,7 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
             const uint64_t r1 = a.barrett[2 * job.table + 1];
             const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
 #pragma unroll
-            for (int j = 0; j < 16; j++) v[j] = barrett64(src[g_far[j]], q, r1);
+            for (int j = 0; j < 16; j++) v[j] = barrett64(src[glob(e_far(j))], q, r1);
         } else if (a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
             const uint64_t r1 = a.barrett[2 * job.table + 1];
             const uint64_t *tsrc = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
@@ -264,40 +294,44 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
             const Shoup w = load_shoup(a.pro_w, job.limb), wlast = load_shoup(a.pro_w, a.pro_last);
 #pragma unroll
             for (int j = 0; j < 16; j++) {
-                const uint64_t r = sub_mod(tsrc[g_far[j]], mul_shoup(dsrc[g_far[j]], wlast, ql), ql);
-                v[j] = add_mod(mul_shoup(job.in[g_far[j]], w, q), barrett64(r, q, r1), q);
+                const uint64_t r = sub_mod(tsrc[glob(e_far(j))], mul_shoup(dsrc[glob(e_far(j))], wlast, ql), ql);
+                v[j] = add_mod(mul_shoup(job.in[glob(e_far(j))], w, q), barrett64(r, q, r1), q);
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < 16; j++) v[j] = job.in[g_far[j]];
+            for (int j = 0; j < 16; j++) v[j] = job.in[glob(e_far(j))];
         }
-        ct_block<4>(v, c.tw, 1u, q);
+        outer(v, [&](uint64_t *w, uint32_t idx) { ct_block<p0>(w, c.tw, idx, q); });
+        if (p1 > 0) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) lds[l_far[j]] = v[j];
-        __syncthreads();
+            for (int j = 0; j < 16; j++) lds[skew(e_far(j))] = v[j];
+            __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 16; j++) v[j] = lds[l_near[j]];
-        ct_block<4>(v, c.tw, 16u + upper, q);
+            for (int j = 0; j < 16; j++) v[j] = lds[skew(e_near(j))];
+            inner(v, [&](uint64_t *w, uint32_t idx) { ct_block<(p1 > 0 ? p1 : 1)>(w, c.tw, idx, q); });
+        }
         // lazy values in [0, 4q) go to the blocks pass
 #pragma unroll
-        for (int j = 0; j < 16; j++) job.out[g_near[j]] = v[j];
+        for (int j = 0; j < 16; j++) job.out[p1 > 0 ? glob(e_near(j)) : glob(e_far(j))] = v[j];
     } else {
 #pragma unroll
-        for (int j = 0; j < 16; j++) v[j] = job.in[g_near[j]];
-        gs_block<4>(v, c.tw, 16u + upper, q);
+        for (int j = 0; j < 16; j++) v[j] = job.in[p1 > 0 ? glob(e_near(j)) : glob(e_far(j))];
+        if (p1 > 0) {
+            inner(v, [&](uint64_t *w, uint32_t idx) { gs_block<(p1 > 0 ? p1 : 1)>(w, c.tw, idx, q); });
 #pragma unroll
-        for (int j = 0; j < 16; j++) lds[l_near[j]] = v[j];
-        __syncthreads();
+            for (int j = 0; j < 16; j++) lds[skew(e_near(j))] = v[j];
+            __syncthreads();
 #pragma unroll
-        for (int j = 0; j < 16; j++) v[j] = lds[l_far[j]];
-        gs_block<4>(v, c.tw, 1u, q);
+            for (int j = 0; j < 16; j++) v[j] = lds[skew(e_far(j))];
+        }
+        outer(v, [&](uint64_t *w, uint32_t idx) { gs_block<p0>(w, c.tw, idx, q); });
         if (a.epi_mode == NTT_EPI_MUL) {
             const Shoup w = load_shoup(a.w, job.limb);
 #pragma unroll
-            for (int j = 0; j < 16; j++) job.out[g_far[j]] = mul_shoup(v[j], w, q);
+            for (int j = 0; j < 16; j++) job.out[glob(e_far(j))] = mul_shoup(v[j], w, q);
         } else {
 #pragma unroll
-            for (int j = 0; j < 16; j++) job.out[g_far[j]] = reduce_2q(v[j], q);
+            for (int j = 0; j < 16; j++) job.out[glob(e_far(j))] = reduce_2q(v[j], q);
         }
     }
 }
@@ -318,9 +352,9 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     const uint32_t lb = logical_block();
     const Job job = decode_job(a, lb / tiles_per_limb);
     const uint32_t col0 = (lb % tiles_per_limb) << LOGC;
-    if constexpr (LD == 8 && (TL == 12 || TL == 10)) {
+    if constexpr (LD >= 4 && tile_elems == 16 * kRowThreads) {
         if (a.rows_direct) {
-            rows_direct<FWD, BE, LOGC>(a, job, col0, lds);
+            rows_direct<LD, FWD, BE, LOGC>(a, job, col0, lds);
             return;
         }
     }
