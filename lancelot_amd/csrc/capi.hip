@@ -66,8 +66,6 @@ struct he_context {
     bool mixed_ok = false;       // mixed launches allowed (at most 64 tables; CAHEL_HIP_NO_MIXED=1 switches them off)
     int rows_direct = 1;         // environment CAHEL_HIP_ROWS_VIA_LDS=1: every register block of the rows pass (and of the
                                  // fused inner-product kernel) takes its operands from LDS
-    bool fuse_modup_rows = true; // environment CAHEL_HIP_NO_FUSED_MODUP=1: base conversion and rows pass as two kernels
-    uint32_t modup_group = 6;    // output limbs per workgroup of the fused kernel (CAHEL_HIP_MODUP_GROUP)
     std::vector<Level> levels;   // indexed by L
     std::vector<void *> owned;
 
@@ -355,12 +353,6 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->mixed_ok = qp <= 64 && !(nx && nx[0] == '1');
         const char *rv = getenv("CAHEL_HIP_ROWS_VIA_LDS");
         ctx->rows_direct = !(rv && rv[0] == '1');
-        const char *nm = getenv("CAHEL_HIP_NO_FUSED_MODUP");
-        ctx->fuse_modup_rows = !(nm && nm[0] == '1');
-        if (const char *g = getenv("CAHEL_HIP_MODUP_GROUP")) {
-            const int v = atoi(g);
-            if (v >= 1 && v <= 64) ctx->modup_group = (uint32_t)v;
-        }
         ctx->fp_ok.assign(qp, 0);
         std::vector<double> psi_fp(qp * n, 0.0), ipsi_fp(qp * n, 0.0), consts(4 * qp, 0.0);
         for (size_t t = 0; t < qp; t++) {
@@ -869,14 +861,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         fwd.n_jobs = lv->n_modup_jobs;
         fwd.groups = lv->d_modup_groups;
         fwd.n_groups = lv->n_modup_groups;
-        const bool fused_rows = ctx->fuse_modup_rows && modup_rows_supported(ctx->log_n);
-        if (fused_rows) {
-            // base conversion and the rows pass of the forward transform in one kernel
-            const uint32_t group = ctx->modup_group;
-            ModupRowsArgs m{tmp, y, lv->d_modup_descs, lv->d_modup_limb, lv->d_modup_table, lv->d_mats_fp,
-                            group, (lv->modup_max_rows + group - 1) / group};
-            HE_HIP(launch_modup_rows(fwd, m, lv->beta, S(s)));
-        } else {
+        {
             BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                          lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts, 1, 0, 0, 0};
             HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
@@ -896,7 +881,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         x.beta = lv->beta;
         x.fold_ct = fold_ct;
         x.fold_w = fold_w;
-        HE_HIP(launch_ntt_forward_inner(fwd, x, fused_rows, S(s)));
+        HE_HIP(launch_ntt_forward_inner(fwd, x, S(s)));
     } else {
         if (int rc = modup_impl(ctx, L, src, galois_elt ? L : c_item_stride, items, y, tmp, s)) return rc;
         EvkPtrs ptrs;

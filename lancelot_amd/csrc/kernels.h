@@ -171,20 +171,6 @@ struct BconvBatch {
 };
 hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s);
 
-// ModUp base conversion fused with the rows pass of the forward transform (FP64 back end, 2^13 <= N <= 2^15): reads the
-// scaled coefficient-form limbs x [L][N], writes the rows-pass output of every converted limb into y
-// [beta][L+K][N] (the layout and tables of BconvBatch for ModUp).  `group` output limbs per workgroup.
-struct ModupRowsArgs {
-    const uint64_t *x;
-    uint64_t *y;
-    const BconvDesc *descs;
-    const uint32_t *out_limb, *out_table;
-    const double *mat_fp;
-    uint32_t group, groups_per_digit;
-};
-bool modup_rows_supported(uint32_t log_n);
-hipError_t launch_modup_rows(const struct NttArgs &a, const ModupRowsArgs &m, uint32_t n_digits, hipStream_t s);
-
 constexpr int kMaxDigits = 64;
 struct EvkPtrs {
     const uint64_t *p[kMaxDigits];
@@ -222,7 +208,7 @@ struct KsFuseArgs {
     const uint64_t *fold_ct;  // [2][L][N]
     const uint64_t *fold_w;   // Shoup pair of P^-1 mod q_{L-1}
 };
-hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, bool rows_done, hipStream_t s);
+hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s);
 
 hipError_t launch_decompose_real(const Tables &t, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,
                                  uint32_t items, size_t out_item_stride, hipStream_t s);

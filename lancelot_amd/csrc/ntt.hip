@@ -487,104 +487,6 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------
-// ModUp base conversion fused with the rows pass of the forward transform (FP64 back end).
-//
-// Workgroup = (tile of 1024 words, digit, group of G output limbs), 256 threads.  Every thread keeps its 4
-// coefficients of the digit's (at most 8) input limbs in registers, so the inputs are read once per group instead
-// of once per output limb; for four output limbs at a time the workgroup forms sum_i x_i M[r][i] straight into
-// four LDS tiles, and each of its four waves then runs the rows-pass stages on one of them.  The converted limbs
-// are never written in coefficient form: 2 limb transfers less per output limb than base conversion followed by
-// the rows pass.
-// ---------------------------------------------------------------------------------------------------
-constexpr int kFuseTileLog = 10;
-constexpr uint32_t kFuseLds = (1u << kFuseTileLog) + (1u << (kFuseTileLog - 4));
-
-template <int LD>
-__global__ __launch_bounds__(256) void modup_rows_fp_kernel(NttArgs a, ModupRowsArgs m) {
-    __shared__ uint64_t lds[4][kFuseLds];
-    constexpr int LOGC = log_cols<LD, kFuseTileLog>();
-    constexpr uint32_t C = 1u << LOGC;
-    constexpr uint32_t tile_elems = 1u << (LD + LOGC);
-    constexpr uint32_t tiles_per_limb = 256u >> LOGC;
-    constexpr uint32_t per_thread = tile_elems / 256;
-    constexpr int p0 = Split<LD>::p0, p1 = Split<LD>::p1;
-    static_assert(tile_elems == 1024, "four coefficients per thread");
-
-    // consecutive logical ids (one XCD, one L2): the groups of one (digit, tile), which read the same inputs, then
-    // the neighbouring tiles, which share their 128-byte lines
-    uint32_t lb = logical_block();
-    const uint32_t grp = lb % m.groups_per_digit;
-    lb /= m.groups_per_digit;
-    const uint32_t tile = lb % tiles_per_limb, dg = lb / tiles_per_limb;
-    const uint32_t col0 = tile << LOGC;
-    const BconvDesc d = m.descs[dg];
-    const uint32_t r_begin = grp * m.group, r_end = r_begin + m.group < d.n_out ? r_begin + m.group : d.n_out;
-    if (r_begin >= d.n_out) return;
-
-    size_t gidx[per_thread];
-#pragma unroll
-    for (uint32_t k = 0; k < per_thread; k++) {
-        const uint32_t e = threadIdx.x + 256 * k;
-        gidx[k] = (size_t)(e >> LOGC) * 256 + col0 + (e & (C - 1));
-    }
-    double xv[8][per_thread];
-    const uint64_t *x = m.x + d.x_off;
-#pragma unroll
-    for (int i = 0; i < 8; i++)
-#pragma unroll
-        for (uint32_t k = 0; k < per_thread; k++)
-            xv[i][k] = (uint32_t)i < d.n_in ? fp_from_u64(x[((size_t)i << a.log_n) + gidx[k]]) : 0.0;
-
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    uint64_t *out = m.y + d.out_off;
-    const double *mat = m.mat_fp + 2 * d.mat_off;
-    for (uint32_t r0 = r_begin; r0 < r_end; r0 += 4) {
-        // conversion of four output limbs, every thread its own coefficients
-#pragma unroll
-        for (uint32_t b = 0; b < 4; b++) {
-            const uint32_t r = r0 + b;
-            if (r >= r_end) break;
-            const FpMod mod = fp_ctx(a, m.out_table[d.map_off + r]).m;
-            const double *row = mat + 2 * (size_t)r * d.n_in;
-            double acc[per_thread];
-#pragma unroll
-            for (uint32_t k = 0; k < per_thread; k++) acc[k] = 0.0;
-#pragma unroll
-            for (int i = 0; i < 8; i++) {
-                if ((uint32_t)i >= d.n_in) break;
-                const FpTw w{row[2 * i], row[2 * i + 1]};
-#pragma unroll
-                for (uint32_t k = 0; k < per_thread; k++) acc[k] += fp_mulmod(xv[i][k], w, mod);
-            }
-            double *ld = reinterpret_cast<double *>(lds[b]);
-#pragma unroll
-            for (uint32_t k = 0; k < per_thread; k++) ld[skew(threadIdx.x + 256 * k)] = acc[k];
-        }
-        lds_barrier();
-        // rows pass: wave w on tile w (the sums are below 6 q in magnitude: the first pass reduces them)
-        const uint32_t r = r0 + wave;
-        const bool active = r < r_end;
-        const FpCtx c = fp_ctx(a, m.out_table[d.map_off + (active ? r : r0)]);
-        if (active) tile_pass_fp<p0, true, true>(lds[wave], tile_elems, LD - p0 + LOGC, 1u, c, lane, 64u);
-        lds_barrier();
-        if (p1 > 0) {
-            if (active) tile_pass_fp<(p1 > 0 ? p1 : 1), true, true>(lds[wave], tile_elems, LOGC, 1u << p0, c, lane, 64u);
-            lds_barrier();
-        }
-        // lazy signed doubles go to the blocks pass
-#pragma unroll
-        for (uint32_t b = 0; b < 4; b++) {
-            const uint32_t rr = r0 + b;
-            if (rr >= r_end) break;
-            uint64_t *dst = out + ((size_t)m.out_limb[d.map_off + rr] << a.log_n);
-#pragma unroll
-            for (uint32_t k = 0; k < per_thread; k++) dst[gidx[k]] = lds[b][skew(threadIdx.x + 256 * k)];
-        }
-        lds_barrier();  // every read of these tiles is done before the next four overwrite them
-    }
-}
-
-// ---------------------------------------------------------------------------------------------------
 // blocks pass: the 8 stages that stay inside 256 consecutive words
 //
 // A workgroup of T threads owns a tile of 16 T consecutive words (T = 128 or 256) and walks through every
@@ -1098,27 +1000,9 @@ hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, h
                                         : launch_blocks<true, NTT_BACKEND_INT>(a, n_polys, s);
 }
 
-// (at N = 2^16 the rows pass with its outer half-pass on registers, after a separate conversion, is faster)
-bool modup_rows_supported(uint32_t log_n) { return log_n >= 13 && log_n <= 15; }
-
-hipError_t launch_modup_rows(const NttArgs &a, const ModupRowsArgs &m, uint32_t n_digits, hipStream_t s) {
-    if (!modup_rows_supported(a.log_n) || m.group == 0 || m.groups_per_digit == 0) return hipErrorInvalidValue;
-    const int ld = (int)a.log_n - 8;
-    const uint32_t tiles = 256u >> (kFuseTileLog - ld);
-    const dim3 grid(n_digits * tiles * m.groups_per_digit);
-    switch (ld) {
-#define HE_CASE(LD) \
-    case LD: hipLaunchKernelGGL(modup_rows_fp_kernel<LD>, grid, dim3(256), 0, s, a, m); break;
-        HE_CASE(5) HE_CASE(6) HE_CASE(7)
-#undef HE_CASE
-        default: return hipErrorInvalidValue;
-    }
-    return hipGetLastError();
-}
-
-hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, bool rows_done, hipStream_t s) {
+hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s) {
     if (a.log_n < 9 || a.log_n > 16 || !a.jobs) return hipErrorInvalidValue;
-    if (a.n_jobs && !rows_done) {
+    if (a.n_jobs) {
         hipError_t e = launch_rows<true, NTT_BACKEND_FP>(a, a.n_jobs, s);
         if (e != hipSuccess) return e;
     }

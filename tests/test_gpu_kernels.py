@@ -177,15 +177,13 @@ def test_mixed_back_end_agrees_with_the_integer_one(oracle, capi, monkeypatch, l
                                                  (14, [50, 49, 48, 50, 47, 50, 50, 50, 50], 3, 5),
                                                  (11, [45, 40, 40, 50], 1, 3), (9, [40, 40, 45, 45], 2, 2)])
 def test_fused_and_separate_key_switch_agree(oracle, capi, monkeypatch, logn, bits, size_p, L):
-    """he_keyswitch with the inner product inside the forward NTT and the base conversion inside its rows pass
-    (defaults for primes below 2^50; the latter for N = 2^13 to 2^15), and, forced by the environment, with the separate
-    kernels: all equal the oracle, with and without a Galois element, with a partial last digit (L = 3 over two
-    special primes, L = 5 over three), with output groups that end inside a round of four, and at the smallest
-    degree."""
-    for no_fuse, no_modup, group in (("0", "0", "8"), ("0", "0", "3"), ("0", "1", "8"), ("1", "0", "8")):
+    """he_keyswitch with the inner product inside the forward NTT (the default for primes below 2^50) and, forced
+    by the environment, with the separate kernels, each with the rows pass on registers and through LDS: all equal
+    the oracle, with and without a Galois element, with a partial last digit (L = 3 over two special primes, L = 5
+    over three), and at the smallest degree."""
+    for no_fuse, via_lds in (("0", "0"), ("0", "1"), ("1", "0"), ("1", "1")):
         monkeypatch.setenv("CAHEL_HIP_NO_FUSED_KS", no_fuse)
-        monkeypatch.setenv("CAHEL_HIP_NO_FUSED_MODUP", no_modup)
-        monkeypatch.setenv("CAHEL_HIP_MODUP_GROUP", group)
+        monkeypatch.setenv("CAHEL_HIP_ROWS_VIA_LDS", via_lds)
         cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
         rng = np.random.default_rng(12)
         lib, h = capi.lib(), ctx.he_handle()
@@ -198,7 +196,7 @@ def test_fused_and_separate_key_switch_agree(oracle, capi, monkeypatch, logn, bi
             capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, elt, ws.ptr, None))
             ks = p.key_switch(p.galois_ntt(c, elt) if elt else c, host_evk)
             want = np.stack([p.add(ct[b], ks[b]) for b in range(2)])
-            assert (dct.numpy() == want).all(), (no_fuse, elt)
+            assert (dct.numpy() == want).all(), (no_fuse, via_lds, elt)
 
 
 @pytest.mark.parametrize("logn,bits,size_p,L", [(13, [50, 50, 49, 50, 50, 50], 2, 4), (13, [50, 50, 49, 50, 50, 50], 2, 3),
