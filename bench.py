@@ -30,7 +30,7 @@ sys.path.insert(0, ROOT)
 LOG_N, SIZE_Q, SIZE_P, BITS, SCALE = 16, 24, 8, 50, 2.0 ** 40
 # HBM bytes of one 72-limb forward NTT call, from the FETCH_SIZE / WRITE_SIZE counters scaled by a copy of known
 # size (profiles/ntt_forward_72limbs_n65536.md)
-NTT72_TRAFFIC_BYTES = 164_006_912
+NTT72_TRAFFIC_BYTES = 164_057_088
 HBM_PEAK_GBS = 8000.0
 
 
