@@ -11,9 +11,12 @@
 //                 columns (C consecutive words per row).
 //   blocks pass : the last 8 stages stay inside one row (256 consecutive words).  A workgroup owns 16
 //                 rows (4096 consecutive words).
-// Inside a pass each thread takes 2^r elements from LDS into registers, runs r stages on them (r <= 4,
-// radix-16) and writes them back; 8 stages cost two LDS round trips.  LDS indices are skewed by one word
-// per 16 so that both the stride-16 and the stride-256 gathers of a wave hit distinct banks.
+// Inside a pass each thread takes 2^r elements into registers, runs r stages on them (r <= 4, radix-16) and
+// hands them on; the stages of a pass form two such register blocks.  In the blocks pass both blocks take
+// their elements from LDS and write them back.  In the rows pass (N >= 2^12) the outer block works on the
+// words that a coalesced access of the tile gives the thread anyway, straight from or to global memory, and
+// only the exchange between the two blocks goes through LDS (rows_direct below).  LDS indices are skewed by
+// one word per 16 so that both the stride-16 and the stride-256 gathers of a wave hit distinct banks.
 // The forward transform runs rows pass then blocks pass, the inverse the other way round.
 //
 // Two arithmetic back ends share this skeleton:
@@ -22,7 +25,8 @@
 //   FP64    : exact integer arithmetic in doubles for primes below 2^50 (8 full-rate operations per
 //             butterfly, see modarith.cuh); values between the two passes are lazy signed doubles stored
 //             in the same 8-byte words; the factor 1/N is folded into the last multiplication
-// A launch uses the FP64 back end when every limb it touches has a prime below 2^50.
+// A launch uses the FP64 back end when every limb it touches has a prime below 2^50, the integer one when none
+// has, and otherwise the mixed instantiations, in which every workgroup follows its own limb's prime.
 #include <type_traits>
 
 #include "kernels.h"
