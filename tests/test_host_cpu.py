@@ -224,3 +224,14 @@ def test_params_record_layout_and_round_trip(cahel):
     with pytest.raises(ValueError):
         q.from_bytes(blob[:17] + struct.pack("<Q", 1) + blob[25:])            # modulus 1
     assert (q.poly_modulus_degree(), q.coeff_modulus()) == (4096, mods)       # failed loads change nothing
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; with --gpus above 1 it says so and exits with an error, before touching a GPU."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
