@@ -160,6 +160,18 @@ int he_galois_ntt(const he_context *ctx, const uint64_t *in, uint64_t *out, uint
 int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_t n_polys, uint32_t L,
                uint64_t *workspace, he_stream stream);
 
+/* he_rescale without a workspace argument, for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc): the coefficient form of the dropped limb goes to a
+ * buffer that is part of the library's device image (4 * 65536 words = 2 MiB on every GPU the library runs on,
+ * held until the process ends), so the call allocates nothing and passes nothing but inputs and outputs.
+ * Limit: n_polys <= 4 (and n_polys * N <= 4 * 65536 words); beyond it the call returns HE_E_UNSUPPORTED and
+ * launches nothing.  Same limbs as he_rescale.  All calls on one GPU share the buffer, on every stream: calls
+ * that overlap in time on one GPU race; calls issued to one stream are ordered and safe.  Nothing in the buffer
+ * has to start at zero (every word read is written earlier in the same call).
+ * No counterpart in the reference, whose rescale takes its temporaries from a memory pool. */
+int he_rescale_static(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_t n_polys, uint32_t L,
+                      he_stream stream);
+
 /* ---- hybrid key switching ---- */
 
 /* c [L][N] (NTT) -> out [beta][L+K][N] (NTT).  workspace: L * N words.

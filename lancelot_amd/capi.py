@@ -50,6 +50,7 @@ SIGNATURES = {
     "he_tensor_square": (C.c_int, [vp, vp, vp, u32, vp]),
     "he_galois_ntt": (C.c_int, [vp, vp, vp, u32, u32, vp]),
     "he_rescale": (C.c_int, [vp, vp, vp, u32, u32, vp, vp]),
+    "he_rescale_static": (C.c_int, [vp, vp, vp, u32, u32, vp]),
     "he_modup": (C.c_int, [vp, u32, vp, vp, vp, vp]),
     "he_ks_inner_product": (C.c_int, [vp, u32, vp, C.POINTER(vp), vp, u32, C.c_int, vp]),
     "he_moddown": (C.c_int, [vp, u32, vp, vp, u32, C.c_int, vp, vp]),

@@ -7,6 +7,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <vector>
 
@@ -43,6 +44,40 @@ struct Level {
     bool batched = false;
     double *d_mats_fp = nullptr;         // (M, M/m) pairs of the digit matrices, when every prime is below 2^50
 };
+
+}  // namespace
+
+// Scratch of he_rescale_static: the coefficient form of the dropped limb of up to kStaticPolys polynomials at
+// N <= 2^16 (2 MiB).  Every GPU the library runs on holds its own copy until the process ends.  In host code the
+// array's name is only a handle for hipGetSymbolAddress: kernels and copies get the per-device address kept in
+// g_static_ptr.
+constexpr uint32_t kStaticPolys = 4;
+constexpr size_t kStaticWords = (size_t)kStaticPolys << 16;
+static __device__ __align__(256) uint64_t scratch[kStaticWords];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+uint64_t *g_static_ptr[kMaxDevices];
+std::mutex g_static_mutex;
+
+// Address of `scratch` on the current device, resolved once per device with that device current.
+int static_scratch(uint64_t **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return HE_E_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    if (!g_static_ptr[dev]) {
+        uint64_t *p = nullptr;
+        e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return HE_E_UNSUPPORTED;
+        g_static_ptr[dev] = p;
+    }
+    *out = g_static_ptr[dev];
+    return HE_OK;
+}
 
 }  // namespace
 
@@ -300,6 +335,11 @@ int he_context_create(const he_context_desc *d, he_context **out) {
     ctx->h_moduli.assign(d->moduli, d->moduli + ctx->size_qp);
     const size_t n = ctx->n(), qp = ctx->size_qp;
     int rc = hipGetDevice(&ctx->device);
+    if (!rc) {
+        // he_rescale_static's scratch on this device: resolved here, so that the entry point itself only looks it up
+        uint64_t *unused = nullptr;
+        rc = static_scratch(&unused);
+    }
     if (!rc) rc = upload(ctx, &ctx->d_moduli, d->moduli, qp);
     if (!rc) rc = upload(ctx, &ctx->d_barrett, d->barrett, 2 * qp);
     if (!rc) rc = upload(ctx, &ctx->d_psi, d->psi, 2 * qp * n);
@@ -655,6 +695,16 @@ int he_rescale(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_
     // the broadcast source is a residue of q_{L-1}: the FP64 back end needs it below 2^50 as well
     HE_HIP(launch_ntt_forward(fwd, n_polys, backend_for(ctx, fwd.map, (int)L - 1), S(s)));
     return HE_OK;
+}
+
+int he_rescale_static(const he_context *ctx, const uint64_t *in, uint64_t *out, uint32_t n_polys, uint32_t L,
+                      he_stream s) {
+    if (!ctx || n_polys == 0) return HE_E_INVALID_ARGUMENT;
+    if (n_polys > kStaticPolys || (size_t)n_polys * ctx->n() > kStaticWords) return HE_E_UNSUPPORTED;
+    uint64_t *ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    // the scratch needs no clearing: the inverse transform writes every word of it that the forward one reads
+    return he_rescale(ctx, in, out, n_polys, L, ws, s);
 }
 
 }  // extern "C"
