@@ -90,6 +90,8 @@ struct he_context {
     std::vector<uint64_t> h_phat_inv;    // host copy of d_phat_inv
     double *d_psi_fp = nullptr, *d_ipsi_fp = nullptr, *d_fp_consts = nullptr;  // FP64 back end tables
     double *d_phat_mod_q_fp = nullptr;   // (M, M/q_j) pairs of the P -> Ql matrix
+    double *d_phat_pinv_fp = nullptr;    // the same matrix times P^-1 mod q_j (merged ModDown + rescale, fused kernel)
+    bool fuse_rows = true;       // environment CAHEL_HIP_NO_FUSED_BCONV=1: conversion kernel, then the rows pass
     uint32_t *d_rot_group = nullptr;     // encoder: 5^j mod 2N
     double2 *d_ksi = nullptr;            // encoder: e^{2 pi i k / 2N}, k <= 2N
     uint64_t *d_garner_inv = nullptr;    // decoder: [size_q][size_q], q_j^-1 mod q_i for j < i
@@ -188,6 +190,11 @@ bool fp_for_level(const he_context *ctx, uint32_t L) {
     for (uint32_t t = 0; t < L + ctx->size_p; t++)
         if (!ctx->fp_ok[table_of(ctx, L, t)]) return false;
     return true;
+}
+
+// base conversion fused with the rows pass of the forward transform that follows it (launch_bconv_rows)
+bool fuse_rows_ok(const he_context *ctx, const Level *lv, uint32_t L) {
+    return ctx->fuse_rows && lv && lv->batched && ctx->log_n >= 12 && fp_for_level(ctx, L);
 }
 
 int check_map(const he_context *ctx, uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail) {
@@ -393,6 +400,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->mixed_ok = qp <= 64 && !(nx && nx[0] == '1');
         const char *rv = getenv("CAHEL_HIP_ROWS_VIA_LDS");
         ctx->rows_direct = !(rv && rv[0] == '1');
+        const char *nb = getenv("CAHEL_HIP_NO_FUSED_BCONV");
+        ctx->fuse_rows = !(nb && nb[0] == '1');
         ctx->fp_ok.assign(qp, 0);
         std::vector<double> psi_fp(qp * n, 0.0), ipsi_fp(qp * n, 0.0), consts(4 * qp, 0.0);
         for (size_t t = 0; t < qp; t++) {
@@ -415,13 +424,23 @@ int he_context_create(const he_context_desc *d, he_context **out) {
             consts[4 * t + 3] = (double)ninv / qd;
         }
         if (d->size_p) {
-            std::vector<double> pfp(2 * (size_t)d->size_q * d->size_p);
+            // (16 doubles of padding: the fused conversion kernel fetches 8 pairs per row whatever the row's length)
+            std::vector<double> pfp(2 * (size_t)d->size_q * d->size_p + 16, 0.0);
             for (size_t jq = 0; jq < d->size_q; jq++)
                 for (size_t k = 0; k < d->size_p; k++) {
                     pfp[2 * (jq * d->size_p + k)] = (double)d->phat_mod_q[jq * d->size_p + k];
                     pfp[2 * (jq * d->size_p + k) + 1] = (double)d->phat_mod_q[jq * d->size_p + k] / (double)d->moduli[jq];
                 }
             rc = upload(ctx, &ctx->d_phat_mod_q_fp, pfp.data(), pfp.size());
+            // (P / p_k) P^-1 mod q_j: delta_j P^-1 straight from the conversion
+            for (size_t jq = 0; jq < d->size_q; jq++)
+                for (size_t k = 0; k < d->size_p; k++) {
+                    const uint64_t q = d->moduli[jq];
+                    const uint64_t v = (uint64_t)((unsigned __int128)d->phat_mod_q[jq * d->size_p + k] * d->pinv_mod_q[2 * jq] % q);
+                    pfp[2 * (jq * d->size_p + k)] = (double)v;
+                    pfp[2 * (jq * d->size_p + k) + 1] = (double)v / (double)q;
+                }
+            if (!rc) rc = upload(ctx, &ctx->d_phat_pinv_fp, pfp.data(), pfp.size());
         }
         if (!rc) rc = upload(ctx, &ctx->d_psi_fp, psi_fp.data(), psi_fp.size());
         if (!rc) rc = upload(ctx, &ctx->d_ipsi_fp, ipsi_fp.data(), ipsi_fp.size());
@@ -527,7 +546,7 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
             if (rc) return rc;
             lv.batched = true;
             if (fp_for_level(ctx, L)) {
-                std::vector<double> mfp(2 * mat_words);
+                std::vector<double> mfp(2 * mat_words + 16, 0.0);   // padded as the P -> Ql matrix is
                 for (uint32_t dg = 0; dg < beta; dg++) {
                     const Digit &g = lv.digits[dg];
                     for (uint32_t r = 0; r < g.n_out; r++) {
@@ -731,7 +750,13 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_part_hat_inv;
     HE_HIP(launch_ntt_inverse(inv, items, backend_for(ctx, inv.map), S(s)));
-    if (lv->batched) {
+    const bool fused = fuse_rows_ok(ctx, lv, L);
+    if (fused) {
+        BconvRows b{ws, out, c, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
+                    lv->beta, lv->modup_max_rows, lv->modup_max_copy,
+                    items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n, 0};
+        HE_HIP(launch_bconv_rows(base_args(ctx, true), b, S(s)));
+    } else if (lv->batched) {
         BconvBatch b{ws, out, c, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                      lv->beta, lv->modup_max_rows, lv->modup_max_copy, lv->d_mats_fp, ctx->d_fp_consts,
                      items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n};
@@ -755,7 +780,7 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     fwd.n_groups = lv->n_modup_groups;
     fwd.items = items;
     fwd.item_stride = (size_t)lv->beta * LK * n;
-    HE_HIP(launch_ntt_forward(fwd, 1, backend_for_level(ctx, L), S(s)));
+    HE_HIP(launch_ntt_forward(fwd, 1, backend_for_level(ctx, L), S(s), fused));
     return HE_OK;
 }
 
@@ -807,12 +832,19 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     const Level *lv = level_of(ctx, L);
     // the conversion tables describe up to 4 polynomials; more of them go as items of 2 (ciphertexts)
     const bool batched = lv && lv->batched && (n_polys <= 4 || n_polys % 2 == 0);
+    const bool fused = batched && fuse_rows_ok(ctx, lv, L);
     if (batched) {
         const uint32_t units = n_polys <= 4 ? n_polys : 2, items = n_polys / units;
-        BconvBatch b{cx, ws, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, units, L, 0,
-                     fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts,
-                     items, (size_t)units * LK * n, (size_t)units * L * n, 0};
-        HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+        if (fused) {
+            BconvRows b{cx, ws, nullptr, ctx->d_phat_mod_q_fp, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, units, L, 0,
+                        items, (size_t)units * LK * n, (size_t)units * L * n, 0, 0};
+            HE_HIP(launch_bconv_rows(base_args(ctx, true), b, S(s)));
+        } else {
+            BconvBatch b{cx, ws, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, units, L, 0,
+                         fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts,
+                         items, (size_t)units * LK * n, (size_t)units * L * n, 0};
+            HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+        }
     }
     for (uint32_t p = 0; p < n_polys && !batched; p++) {
         BconvArgs b{cx + ((size_t)p * LK + L) * n, ws + (size_t)p * L * n, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, K, L};
@@ -832,7 +864,7 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     fwd.w = ctx->d_pinv_mod_q;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L;
-    HE_HIP(launch_ntt_forward(fwd, n_polys, backend_for(ctx, fwd.map), S(s)));
+    HE_HIP(launch_ntt_forward(fwd, n_polys, backend_for(ctx, fwd.map), S(s), fused));
     return HE_OK;
 }
 
@@ -911,7 +943,12 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         fwd.n_jobs = lv->n_modup_jobs;
         fwd.groups = lv->d_modup_groups;
         fwd.n_groups = lv->n_modup_groups;
-        {
+        const bool rows_done = fuse_rows_ok(ctx, lv, L);
+        if (rows_done) {
+            BconvRows b{tmp, y, nullptr, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
+                        lv->beta, lv->modup_max_rows, 0, 1, 0, 0, 0, 0};
+            HE_HIP(launch_bconv_rows(fwd, b, S(s)));
+        } else {
             BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                          lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts, 1, 0, 0, 0};
             HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
@@ -931,7 +968,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         x.beta = lv->beta;
         x.fold_ct = fold_ct;
         x.fold_w = fold_w;
-        HE_HIP(launch_ntt_forward_inner(fwd, x, S(s)));
+        HE_HIP(launch_ntt_forward_inner(fwd, x, S(s), rows_done));
     } else {
         if (int rc = modup_impl(ctx, L, src, galois_elt ? L : c_item_stride, items, y, tmp, s)) return rc;
         EvkPtrs ptrs;
@@ -1038,7 +1075,13 @@ int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items
     inv.w = lv->d_mdr_w;
     HE_HIP(launch_ntt_inverse(inv, polys, backend_for(ctx, inv.map), S(s)));
     // (3) delta = P -> Ql conversion of the special limbs
-    if (lv->batched) {
+    const bool fused = fuse_rows_ok(ctx, lv, L);
+    if (fused) {
+        // with the prologue of (4) and the rows pass of its transform
+        BconvRows b{cx, delta, nullptr, ctx->d_phat_pinv_fp, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
+                    items, 2 * (size_t)LK * n, 2 * (size_t)L * n, 0, 1};
+        HE_HIP(launch_bconv_rows(base_args(ctx, true), b, S(s)));
+    } else if (lv->batched) {
         BconvBatch b{cx, delta, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
                      fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts,
                      items, 2 * (size_t)LK * n, 2 * (size_t)L * n, 0};
@@ -1070,7 +1113,7 @@ int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items
     fwd.w = lv->d_qlast_inv;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L - 1;
-    HE_HIP(launch_ntt_forward(fwd, polys, backend_for(ctx, fwd.map, (int)L - 1), S(s)));
+    HE_HIP(launch_ntt_forward(fwd, polys, backend_for(ctx, fwd.map, (int)L - 1), S(s), fused));
     return HE_OK;
 }
 

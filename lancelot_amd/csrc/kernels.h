@@ -100,7 +100,8 @@ struct NttArgs {
 // NTT_BACKEND_MIXED (every workgroup picks the FP64 back end when its limb's bit of fp_mask is set, the integer
 // one otherwise: for chains that mix primes below and above 2^50, tables below 64 only).
 enum : int { NTT_BACKEND_INT = 0, NTT_BACKEND_FP = 1, NTT_BACKEND_MIXED = 2 };
-hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s);
+// rows_done: the rows pass has run already (launch_bconv_rows), only the blocks pass is launched.
+hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool rows_done = false);
 // Inverse transform: phase A (contiguous blocks, reads a.in writes a.out) then phase B (rows, in place on
 // a.out, epilogue NTT_EPI_MUL optional).
 hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s);
@@ -171,6 +172,26 @@ struct BconvBatch {
 };
 hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s);
 
+// Base conversion fused with the rows pass of the forward transform of its output limbs (FP64 back end, N >= 2^12,
+// n_in <= 8): the units of a BconvBatch, with the results left as the lazy words that the blocks pass continues on.
+struct BconvRows {
+    const uint64_t *x_base;
+    uint64_t *out_base;
+    const uint64_t *copy_base;   // limbs copied unchanged (descs' copy_first / copy_count), or nullptr
+    const double *mat_fp;        // (M, M/m) pairs at 2 * mat_off
+    const uint32_t *out_limb;
+    const uint32_t *out_table;
+    const BconvDesc *descs;      // device memory
+    uint32_t n_units, max_rows, max_copy;
+    uint32_t items;              // 0 = 1
+    size_t x_item_stride, out_item_stride, copy_item_stride;
+    // merged ModDown + rescale: the last row of every unit's matrix is the limb that is dropped; the other output
+    // limbs receive sum_i x_i M[j][i] + ((t - sum_i x_i M[last][i] mod q_last) mod q_j), t = the limb before x
+    int mdr;
+};
+// `a` supplies the FP64 twiddles and constants of a forward transform (base_args)
+hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s);
+
 constexpr int kMaxDigits = 64;
 struct EvkPtrs {
     const uint64_t *p[kMaxDigits];
@@ -208,7 +229,7 @@ struct KsFuseArgs {
     const uint64_t *fold_ct;  // [2][L][N]
     const uint64_t *fold_w;   // Shoup pair of P^-1 mod q_{L-1}
 };
-hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s);
+hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s, bool rows_done = false);
 
 hipError_t launch_decompose_real(const Tables &t, const double *coeffs, uint64_t *out, uint32_t limbs, uint32_t first,
                                  uint32_t items, size_t out_item_stride, hipStream_t s);

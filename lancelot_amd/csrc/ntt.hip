@@ -27,6 +27,7 @@
 //             in the same 8-byte words; the factor 1/N is folded into the last multiplication
 // A launch uses the FP64 back end when every limb it touches has a prime below 2^50, the integer one when none
 // has, and otherwise the mixed instantiations, in which every workgroup follows its own limb's prime.
+#include <cstdlib>
 #include <type_traits>
 
 #include "kernels.h"
@@ -487,6 +488,198 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
                 job.out[(size_t)row * 256 + col0 + col] = reduce_2q(lds[skew(e)], q);
             }
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Base conversion fused with the rows pass of the forward transform that follows it (FP64 back end, N >= 2^12).
+//
+// Both operate on the same set of coefficients: a tile of all 2^LD rows x C columns of the limb's (N / 256) x 256
+// view.  A workgroup of 256 threads owns a tile of 2048 coefficients (8 per thread) of one unit (a ModUp digit or a
+// ModDown polynomial) and a group of the unit's output limbs.  Every thread keeps its 8 coefficients of the unit's
+// (at most 8) input limbs in registers; for each output limb of the group it forms sum_i x_i M[r][i] for its
+// coefficients, which are exactly the 8 words of its first register block of the rows pass (rows 2^(LD-3) apart),
+// runs the first three stages on them, and the tile then crosses LDS between the remaining register blocks.  The
+// converted limbs never exist in coefficient form in memory: 2 limb transfers and one launch less per output limb
+// than conversion kernel + rows pass.  The groups of one tile re-read the same inputs (from L2: they run on one XCD).
+//
+// mdr (merged ModDown + rescale): the last matrix row belongs to the limb that the rescale drops; with
+// r = t - sum_i x_i M[last][i] mod q_last (t: the limb right before the unit's inputs), output limb j receives
+// sum_i x_i M[j][i] + (r mod q_j); the matrix carries the factor P^-1.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kFuseLog = 11;
+constexpr uint32_t kFuseWords = 1u << kFuseLog, kFuseThreads = kFuseWords / 8;
+
+// LDS index of tile word e: 8 words of padding per 32, so that the 32 lanes of a half-wave that read the words
+// {32 a + 8 j + c} or {256 u + 32 j + c'} of one register slot j hit distinct 8-byte banks
+__device__ __forceinline__ uint32_t skew8(uint32_t e) { return e + ((e >> 5) << 3); }
+
+struct BconvRowsK {
+    BconvRows b;
+    uint32_t compute_groups, copy_groups, rows_per;
+};
+
+// register block of LOGR stages on the groups of a tile that lives in LDS (tile index bits: [upper][LOGR bits][low_bits]);
+// twl: entries 0..255 of the limb's twiddle table, in LDS; LAST: the results go to global memory (lazy signed doubles
+// for the blocks pass), else back to LDS
+template <int LD, int LOGR, bool LAST>
+__device__ __forceinline__ void fuse_block(double *ld, const double *twl, uint32_t s0, FpMod m, uint64_t *dst, uint32_t col0) {
+    constexpr int LOGC = kFuseLog - LD;
+    constexpr uint32_t C = 1u << LOGC;
+    constexpr int R = 1 << LOGR, PER = 8 >> LOGR;
+    const uint32_t low_bits = (uint32_t)(LD - LOGR + LOGC) - s0;
+    const uint32_t low_mask = (1u << low_bits) - 1;
+#pragma unroll
+    for (int gi = 0; gi < PER; gi++) {
+        const uint32_t g = threadIdx.x + kFuseThreads * gi;
+        const uint32_t upper = g >> low_bits;
+        const uint32_t base = (upper << (low_bits + LOGR)) | (g & low_mask);
+        double v[R];
+#pragma unroll
+        for (int j = 0; j < R; j++) v[j] = ld[skew8(base + ((uint32_t)j << low_bits))];
+        fp_ct_block<LOGR, true>(v, twl, (1u << s0) + upper, m);
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+            const uint32_t e = base + ((uint32_t)j << low_bits);
+            if (LAST)
+                dst[(size_t)(e >> LOGC) * 256 + col0 + (e & (C - 1))] = (uint64_t)__double_as_longlong(v[j]);
+            else
+                ld[skew8(e)] = v[j];
+        }
+    }
+}
+
+// what the loop over a group's output limbs fetches one iteration ahead (uniform values: scalar registers)
+struct FuseRow {
+    double q, qinv;
+    uint32_t limb;
+};
+
+template <int LD>
+__global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(2))) void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
+    __shared__ double ld[kFuseWords + (kFuseWords >> 2)];
+    __shared__ double twl[2][256];
+    static_assert(LD >= 4 && LD <= 8, "N from 2^12 to 2^16");
+    constexpr int LOGC = kFuseLog - LD;
+    constexpr uint32_t C = 1u << LOGC, tiles_per_limb = 256u >> LOGC, row_step = kFuseThreads >> LOGC;
+    const size_t n = (size_t)1 << a.log_n;
+
+    // consecutive logical ids (one XCD, one L2): the groups of one tile, which read the same inputs
+    uint32_t lb = logical_block();
+    const uint32_t groups = p.compute_groups + p.copy_groups;
+    const uint32_t grp = lb % groups;
+    lb /= groups;
+    const uint32_t tile = lb % tiles_per_limb, uidx = lb / tiles_per_limb;
+    const uint32_t item = uidx / p.b.n_units;
+    const BconvDesc d = p.b.descs[uidx - item * p.b.n_units];
+    const uint32_t col0 = tile << LOGC;
+    // word i of this thread: tile word t + 256 i = row (t >> LOGC) + i row_step, column t mod C
+    const size_t g0 = (size_t)(threadIdx.x >> LOGC) * 256 + col0 + (threadIdx.x & (C - 1));
+    constexpr size_t gstep = (size_t)row_step * 256;
+    uint64_t *out = p.b.out_base + item * p.b.out_item_stride + d.out_off;
+
+    if (grp >= p.compute_groups) {
+        // limbs that pass through unchanged (a digit's own limbs keep their NTT form)
+        const uint64_t *from = p.b.copy_base + item * p.b.copy_item_stride;
+        const uint32_t first = (grp - p.compute_groups) * p.rows_per;
+        for (uint32_t r = first; r < first + p.rows_per && r < d.copy_count; r++) {
+            const size_t limb = (size_t)(d.copy_first + r) << a.log_n;
+#pragma unroll
+            for (int i = 0; i < 8; i++) out[limb + g0 + gstep * i] = from[limb + g0 + gstep * i];
+        }
+        return;
+    }
+    const uint32_t n_rows = p.b.mdr ? d.n_out - 1 : d.n_out;
+    const uint32_t r_begin = grp * p.rows_per;
+    const uint32_t r_end = r_begin + p.rows_per < n_rows ? r_begin + p.rows_per : n_rows;
+    if (r_begin >= n_rows) return;
+
+    const double *mat = p.b.mat_fp + 2 * d.mat_off;
+    auto fetch_row = [&](uint32_t r, FuseRow &f, double &tw) {
+        const uint32_t table = p.b.out_table[d.map_off + r];
+        f.q = a.fp_consts[4 * (size_t)table];
+        f.qinv = a.fp_consts[4 * (size_t)table + 1];
+        f.limb = p.b.out_limb[d.map_off + r];
+        tw = a.tw_fp[((size_t)table << a.log_n) + threadIdx.x];   // entries 1..255: every twiddle of the rows pass
+    };
+    FuseRow cur;
+    double tw_cur;
+    fetch_row(r_begin, cur, tw_cur);
+
+    // the unit's inputs at this thread's 8 coefficients (limbs past n_in repeat the last one; their matrix entries
+    // are replaced by zero below), all loads in flight together
+    const uint64_t *x = p.b.x_base + item * p.b.x_item_stride + d.x_off;
+    double xv[8][8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        const uint32_t kk = (uint32_t)k < d.n_in ? (uint32_t)k : d.n_in - 1;
+#pragma unroll
+        for (int i = 0; i < 8; i++) xv[k][i] = fp_from_u64(x[((size_t)kk << a.log_n) + g0 + gstep * i]);
+    }
+
+    double rr[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+    if (p.b.mdr) {
+        // coefficients of the dropped limb of the ModDown result, canonical mod q_last
+        const uint32_t last = d.n_out - 1;
+        const FpMod ml = fp_ctx(a, p.b.out_table[d.map_off + last]).m;
+        const double *row = mat + 2 * (size_t)last * d.n_in;
+        const uint64_t *tsrc = x - n;
+#pragma unroll
+        for (int i = 0; i < 8; i++) rr[i] = fp_from_u64(tsrc[g0 + gstep * i]);
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const bool on = (uint32_t)k < d.n_in;
+            const FpTw w{on ? row[2 * k] : 0.0, on ? row[2 * k + 1] : 0.0};
+#pragma unroll
+            for (int i = 0; i < 8; i++) rr[i] -= fp_mulmod(xv[k][i], w, ml);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) rr[i] = fp_canonical(rr[i], ml);
+    }
+    twl[r_begin & 1][threadIdx.x] = tw_cur;
+    lds_barrier();
+
+    for (uint32_t r = r_begin; r < r_end; r++) {
+        // the next output limb's constants travel while this one is computed
+        FuseRow nxt = cur;
+        double tw_nxt = 0.0;
+        const bool more = r + 1 < r_end;
+        if (more) fetch_row(r + 1, nxt, tw_nxt);
+        const FpMod mod{cur.q, cur.qinv};
+        const double *tws = twl[r & 1];
+        // (the matrices are padded: 8 pairs can be fetched whatever the row's length)
+        const double *row = mat + 2 * (size_t)r * d.n_in;
+        double v[8];
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = p.b.mdr ? fp_reduce(rr[i], mod) : 0.0;
+        // every product is reduced to |r| <= 0.75 m: the sums stay exact integers below 7 m < 2^53
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const bool on = (uint32_t)k < d.n_in;
+            const FpTw w{on ? row[2 * k] : 0.0, on ? row[2 * k + 1] : 0.0};
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] += fp_mulmod(xv[k][i], w, mod);
+        }
+        // stages 0..2 pair rows that differ in their top three bits: this thread's own 8 words
+        fp_ct_block<3, true>(v, tws, 1u, mod);
+#pragma unroll
+        for (int i = 0; i < 8; i++) ld[skew8(threadIdx.x + kFuseThreads * i)] = v[i];
+        lds_barrier();
+        uint64_t *dst = out + ((size_t)cur.limb << a.log_n);
+        if constexpr (LD == 8) {
+            fuse_block<LD, 3, false>(ld, tws, 3, mod, dst, col0);
+            lds_barrier();
+            fuse_block<LD, 2, true>(ld, tws, 6, mod, dst, col0);
+        } else if constexpr (LD == 7) {
+            fuse_block<LD, 2, false>(ld, tws, 3, mod, dst, col0);
+            lds_barrier();
+            fuse_block<LD, 2, true>(ld, tws, 5, mod, dst, col0);
+        } else {
+            fuse_block<LD, LD - 3, true>(ld, tws, 3, mod, dst, col0);
+        }
+        if (more) twl[(r + 1) & 1][threadIdx.x] = tw_nxt;
+        lds_barrier();  // every read of this tile is done before the next output limb overwrites it
+        cur = nxt;
     }
 }
 
@@ -991,11 +1184,39 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
 
 }  // namespace
 
-hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s) {
+hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s) {
+    if (a.log_n < 12 || a.log_n > 16 || !b.mat_fp || b.n_units == 0) return hipErrorInvalidValue;
+    static const uint32_t target = [] {
+        const char *e = getenv("CAHEL_HIP_FUSE_ROWS");
+        const int v = e ? atoi(e) : 3;
+        return (uint32_t)(v >= 1 && v <= 64 ? v : 3);
+    }();
+    const uint32_t rows = b.mdr ? b.max_rows - 1 : b.max_rows;
+    if (rows == 0) return hipErrorInvalidValue;
+    BconvRowsK p{b, (rows + target - 1) / target, 0, target};
+    p.copy_groups = b.copy_base ? (b.max_copy + target - 1) / target : 0;
+    const uint32_t items = b.items ? b.items : 1;
+    const int ld = (int)a.log_n - 8;
+    const uint32_t tiles = 256u >> (kFuseLog - ld);
+    const uint64_t wgs = (uint64_t)b.n_units * items * tiles * (p.compute_groups + p.copy_groups);
+    if (wgs > 0x7fffffffu) return hipErrorInvalidValue;
+    const dim3 grid((uint32_t)wgs);
+    switch (ld) {
+#define HE_CASE(LD) \
+    case LD: hipLaunchKernelGGL(bconv_rows_fp_kernel<LD>, grid, dim3(kFuseThreads), 0, s, a, p); break;
+        HE_CASE(4) HE_CASE(5) HE_CASE(6) HE_CASE(7) HE_CASE(8)
+#undef HE_CASE
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool rows_done) {
     if (a.log_n < 9 || a.log_n > 16 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
-    hipError_t e = backend == NTT_BACKEND_MIXED ? launch_rows<true, NTT_BACKEND_MIXED>(a, n_jobs, s)
+    hipError_t e = rows_done                    ? hipSuccess
+                   : backend == NTT_BACKEND_MIXED ? launch_rows<true, NTT_BACKEND_MIXED>(a, n_jobs, s)
                    : backend                    ? launch_rows<true, NTT_BACKEND_FP>(a, n_jobs, s)
                                                 : launch_rows<true, NTT_BACKEND_INT>(a, n_jobs, s);
     if (e != hipSuccess) return e;
@@ -1004,9 +1225,9 @@ hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, h
                                         : launch_blocks<true, NTT_BACKEND_INT>(a, n_polys, s);
 }
 
-hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s) {
+hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s, bool rows_done) {
     if (a.log_n < 9 || a.log_n > 16 || !a.jobs) return hipErrorInvalidValue;
-    if (a.n_jobs) {
+    if (a.n_jobs && !rows_done) {
         hipError_t e = launch_rows<true, NTT_BACKEND_FP>(a, a.n_jobs, s);
         if (e != hipSuccess) return e;
     }

@@ -1,0 +1,95 @@
+"""Base conversion fused with the rows pass of the forward transform (bconv_rows_fp_kernel: every prime below 2^50,
+N >= 2^12) against the oracle, through the C-ABI entry points that use it: he_modup (with the copy of a digit's own
+limbs), he_moddown (1 to 6 polynomials, overwriting and adding), he_keyswitch, he_keyswitch_rescale (the merged
+ModDown + rescale prologue) and its batch form; every degree from 2^12 to 2^16, full and partial last digits, and
+the same calls with the fusion switched off by the environment."""
+import numpy as np
+import pytest
+
+from gpu_util import DeviceArray, make_pair, rand_limbs
+
+pytestmark = pytest.mark.gpu
+
+CASES = [  # logn, bits, size_p, levels
+    (12, [50, 49, 48, 50, 47, 50, 50, 50], 2, (6, 5, 2)),
+    (13, [45, 50, 49, 50, 50, 40, 50, 50, 50], 3, (6, 4)),
+    (14, [50, 49, 48, 50, 50, 50], 2, (4, 3)),
+    (15, [50, 50, 49, 50, 48], 1, (4, 2)),
+    (16, [50] * 16, 8, (8, 3)),
+    (16, [50, 49, 50, 50, 50, 50], 2, (4,)),
+]
+
+
+@pytest.fixture(scope="module")
+def capi():
+    from lancelot_amd import capi as c
+    c.lib()
+    return c
+
+
+def _evk(p, rng, capi):
+    dnum = p.size_q // p.size_p
+    host = [rand_limbs(p, rng, range(p.size_qp), n_polys=2) for _ in range(dnum)]
+    dev = [DeviceArray(capi, host=k) for k in host]
+    return host, dev, capi.evk_array([d.ptr for d in dev])
+
+
+@pytest.mark.parametrize("no_fused", ["0", "1"])
+@pytest.mark.parametrize("logn,bits,size_p,levels", CASES)
+def test_entry_points_with_fused_conversion(oracle, capi, monkeypatch, logn, bits, size_p, levels, no_fused):
+    monkeypatch.setenv("CAHEL_HIP_NO_FUSED_BCONV", no_fused)
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(100 + logn)
+    lib, h = capi.lib(), ctx.he_handle()
+    K, n = p.size_p, p.n
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    for L in levels:
+        beta = -(-L // K)
+        tables = [p.table_index(L, t) for t in range(L + K)]
+        # ModUp (the digits' own limbs are copied by the same launch)
+        c = rand_limbs(p, rng, range(L))
+        c[0, :4] = [0, 1, p.moduli[0] - 1, p.moduli[0] - 2]          # edge residues
+        dc = DeviceArray(capi, host=c)
+        dy = DeviceArray(capi, shape=(beta, L + K, n))
+        ws = DeviceArray(capi, shape=(2 * L, n))
+        capi.check(lib.he_modup(h, L, dc.ptr, dy.ptr, ws.ptr, None))
+        assert (dy.numpy() == p.modup(c)).all(), ("modup", L)
+        # ModDown of 1, 2, 3 and 6 polynomials, overwriting and adding
+        for n_polys in (1, 2, 3, 6):
+            cx = np.stack([rand_limbs(p, rng, tables) for _ in range(n_polys)])
+            md = np.stack([p.moddown(cx[b]) for b in range(n_polys)])
+            wsd = DeviceArray(capi, shape=(n_polys, L, n))
+            dcx, dout = DeviceArray(capi, host=cx), DeviceArray(capi, shape=(n_polys, L, n))
+            capi.check(lib.he_moddown(h, L, dcx.ptr, dout.ptr, n_polys, 0, wsd.ptr, None))
+            assert (dout.numpy() == md).all(), ("moddown", L, n_polys)
+            base = rand_limbs(p, rng, range(L), n_polys=n_polys)
+            dcx, dacc = DeviceArray(capi, host=cx), DeviceArray(capi, host=base)
+            capi.check(lib.he_moddown(h, L, dcx.ptr, dacc.ptr, n_polys, 1, wsd.ptr, None))
+            assert (dacc.numpy() == np.stack([p.add(base[b], md[b]) for b in range(n_polys)])).all(), ("moddown+", L, n_polys)
+        # key switch, and key switch + rescale, with and without a Galois element
+        kws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+        for elt in (0, 5):
+            c = rand_limbs(p, rng, range(L))
+            ct = rand_limbs(p, rng, range(L), n_polys=2)
+            ks = p.key_switch(p.galois_ntt(c, elt) if elt else c, host_evk)
+            want = np.stack([p.add(ct[b], ks[b]) for b in range(2)])
+            dc, dct = DeviceArray(capi, host=c), DeviceArray(capi, host=ct)
+            capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, elt, kws.ptr, None))
+            assert (dct.numpy() == want).all(), ("keyswitch", L, elt)
+            if L >= 2:
+                dct, dout = DeviceArray(capi, host=ct), DeviceArray(capi, shape=(2, L - 1, n))
+                capi.check(lib.he_keyswitch_rescale(h, L, dc.ptr, ptrs, dct.ptr, dout.ptr, elt, kws.ptr, None))
+                assert (dout.numpy() == p.rescale(want)).all(), ("keyswitch_rescale", L, elt)
+        # the batch form over three inputs (separate kernels for the inner product, same conversions)
+        if L >= 2:
+            items = 3
+            c3 = rand_limbs(p, rng, range(L), n_polys=items)
+            ct3 = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
+            bws = DeviceArray(capi, shape=(lib.he_keyswitch_batch_workspace_words(h, L, items),))
+            dc3, dct3 = DeviceArray(capi, host=c3), DeviceArray(capi, host=ct3)
+            dout3 = DeviceArray(capi, shape=(items, 2, L - 1, n))
+            capi.check(lib.he_keyswitch_rescale_batch(h, L, items, dc3.ptr, L, ptrs, dct3.ptr, dout3.ptr, 0, bws.ptr, None))
+            got = dout3.numpy()
+            for k in range(items):
+                ks = p.key_switch(c3[k], host_evk)
+                assert (got[k] == p.rescale(np.stack([p.add(ct3[k][b], ks[b]) for b in range(2)]))).all(), ("batch", L, k)
