@@ -909,23 +909,26 @@ KsWorkspace ks_workspace(const he_context *ctx, const Level *lv, uint32_t L, uin
 
 // ModUp and inner product of a key switch over `items` inputs (item k at c + k * c_item_stride * N): ws -> cx.
 // fold_ct != nullptr: limb L-1 of cx becomes cx * P^-1 + fold_ct (see KsFuseArgs); fold_ct holds [items][2][L][N].
+// add_c0 != nullptr (a rotation, items = 1): polynomial 0 of cx gains P sigma(add_c0) on its data limbs, sigma =
+// X -> X^galois_elt, so that the ModDown of cx yields sigma(add_c0) + KeySwitch(sigma(c)) with no pass for sigma.
 int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint64_t *c, uint32_t c_item_stride,
                   uint32_t items, const uint64_t *const *evk, uint32_t galois_elt, const uint64_t *fold_ct, uint64_t *ws,
-                  he_stream s) {
-    if (items == 0 || (items > 1 && galois_elt)) return HE_E_INVALID_ARGUMENT;
+                  he_stream s, const uint64_t *add_c0 = nullptr) {
+    if (items == 0 || (items > 1 && (galois_elt || add_c0))) return HE_E_INVALID_ARGUMENT;
     const uint64_t *fold_w = fold_ct ? ctx->d_pinv_mod_q + 2 * (size_t)(L - 1) : nullptr;
     const size_t n = ctx->n();
     const KsWorkspace w = ks_workspace(ctx, lv, L, items, ws);
     uint64_t *y = w.y, *cx = w.cx, *tmp = w.tmp;
     const uint64_t *src = c;
-    if (galois_elt) {
+    const bool fused_inner = items == 1 && ctx->fuse_inner && lv->batched && fp_for_level(ctx, L);
+    if (galois_elt && !fused_inner) {
         // sigma(c) is staged in the second half of the ModDown workspace, which ModUp leaves alone and ModDown
-        // only touches after the inner product has read it
+        // only touches after the inner product has read it (the fused path gathers sigma(c) where it reads c)
         uint64_t *staged = tmp + (size_t)L * n;
         if (int rc = he_galois_ntt(ctx, c, staged, L, galois_elt, s)) return rc;
         src = staged;
     }
-    if (items == 1 && ctx->fuse_inner && lv->batched && fp_for_level(ctx, L)) {
+    if (fused_inner) {
         // ModUp without the copy of a digit's own limbs, then the forward NTT fused with the inner product: the
         // transformed digits are never written (216 limb transfers less at L = 24, K = 8)
         NttArgs inv = base_args(ctx, false);
@@ -935,6 +938,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         inv.map = plain_map(L, 0);
         inv.epi_mode = NTT_EPI_MUL;
         inv.w = lv->d_part_hat_inv;
+        inv.in_galois = galois_elt;
         HE_HIP(launch_ntt_inverse(inv, 1, true, S(s)));
         NttArgs fwd = base_args(ctx, true);
         fwd.in = y;
@@ -960,6 +964,9 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
             x.evk.p[d] = evk[d];
         }
         x.own = src;
+        x.own_galois = galois_elt;
+        x.add_c0 = add_c0;
+        x.p_mod_q = ctx->d_p_mod_q;
         x.out = cx;
         x.L = L;
         x.K = ctx->size_p;
@@ -978,7 +985,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
             ptrs.p[d] = evk[d];
         }
         HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, cx, L, ctx->size_p, ctx->size_q, lv->beta, 0, false,
-                                    fold_ct, fold_w, items, 2 * (size_t)L * n, S(s)));
+                                    fold_ct, fold_w, items, 2 * (size_t)L * n, S(s), add_c0, galois_elt, ctx->d_p_mod_q));
     }
     return HE_OK;
 }
@@ -1004,11 +1011,12 @@ int he_rotate(const he_context *ctx, uint32_t L, const uint64_t *ct_in, const ui
     if (!lv) return HE_E_LEVEL_NOT_SET;
     const size_t n = ctx->n();
     const KsWorkspace w = ks_workspace(ctx, lv, L, 1, ws);
-    // (sigma(c0), sigma(c1)) in one pass; sigma(c1) is the key-switch input and is overwritten at the end
-    if (int rc = he_galois_ntt(ctx, ct_in, ct_out, 2 * L, galois_elt, s)) return rc;
-    if (int rc = ks_accumulate(ctx, lv, L, ct_out + (size_t)L * n, L, 1, evk, 0, nullptr, ws, s)) return rc;
-    // out0 = sigma(c0) + ks0, out1 = ks1
-    return moddown_impl(ctx, L, w.cx, ct_out, 2, 1u, w.tmp, s);
+    if (!(galois_elt & 1) || galois_elt >= (2u << ctx->log_n)) return HE_E_INVALID_ARGUMENT;
+    // the automorphism is never a pass of its own: sigma(c1) is gathered where the key switch reads its input,
+    // sigma(c0) where the inner product adds P sigma(c0) to its first polynomial
+    if (int rc = ks_accumulate(ctx, lv, L, ct_in + (size_t)L * n, L, 1, evk, galois_elt, nullptr, ws, s, ct_in)) return rc;
+    // out0 = sigma(c0) + ks0 (the inner product carries P sigma(c0)), out1 = ks1
+    return moddown_impl(ctx, L, w.cx, ct_out, 2, 0u, w.tmp, s);
 }
 
 int he_hoisted_rotations_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *ct_in,

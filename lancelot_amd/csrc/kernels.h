@@ -85,6 +85,7 @@ struct NttArgs {
     const uint64_t *epi_b;
     uint32_t epi_b_poly_stride;
     uint32_t epi_b_mask;      // NTT_EPI_SUB_MUL_ADD: bit (poly mod 32) set = that polynomial has an addend
+    uint32_t in_galois;       // inverse transform, map mode: the input is sigma(in), gathered by the blocks pass
     const uint64_t *pro_w;    // [limbs][2] Shoup constants of the scaling prologue / epilogue, indexed like w
     const uint64_t *pro_src2; // NTT_PRO_MODDOWN_RESCALE: second source, limb (poly) at pro_src2 + poly * pro2_poly_stride * N
     uint32_t pro2_poly_stride;
@@ -199,10 +200,12 @@ struct EvkPtrs {
 // (2, L+K, N) <- sum_d y_d * evk_d ; galois_elt != 0 applies the NTT-domain automorphism to y on load.
 // items inputs (y and out dense, fold_ct fold_item_stride words apart) in one launch.
 // fold_ct / fold_w as in KsFuseArgs (nullptr: plain inner product).
+// add_c0 / add_elt / p_mod_q as in KsFuseArgs (add_elt = 0: add_c0 is added as it is; items must be 1).
 hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
                                 const uint64_t *fold_ct, const uint64_t *fold_w, uint32_t items, size_t fold_item_stride,
-                                hipStream_t s);
+                                hipStream_t s, const uint64_t *add_c0 = nullptr, uint32_t add_elt = 0,
+                                const uint64_t *p_mod_q = nullptr);
 
 // Hoisted rotations: out (2, L+K, N) (+)= sum over steps of the inner product of sigma_s(y) with the step's key, and
 // c0_out (L, N) (+)= sum_s sigma_s(c0).  with_self: c0_out also receives c0 itself and the L limbs after it a copy
@@ -222,6 +225,11 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
 struct KsFuseArgs {
     EvkPtrs evk;          // per digit: [2][size_qp][N], NTT form
     const uint64_t *own;  // the key-switch input c, [L][N], NTT form
+    uint32_t own_galois;  // != 0: the input is sigma(own), gathered while it is read
+    // optional (a rotation): out[0][t] += P * sigma(add_c0)[t] on the data limbs, with the same sigma; the ModDown that
+    // follows divides by P, so the rotated c0 arrives in the result without a pass of its own
+    const uint64_t *add_c0;   // [L][N], NTT form
+    const uint64_t *p_mod_q;  // [size_q][2] Shoup pairs of P mod q_i
     uint64_t *out;        // [2][L+K][N]
     uint32_t L, K, size_q, size_qp, beta;
     // optional: limb L-1 of the result becomes out * fold_w + fold_ct[k][L-1] (what the merged ModDown + rescale

@@ -113,6 +113,14 @@ __device__ __forceinline__ Shoup load_shoup(const uint64_t *table, size_t idx) {
     return Shoup{v.x, v.y};
 }
 
+// NTT-domain automorphism X -> X^elt as a gather: out[i] = in[pi(i)],
+// pi(i) = bitrev(((elt * (2 bitrev(i) + 1)) >> 1) mod N)   (table of cahel-main/include/galois.cuh:45-57, on the fly)
+__device__ __forceinline__ uint32_t galois_index(uint32_t i, uint32_t elt, uint32_t log_n) {
+    const uint32_t r = __brev(i) >> (32 - log_n);
+    const uint32_t raw = (uint32_t)(((uint64_t)elt * (2 * r + 1)) >> 1) & ((1u << log_n) - 1);
+    return __brev(raw) >> (32 - log_n);
+}
+
 // R = 2^LOGR point decimation-in-time block: LOGR consecutive forward stages on register values.
 // v[j] are the elements whose index differs in the LOGR bits that these stages pair, most significant
 // first; idx = 2^s0 + (group number at the first stage s0); twiddle of local stage l, sub-block b is

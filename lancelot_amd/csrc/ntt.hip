@@ -739,7 +739,9 @@ constexpr int kMaxGroup = 4;  // most jobs in one LimbGroup
 // FP64 back end.  EPI compiles the fused forward epilogues in (they cost 64 registers).  Two waves per SIMD: with
 // the epilogues the kernel needs 254 registers; left to itself the compiler spreads into the accumulation registers
 // and a single wave, which costs a third more time (three waves would spill, and measure slower).
-template <bool FWD, bool EPI>
+// GAL: the inverse pass gathers its input through a Galois permutation (a.in_galois); an instantiation of its own, so
+// that the index arithmetic costs the other launches no registers
+template <bool FWD, bool EPI, bool GAL>
 __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *lds) {
     const uint32_t nthreads = blockDim.x;
     const BlocksGeom g = blocks_geom(a);
@@ -788,11 +790,20 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
         }
         lds_barrier();
     };
-    {
-        const uint64_t *src = (FWD ? job.out : job.in) + off;  // the forward blocks pass continues on the rows pass's output
+    // inverse pass of a rotation: the input is sigma(in), gathered here (map mode only)
+    const uint32_t in_elt = (FWD || !GAL) ? 0u : a.in_galois;
+    auto fetch = [&](const Job &j) {
+        const uint64_t *src = (FWD ? j.out : j.in) + off;  // the forward blocks pass continues on the rows pass's output
+        if (!FWD && GAL && in_elt) {
 #pragma unroll
-        for (int i = 0; i < kPer; i++) nx[i] = src[threadIdx.x + i * nthreads];
-    }
+            for (int i = 0; i < kPer; i++)
+                nx[i] = j.in[galois_index((uint32_t)off + threadIdx.x + i * nthreads, in_elt, a.log_n)];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kPer; i++) nx[i] = src[threadIdx.x + i * nthreads];
+        }
+    };
+    fetch(job);
     // the twiddles have arrived before the loop starts: inside it only the prefetch is in flight
 #pragma unroll
     for (int i = 0; i < 15; i++) asm volatile("" ::"v"(tw0[i]), "v"(tw1[i]));
@@ -804,11 +815,7 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
         // (with a fused epilogue the registers go to its operands instead and the next tile is fetched late)
         Job next = job;
         if (more) next = entry(b + 1);
-        if (more && !EPI) {
-            const uint64_t *src = (FWD ? next.out : next.in) + off;
-#pragma unroll
-            for (int i = 0; i < kPer; i++) nx[i] = src[threadIdx.x + i * nthreads];
-        }
+        if (more && !EPI) fetch(next);
         const size_t epi_off = off + (size_t)job.limb * n;
         // SUB_MUL_ADD adds onto the polynomials named by epi_b_mask only (a rotation adds onto c0, not c1)
         const bool add_b = has_addend && (fma_mode || ((a.epi_b_mask >> (job.poly & 31)) & 1));
@@ -818,10 +825,9 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
             const uint64_t *minuend = a.epi_a + (size_t)job.poly * a.epi_a_poly_stride * n + epi_off;
             const uint64_t *addend = add_b ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
 #pragma unroll
-            for (int i = 0; i < kPer; i++) {
-                pre_a[EPI ? i : 0] = minuend[threadIdx.x + i * nthreads];
-                pre_b[EPI ? i : 0] = addend[threadIdx.x + i * nthreads];
-            }
+            for (int i = 0; i < kPer; i++) pre_a[EPI ? i : 0] = minuend[threadIdx.x + i * nthreads];
+#pragma unroll
+            for (int i = 0; i < kPer; i++) pre_b[EPI ? i : 0] = addend[threadIdx.x + i * nthreads];
         }
 
         double v[16];
@@ -883,21 +889,17 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
             for (int i = 0; i < kPer; i++) dst[threadIdx.x + i * nthreads] = o[i];
         }
         if (!more) break;
-        if (EPI) {
-            const uint64_t *src = (FWD ? next.out : next.in) + off;
-#pragma unroll
-            for (int i = 0; i < kPer; i++) nx[i] = src[threadIdx.x + i * nthreads];
-        }
+        if (EPI) fetch(next);
         lds_barrier();  // every read of this tile is done before the next one overwrites it
         stage();
         job = next;
     }
 }
 
-template <bool FWD, bool EPI>
+template <bool FWD, bool EPI, bool GAL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void ntt_blocks_fp_kernel(NttArgs a) {
     __shared__ uint64_t lds[kLdsWords];
-    ntt_blocks_fp_body<FWD, EPI>(a, lds);
+    ntt_blocks_fp_body<FWD, EPI, GAL>(a, lds);
 }
 
 // Forward blocks pass of ModUp fused with the key-switch inner product.  Workgroup = (limb t of Ql u P, tile of
@@ -934,12 +936,14 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
     const size_t key_off = ((size_t)role * x.size_qp + table) * n + off;
     double acc[kPer];
     if (own != 0xffffffffu) {
-        const uint64_t *src = x.own + (size_t)t * n + off;
+        const uint64_t *src = x.own + (size_t)t * n;
         const uint64_t *key = x.evk.p[own] + key_off;
 #pragma unroll
         for (int i = 0; i < kPer; i++) {
             const double w = fp_from_u64(key[tid + i * half]);
-            acc[i] = fp_mulmod(fp_from_u64(src[tid + i * half]), FpTw{w, w * m.qinv}, m);
+            const uint32_t e = (uint32_t)off + tid + i * half;
+            const uint64_t c = src[x.own_galois ? galois_index(e, x.own_galois, a.log_n) : e];
+            acc[i] = fp_mulmod(fp_from_u64(c), FpTw{w, w * m.qinv}, m);
         }
     } else {
 #pragma unroll
@@ -1002,6 +1006,17 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
         }
         lds_barrier();  // every read of this tile is done before the next one overwrites it
     }
+    if (x.add_c0 && !role && t < x.L) {
+        // a rotation: polynomial 0 gains P sigma(c0), which ModDown's division by P turns into sigma(c0)
+        const uint64_t *c0 = x.add_c0 + (size_t)t * n;
+        const double pd = fp_from_u64(x.p_mod_q[2 * t]);
+        const FpTw pw{pd, pd * m.qinv};
+#pragma unroll
+        for (int i = 0; i < kPer; i++) {
+            const uint32_t e = (uint32_t)off + tid + i * half;
+            acc[i] += fp_mulmod(fp_from_u64(c0[x.own_galois ? galois_index(e, x.own_galois, a.log_n) : e]), pw, m);
+        }
+    }
     uint64_t *o = x.out + ((size_t)role * LK + t) * n + off;
     if (x.fold_ct && t == x.L - 1) {
         const uint64_t *cl = x.fold_ct + ((size_t)role * x.L + t) * n + off;
@@ -1018,7 +1033,7 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
 // Integer back end (twiddles stay in the table: 30 Shoup pairs per thread do not fit in registers).  Three waves
 // per SIMD (168 registers, 24 bytes of spill in the forward kernel) hide the latency of the epilogue's operand loads
 // better than the two waves that 196 registers allow.
-template <bool FWD>
+template <bool FWD, bool GAL>
 __device__ __forceinline__ void ntt_blocks_int_body(const NttArgs &a, uint64_t *lds) {
     const uint32_t nthreads = blockDim.x;
     const uint32_t tile_elems = nthreads << 4;
@@ -1034,8 +1049,14 @@ __device__ __forceinline__ void ntt_blocks_int_body(const NttArgs &a, uint64_t *
         const IntCtx ic = int_ctx(a, job.table);
         const uint64_t q = ic.q;
         const uint64_t *src = (FWD ? job.out : job.in) + off;
+        if (!FWD && GAL && a.in_galois) {
 #pragma unroll
-        for (int i = 0; i < kPer; i++) lds[skew(threadIdx.x + i * nthreads)] = src[threadIdx.x + i * nthreads];
+            for (int i = 0; i < kPer; i++)
+                lds[skew(threadIdx.x + i * nthreads)] = job.in[galois_index((uint32_t)off + threadIdx.x + i * nthreads, a.in_galois, a.log_n)];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kPer; i++) lds[skew(threadIdx.x + i * nthreads)] = src[threadIdx.x + i * nthreads];
+        }
         __syncthreads();
         const size_t epi_off = off + (size_t)job.limb * n;
         if (FWD) {
@@ -1086,23 +1107,23 @@ __device__ __forceinline__ void ntt_blocks_int_body(const NttArgs &a, uint64_t *
     }
 }
 
-template <bool FWD>
+template <bool FWD, bool GAL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3, 3))) void ntt_blocks_int_kernel(NttArgs a) {
     __shared__ uint64_t lds[kLdsWords];
-    ntt_blocks_int_body<FWD>(a, lds);
+    ntt_blocks_int_body<FWD, GAL>(a, lds);
 }
 
 // Mixed back end: the limbs of a unit share a modulus, so the whole workgroup takes one branch.  EPI as in
 // ntt_blocks_fp_kernel: the FP64 body compiled with the fused epilogues addresses their operands unconditionally,
 // so it is only launched when the launch has an epilogue.
-template <bool FWD, bool EPI>
+template <bool FWD, bool EPI, bool GAL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void ntt_blocks_mixed_kernel(NttArgs a) {
     __shared__ uint64_t lds[kLdsWords];
     const Job first = decode_job(a, blocks_geom(a).unit.j0);
     if ((a.fp_mask >> first.table) & 1)
-        ntt_blocks_fp_body<FWD, EPI>(a, lds);
+        ntt_blocks_fp_body<FWD, EPI, GAL>(a, lds);
     else
-        ntt_blocks_int_body<FWD>(a, lds);
+        ntt_blocks_int_body<FWD, GAL>(a, lds);
 }
 
 template <bool FWD, int FP>
@@ -1169,16 +1190,26 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
     a.n_polys = n_polys;
     const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD ||
                              a.epi_mode == NTT_EPI_FMA_SUB_MUL);
-    if (FP == NTT_BACKEND_MIXED && epi)
-        hipLaunchKernelGGL((ntt_blocks_mixed_kernel<FWD, FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
+    // the Galois gather of an inverse pass's input lives in instantiations of its own
+    const bool gal = !FWD && a.in_galois != 0 && !a.jobs;
+    const dim3 grid(p.grid), block(p.threads);
+    if (gal) {
+        if (FP == NTT_BACKEND_MIXED)
+            hipLaunchKernelGGL((ntt_blocks_mixed_kernel<false, false, true>), grid, block, 0, s, a);
+        else if (!FP)
+            hipLaunchKernelGGL((ntt_blocks_int_kernel<false, true>), grid, block, 0, s, a);
+        else
+            hipLaunchKernelGGL((ntt_blocks_fp_kernel<false, false, true>), grid, block, 0, s, a);
+    } else if (FP == NTT_BACKEND_MIXED && epi)
+        hipLaunchKernelGGL((ntt_blocks_mixed_kernel<FWD, FWD, false>), grid, block, 0, s, a);
     else if (FP == NTT_BACKEND_MIXED)
-        hipLaunchKernelGGL((ntt_blocks_mixed_kernel<FWD, false>), dim3(p.grid), dim3(p.threads), 0, s, a);
+        hipLaunchKernelGGL((ntt_blocks_mixed_kernel<FWD, false, false>), grid, block, 0, s, a);
     else if (!FP)
-        hipLaunchKernelGGL((ntt_blocks_int_kernel<FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
+        hipLaunchKernelGGL((ntt_blocks_int_kernel<FWD, false>), grid, block, 0, s, a);
     else if (epi)
-        hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, FWD>), dim3(p.grid), dim3(p.threads), 0, s, a);
+        hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, FWD, false>), grid, block, 0, s, a);
     else
-        hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, false>), dim3(p.grid), dim3(p.threads), 0, s, a);
+        hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, false, false>), grid, block, 0, s, a);
     return hipGetLastError();
 }
 

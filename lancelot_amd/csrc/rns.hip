@@ -173,14 +173,6 @@ __global__ __launch_bounds__(kThreads) void pair_square_sum_kernel(PairSquareArg
     p.out2[(size_t)blockIdx.z * poly + idx] = d2;
 }
 
-// NTT-domain automorphism X -> X^elt as a gather: out[i] = in[pi(i)],
-// pi(i) = bitrev(((elt * (2 bitrev(i) + 1)) >> 1) mod N)
-__device__ __forceinline__ uint32_t galois_index(uint32_t i, uint32_t elt, uint32_t log_n) {
-    const uint32_t r = __brev(i) >> (32 - log_n);
-    const uint32_t raw = (uint32_t)(((uint64_t)elt * (2 * r + 1)) >> 1) & ((1u << log_n) - 1);
-    return __brev(raw) >> (32 - log_n);
-}
-
 // grid: (N / 256, total limbs)
 __global__ __launch_bounds__(kThreads) void galois_kernel(const uint64_t *in, uint64_t *out, uint32_t elt,
                                                           uint32_t log_n) {
@@ -319,6 +311,8 @@ struct InnerArgs {
     int accumulate;
     const uint64_t *fold_ct, *fold_w;
     size_t y_item_stride, out_item_stride, fold_item_stride;   // blockIdx.z = item (words between items)
+    const uint64_t *add_c0, *p_mod_q;
+    uint32_t add_elt;
 };
 
 // grid: (N / 256, L + K, items).  Streams beta digit limbs of y and 2 beta key limbs, writes (or accumulates) the
@@ -350,6 +344,11 @@ __global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
     if (p.accumulate) {
         o0 = add_mod(o0, out[o], q);
         o1 = add_mod(o1, out[o + opoly], q);
+    }
+    if (p.add_c0 && t < p.L) {
+        // a rotation: polynomial 0 gains P sigma(c0), which ModDown's division by P turns into sigma(c0)
+        const uint32_t g = p.add_elt ? galois_index(j, p.add_elt, p.log_n) : j;
+        o0 = add_mod(o0, mul_shoup(p.add_c0[((size_t)t << p.log_n) + g], load_shoup(p.p_mod_q, t), q), q);
     }
     if (p.fold_ct && t == p.L - 1) {
         const Shoup w = load_shoup(p.fold_w, 0);
@@ -644,11 +643,12 @@ hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_
 hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
                                 const uint64_t *fold_ct, const uint64_t *fold_w, uint32_t items, size_t fold_item_stride,
-                                hipStream_t s) {
+                                hipStream_t s, const uint64_t *add_c0, uint32_t add_elt, const uint64_t *p_mod_q) {
     const size_t n = (size_t)1 << t.log_n;
     InnerArgs p{y, out, t.moduli, t.barrett, evk, L, K, size_q, beta, t.log_n, galois_elt, accumulate ? 1 : 0,
-                fold_ct, fold_w, (size_t)beta * (L + K) * n, 2 * (size_t)(L + K) * n, fold_item_stride};
-    if (items == 0 || items > 65535) return hipErrorInvalidValue;
+                fold_ct, fold_w, (size_t)beta * (L + K) * n, 2 * (size_t)(L + K) * n, fold_item_stride,
+                add_c0, p_mod_q, add_elt};
+    if (items == 0 || items > 65535 || (add_c0 && (items != 1 || !p_mod_q))) return hipErrorInvalidValue;
     hipLaunchKernelGGL(inner_product_kernel, dim3((1u << t.log_n) / kThreads, L + K, items), dim3(kThreads), 0, s, p);
     return hipGetLastError();
 }
