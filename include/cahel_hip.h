@@ -258,6 +258,25 @@ int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, c
                          const uint64_t *ct, uint64_t *out, uint32_t galois_elt, uint64_t *workspace,
                          he_stream stream);
 
+/* out [2][L-1][N] = rescale(relinearize(ct1 * ct2)) for two size-2 ciphertexts ct1, ct2 [2][L][N] (ct2 == ct1
+ * squares): he_tensor, he_keyswitch and he_rescale with the same limbs in one call; when every prime of the level
+ * is below 2^50 the tensor product is formed by the first pass of the key switch's inverse transform (its third
+ * polynomial is never read back).  workspace: he_multiply_relin_rescale_workspace_words words.
+ * Replaces the sequence multiply (src/evaluate.cu:447-501: tensor_prod_2x2_rns_poly), relinearize_inplace
+ * (src/eval_key_switch.cu:80-216) and rescale_to_next (src/evaluate.cu:2058-2085). */
+size_t he_multiply_relin_rescale_workspace_words(const he_context *ctx, uint32_t L);
+int he_multiply_relin_rescale(const he_context *ctx, uint32_t L, const uint64_t *ct1, const uint64_t *ct2,
+                              const uint64_t *const *evk, uint64_t *out, uint64_t *workspace, he_stream stream);
+
+/* he_multiply_relin_rescale over `items` independent products with one launch per stage: ct1, ct2 [items][2][L][N]
+ * -> out [items][2][L-1][N] (ct2 == ct1 squares every item), all with the same relinearisation key.  The limbs are
+ * those of `items` separate calls.  No counterpart in the reference, which multiplies one pair per call.
+ * workspace: he_multiply_relin_rescale_batch_workspace_words words. */
+size_t he_multiply_relin_rescale_batch_workspace_words(const he_context *ctx, uint32_t L, uint32_t items);
+int he_multiply_relin_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *ct1,
+                                    const uint64_t *ct2, const uint64_t *const *evk, uint64_t *out, uint64_t *workspace,
+                                    he_stream stream);
+
 /* ---- encoder support ----
  * coeffs: DEVICE array of N doubles holding integers (already rounded, |c| < 2^63); out [limbs][N]:
  * out[l][i] = c_i mod q_{first_table + l} (negative values wrap to q - |c| mod q).

@@ -63,6 +63,10 @@ SIGNATURES = {
     "he_keyswitch_rescale_batch": (C.c_int, [vp, u32, u32, vp, u32, C.POINTER(vp), vp, vp, u32, vp, vp]),
     "he_pair_square_sum": (C.c_int, [vp, u32, u32, u32, vp, vp, vp, vp]),
     "he_keyswitch_rescale": (C.c_int, [vp, u32, vp, C.POINTER(vp), vp, vp, u32, vp, vp]),
+    "he_multiply_relin_rescale_workspace_words": (C.c_size_t, [vp, u32]),
+    "he_multiply_relin_rescale": (C.c_int, [vp, u32, vp, vp, C.POINTER(vp), vp, vp, vp]),
+    "he_multiply_relin_rescale_batch_workspace_words": (C.c_size_t, [vp, u32, u32]),
+    "he_multiply_relin_rescale_batch": (C.c_int, [vp, u32, u32, vp, vp, C.POINTER(vp), vp, vp, vp]),
     "he_decompose_real": (C.c_int, [vp, vp, vp, u32, u32, vp]),
     "he_ckks_encode": (C.c_int, [vp, vp, vp, u32, u32, C.c_double, u32, vp, vp, vp]),
     "he_ckks_decode": (C.c_int, [vp, vp, u32, u32, C.c_double, vp, vp, vp]),

@@ -92,6 +92,7 @@ struct he_context {
     double *d_phat_mod_q_fp = nullptr;   // (M, M/q_j) pairs of the P -> Ql matrix
     double *d_phat_pinv_fp = nullptr;    // the same matrix times P^-1 mod q_j (merged ModDown + rescale, fused kernel)
     bool fuse_rows = true;       // environment CAHEL_HIP_NO_FUSED_BCONV=1: conversion kernel, then the rows pass
+    bool fuse_tensor = true;     // environment CAHEL_HIP_NO_FUSED_TENSOR=1: he_multiply_relin_rescale as tensor kernel + key switch
     uint32_t *d_rot_group = nullptr;     // encoder: 5^j mod 2N
     double2 *d_ksi = nullptr;            // encoder: e^{2 pi i k / 2N}, k <= 2N
     uint64_t *d_garner_inv = nullptr;    // decoder: [size_q][size_q], q_j^-1 mod q_i for j < i
@@ -402,6 +403,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->rows_direct = !(rv && rv[0] == '1');
         const char *nb = getenv("CAHEL_HIP_NO_FUSED_BCONV");
         ctx->fuse_rows = !(nb && nb[0] == '1');
+        const char *nt = getenv("CAHEL_HIP_NO_FUSED_TENSOR");
+        ctx->fuse_tensor = !(nt && nt[0] == '1');
         ctx->fp_ok.assign(qp, 0);
         std::vector<double> psi_fp(qp * n, 0.0), ipsi_fp(qp * n, 0.0), consts(4 * qp, 0.0);
         for (size_t t = 0; t < qp; t++) {
@@ -658,13 +661,15 @@ int he_add_p_multiple(const he_context *ctx, const uint64_t *a, const uint64_t *
 int he_tensor(const he_context *ctx, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
               he_stream s) {
     if (!ctx || !ct1 || !ct2 || !out || L == 0 || L > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
-    HE_HIP(launch_tensor(ctx->tables(), ct1, ct2, out, L, false, S(s)));
+    HE_HIP(launch_tensor(ctx->tables(), ct1, ct2, out, L, false, S(s),
+                         L <= ctx->size_q && fp_for(ctx, plain_map(L)) ? ctx->d_fp_consts : nullptr));
     return HE_OK;
 }
 
 int he_tensor_square(const he_context *ctx, const uint64_t *ct, uint64_t *out, uint32_t L, he_stream s) {
     if (!ctx || !ct || !out || L == 0 || L > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
-    HE_HIP(launch_tensor(ctx->tables(), ct, ct, out, L, true, S(s)));
+    HE_HIP(launch_tensor(ctx->tables(), ct, ct, out, L, true, S(s),
+                         L <= ctx->size_q && fp_for(ctx, plain_map(L)) ? ctx->d_fp_consts : nullptr));
     return HE_OK;
 }
 
@@ -913,7 +918,7 @@ KsWorkspace ks_workspace(const he_context *ctx, const Level *lv, uint32_t L, uin
 // X -> X^galois_elt, so that the ModDown of cx yields sigma(add_c0) + KeySwitch(sigma(c)) with no pass for sigma.
 int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint64_t *c, uint32_t c_item_stride,
                   uint32_t items, const uint64_t *const *evk, uint32_t galois_elt, const uint64_t *fold_ct, uint64_t *ws,
-                  he_stream s, const uint64_t *add_c0 = nullptr) {
+                  he_stream s, const uint64_t *add_c0 = nullptr, const TensorFuse *tin = nullptr) {
     if (items == 0 || (items > 1 && (galois_elt || add_c0))) return HE_E_INVALID_ARGUMENT;
     const uint64_t *fold_w = fold_ct ? ctx->d_pinv_mod_q + 2 * (size_t)(L - 1) : nullptr;
     const size_t n = ctx->n();
@@ -939,7 +944,9 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         inv.epi_mode = NTT_EPI_MUL;
         inv.w = lv->d_part_hat_inv;
         inv.in_galois = galois_elt;
-        HE_HIP(launch_ntt_inverse(inv, 1, true, S(s)));
+        // tin: c is the third polynomial of a tensor product that has not been formed yet; the blocks pass forms it
+        if (tin) HE_HIP(launch_tensor_intt_blocks(inv, *tin, S(s)));
+        HE_HIP(launch_ntt_inverse(inv, 1, NTT_BACKEND_FP, S(s), tin != nullptr));
         NttArgs fwd = base_args(ctx, true);
         fwd.in = y;
         fwd.out = y;
@@ -977,6 +984,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         x.fold_w = fold_w;
         HE_HIP(launch_ntt_forward_inner(fwd, x, S(s), rows_done));
     } else {
+        if (tin) return HE_E_INVALID_ARGUMENT;
         if (int rc = modup_impl(ctx, L, src, galois_elt ? L : c_item_stride, items, y, tmp, s)) return rc;
         EvkPtrs ptrs;
         memset(&ptrs, 0, sizeof(ptrs));
@@ -1053,9 +1061,18 @@ int he_hoisted_rotations(const he_context *ctx, uint32_t L, const uint64_t *ct_i
     return he_hoisted_rotations_batch(ctx, L, 1, ct_in, evk, galois_elts, n_steps, 0, ct_out, ws, s);
 }
 
-int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *c,
-                               uint32_t c_item_stride, const uint64_t *const *evk, const uint64_t *ct, uint64_t *out,
-                               uint32_t galois_elt, uint64_t *ws, he_stream s) {
+}  // extern "C"
+
+namespace {
+
+// the fused tensor + key switch of he_multiply_relin_rescale applies: one input, FP64 back end, fused inner product
+bool tensor_fusion_ok(const he_context *ctx, const Level *lv, uint32_t L) {
+    return lv && ctx->fuse_tensor && ctx->fuse_inner && lv->batched && fp_for_level(ctx, L);
+}
+
+int ksr_impl(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *c, uint32_t c_item_stride,
+             const uint64_t *const *evk, const uint64_t *ct, uint64_t *out, uint32_t galois_elt, uint64_t *ws, he_stream s,
+             const TensorFuse *tin) {
     if (!ctx || !c || !evk || !ct || !out || !ws || ctx->size_p == 0 || L < 2 || items == 0 || items > 16384 ||
         c_item_stride < L)
         return HE_E_INVALID_ARGUMENT;
@@ -1072,7 +1089,7 @@ int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items
     // so ModDown and rescale share one inverse and one forward transform.  Every step is exact modular arithmetic:
     // the limbs equal he_keyswitch followed by he_rescale.
     // (1) inner product; limb L-1 of cx leaves as cx_{L-1} P^-1 + ct_{L-1}
-    if (int rc = ks_accumulate(ctx, lv, L, c, c_item_stride, items, evk, galois_elt, ct, ws, s)) return rc;
+    if (int rc = ks_accumulate(ctx, lv, L, c, c_item_stride, items, evk, galois_elt, ct, ws, s, nullptr, tin)) return rc;
     // (2) limb L-1 and the special limbs -> coefficient form, the latter scaled by (P / p_k)^-1
     NttArgs inv = base_args(ctx, false);
     inv.in = cx + (size_t)(L - 1) * n;
@@ -1123,6 +1140,61 @@ int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items
     fwd.epi_dst_poly_stride = L - 1;
     HE_HIP(launch_ntt_forward(fwd, polys, backend_for(ctx, fwd.map, (int)L - 1), S(s), fused));
     return HE_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int he_keyswitch_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *c,
+                               uint32_t c_item_stride, const uint64_t *const *evk, const uint64_t *ct, uint64_t *out,
+                               uint32_t galois_elt, uint64_t *ws, he_stream s) {
+    return ksr_impl(ctx, L, items, c, c_item_stride, evk, ct, out, galois_elt, ws, s, nullptr);
+}
+
+size_t he_multiply_relin_rescale_workspace_words(const he_context *ctx, uint32_t L) {
+    const size_t ks = he_keyswitch_workspace_words(ctx, L);
+    return ks ? ks + 3 * (size_t)L * ctx->n() : 0;
+}
+
+int he_multiply_relin_rescale(const he_context *ctx, uint32_t L, const uint64_t *ct1, const uint64_t *ct2,
+                              const uint64_t *const *evk, uint64_t *out, uint64_t *ws, he_stream s) {
+    if (!ctx || !ct1 || !ct2 || !evk || !out || !ws || ctx->size_p == 0 || L < 2 || L > ctx->size_q)
+        return HE_E_INVALID_ARGUMENT;
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    const size_t n = ctx->n();
+    uint64_t *d01 = ws + he_keyswitch_workspace_words(ctx, L), *d2 = d01 + 2 * (size_t)L * n;
+    if (tensor_fusion_ok(ctx, lv, L)) {
+        const TensorFuse tin{ct1, ct2, d01, d2, L, ct1 == ct2 ? 1 : 0};
+        return ksr_impl(ctx, L, 1, d2, L, evk, d01, out, 0, ws, s, &tin);
+    }
+    // (d0, d1 | d2) are contiguous: the layout of he_tensor's output
+    if (int rc = ct1 == ct2 ? he_tensor_square(ctx, ct1, d01, L, s) : he_tensor(ctx, ct1, ct2, d01, L, s)) return rc;
+    return ksr_impl(ctx, L, 1, d2, L, evk, d01, out, 0, ws, s, nullptr);
+}
+
+size_t he_multiply_relin_rescale_batch_workspace_words(const he_context *ctx, uint32_t L, uint32_t items) {
+    const size_t ks = he_keyswitch_workspace_words(ctx, L);
+    return ks ? (size_t)items * (ks + 3 * (size_t)L * ctx->n()) : 0;
+}
+
+int he_multiply_relin_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *ct1,
+                                    const uint64_t *ct2, const uint64_t *const *evk, uint64_t *out, uint64_t *ws,
+                                    he_stream s) {
+    if (!ctx || !ct1 || !ct2 || !evk || !out || !ws || ctx->size_p == 0 || L < 2 || L > ctx->size_q || items == 0 ||
+        items > 16384)
+        return HE_E_INVALID_ARGUMENT;
+    if (items == 1) return he_multiply_relin_rescale(ctx, L, ct1, ct2, evk, out, ws, s);
+    const Level *lv = level_of(ctx, L);
+    if (!lv) return HE_E_LEVEL_NOT_SET;
+    if (!lv->batched) return HE_E_UNSUPPORTED;
+    const size_t n = ctx->n();
+    // [items] key-switch workspaces | (d0, d1) [items][2][L][N] | d2 [items][L][N]
+    uint64_t *d01 = ws + (size_t)items * he_keyswitch_workspace_words(ctx, L), *d2 = d01 + (size_t)items * 2 * L * n;
+    HE_HIP(launch_tensor(ctx->tables(), ct1, ct2, d01, L, ct1 == ct2, S(s),
+                         fp_for(ctx, plain_map(L)) ? ctx->d_fp_consts : nullptr, items, d2));
+    return ksr_impl(ctx, L, items, d2, L, evk, d01, out, 0, ws, s, nullptr);
 }
 
 int he_keyswitch_rescale(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk,

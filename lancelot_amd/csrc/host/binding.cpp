@@ -328,6 +328,7 @@ PYBIND11_MODULE(pyCAHEL, m) {
     m.def("relinearize", &relinearize, nogil);
     m.def("relinearize_inplace", &relinearize_inplace, nogil);
     m.def("relinearize_rescale_inplace", &relinearize_rescale_inplace, nogil);
+    m.def("multiply_relin_rescale", &multiply_relin_rescale, nogil);
     m.def("pair_square_distances", &pair_square_distances, py::arg("context"), py::arg("clients"), py::arg("pairs"),
           py::arg("relin_key"), py::arg("galois_key"), py::arg("rounds"), py::arg("scale") = 0.0, py::arg("drop_levels") = 0,
           nogil);

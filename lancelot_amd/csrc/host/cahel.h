@@ -432,7 +432,10 @@ std::vector<CAHELGPUCiphertext> pair_square_distances(
     const std::vector<std::pair<std::size_t, std::size_t>> &pairs, const CAHELGPURelinKey &rlk,
     const CAHELGPUGaloisKey &glk, const std::vector<std::vector<int>> &rounds, double scale, std::size_t drop_levels = 0);
 void relinearize_rescale_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted,
-                                 const CAHELGPURelinKey &relin_keys);  // this build's addition
+                                 const CAHELGPURelinKey &relin_keys);
+void multiply_relin_rescale(const CAHELGPUContext &context, const CAHELGPUCiphertext &encrypted1,
+                            const CAHELGPUCiphertext &encrypted2, const CAHELGPURelinKey &relin_keys,
+                            CAHELGPUCiphertext &destination);  // this build's addition
 void relinearize(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, CAHELGPUCiphertext &destination,
                  const CAHELGPURelinKey &relin_keys);
 void mod_switch_to_next_inplace(const CAHELGPUContext &context, CAHELGPUPlaintext &plain);

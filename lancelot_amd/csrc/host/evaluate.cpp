@@ -271,6 +271,48 @@ void relinearize_rescale_inplace(const CAHELGPUContext &context, CAHELGPUCiphert
     encrypted.scale() = scale;
 }
 
+// multiply + relinearize_inplace + rescale_to_next_inplace of two size-2 ciphertexts in one device call
+// (he_multiply_relin_rescale): the same limbs as the three calls, with the tensor product formed inside the first
+// pass of the key switch.  Not in the reference, whose callers run the three back to back (src/evaluate.cu:447-501,
+// src/eval_key_switch.cu:80-216, src/evaluate.cu:2058-2085).
+void multiply_relin_rescale(const CAHELGPUContext &context, const CAHELGPUCiphertext &encrypted1,
+                            const CAHELGPUCiphertext &encrypted2, const CAHELGPURelinKey &relin_keys,
+                            CAHELGPUCiphertext &destination) {
+    require_ckks(context);
+    if (encrypted1.parms_id() != encrypted2.parms_id()) throw std::invalid_argument("encrypted1 and encrypted2 parameter mismatch");
+    check_same(encrypted1, encrypted2, true);
+    if (!(encrypted1.is_ntt_form() && encrypted2.is_ntt_form()))
+        throw std::invalid_argument("encrypted1 or encrypted2 must be in NTT form");
+    if (encrypted1.size() != 2 || encrypted2.size() != 2)
+        throw std::invalid_argument("multiply_relin_rescale takes size-2 operands");
+    if (relin_keys.parms_id() != context.key_parms_id())
+        throw std::invalid_argument("relin_keys is not valid for encryption parameters");
+    if (!context.using_keyswitching()) throw std::logic_error("keyswitching is not supported by the context");
+    const std::size_t chain = encrypted1.chain_index();
+    if (chain == 0) throw std::invalid_argument("key switching needs a data-level ciphertext");
+    if (chain == context.max_chain_index()) throw std::invalid_argument("end of modulus switching chain reached");
+    const double product_scale = encrypted1.scale() * encrypted2.scale();
+    if (!scale_within_bounds(context, product_scale, chain)) throw std::invalid_argument("scale out of bounds");
+    const std::size_t n = context.poly_degree();
+    const uint32_t L = (uint32_t)encrypted1.coeff_modulus_size();
+    auto ptrs = relin_keys.key_ptrs();
+    const std::size_t beta = (L + context.size_p() - 1) / context.size_p();
+    if (ptrs.size() < beta) throw std::invalid_argument("key_poly_num != 2");
+    DeviceBuffer ws(he_multiply_relin_rescale_workspace_words(context.handle(), L)), out(2 * (std::size_t)(L - 1) * n);
+    check_status(he_multiply_relin_rescale(context.handle(), L, encrypted1.data(), encrypted2.data(), ptrs.data(), out.get(),
+                                           ws.get(), context.stream()),
+                 "he_multiply_relin_rescale");
+    destination.is_ntt_form() = true;
+    destination.is_asymmetric_ = encrypted1.is_asymmetric_;
+    destination.data_ = std::move(out);
+    destination.size_ = 2;
+    destination.coeff_modulus_size_ = L - 1;
+    destination.poly_modulus_degree_ = n;
+    destination.chain_index() = chain + 1;
+    destination.parms_id() = context.parms_id_at(chain + 1);
+    destination.scale() = product_scale / static_cast<double>(context.key_modulus()[L - 1].value());
+}
+
 void relinearize(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, CAHELGPUCiphertext &destination,
                  const CAHELGPURelinKey &relin_keys) {
     if (&encrypted != &destination) destination = encrypted;

@@ -105,7 +105,21 @@ enum : int { NTT_BACKEND_INT = 0, NTT_BACKEND_FP = 1, NTT_BACKEND_MIXED = 2 };
 hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool rows_done = false);
 // Inverse transform: phase A (contiguous blocks, reads a.in writes a.out) then phase B (rows, in place on
 // a.out, epilogue NTT_EPI_MUL optional).
-hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s);
+// blocks_done: the blocks pass has run already (launch_tensor_intt_blocks left its lazy words in a.out), only the
+// rows pass is launched.
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool blocks_done = false);
+
+// Tensor product of two size-2 ciphertexts fused with the blocks pass of the inverse transform of its third polynomial
+// (FP64 back end; every prime of the L limbs below 2^50).  `a`: inverse base arguments with map = the L data limbs
+// and out = where the lazy words of INTT(d2) go ([L][N]); finish with launch_ntt_inverse(a, 1, FP, s, true).
+struct TensorFuse {
+    const uint64_t *ct1, *ct2;   // [2][L][N]
+    uint64_t *d01;               // [2][L][N]: d0, d1
+    uint64_t *d2;                // [L][N]: d2 in NTT form
+    uint32_t L;
+    int square;                  // ct2 is ignored, (d0, d1, d2) = (a0^2, 2 a0 a1, a1^2)
+};
+hipError_t launch_tensor_intt_blocks(NttArgs a, const TensorFuse &x, hipStream_t s);
 
 struct Tables {
     const uint64_t *moduli;
@@ -120,8 +134,11 @@ hipError_t launch_elementwise(const Tables &t, int op, const uint64_t *a, const 
 // out = a + b * w[limb] on limbs first .. first+limbs-1 (pointers already offset to limb `first`)
 hipError_t launch_scalar_mul_add(const Tables &t, const uint64_t *a, const uint64_t *b, uint64_t *out,
                                  const uint64_t *w, uint32_t first, uint32_t limbs, hipStream_t s);
+// fp_consts != nullptr: exact FP64 arithmetic (every prime of limbs 0 .. L-1 below 2^50; [tables][4] as in NttArgs)
+// items > 1: that many dense inputs [items][2][L][N] -> (d0, d1) in out [items][2][L][N], d2 in out2 [items][L][N]
 hipError_t launch_tensor(const Tables &t, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
-                         bool square, hipStream_t s);
+                         bool square, hipStream_t s, const double *fp_consts = nullptr, uint32_t items = 1,
+                         uint64_t *out2 = nullptr);
 // (out01 [items][2][L][N], out2 [items][L][N]) = sum over chunks of (a - b)^2 for the pairs of ciphertexts in the
 // device pointer table pairs [items][chunks][2]
 hipError_t launch_pair_square_sum(const Tables &t, const uint64_t *const *pairs, uint64_t *out01, uint64_t *out2,

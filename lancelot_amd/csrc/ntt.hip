@@ -508,11 +508,13 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
 // sum_i x_i M[j][i] + (r mod q_j); the matrix carries the factor P^-1.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kFuseLog = 11;
-constexpr uint32_t kFuseWords = 1u << kFuseLog, kFuseThreads = kFuseWords / 8;
+constexpr uint32_t kFuseWords = 1u << kFuseLog;
 
-// LDS index of tile word e: 8 words of padding per 32, so that the 32 lanes of a half-wave that read the words
-// {32 a + 8 j + c} or {256 u + 32 j + c'} of one register slot j hit distinct 8-byte banks
-__device__ __forceinline__ uint32_t skew8(uint32_t e) { return e + ((e >> 5) << 3); }
+// LDS index of tile word e: 8 words of padding per 32 and 8 more per 256, so that the 32 lanes of a half-wave that
+// read the words {32 a + 8 j + c}, {256 u + 32 j + c'} or {256 u + 32 j + 8 w + c} of one register slot j hit distinct
+// 8-byte banks
+__device__ __forceinline__ uint32_t skew8(uint32_t e) { return e + ((e >> 5) << 3) + ((e >> 8) << 3); }
+constexpr uint32_t kFuseLds = kFuseWords + (kFuseWords >> 2) + (kFuseWords >> 5);
 
 struct BconvRowsK {
     BconvRows b;
@@ -520,18 +522,18 @@ struct BconvRowsK {
 };
 
 // register block of LOGR stages on the groups of a tile that lives in LDS (tile index bits: [upper][LOGR bits][low_bits]);
-// twl: entries 0..255 of the limb's twiddle table, in LDS; LAST: the results go to global memory (lazy signed doubles
-// for the blocks pass), else back to LDS
-template <int LD, int LOGR, bool LAST>
+// P words per thread; twl: entries 0..255 of the limb's twiddle table, in LDS; LAST: the results go to global memory
+// (lazy signed doubles for the blocks pass), else back to LDS
+template <int LD, int P, int LOGR, bool LAST>
 __device__ __forceinline__ void fuse_block(double *ld, const double *twl, uint32_t s0, FpMod m, uint64_t *dst, uint32_t col0) {
     constexpr int LOGC = kFuseLog - LD;
-    constexpr uint32_t C = 1u << LOGC;
-    constexpr int R = 1 << LOGR, PER = 8 >> LOGR;
+    constexpr uint32_t C = 1u << LOGC, T = kFuseWords / P;
+    constexpr int R = 1 << LOGR, PER = P >> LOGR;
     const uint32_t low_bits = (uint32_t)(LD - LOGR + LOGC) - s0;
     const uint32_t low_mask = (1u << low_bits) - 1;
 #pragma unroll
     for (int gi = 0; gi < PER; gi++) {
-        const uint32_t g = threadIdx.x + kFuseThreads * gi;
+        const uint32_t g = threadIdx.x + T * gi;
         const uint32_t upper = g >> low_bits;
         const uint32_t base = (upper << (low_bits + LOGR)) | (g & low_mask);
         double v[R];
@@ -549,19 +551,50 @@ __device__ __forceinline__ void fuse_block(double *ld, const double *twl, uint32
     }
 }
 
-// what the loop over a group's output limbs fetches one iteration ahead (uniform values: scalar registers)
-struct FuseRow {
-    double q, qinv;
-    uint32_t limb;
-};
+// the stages S0 .. LD-1 of the rows pass, in register blocks of at most log2(P) stages with the tile in LDS between them
+template <int LD, int P, int S0>
+__device__ __forceinline__ void fuse_rest(double *ld, const double *twl, FpMod m, uint64_t *dst, uint32_t col0) {
+    constexpr int LOGP = P == 8 ? 3 : 2;
+    constexpr int LOGR = (LD - S0) < LOGP ? (LD - S0) : LOGP;
+    constexpr bool LAST = S0 + LOGR == LD;
+    fuse_block<LD, P, LOGR, LAST>(ld, twl, S0, m, dst, col0);
+    if constexpr (!LAST) {
+        lds_barrier();
+        fuse_rest<LD, P, S0 + LOGR>(ld, twl, m, dst, col0);
+    }
+}
 
-template <int LD>
-__global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(2))) void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
-    __shared__ double ld[kFuseWords + (kFuseWords >> 2)];
-    __shared__ double twl[2][256];
-    static_assert(LD >= 4 && LD <= 8, "N from 2^12 to 2^16");
-    constexpr int LOGC = kFuseLog - LD;
-    constexpr uint32_t C = 1u << LOGC, tiles_per_limb = 256u >> LOGC, row_step = kFuseThreads >> LOGC;
+// a value that every lane of the wave holds (read from LDS with one address) as a scalar
+__device__ __forceinline__ double uniform_f64(double v) {
+    const long long b = __double_as_longlong(v);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b), hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+}
+
+constexpr uint32_t kFuseMaxRows = 8;   // output limbs per workgroup, at most
+
+// P = coefficients per thread.  8: 256 threads, two waves per SIMD.  (4, with 512 threads and four waves per SIMD,
+// compiles but measured 1.7 times slower at N = 2^16: the inputs' registers spill, and a tile needs twice the LDS
+// exchanges and barriers.)
+//
+// Thread -> coefficient mapping.  The thread's P words are rows row0 + i 2^(LD-3) of one column (the first register
+// block pairs exactly these).  At N = 2^16 (LD = 8: 256 rows x 8 columns) wave w takes row0 = w + 4 j, j = lane / 8:
+// the second register block (stages 3..5, rows that differ in bits 2..4) then exchanges words inside the wave only, so
+// the tile needs one workgroup barrier per output limb (before the last block) instead of three; the tile and the
+// twiddles are double / triple buffered so that the next limb's first block never waits for this limb's last one.
+// Other degrees use row0 = thread / C and a barrier after every block.
+template <int LD, int P>
+__global__ __launch_bounds__(kFuseWords / P) __attribute__((amdgpu_waves_per_eu(P == 8 ? 2 : 4)))
+void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
+    constexpr bool WAVE_B = LD == 8 && P == 8;
+    __shared__ double ld[WAVE_B ? 2 : 1][kFuseLds];
+    __shared__ double twl[3][256];
+    __shared__ double mrow[kFuseMaxRows][18];
+    __shared__ uint32_t mlimb[kFuseMaxRows], mtable[kFuseMaxRows];
+    static_assert(LD >= 4 && LD <= 8 && (P == 8 || P == 4), "N from 2^12 to 2^16");
+    constexpr int LOGC = kFuseLog - LD, LOGP = P == 8 ? 3 : 2;
+    constexpr uint32_t T = kFuseWords / P;
+    constexpr uint32_t C = 1u << LOGC, tiles_per_limb = 256u >> LOGC, row_step = T >> LOGC;
     const size_t n = (size_t)1 << a.log_n;
 
     // consecutive logical ids (one XCD, one L2): the groups of one tile, which read the same inputs
@@ -573,8 +606,12 @@ __global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(2)
     const uint32_t item = uidx / p.b.n_units;
     const BconvDesc d = p.b.descs[uidx - item * p.b.n_units];
     const uint32_t col0 = tile << LOGC;
-    // word i of this thread: tile word t + 256 i = row (t >> LOGC) + i row_step, column t mod C
-    const size_t g0 = (size_t)(threadIdx.x >> LOGC) * 256 + col0 + (threadIdx.x & (C - 1));
+    // word i of this thread: row row0 + i row_step, column col of the tile = tile word e0 + T i
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t row0 = WAVE_B ? wave + 4 * (lane >> 3) : threadIdx.x >> LOGC;
+    const uint32_t col = threadIdx.x & (C - 1);
+    const uint32_t e0 = (row0 << LOGC) + col;
+    const size_t g0 = (size_t)row0 * 256 + col0 + col;
     constexpr size_t gstep = (size_t)row_step * 256;
     uint64_t *out = p.b.out_base + item * p.b.out_item_stride + d.out_off;
 
@@ -584,8 +621,11 @@ __global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(2)
         const uint32_t first = (grp - p.compute_groups) * p.rows_per;
         for (uint32_t r = first; r < first + p.rows_per && r < d.copy_count; r++) {
             const size_t limb = (size_t)(d.copy_first + r) << a.log_n;
+            uint64_t w[P];
 #pragma unroll
-            for (int i = 0; i < 8; i++) out[limb + g0 + gstep * i] = from[limb + g0 + gstep * i];
+            for (int i = 0; i < P; i++) w[i] = from[limb + g0 + gstep * i];
+#pragma unroll
+            for (int i = 0; i < P; i++) out[limb + g0 + gstep * i] = w[i];
         }
         return;
     }
@@ -594,30 +634,36 @@ __global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(2)
     const uint32_t r_end = r_begin + p.rows_per < n_rows ? r_begin + p.rows_per : n_rows;
     if (r_begin >= n_rows) return;
 
+    // The constants of this group's output limbs (matrix row, modulus, output limb, table) go to LDS once, and are
+    // read back into scalar registers limb by limb: a scalar load per limb would stall the workgroup for a cache miss.
     const double *mat = p.b.mat_fp + 2 * d.mat_off;
-    auto fetch_row = [&](uint32_t r, FuseRow &f, double &tw) {
+    if (threadIdx.x < (r_end - r_begin) * 18) {
+        const uint32_t rl = threadIdx.x / 18, c = threadIdx.x - rl * 18, r = r_begin + rl;
         const uint32_t table = p.b.out_table[d.map_off + r];
-        f.q = a.fp_consts[4 * (size_t)table];
-        f.qinv = a.fp_consts[4 * (size_t)table + 1];
-        f.limb = p.b.out_limb[d.map_off + r];
-        tw = a.tw_fp[((size_t)table << a.log_n) + threadIdx.x];   // entries 1..255: every twiddle of the rows pass
-    };
-    FuseRow cur;
-    double tw_cur;
-    fetch_row(r_begin, cur, tw_cur);
+        // (the matrices are padded: 8 pairs can be fetched whatever the row's length)
+        mrow[rl][c] = c < 16 ? mat[2 * (size_t)r * d.n_in + c] : a.fp_consts[4 * (size_t)table + (c - 16)];
+        if (c == 0) {
+            mlimb[rl] = p.b.out_limb[d.map_off + r];
+            mtable[rl] = table;
+        }
+    }
+    // entries 1..255 of the first limb's table: every twiddle of the rows pass
+    double tw_cur = a.tw_fp[((size_t)p.b.out_table[d.map_off + r_begin] << a.log_n) + (threadIdx.x & 255)];
 
-    // the unit's inputs at this thread's 8 coefficients (limbs past n_in repeat the last one; their matrix entries
+    // the unit's inputs at this thread's P coefficients (limbs past n_in repeat the last one; their matrix entries
     // are replaced by zero below), all loads in flight together
     const uint64_t *x = p.b.x_base + item * p.b.x_item_stride + d.x_off;
-    double xv[8][8];
+    double xv[8][P];
 #pragma unroll
     for (int k = 0; k < 8; k++) {
         const uint32_t kk = (uint32_t)k < d.n_in ? (uint32_t)k : d.n_in - 1;
 #pragma unroll
-        for (int i = 0; i < 8; i++) xv[k][i] = fp_from_u64(x[((size_t)kk << a.log_n) + g0 + gstep * i]);
+        for (int i = 0; i < P; i++) xv[k][i] = fp_from_u64(x[((size_t)kk << a.log_n) + g0 + gstep * i]);
     }
 
-    double rr[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+    double rr[P];
+#pragma unroll
+    for (int i = 0; i < P; i++) rr[i] = 0.0;
     if (p.b.mdr) {
         // coefficients of the dropped limb of the ModDown result, canonical mod q_last
         const uint32_t last = d.n_out - 1;
@@ -625,61 +671,67 @@ __global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(2)
         const double *row = mat + 2 * (size_t)last * d.n_in;
         const uint64_t *tsrc = x - n;
 #pragma unroll
-        for (int i = 0; i < 8; i++) rr[i] = fp_from_u64(tsrc[g0 + gstep * i]);
+        for (int i = 0; i < P; i++) rr[i] = fp_from_u64(tsrc[g0 + gstep * i]);
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             const bool on = (uint32_t)k < d.n_in;
             const FpTw w{on ? row[2 * k] : 0.0, on ? row[2 * k + 1] : 0.0};
 #pragma unroll
-            for (int i = 0; i < 8; i++) rr[i] -= fp_mulmod(xv[k][i], w, ml);
+            for (int i = 0; i < P; i++) rr[i] -= fp_mulmod(xv[k][i], w, ml);
         }
 #pragma unroll
-        for (int i = 0; i < 8; i++) rr[i] = fp_canonical(rr[i], ml);
+        for (int i = 0; i < P; i++) rr[i] = fp_canonical(rr[i], ml);
     }
-    twl[r_begin & 1][threadIdx.x] = tw_cur;
+    if (threadIdx.x < 256) twl[r_begin % 3][threadIdx.x] = tw_cur;
     lds_barrier();
 
     for (uint32_t r = r_begin; r < r_end; r++) {
-        // the next output limb's constants travel while this one is computed
-        FuseRow nxt = cur;
+        const uint32_t rl = r - r_begin;
+        // the next output limb's twiddles travel while this one is computed
         double tw_nxt = 0.0;
         const bool more = r + 1 < r_end;
-        if (more) fetch_row(r + 1, nxt, tw_nxt);
-        const FpMod mod{cur.q, cur.qinv};
-        const double *tws = twl[r & 1];
-        // (the matrices are padded: 8 pairs can be fetched whatever the row's length)
-        const double *row = mat + 2 * (size_t)r * d.n_in;
-        double v[8];
+        if (more) tw_nxt = a.tw_fp[((size_t)mtable[rl + 1] << a.log_n) + (threadIdx.x & 255)];
+        const FpMod mod{uniform_f64(mrow[rl][16]), uniform_f64(mrow[rl][17])};
+        const uint32_t limb = __builtin_amdgcn_readfirstlane(mlimb[rl]);
+        const double *tws = twl[r % 3];
+        double *tile_ld = ld[WAVE_B ? (r & 1) : 0];
+        double v[P];
 #pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = p.b.mdr ? fp_reduce(rr[i], mod) : 0.0;
+        for (int i = 0; i < P; i++) v[i] = p.b.mdr ? fp_reduce(rr[i], mod) : 0.0;
         // every product is reduced to |r| <= 0.75 m: the sums stay exact integers below 7 m < 2^53
 #pragma unroll
         for (int k = 0; k < 8; k++) {
             const bool on = (uint32_t)k < d.n_in;
-            const FpTw w{on ? row[2 * k] : 0.0, on ? row[2 * k + 1] : 0.0};
+            const FpTw w{on ? uniform_f64(mrow[rl][2 * k]) : 0.0, on ? uniform_f64(mrow[rl][2 * k + 1]) : 0.0};
 #pragma unroll
-            for (int i = 0; i < 8; i++) v[i] += fp_mulmod(xv[k][i], w, mod);
+            for (int i = 0; i < P; i++) v[i] += fp_mulmod(xv[k][i], w, mod);
         }
-        // stages 0..2 pair rows that differ in their top three bits: this thread's own 8 words
-        fp_ct_block<3, true>(v, tws, 1u, mod);
+        // the first log2(P) stages pair rows that differ in their top bits: this thread's own P words
+        fp_ct_block<LOGP, true>(v, tws, 1u, mod);
 #pragma unroll
-        for (int i = 0; i < 8; i++) ld[skew8(threadIdx.x + kFuseThreads * i)] = v[i];
-        lds_barrier();
-        uint64_t *dst = out + ((size_t)cur.limb << a.log_n);
-        if constexpr (LD == 8) {
-            fuse_block<LD, 3, false>(ld, tws, 3, mod, dst, col0);
+        for (int i = 0; i < P; i++) tile_ld[skew8(e0 + T * i)] = v[i];
+        uint64_t *dst = out + ((size_t)limb << a.log_n);
+        if constexpr (WAVE_B) {
+            // stages 3..5 inside the wave: lane (u, col) takes rows 32 u + 4 j + wave, which lanes of this wave wrote
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            const uint32_t u = lane >> 3;
+            const uint32_t base = ((32 * u + wave) << LOGC) + col;
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = tile_ld[skew8(base + ((uint32_t)(4 * j) << LOGC))];
+            fp_ct_block<3, true>(v, tws, 8u + u, mod);
+#pragma unroll
+            for (int j = 0; j < 8; j++) tile_ld[skew8(base + ((uint32_t)(4 * j) << LOGC))] = v[j];
+            // the twiddles of the next limb become visible with the same barrier (their buffer was last read two
+            // limbs ago, and every wave has passed the barrier of the limb in between)
+            if (more) twl[(r + 1) % 3][threadIdx.x] = tw_nxt;
             lds_barrier();
-            fuse_block<LD, 2, true>(ld, tws, 6, mod, dst, col0);
-        } else if constexpr (LD == 7) {
-            fuse_block<LD, 2, false>(ld, tws, 3, mod, dst, col0);
-            lds_barrier();
-            fuse_block<LD, 2, true>(ld, tws, 5, mod, dst, col0);
+            fuse_block<LD, P, 2, true>(tile_ld, tws, 6, mod, dst, col0);
         } else {
-            fuse_block<LD, LD - 3, true>(ld, tws, 3, mod, dst, col0);
+            lds_barrier();
+            fuse_rest<LD, P, LOGP>(tile_ld, tws, mod, dst, col0);
+            if (more && threadIdx.x < 256) twl[(r + 1) % 3][threadIdx.x] = tw_nxt;
+            lds_barrier();  // every read of this tile is done before the next output limb overwrites it
         }
-        if (more) twl[(r + 1) & 1][threadIdx.x] = tw_nxt;
-        lds_barrier();  // every read of this tile is done before the next output limb overwrites it
-        cur = nxt;
     }
 }
 
@@ -1030,6 +1082,79 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
     for (int i = 0; i < kPer; i++) o[tid + i * half] = fp_to_u64(fp_canonical(acc[i], m));
 }
 
+// Tensor product fused with the blocks pass of the inverse transform of its third polynomial (FP64 back end, one
+// workgroup per (limb, tile of 16 T words)): (d0, d1, d2) = (a0 b0, a0 b1 + a1 b0, a1 b1) from the four input tiles,
+// all three written as canonical residues (d2 in NTT form is what the key switch multiplies by its own digit's key),
+// and d2 goes on through the 8 inverse stages inside 256 consecutive words; the lazy words are left in a.out for the
+// rows pass.  One read of d2 and one launch less than tensor kernel + inverse transform.
+template <bool SQUARE>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void tensor_intt_blocks_fp_kernel(NttArgs a, TensorFuse x) {
+    __shared__ uint64_t lds[kLdsWords];
+    double *ld = reinterpret_cast<double *>(lds);
+    const uint32_t nthreads = blockDim.x;
+    const BlocksGeom g = blocks_geom(a);
+    const Job job = decode_job(a, g.unit.j0);
+    const FpCtx fc = fp_ctx(a, job.table);
+    const FpMod m = fc.m;
+    const size_t n = (size_t)1 << a.log_n;
+    const uint32_t gi = threadIdx.x;
+    const uint32_t base0 = ((gi >> 4) << 8) | (gi & 15);
+    const uint32_t base1 = gi << 4;
+    double tw0[15], tw1[15];
+    fp_load_block_tw<4>(tw0, fc.tw, g.idx0 + (gi >> 4));
+    fp_load_block_tw<4>(tw1, fc.tw, g.idx1 + gi);
+
+    const size_t lo = (size_t)job.limb * n + g.off, poly = (size_t)x.L * n;
+#pragma unroll 4
+    for (int i = 0; i < kPer; i++) {
+        const uint32_t e = threadIdx.x + i * nthreads;
+        const double a0 = fp_from_u64(x.ct1[lo + e]), a1 = fp_from_u64(x.ct1[poly + lo + e]);
+        double d0, d1, d2;
+        if (SQUARE) {
+            d0 = fp_canonical(fp_mulmod(a0, FpTw{a0, a0 * m.qinv}, m), m);
+            d2 = fp_canonical(fp_mulmod(a1, FpTw{a1, a1 * m.qinv}, m), m);
+            const double mm = fp_mulmod(a0, FpTw{a1, a1 * m.qinv}, m);
+            d1 = fp_canonical(mm + mm, m);
+        } else {
+            const double b0 = fp_from_u64(x.ct2[lo + e]), b1 = fp_from_u64(x.ct2[poly + lo + e]);
+            d0 = fp_canonical(fp_mulmod(a0, FpTw{b0, b0 * m.qinv}, m), m);
+            d2 = fp_canonical(fp_mulmod(a1, FpTw{b1, b1 * m.qinv}, m), m);
+            // Karatsuba: (a0 + a1)(b0 + b1) - d0 - d2; both factors are below 2 q, the product is reduced to
+            // |r| <= 2 q and the difference stays below 4 q < 2^53
+            const double sb = b0 + b1;
+            const double mm = fp_mulmod(a0 + a1, FpTw{sb, sb * m.qinv}, m);
+            d1 = fp_canonical(mm - d0 - d2, m);
+        }
+        x.d01[lo + e] = fp_to_u64(d0);
+        x.d01[poly + lo + e] = fp_to_u64(d1);
+        x.d2[lo + e] = fp_to_u64(d2);
+        ld[skew(e)] = d2;
+    }
+#pragma unroll
+    for (int i = 0; i < 15; i++) asm volatile("" ::"v"(tw0[i]), "v"(tw1[i]));
+    lds_barrier();
+    double v[16];
+#pragma unroll
+    for (int j = 0; j < 16; j++) v[j] = ld[skew(base1 + j)];
+    fp_gs_block_tw<4, false>(v, tw1, m);
+#pragma unroll
+    for (int j = 0; j < 16; j++) ld[skew(base1 + j)] = v[j];
+    lds_barrier();
+#pragma unroll
+    for (int j = 0; j < 16; j++) v[j] = ld[skew(base0 + (j << 4))];
+    fp_gs_block_tw<4, true>(v, tw0, m);
+#pragma unroll
+    for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
+    lds_barrier();
+    // lazy signed doubles go to the rows pass
+    uint64_t *dst = job.out + g.off;
+    uint64_t o[kPer];
+#pragma unroll
+    for (int i = 0; i < kPer; i++) o[i] = lds[skew(threadIdx.x + i * nthreads)];
+#pragma unroll
+    for (int i = 0; i < kPer; i++) dst[threadIdx.x + i * nthreads] = o[i];
+}
+
 // Integer back end (twiddles stay in the table: 30 Shoup pairs per thread do not fit in registers).  Three waves
 // per SIMD (168 registers, 24 bytes of spill in the forward kernel) hide the latency of the epilogue's operand loads
 // better than the two waves that 196 registers allow.
@@ -1220,7 +1345,7 @@ hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s
     static const uint32_t target = [] {
         const char *e = getenv("CAHEL_HIP_FUSE_ROWS");
         const int v = e ? atoi(e) : 3;
-        return (uint32_t)(v >= 1 && v <= 64 ? v : 3);
+        return (uint32_t)(v >= 1 && v <= (int)kFuseMaxRows ? v : 3);
     }();
     const uint32_t rows = b.mdr ? b.max_rows - 1 : b.max_rows;
     if (rows == 0) return hipErrorInvalidValue;
@@ -1234,7 +1359,7 @@ hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s
     const dim3 grid((uint32_t)wgs);
     switch (ld) {
 #define HE_CASE(LD) \
-    case LD: hipLaunchKernelGGL(bconv_rows_fp_kernel<LD>, grid, dim3(kFuseThreads), 0, s, a, p); break;
+    case LD: hipLaunchKernelGGL((bconv_rows_fp_kernel<LD, 8>), grid, dim3(kFuseWords / 8), 0, s, a, p); break;
         HE_CASE(4) HE_CASE(5) HE_CASE(6) HE_CASE(7) HE_CASE(8)
 #undef HE_CASE
         default: return hipErrorInvalidValue;
@@ -1274,11 +1399,24 @@ hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipSt
     return hipGetLastError();
 }
 
-hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s) {
+hipError_t launch_tensor_intt_blocks(NttArgs a, const TensorFuse &x, hipStream_t s) {
+    if (a.log_n < 9 || a.log_n > 16 || a.jobs || a.map.limbs != x.L || x.L == 0) return hipErrorInvalidValue;
+    const BlocksPlan p = plan_blocks(a, 1);
+    a.batch = 1;
+    a.n_polys = 1;
+    if (x.square)
+        hipLaunchKernelGGL(tensor_intt_blocks_fp_kernel<true>, dim3(p.grid), dim3(p.threads), 0, s, a, x);
+    else
+        hipLaunchKernelGGL(tensor_intt_blocks_fp_kernel<false>, dim3(p.grid), dim3(p.threads), 0, s, a, x);
+    return hipGetLastError();
+}
+
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool blocks_done) {
     if (a.log_n < 9 || a.log_n > 16 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
-    hipError_t e = backend == NTT_BACKEND_MIXED ? launch_blocks<false, NTT_BACKEND_MIXED>(a, n_polys, s)
+    hipError_t e = blocks_done                    ? hipSuccess
+                   : backend == NTT_BACKEND_MIXED ? launch_blocks<false, NTT_BACKEND_MIXED>(a, n_polys, s)
                    : backend                    ? launch_blocks<false, NTT_BACKEND_FP>(a, n_polys, s)
                                                 : launch_blocks<false, NTT_BACKEND_INT>(a, n_polys, s);
     if (e != hipSuccess) return e;

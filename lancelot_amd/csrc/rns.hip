@@ -95,6 +95,8 @@ struct TensorArgs {
     uint64_t *out;
     const uint64_t *moduli, *barrett;
     uint32_t L, log_n;
+    uint64_t *out2;                           // d2 (out + 2 polynomials for a dense size-3 result)
+    size_t in_item_stride, out_item_stride, out2_item_stride;   // blockIdx.z = item (words between items)
 };
 
 // grid: (N / 256, L).  Reads the four input limbs once, writes the three outputs: (d0, d1, d2) =
@@ -105,7 +107,9 @@ __global__ __launch_bounds__(kThreads) void tensor_kernel(TensorArgs p) {
     const uint64_t q = p.moduli[limb], r0 = p.barrett[2 * limb], r1 = p.barrett[2 * limb + 1];
     const size_t poly = (size_t)p.L << p.log_n;
     const size_t idx = ((size_t)limb << p.log_n) + blockIdx.x * kThreads + threadIdx.x;
-    const uint64_t a0 = p.ct1[idx], a1 = p.ct1[idx + poly];
+    const uint64_t *ct1 = p.ct1 + blockIdx.z * p.in_item_stride, *ct2 = p.ct2 + blockIdx.z * p.in_item_stride;
+    uint64_t *out = p.out + blockIdx.z * p.out_item_stride, *out2 = p.out2 + blockIdx.z * p.out2_item_stride;
+    const uint64_t a0 = ct1[idx], a1 = ct1[idx + poly];
     uint64_t d0, d1, d2;
     if (SQUARE) {
         d0 = mul_mod(a0, a0, q, r0, r1);
@@ -113,16 +117,46 @@ __global__ __launch_bounds__(kThreads) void tensor_kernel(TensorArgs p) {
         uint64_t m = mul_mod(a0, a1, q, r0, r1);
         d1 = add_mod(m, m, q);
     } else {
-        const uint64_t b0 = p.ct2[idx], b1 = p.ct2[idx + poly];
+        const uint64_t b0 = ct2[idx], b1 = ct2[idx + poly];
         d0 = mul_mod(a0, b0, q, r0, r1);
         d2 = mul_mod(a1, b1, q, r0, r1);
         // Karatsuba: (a0 + a1)(b0 + b1) - d0 - d2; the sums stay below 2^62
         uint64_t m = mul_mod(a0 + a1, b0 + b1, q, r0, r1);
         d1 = sub_mod(sub_mod(m, d0, q), d2, q);
     }
-    p.out[idx] = d0;
-    p.out[idx + poly] = d1;
-    p.out[idx + 2 * poly] = d2;
+    out[idx] = d0;
+    out[idx + poly] = d1;
+    out2[idx] = d2;
+}
+
+// The same in exact FP64 arithmetic (every prime below 2^50): about 60 instructions per coefficient instead of
+// about 260, the same canonical residues.
+template <bool SQUARE>
+__global__ __launch_bounds__(kThreads) void tensor_fp_kernel(TensorArgs p, const double *fp_consts) {
+    const uint32_t limb = blockIdx.y;
+    const FpMod m{fp_consts[4 * limb], fp_consts[4 * limb + 1]};
+    const size_t poly = (size_t)p.L << p.log_n;
+    const size_t idx = ((size_t)limb << p.log_n) + blockIdx.x * kThreads + threadIdx.x;
+    const uint64_t *ct1 = p.ct1 + blockIdx.z * p.in_item_stride, *ct2 = p.ct2 + blockIdx.z * p.in_item_stride;
+    uint64_t *out = p.out + blockIdx.z * p.out_item_stride, *out2 = p.out2 + blockIdx.z * p.out2_item_stride;
+    const double a0 = fp_from_u64(ct1[idx]), a1 = fp_from_u64(ct1[idx + poly]);
+    double d0, d1, d2;
+    if (SQUARE) {
+        d0 = fp_canonical(fp_mulmod(a0, FpTw{a0, a0 * m.qinv}, m), m);
+        d2 = fp_canonical(fp_mulmod(a1, FpTw{a1, a1 * m.qinv}, m), m);
+        const double mm = fp_mulmod(a0, FpTw{a1, a1 * m.qinv}, m);
+        d1 = fp_canonical(mm + mm, m);
+    } else {
+        const double b0 = fp_from_u64(ct2[idx]), b1 = fp_from_u64(ct2[idx + poly]);
+        d0 = fp_canonical(fp_mulmod(a0, FpTw{b0, b0 * m.qinv}, m), m);
+        d2 = fp_canonical(fp_mulmod(a1, FpTw{b1, b1 * m.qinv}, m), m);
+        const double sb = b0 + b1;
+        const double mm = fp_mulmod(a0 + a1, FpTw{sb, sb * m.qinv}, m);
+        d1 = fp_canonical(mm - d0 - d2, m);
+    }
+    out[idx] = fp_to_u64(d0);
+    out[idx + poly] = fp_to_u64(d1);
+    out2[idx] = fp_to_u64(d2);
 }
 
 // grid: (N / 256, limbs, items).  out[item][limb] = c0 + c1 * s (+ noise[item][limb]) for the ciphertext cts[item]
@@ -571,10 +605,16 @@ hipError_t launch_encrypt_fma(const Tables &t, const uint64_t *u, const uint64_t
 }
 
 hipError_t launch_tensor(const Tables &t, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
-                         bool square, hipStream_t s) {
-    TensorArgs p{ct1, ct2, out, t.moduli, t.barrett, L, t.log_n};
-    dim3 grid((1u << t.log_n) / kThreads, L);
-    if (square)
+                         bool square, hipStream_t s, const double *fp_consts, uint32_t items, uint64_t *out2) {
+    if (items == 0 || items > 65535 || (items > 1 && !out2)) return hipErrorInvalidValue;
+    const size_t poly = (size_t)L << t.log_n;
+    TensorArgs p{ct1, ct2, out, t.moduli, t.barrett, L, t.log_n, out2 ? out2 : out + 2 * poly, 2 * poly, 2 * poly, poly};
+    dim3 grid((1u << t.log_n) / kThreads, L, items);
+    if (fp_consts && square)
+        hipLaunchKernelGGL(tensor_fp_kernel<true>, grid, dim3(kThreads), 0, s, p, fp_consts);
+    else if (fp_consts)
+        hipLaunchKernelGGL(tensor_fp_kernel<false>, grid, dim3(kThreads), 0, s, p, fp_consts);
+    else if (square)
         hipLaunchKernelGGL(tensor_kernel<true>, grid, dim3(kThreads), 0, s, p);
     else
         hipLaunchKernelGGL(tensor_kernel<false>, grid, dim3(kThreads), 0, s, p);

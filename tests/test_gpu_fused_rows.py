@@ -93,3 +93,68 @@ def test_entry_points_with_fused_conversion(oracle, capi, monkeypatch, logn, bit
             for k in range(items):
                 ks = p.key_switch(c3[k], host_evk)
                 assert (got[k] == p.rescale(np.stack([p.add(ct3[k][b], ks[b]) for b in range(2)]))).all(), ("batch", L, k)
+
+
+@pytest.mark.parametrize("no_fused", ["0", "1"])
+@pytest.mark.parametrize("logn,bits,size_p,levels", CASES + [(11, [45, 40, 40, 50], 1, (3, 2)), (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, (6, 3))])
+def test_multiply_relin_rescale_entry_point(oracle, capi, monkeypatch, logn, bits, size_p, levels, no_fused):
+    """he_multiply_relin_rescale (tensor product formed inside the key switch's first pass when every prime is below
+    2^50; tensor kernel + key switch otherwise or when switched off) against the oracle's tensor, relinearize and
+    rescale; a product of two ciphertexts and a square."""
+    monkeypatch.setenv("CAHEL_HIP_NO_FUSED_TENSOR", no_fused)
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(200 + logn)
+    lib, h = capi.lib(), ctx.he_handle()
+    n = p.n
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    for L in levels:
+        if L < 2:
+            continue
+        a = rand_limbs(p, rng, range(L), n_polys=2)
+        b = rand_limbs(p, rng, range(L), n_polys=2)
+        a[0, 0, :3] = [0, p.moduli[0] - 1, 1]
+        b[1, 0, :3] = [p.moduli[0] - 1, p.moduli[0] - 1, 0]
+        da, db = DeviceArray(capi, host=a), DeviceArray(capi, host=b)
+        ws = DeviceArray(capi, shape=(lib.he_multiply_relin_rescale_workspace_words(h, L),))
+        dout = DeviceArray(capi, shape=(2, L - 1, n))
+        capi.check(lib.he_multiply_relin_rescale(h, L, da.ptr, db.ptr, ptrs, dout.ptr, ws.ptr, None))
+        t3 = p.tensor(a, b)
+        ks = p.key_switch(t3[2], host_evk)
+        want = p.rescale(np.stack([p.add(t3[k], ks[k]) for k in range(2)]))
+        assert (dout.numpy() == want).all(), ("product", L)
+        assert (da.numpy() == a).all() and (db.numpy() == b).all()
+        capi.check(lib.he_multiply_relin_rescale(h, L, da.ptr, da.ptr, ptrs, dout.ptr, ws.ptr, None))
+        t3 = p.tensor(a, a)
+        ks = p.key_switch(t3[2], host_evk)
+        want = p.rescale(np.stack([p.add(t3[k], ks[k]) for k in range(2)]))
+        assert (dout.numpy() == want).all(), ("square", L)
+    assert lib.he_multiply_relin_rescale(h, 1, da.ptr, db.ptr, ptrs, dout.ptr, ws.ptr, None) == -1
+
+
+@pytest.mark.parametrize("logn,bits,size_p,L,items", [(13, [45, 50, 49, 50, 50, 40, 50, 50, 50], 3, 6, 3),
+                                                       (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5, 4),
+                                                       (16, [50, 49, 50, 50, 50, 50], 2, 4, 2)])
+def test_multiply_relin_rescale_batch_equals_single_calls(oracle, capi, logn, bits, size_p, L, items):
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(300 + logn)
+    lib, h = capi.lib(), ctx.he_handle()
+    n = p.n
+    host_evk, dev_evk, ptrs = _evk(p, rng, capi)
+    a = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
+    b = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
+    da, db = DeviceArray(capi, host=a), DeviceArray(capi, host=b)
+    ws = DeviceArray(capi, shape=(lib.he_multiply_relin_rescale_batch_workspace_words(h, L, items),))
+    dout = DeviceArray(capi, shape=(items, 2, L - 1, n))
+    capi.check(lib.he_multiply_relin_rescale_batch(h, L, items, da.ptr, db.ptr, ptrs, dout.ptr, ws.ptr, None))
+    got = dout.numpy()
+    for k in range(items):
+        t3 = p.tensor(a[k], b[k])
+        ks = p.key_switch(t3[2], host_evk)
+        assert (got[k] == p.rescale(np.stack([p.add(t3[j], ks[j]) for j in range(2)]))).all(), k
+    # squares of every item
+    capi.check(lib.he_multiply_relin_rescale_batch(h, L, items, da.ptr, da.ptr, ptrs, dout.ptr, ws.ptr, None))
+    got = dout.numpy()
+    for k in range(items):
+        t3 = p.tensor(a[k], a[k])
+        ks = p.key_switch(t3[2], host_evk)
+        assert (got[k] == p.rescale(np.stack([p.add(t3[j], ks[j]) for j in range(2)]))).all(), ("square", k)
