@@ -86,6 +86,8 @@ public:
     ~DeviceBuffer() { release(); }
     void allocate(std::size_t words);
     void release();
+    // becomes a copy of the first `words` words of `src`; keeps its own block when that is large enough
+    void assign(const DeviceBuffer &src, std::size_t words);
     uint64_t *get() const { return ptr_; }
     std::size_t words() const { return words_; }
     static void trim_pool();  // return every cached block to the driver
@@ -214,6 +216,12 @@ class CAHELGPUCiphertext {
 public:
     CAHELGPUCiphertext() = default;
     explicit CAHELGPUCiphertext(const CAHELGPUContext &) {}
+    // copies move size() polynomials; the buffer behind data() may be larger than that (resize keeps a block that is
+    // large enough, so that relinearize_inplace's 3 -> 2 polynomials and a later growth back cost no device copy)
+    CAHELGPUCiphertext(const CAHELGPUCiphertext &o) { *this = o; }
+    CAHELGPUCiphertext &operator=(const CAHELGPUCiphertext &o);
+    CAHELGPUCiphertext(CAHELGPUCiphertext &&) noexcept = default;
+    CAHELGPUCiphertext &operator=(CAHELGPUCiphertext &&) noexcept = default;
     // keeps the leading min(old, new) words (include/ciphertext.h:303-333)
     void resize(const CAHELGPUContext &context, std::size_t chain_index, std::size_t size);
     void resize(std::size_t size, std::size_t coeff_modulus_size, std::size_t poly_modulus_degree);

@@ -153,6 +153,13 @@ DeviceBuffer &DeviceBuffer::operator=(const DeviceBuffer &o) {
     return *this;
 }
 
+void DeviceBuffer::assign(const DeviceBuffer &src, std::size_t words) {
+    if (this == &src) return;
+    if (words > src.words_) throw std::logic_error("DeviceBuffer::assign: source too small");
+    if (words_ < words || !ptr_) allocate(words);
+    if (words) check_status(he_memcpy_d2d(ptr_, src.ptr_, words * sizeof(uint64_t), current_stream()), "device copy failed");
+}
+
 DeviceBuffer &DeviceBuffer::operator=(DeviceBuffer &&o) noexcept {
     if (this != &o) {
         release();
@@ -223,10 +230,26 @@ void CAHELGPUPlaintext::resize(std::size_t coeff_modulus_size, std::size_t poly_
     poly_modulus_degree_ = poly_modulus_degree;
 }
 
+CAHELGPUCiphertext &CAHELGPUCiphertext::operator=(const CAHELGPUCiphertext &o) {
+    if (this == &o) return *this;
+    data_.assign(o.data_, o.size_ * o.coeff_modulus_size_ * o.poly_modulus_degree_);
+    size_ = o.size_;
+    chain_index_ = o.chain_index_;
+    coeff_modulus_size_ = o.coeff_modulus_size_;
+    poly_modulus_degree_ = o.poly_modulus_degree_;
+    scale_ = o.scale_;
+    is_ntt_form_ = o.is_ntt_form_;
+    is_asymmetric_ = o.is_asymmetric_;
+    parms_id_ = o.parms_id_;
+    prng_seed_ = o.prng_seed_;
+    return *this;
+}
+
 void CAHELGPUCiphertext::resize(std::size_t size, std::size_t coeff_modulus_size, std::size_t poly_modulus_degree) {
     const std::size_t old_words = size_ * coeff_modulus_size_ * poly_modulus_degree_;
     const std::size_t new_words = size * coeff_modulus_size * poly_modulus_degree;
-    if (new_words != data_.words()) {
+    // a block that is large enough stays: the leading words are the ones to keep anyway
+    if (new_words > data_.words() || !data_.get()) {
         DeviceBuffer fresh(new_words);
         const std::size_t keep = old_words < new_words ? old_words : new_words;
         if (keep && data_.get())

@@ -143,7 +143,10 @@ void multiply_plain(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypte
     multiply_plain_inplace(context, destination, plain);
 }
 
-void multiply_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted1, const CAHELGPUCiphertext &encrypted2) {
+// destination = encrypted1 * encrypted2 as a size-3 ciphertext; destination may be either operand.  The product is
+// written into a fresh block, so neither an in-place call nor a distinct destination costs a device copy.
+static void multiply_into(const CAHELGPUContext &context, const CAHELGPUCiphertext &encrypted1,
+                          const CAHELGPUCiphertext &encrypted2, CAHELGPUCiphertext &destination) {
     require_ckks(context);
     if (encrypted1.parms_id() != encrypted2.parms_id()) throw std::invalid_argument("encrypted1 and encrypted2 parameter mismatch");
     check_same(encrypted1, encrypted2, true);
@@ -152,28 +155,36 @@ void multiply_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encryp
     if (encrypted1.size() != 2 || encrypted2.size() != 2)
         throw std::invalid_argument("ciphertext multiplication is implemented for size-2 operands");
     const uint32_t L = (uint32_t)encrypted1.coeff_modulus_size();
-    const std::size_t chain = encrypted1.chain_index();
-    if (&encrypted1 == &encrypted2) {
-        encrypted1.resize(context, chain, 3);
-        check_status(he_tensor_square(context.handle(), encrypted1.data(), encrypted1.data(), L, context.stream()),
+    const std::size_t chain = encrypted1.chain_index(), n = encrypted1.poly_modulus_degree();
+    const double scale = encrypted1.scale() * encrypted2.scale();
+    DeviceBuffer product(3 * (std::size_t)L * n);
+    if (&encrypted1 == &encrypted2)
+        check_status(he_tensor_square(context.handle(), encrypted1.data(), product.get(), L, context.stream()),
                      "he_tensor_square");
-    } else {
-        encrypted1.resize(context, chain, 3);
-        check_status(he_tensor(context.handle(), encrypted1.data(), encrypted2.data(), encrypted1.data(), L, context.stream()),
+    else
+        check_status(he_tensor(context.handle(), encrypted1.data(), encrypted2.data(), product.get(), L, context.stream()),
                      "he_tensor");
-    }
-    encrypted1.scale() *= encrypted2.scale();
-    if (!scale_within_bounds(context, encrypted1.scale(), chain)) throw std::invalid_argument("scale out of bounds");
+    const bool asym = encrypted1.is_asymmetric_;
+    const auto id = encrypted1.parms_id();
+    destination.data_ = std::move(product);
+    destination.size_ = 3;
+    destination.coeff_modulus_size_ = L;
+    destination.poly_modulus_degree_ = n;
+    destination.chain_index() = chain;
+    destination.parms_id() = id;
+    destination.is_ntt_form() = true;
+    destination.is_asymmetric_ = asym;
+    destination.scale() = scale;
+    if (!scale_within_bounds(context, scale, chain)) throw std::invalid_argument("scale out of bounds");
+}
+
+void multiply_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted1, const CAHELGPUCiphertext &encrypted2) {
+    multiply_into(context, encrypted1, encrypted2, encrypted1);
 }
 
 void multiply(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted1, const CAHELGPUCiphertext &encrypted2,
               CAHELGPUCiphertext &destination) {
-    if (&encrypted2 == &destination) {
-        multiply_inplace(context, destination, encrypted1);
-    } else {
-        if (&encrypted1 != &destination) destination = encrypted1;
-        multiply_inplace(context, destination, encrypted2);
-    }
+    multiply_into(context, encrypted1, encrypted2, destination);
 }
 
 void multiply_and_relin_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted1,
@@ -187,21 +198,15 @@ void multiply_many(const CAHELGPUContext &, std::vector<CAHELGPUCiphertext> &, C
 }
 
 void square_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted) {
-    require_ckks(context);
     if (!encrypted.is_ntt_form()) throw std::invalid_argument("encrypted must be in NTT form");
     if (encrypted.size() != 2) throw std::invalid_argument("ciphertext squaring is implemented for size-2 operands");
-    const uint32_t L = (uint32_t)encrypted.coeff_modulus_size();
-    const std::size_t chain = encrypted.chain_index();
-    encrypted.resize(context, chain, 3);
-    check_status(he_tensor_square(context.handle(), encrypted.data(), encrypted.data(), L, context.stream()),
-                 "he_tensor_square");
-    encrypted.scale() *= encrypted.scale();
-    if (!scale_within_bounds(context, encrypted.scale(), chain)) throw std::invalid_argument("scale out of bounds");
+    multiply_into(context, encrypted, encrypted, encrypted);
 }
 
 void square(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, CAHELGPUCiphertext &destination) {
-    if (&encrypted != &destination) destination = encrypted;
-    square_inplace(context, destination);
+    if (!encrypted.is_ntt_form()) throw std::invalid_argument("encrypted must be in NTT form");
+    if (encrypted.size() != 2) throw std::invalid_argument("ciphertext squaring is implemented for size-2 operands");
+    multiply_into(context, encrypted, encrypted, destination);
 }
 
 void exponentiate_inplace(const CAHELGPUContext &, CAHELGPUCiphertext &, uint64_t, CAHELGPURelinKey &) {
