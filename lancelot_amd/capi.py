@@ -48,6 +48,7 @@ SIGNATURES = {
     "he_add_p_multiple": (C.c_int, [vp, vp, vp, vp, u32, u32, vp]),
     "he_tensor": (C.c_int, [vp, vp, vp, vp, u32, vp]),
     "he_tensor_square": (C.c_int, [vp, vp, vp, u32, vp]),
+    "he_tensor_mxn": (C.c_int, [vp, vp, u32, vp, u32, vp, u32, vp]),
     "he_galois_ntt": (C.c_int, [vp, vp, vp, u32, u32, vp]),
     "he_rescale": (C.c_int, [vp, vp, vp, u32, u32, vp, vp]),
     "he_rescale_static": (C.c_int, [vp, vp, vp, u32, u32, vp]),

@@ -673,6 +673,15 @@ int he_tensor_square(const he_context *ctx, const uint64_t *ct, uint64_t *out, u
     return HE_OK;
 }
 
+int he_tensor_mxn(const he_context *ctx, const uint64_t *ct1, uint32_t size1, const uint64_t *ct2, uint32_t size2,
+                  uint64_t *out, uint32_t L, he_stream s) {
+    if (!ctx || !ct1 || !ct2 || !out || L == 0 || L > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
+    if (size1 == 0 || size2 == 0) return HE_E_INVALID_ARGUMENT;
+    if (size1 > 3 || size2 > 3) return HE_E_UNSUPPORTED;
+    HE_HIP(launch_tensor_mxn(ctx->tables(), ct1, size1, ct2, size2, out, L, S(s)));
+    return HE_OK;
+}
+
 int he_pair_square_sum(const he_context *ctx, uint32_t L, uint32_t items, uint32_t chunks,
                        const uint64_t *const *d_pairs, uint64_t *out01, uint64_t *out2, he_stream s) {
     if (!ctx || !d_pairs || !out01 || !out2 || L == 0 || L > ctx->size_q || items == 0 || items > 16384 || chunks == 0)

@@ -152,13 +152,21 @@ static void multiply_into(const CAHELGPUContext &context, const CAHELGPUCipherte
     check_same(encrypted1, encrypted2, true);
     if (!(encrypted1.is_ntt_form() && encrypted2.is_ntt_form()))
         throw std::invalid_argument("encrypted1 or encrypted2 must be in NTT form");
-    if (encrypted1.size() != 2 || encrypted2.size() != 2)
-        throw std::invalid_argument("ciphertext multiplication is implemented for size-2 operands");
+    const std::size_t size1 = encrypted1.size(), size2 = encrypted2.size();
+    if (size1 < 2 || size2 < 2) throw std::invalid_argument("ciphertext size must be at least 2");
+    // the reference takes operands of any size (src/evaluate.cu:474-488: tensor_prod_mxn_rns_poly); here a size-3
+    // operand is the largest (what a multiplication without relinearisation leaves)
+    if (size1 > 3 || size2 > 3) throw std::invalid_argument("ciphertext multiplication takes operands of size 2 or 3");
+    const std::size_t dest_size = size1 + size2 - 1;
     const uint32_t L = (uint32_t)encrypted1.coeff_modulus_size();
     const std::size_t chain = encrypted1.chain_index(), n = encrypted1.poly_modulus_degree();
     const double scale = encrypted1.scale() * encrypted2.scale();
-    DeviceBuffer product(3 * (std::size_t)L * n);
-    if (&encrypted1 == &encrypted2)
+    DeviceBuffer product(dest_size * (std::size_t)L * n);
+    if (dest_size != 3)
+        check_status(he_tensor_mxn(context.handle(), encrypted1.data(), (uint32_t)size1, encrypted2.data(), (uint32_t)size2,
+                                   product.get(), L, context.stream()),
+                     "he_tensor_mxn");
+    else if (&encrypted1 == &encrypted2)
         check_status(he_tensor_square(context.handle(), encrypted1.data(), product.get(), L, context.stream()),
                      "he_tensor_square");
     else
@@ -167,7 +175,7 @@ static void multiply_into(const CAHELGPUContext &context, const CAHELGPUCipherte
     const bool asym = encrypted1.is_asymmetric_;
     const auto id = encrypted1.parms_id();
     destination.data_ = std::move(product);
-    destination.size_ = 3;
+    destination.size_ = dest_size;
     destination.coeff_modulus_size_ = L;
     destination.poly_modulus_degree_ = n;
     destination.chain_index() = chain;
@@ -197,15 +205,14 @@ void multiply_many(const CAHELGPUContext &, std::vector<CAHELGPUCiphertext> &, C
     throw std::logic_error("unsupported scheme");  // BFV only in the reference (src/evaluate.cu:305-306)
 }
 
+// a size-3 operand goes through the general tensor product, as in the reference (src/evaluate.cu:531-545)
 void square_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted) {
     if (!encrypted.is_ntt_form()) throw std::invalid_argument("encrypted must be in NTT form");
-    if (encrypted.size() != 2) throw std::invalid_argument("ciphertext squaring is implemented for size-2 operands");
     multiply_into(context, encrypted, encrypted, encrypted);
 }
 
 void square(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, CAHELGPUCiphertext &destination) {
     if (!encrypted.is_ntt_form()) throw std::invalid_argument("encrypted must be in NTT form");
-    if (encrypted.size() != 2) throw std::invalid_argument("ciphertext squaring is implemented for size-2 operands");
     multiply_into(context, encrypted, encrypted, destination);
 }
 

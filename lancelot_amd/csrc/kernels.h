@@ -139,6 +139,9 @@ hipError_t launch_scalar_mul_add(const Tables &t, const uint64_t *a, const uint6
 hipError_t launch_tensor(const Tables &t, const uint64_t *ct1, const uint64_t *ct2, uint64_t *out, uint32_t L,
                          bool square, hipStream_t s, const double *fp_consts = nullptr, uint32_t items = 1,
                          uint64_t *out2 = nullptr);
+// ct1 [s1][L][N] x ct2 [s2][L][N] -> out [s1 + s2 - 1][L][N], 1 <= s1, s2 <= 3
+hipError_t launch_tensor_mxn(const Tables &t, const uint64_t *ct1, uint32_t s1, const uint64_t *ct2, uint32_t s2,
+                             uint64_t *out, uint32_t L, hipStream_t s);
 // (out01 [items][2][L][N], out2 [items][L][N]) = sum over chunks of (a - b)^2 for the pairs of ciphertexts in the
 // device pointer table pairs [items][chunks][2]
 hipError_t launch_pair_square_sum(const Tables &t, const uint64_t *const *pairs, uint64_t *out01, uint64_t *out2,

@@ -159,6 +159,33 @@ __global__ __launch_bounds__(kThreads) void tensor_fp_kernel(TensorArgs p, const
     out2[idx] = fp_to_u64(d2);
 }
 
+// General tensor product: grid (N / 256, L); ct1 [S1][L][N], ct2 [S2][L][N] -> out [S1 + S2 - 1][L][N],
+// out_j = sum over a + b = j of ct1_a * ct2_b with the products summed in 128 bits and reduced once (at most three
+// products of 61-bit factors).  Sizes are template parameters: the operands stay in registers, nothing is allocated
+// on the device.  out may be ct1's buffer: every coefficient is read before it is written.
+template <int S1, int S2>
+__global__ __launch_bounds__(kThreads) void tensor_mxn_kernel(TensorArgs p) {
+    const uint32_t limb = blockIdx.y;
+    const uint64_t q = p.moduli[limb], r0 = p.barrett[2 * limb], r1 = p.barrett[2 * limb + 1];
+    const size_t poly = (size_t)p.L << p.log_n;
+    const size_t idx = ((size_t)limb << p.log_n) + blockIdx.x * kThreads + threadIdx.x;
+    uint64_t c1[S1], c2[S2], o[S1 + S2 - 1];
+#pragma unroll
+    for (int a = 0; a < S1; a++) c1[a] = p.ct1[idx + poly * a];
+#pragma unroll
+    for (int b = 0; b < S2; b++) c2[b] = p.ct2[idx + poly * b];
+#pragma unroll
+    for (int j = 0; j < S1 + S2 - 1; j++) {
+        U128 acc{0, 0};
+#pragma unroll
+        for (int a = 0; a < S1; a++)
+            if (j - a >= 0 && j - a < S2) mac128(acc, c1[a], c2[j - a]);
+        o[j] = barrett128(acc.lo, acc.hi, q, r0, r1);
+    }
+#pragma unroll
+    for (int j = 0; j < S1 + S2 - 1; j++) p.out[idx + poly * j] = o[j];
+}
+
 // grid: (N / 256, limbs, items).  out[item][limb] = c0 + c1 * s (+ noise[item][limb]) for the ciphertext cts[item]
 __global__ __launch_bounds__(kThreads) void decrypt_gather_kernel(const uint64_t *const *cts, const uint64_t *sk,
                                                                   const uint64_t *noise, uint64_t *out,
@@ -618,6 +645,19 @@ hipError_t launch_tensor(const Tables &t, const uint64_t *ct1, const uint64_t *c
         hipLaunchKernelGGL(tensor_kernel<true>, grid, dim3(kThreads), 0, s, p);
     else
         hipLaunchKernelGGL(tensor_kernel<false>, grid, dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_tensor_mxn(const Tables &t, const uint64_t *ct1, uint32_t s1, const uint64_t *ct2, uint32_t s2,
+                             uint64_t *out, uint32_t L, hipStream_t s) {
+    const size_t poly = (size_t)L << t.log_n;
+    TensorArgs p{ct1, ct2, out, t.moduli, t.barrett, L, t.log_n, out, 0, 0, poly};
+    dim3 grid((1u << t.log_n) / kThreads, L);
+#define HE_CASE(A, B) \
+    if (s1 == A && s2 == B) hipLaunchKernelGGL((tensor_mxn_kernel<A, B>), grid, dim3(kThreads), 0, s, p); else
+    HE_CASE(1, 1) HE_CASE(1, 2) HE_CASE(1, 3) HE_CASE(2, 1) HE_CASE(2, 2) HE_CASE(2, 3) HE_CASE(3, 1) HE_CASE(3, 2)
+    HE_CASE(3, 3) return hipErrorInvalidValue;
+#undef HE_CASE
     return hipGetLastError();
 }
 

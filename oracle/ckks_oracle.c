@@ -275,6 +275,32 @@ void orc_tensor_square(const orc_params *p, const uint64_t *ct, uint64_t *out, u
     }
 }
 
+/* src/polymath.cu:614-672  tensor_prod_mxn_rns_poly: out_j = sum over a + b = j of ct1_a * ct2_b, the products
+ * summed in 128 bits and reduced once.  ct1 [s1][L][N], ct2 [s2][L][N], out [s1 + s2 - 1][L][N]; out may be ct1's
+ * buffer when that has room (every coefficient is read before it is written, as in the reference). */
+void orc_tensor_mxn(const orc_params *p, const uint64_t *ct1, uint32_t s1, const uint64_t *ct2, uint32_t s2,
+                    uint64_t *out, uint32_t L) {
+    size_t n = (size_t)1 << p->logn, poly = (size_t)L * n;
+    uint32_t res = s1 + s2 - 1;
+#pragma omp parallel for
+    for (uint32_t l = 0; l < L; l++) {
+        uint64_t q = p->mod[l];
+        const uint64_t *r = p->ratio + 2 * (size_t)l;
+        for (size_t i = (size_t)l * n; i < (size_t)(l + 1) * n; i++) {
+            uint64_t c1[8], c2[8], o[16];
+            for (uint32_t a = 0; a < s1; a++) c1[a] = ct1[i + poly * a];
+            for (uint32_t b = 0; b < s2; b++) c2[b] = ct2[i + poly * b];
+            for (uint32_t j = 0; j < res; j++) {
+                uint32_t last1 = j < s1 - 1 ? j : s1 - 1, first2 = j < s2 - 1 ? j : s2 - 1, first1 = j - first2;
+                u128 acc = 0;
+                for (uint32_t k = 0; k + first1 <= last1; k++) acc += (u128)c1[first1 + k] * c2[first2 - k];
+                o[j] = barrett128(acc, q, r);
+            }
+            for (uint32_t j = 0; j < res; j++) out[i + poly * j] = o[j];
+        }
+    }
+}
+
 /* src/galois.cu:20-30  apply_galois_ntt_permutation: out[limb][i] = in[limb][table[i]] */
 void orc_galois_ntt(const orc_params *p, const uint64_t *in, uint64_t *out, const uint32_t *table,
                     uint32_t nlimbs) {

@@ -57,7 +57,7 @@ def lib():
         _lib.orc_mulmod.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64, u64p]
         for name in ("orc_power_table", "orc_shoup_table", "orc_ntt_fwd", "orc_ntt_inv", "orc_ntt_fwd_limbs",
                      "orc_ntt_inv_limbs", "orc_elementwise", "orc_negate", "orc_mul_add", "orc_tensor_2x2",
-                     "orc_tensor_square", "orc_galois_ntt", "orc_galois_table", "orc_rescale", "orc_modup",
+                     "orc_tensor_square", "orc_tensor_mxn", "orc_galois_ntt", "orc_galois_table", "orc_rescale", "orc_modup",
                      "orc_inner_prod", "orc_moddown", "orc_evk_add_ps", "orc_chacha20_block", "orc_sample_ternary",
                      "orc_sample_error", "orc_sample_uniform", "orc_sample_gauss", "orc_decompose_coeffs"):
             getattr(_lib, name).restype = None
@@ -334,6 +334,16 @@ class Params:
         L = ct1.shape[1]
         out = np.empty((3, L, self.n), dtype=np.uint64)
         lib().orc_tensor_2x2(C.byref(self.c), _p64(ct1.reshape(-1)), _p64(ct2.reshape(-1)), _p64(out.reshape(-1)),
+                             C.c_uint32(L))
+        return out
+
+    def tensor_mxn(self, ct1: np.ndarray, ct2: np.ndarray) -> np.ndarray:
+        """(s1,L,N) x (s2,L,N) -> (s1+s2-1,L,N), sizes up to 8 (src/polymath.cu:614-672)."""
+        s1, L = ct1.shape[0], ct1.shape[1]
+        s2 = ct2.shape[0]
+        out = np.empty((s1 + s2 - 1, L, self.n), dtype=np.uint64)
+        lib().orc_tensor_mxn(C.byref(self.c), _p64(np.ascontiguousarray(ct1).reshape(-1)), C.c_uint32(s1),
+                             _p64(np.ascontiguousarray(ct2).reshape(-1)), C.c_uint32(s2), _p64(out.reshape(-1)),
                              C.c_uint32(L))
         return out
 

@@ -474,6 +474,35 @@ def test_tensor_and_square(small, capi):
         assert (dbuf.numpy() == p.tensor(a, b)).all()
 
 
+@pytest.mark.parametrize("s1,s2", [(2, 3), (3, 2), (3, 3), (2, 2), (1, 2)])
+def test_tensor_mxn(small, capi, s1, s2):
+    """he_tensor_mxn against the oracle for every operand size up to 3 x 3, out of place and into the first operand's
+    buffer, with edge residues; sizes beyond 3 are refused."""
+    cahel, parms, ctx, p = small
+    rng = np.random.default_rng(70 + 10 * s1 + s2)
+    L = 5
+    a = rand_limbs(p, rng, range(L), n_polys=s1)
+    b = rand_limbs(p, rng, range(L), n_polys=s2)
+    for i in range(L):
+        a[:, i, 0] = p.moduli[i] - 1
+        b[:, i, 0] = p.moduli[i] - 1
+        b[:, i, 1] = 0
+    want = p.tensor_mxn(a, b)
+    lib, h = capi.lib(), ctx.he_handle()
+    da, db = DeviceArray(capi, host=a), DeviceArray(capi, host=b)
+    dout = DeviceArray(capi, shape=want.shape)
+    capi.check(lib.he_tensor_mxn(h, da.ptr, s1, db.ptr, s2, dout.ptr, L, None))
+    assert (dout.numpy() == want).all()
+    # in place: the first operand sits at the start of a buffer with room for the result
+    big = np.zeros(want.shape, dtype=np.uint64)
+    big[:s1] = a
+    dbig = DeviceArray(capi, host=big)
+    capi.check(lib.he_tensor_mxn(h, dbig.ptr, s1, db.ptr, s2, dbig.ptr, L, None))
+    assert (dbig.numpy() == want).all()
+    assert lib.he_tensor_mxn(h, da.ptr, 4, db.ptr, s2, dout.ptr, L, None) == -2
+    assert lib.he_tensor_mxn(h, da.ptr, 0, db.ptr, s2, dout.ptr, L, None) == -1
+
+
 @pytest.mark.parametrize("step", [1, -1, 7, 0, 1000])
 def test_galois(small, capi, oracle, step):
     cahel, parms, ctx, p = small

@@ -258,6 +258,46 @@ def test_hoisting_bit_exact(world):
         c.hoisting(ctx, ct, w["glk"], [7])
 
 
+def test_multiply_with_size_three_operands(world):
+    """multiply / square of ciphertexts that were not relinearised (size 3): the general tensor product of
+    src/evaluate.cu:474-488, 531-545.  Limbs against the oracle, and the size-5 results decrypt (c0 + c1 s + ... +
+    c4 s^4) to the product of the slots.  As in the reference, operands of different sizes are refused
+    (src/evaluate.cu:369-370)."""
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    rng = np.random.default_rng(21)
+    x, y, z, v = (rng.uniform(-1, 1, p.n // 2) for _ in range(4))
+    scale = 2.0 ** 25
+    _, _, cx, o_cx = _encrypt_both(w, x, scale)
+    _, _, cy, o_cy = _encrypt_both(w, y, scale)
+    _, _, cz, o_cz = _encrypt_both(w, z, scale)
+    _, _, cv, o_cv = _encrypt_both(w, v, scale)
+    xy, zv = c.ciphertext(ctx), c.ciphertext(ctx)
+    c.multiply(ctx, cx, cy, xy)
+    c.multiply(ctx, cz, cv, zv)
+    o_xy, o_zv = p.tensor(o_cx, o_cy), p.tensor(o_cz, o_cv)
+    same_scale = _encrypt_product_only(w, z, scale * scale)
+    with pytest.raises(ValueError, match="poly number mismatch"):
+        c.multiply_inplace(ctx, xy, same_scale)
+    prod = c.ciphertext(ctx)
+    c.multiply(ctx, xy, zv, prod)
+    assert prod.size() == 5 and (prod.to_numpy() == p.tensor_mxn(o_xy, o_zv)).all()
+    assert prod.scale() == scale ** 4
+    w["sk"].set_noise_flooding(False)
+    try:
+        got = np.array(w["enc"].decode(ctx, w["sk"].decrypt(ctx, prod)))
+        assert np.max(np.abs(got - x * y * z * v)) < 1e-3
+        # squaring a size-3 ciphertext in place
+        c.square_inplace(ctx, xy)
+        assert xy.size() == 5 and (xy.to_numpy() == p.tensor_mxn(o_xy, o_xy)).all()
+        got = np.array(w["enc"].decode(ctx, w["sk"].decrypt(ctx, xy)))
+        assert np.max(np.abs(got - (x * y) ** 2)) < 1e-3
+    finally:
+        w["sk"].set_noise_flooding(True)
+    with pytest.raises(ValueError, match="operands of size 2 or 3"):
+        c.square_inplace(ctx, xy)
+
+
 def test_error_behaviour(world):
     w = world
     c, ctx, p = w["cahel"], w["ctx"], w["p"]

@@ -263,6 +263,34 @@ def test_tensor_and_square_bigint(small):
             assert [int(s[k][i][j]) for k in range(3)] == [a0 * a0 % q, 2 * a0 * a1 % q, a1 * a1 % q]
 
 
+@pytest.mark.parametrize("s1,s2", [(2, 2), (2, 3), (3, 2), (3, 3), (1, 3)])
+def test_tensor_mxn_is_the_convolution_of_the_operands(small, s1, s2):
+    """orc_tensor_mxn against Python integers: polynomial j of the product is the sum of ct1_a ct2_b over a + b = j
+    (the ciphertexts multiplied as polynomials in the secret key), coefficient by coefficient and limb by limb, with
+    both operands at q - 1 in one position so that the 128-bit sum is as large as it gets; the 2 x 2 case must equal
+    the dedicated 2 x 2 routine, and squaring a size-2 operand the squaring routine."""
+    p, rng = small, random.Random(60 + 10 * s1 + s2)
+    L = 4
+    a = np.stack([rand_poly(p, rng, range(L)) for _ in range(s1)])
+    b = np.stack([rand_poly(p, rng, range(L)) for _ in range(s2)])
+    for i in range(L):
+        a[:, i, 0] = p.moduli[i] - 1
+        b[:, i, 0] = p.moduli[i] - 1
+        a[:, i, 1] = 0
+    t = p.tensor_mxn(a, b)
+    assert t.shape == (s1 + s2 - 1, L, p.n)
+    for i in range(L):
+        q = p.moduli[i]
+        for j in range(0, p.n, 7):
+            av = [int(a[k][i][j]) for k in range(s1)]
+            bv = [int(b[k][i][j]) for k in range(s2)]
+            want = [sum(av[x] * bv[k - x] for x in range(s1) if 0 <= k - x < s2) % q for k in range(s1 + s2 - 1)]
+            assert [int(t[k][i][j]) for k in range(s1 + s2 - 1)] == want
+    if (s1, s2) == (2, 2):
+        assert (t == p.tensor(a, b)).all()
+        assert (p.tensor_mxn(a, a) == p.square(a)).all()
+
+
 def test_elementwise_bigint(small):
     p, rng = small, random.Random(8)
     a, b, c = (rand_poly(p, rng, range(5)) for _ in range(3))
