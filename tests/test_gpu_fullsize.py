@@ -194,6 +194,8 @@ def test_c5_krum_round_full_shape():
     chosen, dist, timings = krum.gpu_krum(updates, krum.KrumConfig(seed=2025))
     want = krum.plain_distance_matrix(updates)
     off = ~np.eye(10, dtype=bool)
-    assert np.max(np.abs(dist[off] - want[off]) / want[off]) < 1e-4
+    # 2^40 / q_last - 1 = 3.6e-6 from set_scale(2^40) after the rescale by q_last = 1099507695617, plus about 2e-6 of
+    # encryption, key-switch and rotation noise relative to the smallest distances
+    assert np.max(np.abs(dist[off] - want[off]) / want[off]) < 2e-5
     assert chosen == krum.krum_select(want) and chosen not in (8, 9)
     assert timings["total"] > 0

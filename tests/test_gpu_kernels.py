@@ -596,6 +596,34 @@ def test_keyswitch(small, capi, L, elt):
     assert (dc.numpy() == c).all()
 
 
+def test_tensor_and_square_benchmark_shape(full, capi):
+    """he_tensor and he_tensor_square at N = 2^16, L = 24 limbs of 50 bits (the exact-FP64 kernels), edge residues
+    included, against the oracle; out of place and into the first operand's buffer."""
+    cahel, parms, ctx, p = full
+    rng = np.random.default_rng(33)
+    lib, h = capi.lib(), ctx.he_handle()
+    L = 24
+    a = rand_limbs(p, rng, range(L), n_polys=2)
+    b = rand_limbs(p, rng, range(L), n_polys=2)
+    for i in range(L):
+        a[:, i, 0] = p.moduli[i] - 1
+        b[:, i, 0] = p.moduli[i] - 1
+        a[:, i, 1] = 0
+        b[0, i, 2], b[1, i, 2] = 1, p.moduli[i] - 1
+    da, db = DeviceArray(capi, host=a), DeviceArray(capi, host=b)
+    dout = DeviceArray(capi, shape=(3, L, p.n))
+    capi.check(lib.he_tensor(h, da.ptr, db.ptr, dout.ptr, L, None))
+    want = p.tensor(a, b)
+    assert (dout.numpy() == want).all()
+    capi.check(lib.he_tensor_square(h, da.ptr, dout.ptr, L, None))
+    assert (dout.numpy() == p.square(a)).all()
+    big = np.zeros((3, L, p.n), dtype=np.uint64)
+    big[:2] = a
+    dbig = DeviceArray(capi, host=big)
+    capi.check(lib.he_tensor(h, dbig.ptr, db.ptr, dbig.ptr, L, None))
+    assert (dbig.numpy() == want).all()
+
+
 def test_keyswitch_benchmark_shape(full, capi):
     """Key switch at N = 2^16, L = 24, K = 8, beta = 3 against the oracle."""
     cahel, parms, ctx, p = full
