@@ -19,6 +19,8 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libckks_oracle.so")
+# a build of the same source to load instead (the sanitizer build of oracle/Makefile)
+_LIB_OVERRIDE = os.environ.get("CKKS_ORACLE_LIB")
 
 u64p = C.POINTER(C.c_uint64)
 u32p = C.POINTER(C.c_uint32)
@@ -43,8 +45,11 @@ _lib = None
 def lib():
     global _lib
     if _lib is None:
-        build()
-        _lib = C.CDLL(_LIB_PATH)
+        if _LIB_OVERRIDE:
+            _lib = C.CDLL(_LIB_OVERRIDE)
+        else:
+            build()
+            _lib = C.CDLL(_LIB_PATH)
         _lib.orc_shoup_quotient.restype = C.c_uint64
         _lib.orc_shoup_quotient.argtypes = [C.c_uint64, C.c_uint64]
         _lib.orc_mul_shoup.restype = C.c_uint64
