@@ -5,20 +5,34 @@
 
 One "step" is one homomorphic multiplication with relinearisation and rescale (tensor product -> hybrid key
 switch with dnum = 3 digits -> rescale) of two fresh ciphertexts at N = 2^16, L = 24 data limbs and 8 special
-limbs of 50 bits, scale 2^40, on buffers that are resident in HBM before the timed region starts; the step goes
-through the C-ABI of libcahel_hip.so exactly as the pyCAHEL evaluator drives it.  Prints ONE JSON line.
+limbs of 50 bits, scale 2^40 (BASELINE.json configs[2]), on buffers that are resident in HBM before the timed region
+starts.  Every figure is the median of BLOCKS timed blocks of K steps each, after W warm-up steps.  Prints ONE JSON
+line.
+
+How the same step is driven (all give the same limbs, `check`):
+  value / throughput   independent operations: dealt round-robin to `--lanes` streams (`streams`), or `--batch`
+                       of them per call through he_multiply_relin_rescale_batch (`batch`); `value` is the better of
+                       the two and `config.value_path` says which
+  single_stream        one he_multiply_relin_rescale after the other on the null stream (HIP events)
+  api_path             what lancelot-main-GPU's byzantine_fl.py gets: pyCAHEL multiply, relinearize_inplace,
+                       rescale_to_next_inplace on the null stream
 
 Extra objects on the line:
-  roofline      the dominant kernel of the step (forward NTT, blocks pass, as launched by the key switch's
-                ModUp) timed alone with HIP events: algorithmic bytes = limbs * N * 8 read + written
+  roofline      the timed step on one stream against the HBM roofline: algorithmic bytes of the step / its duration
+                (HIP events on the stream the kernels run on), with the VALU bound beside it (`valu`: wave
+                instructions of the step's kernels from the committed counter profile, priced against the FP64
+                issue rate that he_probe_fp64_issue_rate measures in this run)
   ntt           config "batched forward + inverse NTT, 24 limbs x 2 polynomials": GB/s of limb data
-  rotate        one rotation with key switch; hoisted and plain rotate-and-sum over 15 steps
-  cpu_baseline  the CPU checker (oracle/, OpenMP) on the same HMult+relin+rescale workload, bounded sample
+  rotate        one rotation with key switch; rotate-and-sum over 15 steps
+  krum          the encrypted Krum round at its real shape, with the CPU checker's time for the same evaluate phase
+  cpu_baseline  the CPU checker (oracle/, OpenMP) on the same HMult+relin+rescale workload, bounded sample; and at
+                BASELINE.json configs[0] (N = 2^14, 4 + 1 primes)
 """
 import argparse
 import ctypes as C
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -28,10 +42,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 LOG_N, SIZE_Q, SIZE_P, BITS, SCALE = 16, 24, 8, 50, 2.0 ** 40
-# HBM bytes of one 72-limb forward NTT call, from the FETCH_SIZE / WRITE_SIZE counters scaled by a copy of known
-# size (profiles/ntt_forward_72limbs_n65536.md)
-NTT72_TRAFFIC_BYTES = 164_057_088
 HBM_PEAK_GBS = 8000.0
+BLOCKS = 5
+# From profiles/hmult_relin_rescale_n65536_l24_k8.md (rocprofv3 --pmc of `bench.py --only step`), per step on one
+# stream: L2-miss traffic (FETCH_SIZE scaled by 2, WRITE_SIZE by 1: the factors a copy of known size gives) and
+# SQ_INSTS_VALU summed over the step's kernels.  Constants of the profile, not measured in this run.
+STEP_TRAFFIC_BYTES = 1158 * 524288
+STEP_VALU_WAVE_INSTR = 35.9e6
 
 
 def sync(capi):
@@ -39,7 +56,7 @@ def sync(capi):
 
 
 class Timer:
-    """HIP-event timer on the null stream (the stream every kernel here is launched on)."""
+    """HIP-event timer on the null stream (the stream the timed kernels are launched on)."""
 
     def __init__(self, capi):
         self.capi, self.lib = capi, capi.lib()
@@ -47,10 +64,7 @@ class Timer:
         capi.check(self.lib.he_event_create(C.byref(self.e0)))
         capi.check(self.lib.he_event_create(C.byref(self.e1)))
 
-    def time(self, fn, iters, warmup=3):
-        for _ in range(warmup):
-            fn()
-        sync(self.capi)
+    def once(self, fn, iters):
         self.capi.check(self.lib.he_event_record(self.e0, None))
         for _ in range(iters):
             fn()
@@ -59,6 +73,12 @@ class Timer:
         ms = C.c_float()
         self.capi.check(self.lib.he_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
         return ms.value / iters
+
+    def time(self, fn, iters, warmup=3, blocks=BLOCKS):
+        for _ in range(warmup):
+            fn()
+        sync(self.capi)
+        return statistics.median(self.once(fn, iters) for _ in range(blocks))
 
 
 class Buf:
@@ -72,12 +92,12 @@ class Buf:
         return self.ptr + 8 * word
 
 
-def cpu_baseline(seconds_budget=12.0):
-    """HMult + relinearise + rescale on the CPU checker at the benchmark's own shape (random residues)."""
+def cpu_hmult(log_n, size_q, size_p, seconds_budget):
+    """HMult + relinearise + rescale on the CPU checker (random residues): (ops/s, iterations, threads)."""
     from oracle import ckks_oracle as O
-    n = 1 << LOG_N
-    mods = O.coeff_modulus_create(n, [BITS] * (SIZE_Q + SIZE_P))
-    p = O.Params(LOG_N, mods, SIZE_P)
+    n = 1 << log_n
+    mods = O.coeff_modulus_create(n, [BITS] * (size_q + size_p))
+    p = O.Params(log_n, mods, size_p)
     rng = np.random.default_rng(1)
 
     def rnd(limbs, polys):
@@ -86,8 +106,8 @@ def cpu_baseline(seconds_budget=12.0):
             out[:, i] = rng.integers(0, mods[i], size=(polys, n), dtype=np.uint64)
         return out
 
-    a, b = rnd(SIZE_Q, 2), rnd(SIZE_Q, 2)
-    evk = [rnd(SIZE_Q + SIZE_P, 2) for _ in range(SIZE_Q // SIZE_P)]
+    a, b = rnd(size_q, 2), rnd(size_q, 2)
+    evk = [rnd(size_q + size_p, 2) for _ in range(size_q // size_p)]
 
     def op():
         return p.rescale(p.relinearize(p.tensor(a, b), evk))
@@ -97,17 +117,67 @@ def cpu_baseline(seconds_budget=12.0):
     while True:
         op()
         iters += 1
-        if time.time() - t0 > seconds_budget or iters >= 2000:
+        if time.time() - t0 > seconds_budget or iters >= 5000:
             break
     dt = (time.time() - t0) / iters
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    return {"value": 1.0 / dt, "unit": "HMult+relin+rescale ops/s", "cores": threads, "kind": "port",
+    return 1.0 / dt, iters, threads
+
+
+def cpu_baseline():
+    v, iters, threads = cpu_hmult(LOG_N, SIZE_Q, SIZE_P, 10.0)
+    v1, iters1, _ = cpu_hmult(14, 4, 1, 4.0)
+    return {"value": v, "unit": "HMult+relin+rescale ops/s", "cores": threads, "kind": "port",
             "sample": "%d iterations of the same workload (N=2^16, L=24, K=8, dnum=3, random residues) on "
                       "oracle/ckks_oracle.c with OpenMP" % iters,
-            "ms_per_op": dt * 1e3}
+            "ms_per_op": 1e3 / v,
+            "config_c1": {"value": v1, "unit": "HMult+relin+rescale ops/s", "cores": threads,
+                          "workload": "BASELINE.json configs[0]: N=2^14, 4 limbs of 50 bits + 1 special prime",
+                          "sample": "%d iterations" % iters1, "ms_per_op": 1e3 / v1}}
 
 
-def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60), sum_drop_levels=0):
+def krum_cpu_evaluate(updates, pairs_sampled=2):
+    """The evaluate phase of the Krum round on the CPU checker: per pair sub, square and add over the chunks,
+    relinearise, rescale, and the slot sum as 15 rotations (each a key switch) + additions, with Lancelot's
+    parameters; `pairs_sampled` pairs are timed and the figure is scaled to the 45 pairs of the round."""
+    from oracle import ckks_oracle as O
+    log_n, n = 16, 1 << 16
+    mods = O.coeff_modulus_create(n, [60, 40, 40, 60])
+    p = O.Params(log_n, mods, 1)
+    ks = O.KeySet(p, seed=2025)
+    ks.gen_secret()
+    rlk = ks.gen_relin()
+    elts = [O.galois_elt_from_step(1 << k, n) for k in range(15)]
+    glk = [ks.gen_galois(e) for e in elts]
+    rng = np.random.default_rng(3)
+    L = p.size_q
+
+    def rnd_ct():
+        out = np.empty((2, L, n), dtype=np.uint64)
+        for i in range(L):
+            out[:, i] = rng.integers(0, mods[i], size=(2, n), dtype=np.uint64)
+        return out
+
+    chunks = 2
+    cts = [[rnd_ct() for _ in range(chunks)] for _ in range(2)]
+    t0 = time.time()
+    for _ in range(pairs_sampled):
+        acc = None
+        for c in range(chunks):
+            d = np.stack([p.sub(cts[1][c][k], cts[0][c][k]) for k in range(2)])
+            sq = p.square(d)
+            acc = sq if acc is None else np.stack([p.add(acc[k], sq[k]) for k in range(3)])
+        r = p.rescale(p.relinearize(acc, rlk))
+        for e, key in zip(elts, glk):
+            rot = p.apply_galois(r, e, key)
+            r = np.stack([p.add(r[k], rot[k]) for k in range(2)])
+    per_pair = (time.time() - t0) / pairs_sampled
+    return {"evaluate_s": per_pair * 45, "sample": "%d of the 45 pairs timed (%.3f s each) on oracle/ckks_oracle.c, "
+            "%d threads; rotations one key switch each (the checker has no hoisting)"
+            % (pairs_sampled, per_pair, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))}
+
+
+def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60), sum_drop_levels=0, with_cpu=False):
     """One encrypted Krum round at its real shape (10 clients x 62,006 parameters, N = 2^16, moduli
     [60, 40, 40, 60], one special prime): seconds per phase and the error against the float64 closed form."""
     from lancelot_amd import krum
@@ -119,20 +189,24 @@ def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60), sum_drop_levels=
     state = krum.gpu_init(krum.KrumConfig(seed=seed, modulus_bits=tuple(modulus_bits), sum_drop_levels=sum_drop_levels))
     setup = time.perf_counter() - t0
     krum.gpu_krum_aggregate(updates, state=state)  # warm-up round (pool growth, first-touch of the keys)
-    # the fastest of three rounds each (a round is about 12 ms of host-driven work: one scheduling hiccup of the host
+    # the fastest of three rounds each (a round is a few ms of host-driven work: one scheduling hiccup of the host
     # threads would otherwise decide the figure)
     chosen_full, weights, full_timings = min((krum.gpu_krum_aggregate(updates, state=state) for _ in range(3)),
                                              key=lambda r: r[2]["total"])
     chosen, dist, timings = min((krum.gpu_krum(updates, state=state) for _ in range(3)), key=lambda r: r[2]["total"])
     plain = krum.plain_distance_matrix(updates)
     off = ~np.eye(10, dtype=bool)
-    return {"workload": "Krum distance round, 10 clients x 62006 parameters, 2 ciphertexts per client, 45 pairs, N=2^16, "
-                        "moduli of %s bits (the last one special); encode and encrypt are one batched pipeline, timed "
-                        "under 'encode'" % (list(modulus_bits),),
-            "setup_s": setup, "round_s": timings, "chosen": chosen, "chosen_plain": krum.krum_select(plain),
-            "full_round_s": full_timings, "full_round_chosen": chosen_full,
-            "aggregate_max_abs_err": float(np.max(np.abs(weights - updates[chosen_full].astype(np.float64)))),
-            "max_rel_err_vs_float64": float(np.max(np.abs(dist[off] - plain[off]) / plain[off]))}
+    out = {"workload": "Krum distance round, 10 clients x 62006 parameters, 2 ciphertexts per client, 45 pairs, N=2^16, "
+                       "moduli of %s bits (the last one special); encode and encrypt are one batched pipeline, timed "
+                       "under 'encode'" % (list(modulus_bits),),
+           "setup_s": setup, "round_s": timings, "chosen": chosen, "chosen_plain": krum.krum_select(plain),
+           "full_round_s": full_timings, "full_round_chosen": chosen_full,
+           "aggregate_max_abs_err": float(np.max(np.abs(weights - updates[chosen_full].astype(np.float64)))),
+           "max_rel_err_vs_float64": float(np.max(np.abs(dist[off] - plain[off]) / plain[off]))}
+    if with_cpu:
+        out["cpu_baseline"] = krum_cpu_evaluate(updates)
+        out["cpu_baseline"]["gpu_evaluate_s"] = timings["evaluate"]
+    return out
 
 
 def main():
@@ -143,12 +217,11 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--lanes", type=int, default=3,
                     help="streams that the timed operations are dealt to (three and the null stream fill the four "
-                         "hardware queues of a process; four measured slower than three or six)")
-    ap.add_argument("--separate-rescale", action="store_true",
-                    help="he_keyswitch then he_rescale instead of the merged he_keyswitch_rescale")
+                         "hardware queues of a process)")
+    ap.add_argument("--batch", type=int, default=8, help="operations per he_multiply_relin_rescale_batch call")
     ap.add_argument("--no-krum", action="store_true", help="skip the encrypted Krum round (BASELINE.json configs[4])")
-    ap.add_argument("--only", choices=["all", "roofline", "krum"], default="all",
-                    help="roofline: run just the kernel the roofline object describes (for rocprofv3)")
+    ap.add_argument("--only", choices=["all", "step", "rotate", "ntt", "krum"], default="all",
+                    help="step / rotate / ntt: run just that workload on the null stream (for rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -158,31 +231,18 @@ def main():
     from lancelot_amd import capi
     lib = capi.lib()
 
+    if args.only == "krum":
+        print(json.dumps(krum_round()))
+        return
     n = 1 << LOG_N
     parms = cahel.params(cahel.scheme_type.ckks)
     parms.set_poly_modulus_degree(n)
     parms.set_coeff_modulus(cahel.coeff_modulus_create(n, [BITS] * (SIZE_Q + SIZE_P)))
     parms.set_special_modulus_size(SIZE_P)
     steps_pow2 = [1 << k for k in range(15)]
-    parms.set_galois_elts(cahel.get_elts_from_steps(steps_pow2, n))
+    parms.set_galois_elts(cahel.get_elts_from_steps(steps_pow2 if args.only in ("all", "rotate") else [1], n))
     ctx = cahel.context(parms, True, cahel.sec_level_type.tc128)
     ctx.set_seed(2025)
-    if args.only == "krum":
-        print(json.dumps(krum_round()))
-        return
-    if args.only == "roofline":
-        # just the kernels the roofline object describes, plus one device-to-device copy of known size that
-        # calibrates the FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run
-        h = ctx.he_handle()
-        words = 3 * (SIZE_Q + SIZE_P) * n
-        big, ref = Buf(capi, words), Buf(capi, words)
-        capi.check(lib.he_memset_zero(big.ptr, 8 * words, None))
-        capi.check(lib.he_memcpy_d2d(ref.ptr, big.ptr, 8 * words, None))
-        ms = Timer(capi).time(lambda: capi.check(lib.he_ntt_forward(h, big.ptr, 3, SIZE_Q + SIZE_P, SIZE_Q, 0, SIZE_Q, 0,
-                                                                    None)), args.steps, args.warmup)
-        print(json.dumps({"kernel": "forward NTT, 72 limbs (ntt_rows_kernel + ntt_blocks_kernel)", "ms_per_launch": ms,
-                          "GBps": 72 * 8 * n * 2 / (ms * 1e-3) / 1e9, "calibration_copy_bytes": 8 * words}))
-        return
     sk = cahel.secret_key(parms)
     sk.gen_secretkey(ctx)
     pk = cahel.public_key(ctx)
@@ -199,101 +259,121 @@ def main():
 
     h = ctx.he_handle()
     L, K = SIZE_Q, SIZE_P
-    LK = L + K
     limb_bytes = 8 * n
     evk = capi.evk_array([rlk.digit_ptr(d) for d in range(rlk.digit_count())])
-    ws = Buf(capi, lib.he_keyswitch_workspace_words(h, L))
-    t3 = Buf(capi, 3 * L * n)
-    res = Buf(capi, 2 * (L - 1) * n)
-    rs_ws = Buf(capi, 2 * n)
+    ws_words = lib.he_multiply_relin_rescale_workspace_words(h, L)
+    ws, res = Buf(capi, ws_words), Buf(capi, 2 * (L - 1) * n)
     a_ptr, b_ptr = ct1.data_ptr(), ct2.data_ptr()
-
-    # relinearise + rescale: one C-ABI call (ModDown's and the rescale's forward transforms merged, same limbs), or,
-    # with --separate-rescale, the two calls that the evaluator's relinearize_inplace / rescale_to_next_inplace make
-    def relin_rescale(t3_, res_, ws_, rs_, st):
-        if args.separate_rescale:
-            capi.check(lib.he_keyswitch(h, L, t3_.at(2 * L * n), evk, t3_.ptr, 0, ws_.ptr, st))
-            capi.check(lib.he_rescale(h, t3_.ptr, res_.ptr, 2, L, rs_.ptr, st))
-        else:
-            capi.check(lib.he_keyswitch_rescale(h, L, t3_.at(2 * L * n), evk, t3_.ptr, res_.ptr, 0, ws_.ptr, st))
+    timer = Timer(capi)
+    K_steps, W = args.steps, args.warmup
 
     def step():
-        capi.check(lib.he_tensor(h, a_ptr, b_ptr, t3.ptr, L, None))
-        relin_rescale(t3, res, ws, rs_ws, None)
+        capi.check(lib.he_multiply_relin_rescale(h, L, a_ptr, b_ptr, evk, res.ptr, ws.ptr, None))
 
-    # (1) one operation after the other on the null stream: the latency of a single HMult + relin + rescale
-    for _ in range(args.warmup):
-        step()
-    sync(capi)
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    sync(capi)
-    single_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    rot_in, rot_out = ct1.copy(), cahel.ciphertext(ctx)
 
-    # (2) the same K independent operations dealt round-robin to `lanes` streams, each with its own workspace and
-    # output: kernels of different operations overlap (one loads while another computes), which a single
-    # operation's kernels, all in the same phase at the same time, cannot do.  This is the throughput figure.
+    def one_rot():
+        cahel.rotate_vector(ctx, rot_in, 1, glk, rot_out)
+
+    two = Buf(capi, 2 * L * n)
+    capi.check(lib.he_memcpy_d2d(two.ptr, a_ptr, 8 * 2 * L * n, None))
+
+    if args.only in ("step", "rotate", "ntt"):
+        fn = {"step": step, "rotate": one_rot,
+              "ntt": lambda: (capi.check(lib.he_ntt_forward(h, two.ptr, 2, L, L, 0, L, 0, None)),
+                              capi.check(lib.he_ntt_inverse(h, two.ptr, 2, L, L, 0, L, 0, None)))}[args.only]
+        # one device-to-device copy of known size calibrates FETCH_SIZE / WRITE_SIZE of a rocprofv3 --pmc run
+        capi.check(lib.he_memcpy_d2d(ws.ptr, ws.at(48 * n), 8 * 48 * n, None))
+        ms = timer.time(fn, K_steps, W, blocks=1)
+        print(json.dumps({"only": args.only, "ms_per_step": ms, "steps": K_steps, "calibration_copy_bytes": 8 * 48 * n}))
+        return
+
+    # (1) one operation after the other on the null stream
+    single_ms = timer.time(step, K_steps, W)
+
+    # (2) the same independent operations dealt round-robin to `lanes` streams, each with its own workspace and output
     lane_bufs, lane_streams = [], []
     for _ in range(args.lanes):
         st = C.c_void_p()
         capi.check(lib.he_stream_create(C.byref(st)))
         lane_streams.append(st)
-        lane_bufs.append((Buf(capi, lib.he_keyswitch_workspace_words(h, L)), Buf(capi, 3 * L * n),
-                          Buf(capi, 2 * (L - 1) * n), Buf(capi, 2 * n)))
+        lane_bufs.append((Buf(capi, ws_words), Buf(capi, 2 * (L - 1) * n)))
 
     def lane_step(k):
-        lws, lt3, lres, lrs = lane_bufs[k]
-        st = lane_streams[k]
-        capi.check(lib.he_tensor(h, a_ptr, b_ptr, lt3.ptr, L, st))
-        relin_rescale(lt3, lres, lws, lrs, st)
+        lws, lres = lane_bufs[k]
+        capi.check(lib.he_multiply_relin_rescale(h, L, a_ptr, b_ptr, evk, lres.ptr, lws.ptr, lane_streams[k]))
 
     def lanes_sync():
         for st in lane_streams:
             capi.check(lib.he_stream_synchronize(st))
 
-    for i in range(args.warmup):
-        lane_step(i % args.lanes)
-    lanes_sync()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        lane_step(i % args.lanes)
-    lanes_sync()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    def timed_wall(issue, count):
+        blocks = []
+        for _ in range(BLOCKS):
+            sync(capi)
+            lanes_sync()
+            t0 = time.perf_counter()
+            for i in range(count):
+                issue(i)
+            lanes_sync()
+            sync(capi)
+            blocks.append((time.perf_counter() - t0) * 1e3 / count)
+        return statistics.median(blocks), blocks
 
-    # the evaluator path must give the same limbs, and decrypt to x * y
+    for i in range(W):
+        lane_step(i % args.lanes)
+    streams_ms, streams_blocks = timed_wall(lambda i: lane_step(i % args.lanes), K_steps)
+
+    # (3) `batch` operations per call, one launch per stage for all of them
+    B = args.batch
+    ba, bb = Buf(capi, B * 2 * L * n), Buf(capi, B * 2 * L * n)
+    for k in range(B):
+        capi.check(lib.he_memcpy_d2d(ba.at(k * 2 * L * n), a_ptr, 8 * 2 * L * n, None))
+        capi.check(lib.he_memcpy_d2d(bb.at(k * 2 * L * n), b_ptr, 8 * 2 * L * n, None))
+    bres = Buf(capi, B * 2 * (L - 1) * n)
+    bws = Buf(capi, lib.he_multiply_relin_rescale_batch_workspace_words(h, L, B))
+
+    def batch_call():
+        capi.check(lib.he_multiply_relin_rescale_batch(h, L, B, ba.ptr, bb.ptr, evk, bres.ptr, bws.ptr, None))
+
+    calls = max(1, -(-K_steps // B))
+    batch_ms = timer.time(batch_call, calls, max(1, W // B)) / B
+
+    # (4) the reference's own call sequence through pyCAHEL on the null stream
     prod = cahel.ciphertext(ctx)
-    cahel.multiply(ctx, ct1, ct2, prod)
-    cahel.relinearize_inplace(ctx, prod, rlk)
-    cahel.rescale_to_next_inplace(ctx, prod)
+
+    def api_step():
+        cahel.multiply(ctx, ct1, ct2, prod)
+        cahel.relinearize_inplace(ctx, prod, rlk)
+        cahel.rescale_to_next_inplace(ctx, prod)
+
+    api_ms = timer.time(api_step, K_steps, W)
+
+    # every path gives the evaluator's limbs, and they decrypt to x * y
+    api_step()
+    want = prod.to_numpy()
     got = np.empty((2, L - 1, n), dtype=np.uint64)
-    capi.check(lib.he_memcpy_d2h(got.ctypes.data, res.ptr, got.nbytes, None))
-    same = bool((got == prod.to_numpy()).all())
-    for lws, lt3, lres, lrs in lane_bufs:
-        capi.check(lib.he_memcpy_d2h(got.ctypes.data, lres.ptr, got.nbytes, None))
-        same = same and bool((got == prod.to_numpy()).all())
+    same = True
+    for buf in [res] + [lres for _, lres in lane_bufs] + [type("B", (), {"ptr": bres.at(k * 2 * (L - 1) * n)}) for k in (0, B - 1)]:
+        capi.check(lib.he_memcpy_d2h(got.ctypes.data, buf.ptr, got.nbytes, None))
+        same = same and bool((got == want).all())
+    fused = cahel.ciphertext(ctx)
+    cahel.multiply_relin_rescale(ctx, ct1, ct2, rlk, fused)
+    same = same and bool((fused.to_numpy() == want).all())
     dec = np.array(enc.decode(ctx, sk.decrypt(ctx, prod)))
     max_err = float(np.max(np.abs(dec - x * y)))
 
-    timer = Timer(capi)
-    # dominant kernel: the forward NTT over the 72 converted limbs of ModUp (beta = 3 digits x 24 limbs); the same
-    # two kernels also run in ModDown and rescale.  Timed alone on a 72-limb buffer.
-    big = Buf(capi, 3 * LK * n)
-    capi.check(lib.he_memset_zero(big.ptr, 8 * 3 * LK * n, None))
-    fwd72 = timer.time(lambda: capi.check(lib.he_ntt_forward(h, big.ptr, 3, LK, L, 0, L, 0, None)), 50)
-    ntt_bytes = 72 * limb_bytes * 2          # each limb read once and written once
-    roof_gbs = ntt_bytes / (fwd72 * 1e-3) / 1e9
+    # measured FP64 issue rate of this GPU (8 waves per SIMD of independent multiply-add chains)
+    rate = C.c_double()
+    capi.check(lib.he_probe_fp64_issue_rate(2048, 2000, C.byref(rate), None))
+    valu_floor_ms = STEP_VALU_WAVE_INSTR * 64 / rate.value * 1e3
 
     # config "NTT alone": 24 limbs x 2 polynomials, forward + inverse
-    two = Buf(capi, 2 * L * n)
-    capi.check(lib.he_memcpy_d2d(two.ptr, a_ptr, 8 * 2 * L * n, None))
     f = timer.time(lambda: capi.check(lib.he_ntt_forward(h, two.ptr, 2, L, L, 0, L, 0, None)), 100)
     i = timer.time(lambda: capi.check(lib.he_ntt_inverse(h, two.ptr, 2, L, L, 0, L, 0, None)), 100)
     ntt = {"forward_ms": f, "inverse_ms": i, "bytes_fwd_plus_inv": 4 * 2 * L * limb_bytes,
            "GBps": 4 * 2 * L * limb_bytes / ((f + i) * 1e-3) / 1e9}
     ntt["frac_of_hbm_peak"] = ntt["GBps"] / HBM_PEAK_GBS
-    # the same kernels over 6 ciphertexts in one call (288 limbs): a launch that spans several rounds of resident
-    # workgroups overlaps the load, butterfly and store phases that a single round runs one after the other
     six = Buf(capi, 12 * L * n)
     capi.check(lib.he_memset_zero(six.ptr, 8 * 12 * L * n, None))
     f6 = timer.time(lambda: capi.check(lib.he_ntt_forward(h, six.ptr, 12, L, L, 0, L, 0, None)), 30)
@@ -302,14 +382,8 @@ def main():
                                        "GBps": 4 * 12 * L * limb_bytes / ((f6 + i6) * 1e-3) / 1e9}
     ntt["six_ciphertexts_per_call"]["frac_of_hbm_peak"] = ntt["six_ciphertexts_per_call"]["GBps"] / HBM_PEAK_GBS
 
-    # rotations (config "rotate-and-sum"): one keyed rotation; 15 dependent rotations + adds; hoisted form
-    rot_in = ct1.copy()
-    rot_out = cahel.ciphertext(ctx)
-
-    def one_rot():
-        cahel.rotate_vector(ctx, rot_in, 1, glk, rot_out)
-
-    rot_ms = timer.time(one_rot, 20)
+    # rotations (config "rotate-and-sum"): one keyed rotation; 15 dependent rotations + adds
+    rot_ms = timer.time(one_rot, 50)
 
     def rotate_and_sum():
         acc = ct1.copy()
@@ -323,33 +397,58 @@ def main():
     total = np.array(enc.decode(ctx, sk.decrypt(ctx, rotate_and_sum())))
     rotate = {"one_rotation_ms": rot_ms, "rotate_and_sum_15_ms": ras_ms,
               "one_rotation_GBps": 288 * limb_bytes / (rot_ms * 1e-3) / 1e9,
+              "one_rotation_frac_of_hbm_roofline": 288 * limb_bytes / (rot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
               "rotate_and_sum_GBps": 15 * 432 * limb_bytes / (ras_ms * 1e-3) / 1e9,
               "slot_sum_rel_err": float(np.max(np.abs(total - x.sum())) / abs(x.sum()))}
 
     alg_bytes = 334 * limb_bytes
+
+    def frac(ms):
+        return alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
+
+    best_ms, path = min((streams_ms, "streams"), (batch_ms, "batch"))
     line = {
         "metric": "HMult+relin+rescale ops/s at N=2^16, L=24 (dnum=3, 8 special primes)",
-        "value": 1e3 / ms_per_step, "unit": "ops/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": 1e3 / best_ms, "unit": "ops/s", "n_gpus": 1, "steps": K_steps, "warmup": W,
+        "ms_per_step": best_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "u64", "data": "synthetic",
-        "arithmetic": "64-bit residues; NTT and base conversion in exact FP64 (primes below 2^50), tensor and inner "
-                      "product in 64-bit integers; every output bit-identical to the integer oracle",
+        "arithmetic": "64-bit residues; every stage in exact FP64 (primes below 2^50) with canonical 64-bit results; "
+                      "every output bit-identical to the integer oracle",
+        "timing": "median of %d blocks of %d steps each" % (BLOCKS, K_steps),
         "config": {"workload": "HMult+relinearize+rescale, N=2^16, L=24 limbs of 50 bits, K=8, dnum=3, scale 2^40, "
                                "two fresh ciphertexts of 32768 uniform[-1,1] slots (BASELINE.json configs[2]); "
-                               "independent operations issued round-robin on %d streams" % args.lanes,
-                   "lanes": args.lanes},
-        "single_stream": {"ms_per_step": single_ms, "ops_per_s": 1e3 / single_ms,
-                          "frac_of_hbm_roofline": alg_bytes / (single_ms * 1e-3) / 1e9 / HBM_PEAK_GBS},
-        "hmult_frac_of_hbm_roofline": alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                               "independent operations, the better of %d streams and batches of %d per call"
+                               % (args.lanes, B),
+                   "value_path": path, "lanes": args.lanes, "batch": B},
+        "hmult_frac_of_hbm_roofline": frac(best_ms),
         "hmult_algorithmic_bytes": alg_bytes,
-        "check": {"c_abi_equals_evaluator": same, "decrypt_max_abs_err_vs_xy": max_err},
-        "roofline": {"bound": "hbm", "kernel": "ntt_rows_kernel + ntt_blocks_kernel (forward NTT, 72 limbs of ModUp)",
-                     "achieved": roof_gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": roof_gbs / HBM_PEAK_GBS,
-                     "traffic": NTT72_TRAFFIC_BYTES, "ms_per_launch": fwd72, "algorithmic_bytes_per_launch": ntt_bytes},
+        "streams": {"ms_per_step": streams_ms, "ops_per_s": 1e3 / streams_ms, "frac_of_hbm_roofline": frac(streams_ms),
+                    "blocks_ms": streams_blocks},
+        "batch": {"ms_per_step": batch_ms, "ops_per_s": 1e3 / batch_ms, "frac_of_hbm_roofline": frac(batch_ms),
+                  "ops_per_call": B},
+        "single_stream": {"ms_per_step": single_ms, "ops_per_s": 1e3 / single_ms, "frac_of_hbm_roofline": frac(single_ms)},
+        "api_path": {"calls": "pyCAHEL multiply, relinearize_inplace, rescale_to_next_inplace on the null stream",
+                     "ms_per_step": api_ms, "ops_per_s": 1e3 / api_ms, "frac_of_hbm_roofline": frac(api_ms)},
+        "check": {"all_paths_equal_the_evaluator": same, "decrypt_max_abs_err_vs_xy": max_err},
+        "roofline": {"bound": "hbm",
+                     "kernel": "the timed step on one stream: tensor_intt_blocks_fp, ntt_rows (inverse), bconv_rows_fp, "
+                               "ntt_blocks_fp_inner, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp with "
+                               "the rescale epilogue",
+                     "achieved": alg_bytes / (single_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": frac(single_ms), "ms_per_launch": single_ms, "algorithmic_bytes_per_launch": alg_bytes,
+                     "traffic": STEP_TRAFFIC_BYTES,
+                     "traffic_source": "profiles/hmult_relin_rescale_n65536_l24_k8.md (counter profile, not this run)",
+                     "frac_of_dataflow_floor": (920 * limb_bytes / 6.0e12 * 1e3) / single_ms,
+                     "dataflow_floor": "920 limbs of traffic (two-pass transforms, every fusion of neighbouring "
+                                       "pointwise stages) at the 6 TB/s a streaming kernel reaches on this GPU",
+                     "valu": {"wave_instructions_per_step": STEP_VALU_WAVE_INSTR,
+                              "source": "SQ_INSTS_VALU summed over the step's kernels, same profile",
+                              "fp64_issue_peak_lane_ops_per_s": rate.value, "issue_bound_ms": valu_floor_ms,
+                              "frac_of_issue_bound": valu_floor_ms / single_ms}},
         "ntt": ntt, "rotate": rotate,
     }
     if not args.no_krum:
-        line["krum"] = krum_round()
+        line["krum"] = krum_round(with_cpu=not args.no_cpu_baseline)
         # The same round with two settings that Lancelot's driver does not use (its own are the ones above): primes
         # below 2^50 (exact FP64 butterflies instead of 64-bit integer ones), and the slot sum one level further down
         # (mod_switch_to_next after the rescale: its key switches run over one limb instead of two).  The two do not

@@ -68,6 +68,12 @@ int he_event_synchronize(he_event event);
 int he_stream_wait_event(he_stream stream, he_event event);
 int he_event_elapsed_ms(he_event start, he_event stop, float *ms);
 
+/* Measures the issue rate of full-rate FP64 vector instructions on this GPU (lane-operations per second, 8
+ * independent fused multiply-add chains per lane over `blocks` workgroups of 256 lanes, `iters` x 64 operations per
+ * lane): the peak that the VALU roofline of the FP64 back end is priced against.  Measurement support; allocates a
+ * 64-byte buffer and two events for the duration of the call.  No counterpart in the reference. */
+int he_probe_fp64_issue_rate(uint32_t blocks, uint32_t iters, double *lane_ops_per_second, he_stream stream);
+
 /* ---- parameter tables ---- */
 
 /* Host-side description of one parameter set; replaces the uploads of CAHELGPUContext's constructor
