@@ -93,6 +93,7 @@ struct he_context {
     double *d_phat_pinv_fp = nullptr;    // the same matrix times P^-1 mod q_j (merged ModDown + rescale, fused kernel)
     bool fuse_rows = true;       // environment CAHEL_HIP_NO_FUSED_BCONV=1: conversion kernel, then the rows pass
     bool fuse_tensor = true;     // environment CAHEL_HIP_NO_FUSED_TENSOR=1: he_multiply_relin_rescale as tensor kernel + key switch
+    bool fp_inner = true;        // environment CAHEL_HIP_NO_FP_INNER=1: a batch's inner product on the integer kernel
     uint32_t *d_rot_group = nullptr;     // encoder: 5^j mod 2N
     double2 *d_ksi = nullptr;            // encoder: e^{2 pi i k / 2N}, k <= 2N
     uint64_t *d_garner_inv = nullptr;    // decoder: [size_q][size_q], q_j^-1 mod q_i for j < i
@@ -405,6 +406,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->fuse_rows = !(nb && nb[0] == '1');
         const char *nt = getenv("CAHEL_HIP_NO_FUSED_TENSOR");
         ctx->fuse_tensor = !(nt && nt[0] == '1');
+        const char *ni = getenv("CAHEL_HIP_NO_FP_INNER");
+        ctx->fp_inner = !(ni && ni[0] == '1');
         ctx->fp_ok.assign(qp, 0);
         std::vector<double> psi_fp(qp * n, 0.0), ipsi_fp(qp * n, 0.0), consts(4 * qp, 0.0);
         for (size_t t = 0; t < qp; t++) {
@@ -747,7 +750,7 @@ namespace {
 // ModUp of `items` polynomials: item k reads c + k * c_item_stride * N (stride in limbs), writes out [k][beta][L+K][N];
 // ws holds items * L limbs
 int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_item_stride, uint32_t items,
-               uint64_t *out, uint64_t *ws, he_stream s) {
+               uint64_t *out, uint64_t *ws, he_stream s, bool skip_own = false) {
     if (!ctx || !c || !out || !ws || ctx->size_p == 0 || items == 0 || c_item_stride < L) return HE_E_INVALID_ARGUMENT;
     const Level *lv = level_of(ctx, L);
     if (!lv) return HE_E_LEVEL_NOT_SET;
@@ -765,14 +768,17 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     inv.w = lv->d_part_hat_inv;
     HE_HIP(launch_ntt_inverse(inv, items, backend_for(ctx, inv.map), S(s)));
     const bool fused = fuse_rows_ok(ctx, lv, L);
+    // skip_own (batched levels only): the consumer reads a digit's own limbs from c, their slots in out stay unwritten
+    if (skip_own && !lv->batched) return HE_E_INVALID_ARGUMENT;
+    const uint32_t copy_rows = skip_own ? 0 : lv->modup_max_copy;
     if (fused) {
         BconvRows b{ws, out, c, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                    lv->beta, lv->modup_max_rows, lv->modup_max_copy,
+                    lv->beta, lv->modup_max_rows, copy_rows,
                     items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n, 0};
         HE_HIP(launch_bconv_rows(base_args(ctx, true), b, S(s)));
     } else if (lv->batched) {
         BconvBatch b{ws, out, c, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                     lv->beta, lv->modup_max_rows, lv->modup_max_copy, lv->d_mats_fp, ctx->d_fp_consts,
+                     lv->beta, lv->modup_max_rows, copy_rows, lv->d_mats_fp, ctx->d_fp_consts,
                      items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n};
         HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
     }
@@ -993,13 +999,23 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         x.fold_w = fold_w;
         HE_HIP(launch_ntt_forward_inner(fwd, x, S(s), rows_done));
     } else {
+        // a batch on the FP64 back end shares each key word among the items of a group and reads a digit's own limbs
+        // where they are
+        const bool fp_batch = items > 1 && ctx->fp_inner && lv->batched && fp_for_level(ctx, L) && n >= 512 &&
+                              !galois_elt && !add_c0;
         if (tin) return HE_E_INVALID_ARGUMENT;
-        if (int rc = modup_impl(ctx, L, src, galois_elt ? L : c_item_stride, items, y, tmp, s)) return rc;
+        if (int rc = modup_impl(ctx, L, src, galois_elt ? L : c_item_stride, items, y, tmp, s, fp_batch)) return rc;
         EvkPtrs ptrs;
         memset(&ptrs, 0, sizeof(ptrs));
         for (uint32_t d = 0; d < lv->beta; d++) {
             if (!evk[d]) return HE_E_INVALID_ARGUMENT;
             ptrs.p[d] = evk[d];
+        }
+        if (fp_batch) {
+            HE_HIP(launch_inner_product_fp(ctx->tables(), ctx->d_fp_consts, y, src, (size_t)c_item_stride * n, ptrs, cx, L,
+                                           ctx->size_p, ctx->size_q, lv->beta, fold_ct, fold_w, items, 2 * (size_t)L * n,
+                                           S(s)));
+            return HE_OK;
         }
         HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, cx, L, ctx->size_p, ctx->size_q, lv->beta, 0, false,
                                     fold_ct, fold_w, items, 2 * (size_t)L * n, S(s), add_c0, galois_elt, ctx->d_p_mod_q));
@@ -1201,6 +1217,8 @@ int he_multiply_relin_rescale_batch(const he_context *ctx, uint32_t L, uint32_t 
     const size_t n = ctx->n();
     // [items] key-switch workspaces | (d0, d1) [items][2][L][N] | d2 [items][L][N]
     uint64_t *d01 = ws + (size_t)items * he_keyswitch_workspace_words(ctx, L), *d2 = d01 + (size_t)items * 2 * L * n;
+    // (a tensor product formed inside the key switch's first pass, as the single call does it, measures slower here:
+    // with many items in one launch the plain tensor kernel streams at a higher rate than the fused one computes)
     HE_HIP(launch_tensor(ctx->tables(), ct1, ct2, d01, L, ct1 == ct2, S(s),
                          fp_for(ctx, plain_map(L)) ? ctx->d_fp_consts : nullptr, items, d2));
     return ksr_impl(ctx, L, items, d2, L, evk, d01, out, 0, ws, s, nullptr);

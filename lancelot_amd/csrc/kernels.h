@@ -227,6 +227,14 @@ hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtr
                                 hipStream_t s, const uint64_t *add_c0 = nullptr, uint32_t add_elt = 0,
                                 const uint64_t *p_mod_q = nullptr);
 
+// The same product for a batch on the FP64 back end (every prime below 2^50, N >= 512): key words are loaded once
+// per group of up to 8 items, and a digit's own limbs come from own (the key switch's input in NTT form, items
+// own_item_stride words apart) instead of a copy inside y, whose own-limb slots are not read.
+hipError_t launch_inner_product_fp(const Tables &t, const double *fp_consts, const uint64_t *y, const uint64_t *own,
+                                   size_t own_item_stride, const EvkPtrs &evk, uint64_t *out, uint32_t L, uint32_t K,
+                                   uint32_t size_q, uint32_t beta, const uint64_t *fold_ct, const uint64_t *fold_w,
+                                   uint32_t items, size_t fold_item_stride, hipStream_t s);
+
 // Hoisted rotations: out (2, L+K, N) (+)= sum over steps of the inner product of sigma_s(y) with the step's key, and
 // c0_out (L, N) (+)= sum_s sigma_s(c0).  with_self: c0_out also receives c0 itself and the L limbs after it a copy
 // of the L limbs after c0 (c1), so that ModDown can add onto the input ciphertext.  items: that many inputs,

@@ -1088,7 +1088,7 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
 // and d2 goes on through the 8 inverse stages inside 256 consecutive words; the lazy words are left in a.out for the
 // rows pass.  One read of d2 and one launch less than tensor kernel + inverse transform.
 template <bool SQUARE>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void tensor_intt_blocks_fp_kernel(NttArgs a, TensorFuse x) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1))) void tensor_intt_blocks_fp_kernel(NttArgs a, TensorFuse x) {
     __shared__ uint64_t lds[kLdsWords];
     double *ld = reinterpret_cast<double *>(lds);
     const uint32_t nthreads = blockDim.x;
@@ -1105,7 +1105,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     fp_load_block_tw<4>(tw1, fc.tw, g.idx1 + gi);
 
     const size_t lo = (size_t)job.limb * n + g.off, poly = (size_t)x.L * n;
-#pragma unroll 4
+    // the launch has 1.5 waves per SIMD at N = 2^16, L = 24: all 64 loads of a thread are in flight at once
+#pragma unroll
     for (int i = 0; i < kPer; i++) {
         const uint32_t e = threadIdx.x + i * nthreads;
         const double a0 = fp_from_u64(x.ct1[lo + e]), a1 = fp_from_u64(x.ct1[poly + lo + e]);

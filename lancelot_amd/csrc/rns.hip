@@ -733,6 +733,104 @@ hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtr
     return hipGetLastError();
 }
 
+struct InnerFpArgs {
+    const uint64_t *y, *own;
+    uint64_t *out;
+    const double *fp_consts;
+    EvkPtrs evk;
+    uint32_t L, K, size_q, beta, log_n, items;
+    const uint64_t *fold_ct, *fold_w;
+    size_t y_item_stride, own_item_stride, out_item_stride, fold_item_stride;
+};
+
+// The inner product of a batch on the FP64 back end (every prime below 2^50).  grid: (N / 512, L + K, groups of I
+// items); a thread holds two coefficients of I items.  A key word is loaded and converted once and multiplies all I
+// items, so the 2 beta key limbs are read once per group instead of once per item; a digit's own limbs are read from
+// the key switch's input (own, NTT form) rather than from a copy inside y.  Terms stay below 0.875 q, eight of them
+// fit between two reductions; the stores are canonical, hence equal to the integer kernel's.
+template <int I>
+__global__ __launch_bounds__(kThreads) void inner_product_fp_kernel(InnerFpArgs p) {
+    const uint32_t t = blockIdx.y;
+    const uint32_t LK = p.L + p.K;
+    const uint32_t table = t < p.L ? t : p.size_q + (t - p.L);
+    const FpMod m{p.fp_consts[4 * table], p.fp_consts[4 * table + 1]};
+    const size_t j = 2 * ((size_t)blockIdx.x * kThreads + threadIdx.x);
+    const size_t key_off = ((size_t)table << p.log_n) + j;
+    const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
+    const uint32_t item0 = blockIdx.z * I;
+    const uint32_t own_digit = t < p.L ? t / p.K : 0xffffffffu;
+    double acc[I][4];
+#pragma unroll
+    for (int i = 0; i < I; i++) acc[i][0] = acc[i][1] = acc[i][2] = acc[i][3] = 0.0;
+    for (uint32_t d = 0; d < p.beta; d++) {
+        const uint64_t *k = p.evk.p[d];
+        const ulonglong2 k0 = *reinterpret_cast<const ulonglong2 *>(k + key_off);
+        const ulonglong2 k1 = *reinterpret_cast<const ulonglong2 *>(k + key_off + key_poly);
+        const double w00 = fp_from_u64(k0.x), w01 = fp_from_u64(k0.y), w10 = fp_from_u64(k1.x), w11 = fp_from_u64(k1.y);
+        const FpTw t00{w00, w00 * m.qinv}, t01{w01, w01 * m.qinv}, t10{w10, w10 * m.qinv}, t11{w11, w11 * m.qinv};
+        const bool is_own = d == own_digit;
+        const uint64_t *src = is_own ? p.own + ((size_t)t << p.log_n) + j : p.y + (((size_t)d * LK + t) << p.log_n) + j;
+        const size_t stride = is_own ? p.own_item_stride : p.y_item_stride;
+#pragma unroll
+        for (int i = 0; i < I; i++) {
+            const uint32_t item = item0 + i < p.items ? item0 + i : p.items - 1;
+            const ulonglong2 v = *reinterpret_cast<const ulonglong2 *>(src + item * stride);
+            const double y0 = fp_from_u64(v.x), y1 = fp_from_u64(v.y);
+            acc[i][0] += fp_mulmod(y0, t00, m);
+            acc[i][1] += fp_mulmod(y1, t01, m);
+            acc[i][2] += fp_mulmod(y0, t10, m);
+            acc[i][3] += fp_mulmod(y1, t11, m);
+        }
+        if ((d & 7) == 7) {
+#pragma unroll
+            for (int i = 0; i < I; i++)
+                for (int c = 0; c < 4; c++) acc[i][c] = fp_reduce(acc[i][c], m);
+        }
+    }
+    const size_t o = ((size_t)t << p.log_n) + j;
+    const size_t opoly = (size_t)LK << p.log_n;
+    const bool fold = p.fold_ct && t == p.L - 1;
+    const double wd = fold ? fp_from_u64(p.fold_w[0]) : 0.0;
+    const FpTw fw{wd, wd * m.qinv};
+#pragma unroll
+    for (int i = 0; i < I; i++) {
+        if (item0 + i >= p.items) break;
+        double r[4];
+        for (int c = 0; c < 4; c++) r[c] = fp_canonical(acc[i][c], m);
+        if (fold) {
+            const uint64_t *f = p.fold_ct + (item0 + i) * p.fold_item_stride + o;
+            const ulonglong2 f0 = *reinterpret_cast<const ulonglong2 *>(f);
+            const ulonglong2 f1 = *reinterpret_cast<const ulonglong2 *>(f + ((size_t)p.L << p.log_n));
+            r[0] = fp_canonical(fp_mulmod(r[0], fw, m) + fp_from_u64(f0.x), m);
+            r[1] = fp_canonical(fp_mulmod(r[1], fw, m) + fp_from_u64(f0.y), m);
+            r[2] = fp_canonical(fp_mulmod(r[2], fw, m) + fp_from_u64(f1.x), m);
+            r[3] = fp_canonical(fp_mulmod(r[3], fw, m) + fp_from_u64(f1.y), m);
+        }
+        uint64_t *out = p.out + (item0 + i) * p.out_item_stride + o;
+        *reinterpret_cast<ulonglong2 *>(out) = ulonglong2{fp_to_u64(r[0]), fp_to_u64(r[1])};
+        *reinterpret_cast<ulonglong2 *>(out + opoly) = ulonglong2{fp_to_u64(r[2]), fp_to_u64(r[3])};
+    }
+}
+
+hipError_t launch_inner_product_fp(const Tables &t, const double *fp_consts, const uint64_t *y, const uint64_t *own,
+                                   size_t own_item_stride, const EvkPtrs &evk, uint64_t *out, uint32_t L, uint32_t K,
+                                   uint32_t size_q, uint32_t beta, const uint64_t *fold_ct, const uint64_t *fold_w,
+                                   uint32_t items, size_t fold_item_stride, hipStream_t s) {
+    const size_t n = (size_t)1 << t.log_n;
+    if (items == 0 || n < 2 * kThreads || !fp_consts || !own) return hipErrorInvalidValue;
+    InnerFpArgs p{y, own, out, fp_consts, evk, L, K, size_q, beta, t.log_n, items, fold_ct, fold_w,
+                  (size_t)beta * (L + K) * n, own_item_stride, 2 * (size_t)(L + K) * n, fold_item_stride};
+    auto grid = [&](uint32_t per) { return dim3((uint32_t)(n / (2 * kThreads)), L + K, (items + per - 1) / per); };
+    if ((items + 7) / 8 > 65535) return hipErrorInvalidValue;
+    if (items >= 7)
+        hipLaunchKernelGGL(inner_product_fp_kernel<8>, grid(8), dim3(kThreads), 0, s, p);
+    else if (items >= 3)
+        hipLaunchKernelGGL(inner_product_fp_kernel<4>, grid(4), dim3(kThreads), 0, s, p);
+    else
+        hipLaunchKernelGGL(inner_product_fp_kernel<2>, grid(2), dim3(kThreads), 0, s, p);
+    return hipGetLastError();
+}
+
 hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
                               const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
                               uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, bool with_self, uint32_t items,
