@@ -44,11 +44,18 @@ sys.path.insert(0, ROOT)
 LOG_N, SIZE_Q, SIZE_P, BITS, SCALE = 16, 24, 8, 50, 2.0 ** 40
 HBM_PEAK_GBS = 8000.0
 BLOCKS = 5
-# From profiles/hmult_relin_rescale_n65536_l24_k8.md (rocprofv3 --pmc of `bench.py --only step`), per step on one
-# stream: L2-miss traffic (FETCH_SIZE scaled by 2, WRITE_SIZE by 1: the factors a copy of known size gives) and
-# SQ_INSTS_VALU summed over the step's kernels.  Constants of the profile, not measured in this run.
-STEP_TRAFFIC_BYTES = 1158 * 524288
-STEP_VALU_WAVE_INSTR = 35.9e6
+# From profiles/hmult_relin_rescale_n65536_l24_k8.md (rocprofv3 --pmc runs of `bench.py --only step` and
+# `--only batch`), per operation: L2-miss traffic in limbs of 8 N bytes (FETCH_SIZE scaled by 2, WRITE_SIZE by 1: the
+# factors a copy of known size gives) and SQ_INSTS_VALU summed over the kernels.  Constants of the profile, not
+# measured in this run.
+PROFILE = {"single": {"traffic_limbs": 1128.5, "valu_wave_instr": 35.89e6,
+                      "kernels": "tensor_intt_blocks_fp, ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp_inner, "
+                                 "ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp with the rescale "
+                                 "epilogue"},
+           "batch": {"traffic_limbs": 1066.6, "valu_wave_instr": 35.2e6,
+                     "kernels": "per call of 8 operations: tensor_fp, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, "
+                                "ntt_blocks_fp, inner_product_fp, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, "
+                                "ntt_blocks_fp with the rescale epilogue"}}
 
 
 def sync(capi):
@@ -220,7 +227,7 @@ def main():
                          "hardware queues of a process)")
     ap.add_argument("--batch", type=int, default=8, help="operations per he_multiply_relin_rescale_batch call")
     ap.add_argument("--no-krum", action="store_true", help="skip the encrypted Krum round (BASELINE.json configs[4])")
-    ap.add_argument("--only", choices=["all", "step", "rotate", "ntt", "krum"], default="all",
+    ap.add_argument("--only", choices=["all", "step", "batch", "rotate", "ntt", "krum"], default="all",
                     help="step / rotate / ntt: run just that workload on the null stream (for rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -278,8 +285,20 @@ def main():
     two = Buf(capi, 2 * L * n)
     capi.check(lib.he_memcpy_d2d(two.ptr, a_ptr, 8 * 2 * L * n, None))
 
-    if args.only in ("step", "rotate", "ntt"):
-        fn = {"step": step, "rotate": one_rot,
+    # operands of the batch entry point: `batch` independent products per call
+    B = args.batch
+    ba, bb = Buf(capi, B * 2 * L * n), Buf(capi, B * 2 * L * n)
+    for k in range(B):
+        capi.check(lib.he_memcpy_d2d(ba.at(k * 2 * L * n), a_ptr, 8 * 2 * L * n, None))
+        capi.check(lib.he_memcpy_d2d(bb.at(k * 2 * L * n), b_ptr, 8 * 2 * L * n, None))
+    bres = Buf(capi, B * 2 * (L - 1) * n)
+    bws = Buf(capi, lib.he_multiply_relin_rescale_batch_workspace_words(h, L, B))
+
+    def batch_call():
+        capi.check(lib.he_multiply_relin_rescale_batch(h, L, B, ba.ptr, bb.ptr, evk, bres.ptr, bws.ptr, None))
+
+    if args.only in ("step", "batch", "rotate", "ntt"):
+        fn = {"step": step, "batch": batch_call, "rotate": one_rot,
               "ntt": lambda: (capi.check(lib.he_ntt_forward(h, two.ptr, 2, L, L, 0, L, 0, None)),
                               capi.check(lib.he_ntt_inverse(h, two.ptr, 2, L, L, 0, L, 0, None)))}[args.only]
         # one device-to-device copy of known size calibrates FETCH_SIZE / WRITE_SIZE of a rocprofv3 --pmc run
@@ -325,17 +344,6 @@ def main():
     streams_ms, streams_blocks = timed_wall(lambda i: lane_step(i % args.lanes), K_steps)
 
     # (3) `batch` operations per call, one launch per stage for all of them
-    B = args.batch
-    ba, bb = Buf(capi, B * 2 * L * n), Buf(capi, B * 2 * L * n)
-    for k in range(B):
-        capi.check(lib.he_memcpy_d2d(ba.at(k * 2 * L * n), a_ptr, 8 * 2 * L * n, None))
-        capi.check(lib.he_memcpy_d2d(bb.at(k * 2 * L * n), b_ptr, 8 * 2 * L * n, None))
-    bres = Buf(capi, B * 2 * (L - 1) * n)
-    bws = Buf(capi, lib.he_multiply_relin_rescale_batch_workspace_words(h, L, B))
-
-    def batch_call():
-        capi.check(lib.he_multiply_relin_rescale_batch(h, L, B, ba.ptr, bb.ptr, evk, bres.ptr, bws.ptr, None))
-
     calls = max(1, -(-K_steps // B))
     batch_ms = timer.time(batch_call, calls, max(1, W // B)) / B
 
@@ -366,7 +374,6 @@ def main():
     # measured FP64 issue rate of this GPU (8 waves per SIMD of independent multiply-add chains)
     rate = C.c_double()
     capi.check(lib.he_probe_fp64_issue_rate(2048, 2000, C.byref(rate), None))
-    valu_floor_ms = STEP_VALU_WAVE_INSTR * 64 / rate.value * 1e3
 
     # config "NTT alone": 24 limbs x 2 polynomials, forward + inverse
     f = timer.time(lambda: capi.check(lib.he_ntt_forward(h, two.ptr, 2, L, L, 0, L, 0, None)), 100)
@@ -406,6 +413,27 @@ def main():
     def frac(ms):
         return alg_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS
 
+    def roofline(ms_per_op, kind, what, ops_per_launch):
+        """The step as the roofline unit: its kernels run back to back, so algorithmic bytes over the step's
+        duration is the traffic-weighted rate of its kernels."""
+        prof = PROFILE[kind]
+        issue_ms = prof["valu_wave_instr"] * 64 / rate.value * 1e3
+        floor_ms = 920 * limb_bytes / 6.0e12 * 1e3
+        return {"bound": "hbm", "kernel": what + prof["kernels"],
+                "achieved": alg_bytes / (ms_per_op * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": frac(ms_per_op), "ms_per_launch": ms_per_op * ops_per_launch,
+                "operations_per_launch": ops_per_launch,
+                "algorithmic_bytes_per_launch": alg_bytes * ops_per_launch,
+                "traffic": int(prof["traffic_limbs"] * limb_bytes * ops_per_launch),
+                "traffic_source": "profiles/hmult_relin_rescale_n65536_l24_k8.md (counter profile, not this run)",
+                "frac_of_dataflow_floor": floor_ms / ms_per_op,
+                "dataflow_floor": "920 limbs of traffic per operation (two-pass transforms, every fusion of "
+                                  "neighbouring pointwise stages) at the 6 TB/s a streaming kernel reaches on this GPU",
+                "valu": {"wave_instructions_per_operation": prof["valu_wave_instr"],
+                         "source": "SQ_INSTS_VALU summed over the kernels, same profile",
+                         "fp64_issue_peak_lane_ops_per_s": rate.value, "issue_bound_ms": issue_ms,
+                         "frac_of_issue_bound": issue_ms / ms_per_op}}
+
     best_ms, path = min((streams_ms, "streams"), (batch_ms, "batch"))
     line = {
         "metric": "HMult+relin+rescale ops/s at N=2^16, L=24 (dnum=3, 8 special primes)",
@@ -430,21 +458,9 @@ def main():
         "api_path": {"calls": "pyCAHEL multiply, relinearize_inplace, rescale_to_next_inplace on the null stream",
                      "ms_per_step": api_ms, "ops_per_s": 1e3 / api_ms, "frac_of_hbm_roofline": frac(api_ms)},
         "check": {"all_paths_equal_the_evaluator": same, "decrypt_max_abs_err_vs_xy": max_err},
-        "roofline": {"bound": "hbm",
-                     "kernel": "the timed step on one stream: tensor_intt_blocks_fp, ntt_rows (inverse), bconv_rows_fp, "
-                               "ntt_blocks_fp_inner, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp with "
-                               "the rescale epilogue",
-                     "achieved": alg_bytes / (single_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": frac(single_ms), "ms_per_launch": single_ms, "algorithmic_bytes_per_launch": alg_bytes,
-                     "traffic": STEP_TRAFFIC_BYTES,
-                     "traffic_source": "profiles/hmult_relin_rescale_n65536_l24_k8.md (counter profile, not this run)",
-                     "frac_of_dataflow_floor": (920 * limb_bytes / 6.0e12 * 1e3) / single_ms,
-                     "dataflow_floor": "920 limbs of traffic (two-pass transforms, every fusion of neighbouring "
-                                       "pointwise stages) at the 6 TB/s a streaming kernel reaches on this GPU",
-                     "valu": {"wave_instructions_per_step": STEP_VALU_WAVE_INSTR,
-                              "source": "SQ_INSTS_VALU summed over the step's kernels, same profile",
-                              "fp64_issue_peak_lane_ops_per_s": rate.value, "issue_bound_ms": valu_floor_ms,
-                              "frac_of_issue_bound": valu_floor_ms / single_ms}},
+        "roofline": roofline(best_ms, "batch" if path == "batch" else "single",
+                             "value path (%s): " % path, B if path == "batch" else 1),
+        "single_stream_roofline": roofline(single_ms, "single", "one operation after the other on one stream: ", 1),
         "ntt": ntt, "rotate": rotate,
     }
     if not args.no_krum:
