@@ -93,6 +93,7 @@ struct he_context {
     double *d_phat_pinv_fp = nullptr;    // the same matrix times P^-1 mod q_j (merged ModDown + rescale, fused kernel)
     bool fuse_rows = true;       // environment CAHEL_HIP_NO_FUSED_BCONV=1: conversion kernel, then the rows pass
     bool fuse_tensor = true;     // environment CAHEL_HIP_NO_FUSED_TENSOR=1: he_multiply_relin_rescale as tensor kernel + key switch
+    bool single_limb_digits = false;  // K = 1 (environment CAHEL_HIP_NO_REDUCE_IN_NTT=1: keep the conversion kernels)
     bool fp_inner = true;        // environment CAHEL_HIP_NO_FP_INNER=1: a batch's inner product on the integer kernel
     uint32_t *d_rot_group = nullptr;     // encoder: 5^j mod 2N
     double2 *d_ksi = nullptr;            // encoder: e^{2 pi i k / 2N}, k <= 2N
@@ -406,6 +407,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->fuse_rows = !(nb && nb[0] == '1');
         const char *nt = getenv("CAHEL_HIP_NO_FUSED_TENSOR");
         ctx->fuse_tensor = !(nt && nt[0] == '1');
+        const char *nr = getenv("CAHEL_HIP_NO_REDUCE_IN_NTT");
+        ctx->single_limb_digits = ctx->size_p == 1 && !(nr && nr[0] == '1');
         const char *ni = getenv("CAHEL_HIP_NO_FP_INNER");
         ctx->fp_inner = !(ni && ni[0] == '1');
         ctx->fp_ok.assign(qp, 0);
@@ -771,7 +774,16 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     // skip_own (batched levels only): the consumer reads a digit's own limbs from c, their slots in out stay unwritten
     if (skip_own && !lv->batched) return HE_E_INVALID_ARGUMENT;
     const uint32_t copy_rows = skip_own ? 0 : lv->modup_max_copy;
-    if (fused) {
+    // digits of one limb each (K = 1): (Q_d / q_d)^-1 and the conversion matrix are all ones, so the conversion is the
+    // reduction of the digit's coefficients modulo each other prime, which the forward transform does where it reads
+    // its input; only the digits' own limbs are copied
+    const bool reduce_in_ntt = ctx->single_limb_digits && !fused;
+    if (reduce_in_ntt) {
+        for (uint32_t d = 0; d < lv->beta && !skip_own; d++)
+            HE_HIP(hipMemcpy2DAsync(out + ((size_t)d * LK + d) * n, (size_t)lv->beta * LK * n * sizeof(uint64_t),
+                                    c + (size_t)d * n, (size_t)c_item_stride * n * sizeof(uint64_t), n * sizeof(uint64_t),
+                                    items, hipMemcpyDeviceToDevice, S(s)));
+    } else if (fused) {
         BconvRows b{ws, out, c, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                     lv->beta, lv->modup_max_rows, copy_rows,
                     items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n, 0};
@@ -782,7 +794,7 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
                      items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n};
         HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
     }
-    for (uint32_t d = 0; d < lv->beta && !lv->batched; d++) {
+    for (uint32_t d = 0; d < lv->beta && !lv->batched && !reduce_in_ntt; d++) {
         const Digit &g = lv->digits[d];
         uint64_t *od = out + (size_t)d * LK * n;
         // the digit's own limbs keep their NTT form
@@ -800,6 +812,12 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     fwd.n_groups = lv->n_modup_groups;
     fwd.items = items;
     fwd.item_stride = (size_t)lv->beta * LK * n;
+    if (reduce_in_ntt) {
+        fwd.pro_mode = NTT_PRO_SOURCE_REDUCE;
+        fwd.pro_src = ws;
+        fwd.pro_item_stride = (size_t)L * n;
+        fwd.pro_lk = LK;
+    }
     HE_HIP(launch_ntt_forward(fwd, 1, backend_for_level(ctx, L), S(s), fused));
     return HE_OK;
 }
@@ -853,7 +871,11 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     // the conversion tables describe up to 4 polynomials; more of them go as items of 2 (ciphertexts)
     const bool batched = lv && lv->batched && (n_polys <= 4 || n_polys % 2 == 0);
     const bool fused = batched && fuse_rows_ok(ctx, lv, L);
-    if (batched) {
+    // one special prime: (P / p)^-1 and the conversion matrix are ones, the conversion is the reduction of the special
+    // limb's coefficients modulo each q_j, done where the forward transform reads its input
+    const bool reduce_in_ntt = ctx->single_limb_digits && !fused;
+    if (reduce_in_ntt) {
+    } else if (batched) {
         const uint32_t units = n_polys <= 4 ? n_polys : 2, items = n_polys / units;
         if (fused) {
             BconvRows b{cx, ws, nullptr, ctx->d_phat_mod_q_fp, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, units, L, 0,
@@ -866,7 +888,7 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
             HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
         }
     }
-    for (uint32_t p = 0; p < n_polys && !batched; p++) {
+    for (uint32_t p = 0; p < n_polys && !batched && !reduce_in_ntt; p++) {
         BconvArgs b{cx + ((size_t)p * LK + L) * n, ws + (size_t)p * L * n, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, K, L};
         HE_HIP(launch_bconv(ctx->tables(), b, S(s)));
     }
@@ -884,6 +906,11 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     fwd.w = ctx->d_pinv_mod_q;
     fwd.epi_dst = out;
     fwd.epi_dst_poly_stride = L;
+    if (reduce_in_ntt) {
+        fwd.pro_mode = NTT_PRO_SOURCE_REDUCE;
+        fwd.pro_src = cx + (size_t)L * n;
+        fwd.pro_poly_stride = LK;
+    }
     HE_HIP(launch_ntt_forward(fwd, n_polys, backend_for(ctx, fwd.map), S(s), fused));
     return HE_OK;
 }

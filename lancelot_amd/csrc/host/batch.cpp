@@ -112,13 +112,13 @@ std::vector<CAHELGPUCiphertext> pair_square_distances(
         std::swap(acc, next);
     }
 
-    // (4) one ciphertext object per pair
+    // (4) one ciphertext object per pair, each a slice of the batch (no copies)
     std::vector<CAHELGPUCiphertext> out(items);
     const std::size_t words = 2 * (std::size_t)L1 * n;
+    auto shared = std::make_shared<DeviceBuffer>(std::move(acc));
     for (uint32_t k = 0; k < items; k++) {
         CAHELGPUCiphertext &ct = out[k];
-        ct.data_.allocate(words);
-        check_status(he_memcpy_d2d(ct.data(), acc.get() + k * words, words * sizeof(uint64_t), st), "copy");
+        ct.data_ = DeviceBuffer::slice(shared, k * words, words);
         ct.size_ = 2;
         ct.coeff_modulus_size_ = L1;
         ct.poly_modulus_degree_ = n;

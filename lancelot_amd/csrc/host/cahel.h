@@ -77,7 +77,7 @@ public:
     DeviceBuffer() = default;
     explicit DeviceBuffer(std::size_t words) { allocate(words); }
     DeviceBuffer(const DeviceBuffer &o);
-    DeviceBuffer(DeviceBuffer &&o) noexcept : ptr_(o.ptr_), words_(o.words_), lane_(o.lane_) {
+    DeviceBuffer(DeviceBuffer &&o) noexcept : ptr_(o.ptr_), words_(o.words_), lane_(o.lane_), parent_(std::move(o.parent_)) {
         o.ptr_ = nullptr;
         o.words_ = 0;
     }
@@ -88,6 +88,10 @@ public:
     void release();
     // becomes a copy of the first `words` words of `src`; keeps its own block when that is large enough
     void assign(const DeviceBuffer &src, std::size_t words);
+    // `words` words of `parent` from word `offset` on, without a copy: the slice keeps the parent's block alive and
+    // returns nothing to the pool itself (batched evaluations hand out their results this way); a copy of a slice
+    // is an ordinary buffer of its own
+    static DeviceBuffer slice(std::shared_ptr<DeviceBuffer> parent, std::size_t offset, std::size_t words);
     uint64_t *get() const { return ptr_; }
     std::size_t words() const { return words_; }
     static void trim_pool();  // return every cached block to the driver
@@ -96,6 +100,7 @@ private:
     uint64_t *ptr_ = nullptr;
     std::size_t words_ = 0;
     int lane_ = 0;  // the lane whose stream orders the reuse of this block
+    std::shared_ptr<DeviceBuffer> parent_;  // set for a slice: the owner of the block that ptr_ points into
 };
 
 // Lanes (not in the reference, which runs everything on the legacy default stream): lane 0 is the null stream,

@@ -136,9 +136,20 @@ void DeviceBuffer::release() {
     // A block goes back to the lane that took it.  Dropped from another lane, it may still be read by work that
     // the dropping thread has enqueued there: wait for that lane before the owner's lane can reuse the block.
     if (ptr_ && g_lane != lane_) (void)he_stream_synchronize(g_lane_streams[g_lane]);
-    if (ptr_) pool().give(ptr_, words_ * sizeof(uint64_t), lane_);
+    if (ptr_ && !parent_) pool().give(ptr_, words_ * sizeof(uint64_t), lane_);
+    parent_.reset();  // the last slice to go releases the parent's block (same rule, in the parent's destructor)
     ptr_ = nullptr;
     words_ = 0;
+}
+
+DeviceBuffer DeviceBuffer::slice(std::shared_ptr<DeviceBuffer> parent, std::size_t offset, std::size_t words) {
+    if (!parent || offset + words > parent->words_) throw std::logic_error("DeviceBuffer::slice: out of range");
+    DeviceBuffer v;
+    v.ptr_ = parent->ptr_ + offset;
+    v.words_ = words;
+    v.lane_ = parent->lane_;
+    v.parent_ = std::move(parent);
+    return v;
 }
 
 DeviceBuffer::DeviceBuffer(const DeviceBuffer &o) {
@@ -166,6 +177,7 @@ DeviceBuffer &DeviceBuffer::operator=(DeviceBuffer &&o) noexcept {
         ptr_ = o.ptr_;
         words_ = o.words_;
         lane_ = o.lane_;
+        parent_ = std::move(o.parent_);
         o.ptr_ = nullptr;
         o.words_ = 0;
     }

@@ -52,6 +52,12 @@ enum : int {
     // forward prologue of the merged ModDown + rescale: with r = pro_src - pro_src2 * pro_w[pro_last] mod q_last
     // (the coefficients of the last limb of the ModDown result), input value = in * pro_w + (r mod q)
     NTT_PRO_MODDOWN_RESCALE = 7,
+    // forward prologue: input value = source limb mod q by integer Barrett reduction (the source may be any 64-bit
+    // residue, also where the limb itself runs on the FP64 back end).  Map mode: the source of polynomial p is
+    // pro_src + p * pro_poly_stride * N.  List mode: the source of job (data_limb, table) of item i is limb
+    // data_limb / pro_lk of pro_src + i * pro_item_stride: the base conversion of digits of one limb each (K = 1),
+    // whose matrix is all ones, done where the forward transform of the converted limb reads its input
+    NTT_PRO_SOURCE_REDUCE = 8,
 };
 
 struct NttArgs {
@@ -80,6 +86,8 @@ struct NttArgs {
     int epi_mode;
     const uint64_t *pro_src;  // [poly][pro_poly_stride limbs], the first limb of each poly is the source
     uint32_t pro_poly_stride;
+    size_t pro_item_stride;   // NTT_PRO_SOURCE_REDUCE in list mode: words between the sources of consecutive items
+    uint32_t pro_lk;          // ... and limbs per digit of the list's buffer (L + K)
     const uint64_t *epi_a;    // limb (poly, i) like `out`, with its own poly stride
     uint32_t epi_a_poly_stride;
     const uint64_t *epi_b;

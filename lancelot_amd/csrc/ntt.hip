@@ -62,6 +62,7 @@ struct Job {
     uint32_t table;
     uint32_t poly;
     uint32_t limb;
+    const uint64_t *src;   // NTT_PRO_SOURCE_REDUCE (rows pass only): the limb that is reduced into this one
 };
 
 __device__ __forceinline__ Job decode_job(const NttArgs &a, uint32_t job) {
@@ -76,12 +77,14 @@ __device__ __forceinline__ Job decode_job(const NttArgs &a, uint32_t job) {
         j.table = lj.table;
         j.poly = 0;
         j.limb = 0;
+        j.src = a.pro_mode == NTT_PRO_SOURCE_REDUCE ? a.pro_src + item * a.pro_item_stride + (size_t)(lj.data_limb / a.pro_lk) * n : nullptr;
     } else {
         j.poly = job / a.map.limbs;
         j.limb = job % a.map.limbs;
         j.in = a.in ? a.in + ((size_t)j.poly * a.in_poly_stride + j.limb) * n : nullptr;
         j.out = a.out + ((size_t)j.poly * a.out_poly_stride + j.limb) * n;
         j.table = map_table(a.map, j.limb);
+        j.src = a.pro_src + ((size_t)j.poly * a.pro_poly_stride << a.log_n);
     }
     return j;
 }
@@ -241,6 +244,11 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
                 const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = fp_from_u64(src[glob(e_far(j))]);
+            } else if (a.pro_mode == NTT_PRO_SOURCE_REDUCE) {
+                const uint64_t q = a.moduli[job.table], r1 = a.barrett[2 * job.table + 1];
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = fp_from_u64(barrett64(job.src[glob(e_far(j))], q, r1));
+                reduce_first = false;
             } else {
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = fp_from_u64(job.in[glob(e_far(j))]);
@@ -286,9 +294,9 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
     const uint64_t q = c.q;
     uint64_t v[16];
     if (FWD) {
-        if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE) {
+        if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE || a.pro_mode == NTT_PRO_SOURCE_REDUCE) {
             const uint64_t r1 = a.barrett[2 * job.table + 1];
-            const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+            const uint64_t *src = a.pro_mode == NTT_PRO_SOURCE_REDUCE ? job.src : a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
 #pragma unroll
             for (int j = 0; j < 16; j++) v[j] = barrett64(src[glob(e_far(j))], q, r1);
         } else if (a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
@@ -385,6 +393,12 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
                     const double r = fp_canonical(fp_from_u64(bsrc[g]) - fp_mulmod(fp_from_u64(dsrc[g]), wlast, ml), ml);
                     ld[skew(e)] = fp_mulmod(fp_from_u64(src[g]), w, c.m) + fp_reduce(r, c.m);
                 }
+            } else if (a.pro_mode == NTT_PRO_SOURCE_REDUCE) {
+                const uint64_t q = a.moduli[job.table], r1 = a.barrett[2 * job.table + 1];
+                for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
+                    uint32_t row = e >> LOGC, col = e & (C - 1);
+                    ld[skew(e)] = fp_from_u64(barrett64(job.src[(size_t)row * 256 + col0 + col], q, r1));
+                }
             } else {
                 for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                     uint32_t row = e >> LOGC, col = e & (C - 1);
@@ -430,9 +444,9 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
 
     const IntCtx c = int_ctx(a, job.table);
     const uint64_t q = c.q;
-    if (FWD && a.pro_mode == NTT_PRO_BROADCAST_REDUCE) {
+    if (FWD && (a.pro_mode == NTT_PRO_BROADCAST_REDUCE || a.pro_mode == NTT_PRO_SOURCE_REDUCE)) {
         const uint64_t r1 = a.barrett[2 * job.table + 1];
-        const uint64_t *src = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
+        const uint64_t *src = a.pro_mode == NTT_PRO_SOURCE_REDUCE ? job.src : a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
         for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
             uint32_t row = e >> LOGC, col = e & (C - 1);
             lds[skew(e)] = barrett64(src[(size_t)row * 256 + col0 + col], q, r1);
@@ -827,7 +841,7 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
         LimbJob lj = pre[0];
 #pragma unroll
         for (int i = 1; i < kMaxGroup; i++) lj = b == (uint32_t)i ? pre[i] : lj;
-        return Job{a.in + item_off + (size_t)lj.data_limb * n, a.out + item_off + (size_t)lj.data_limb * n, lj.table, 0, 0};
+        return Job{a.in + item_off + (size_t)lj.data_limb * n, a.out + item_off + (size_t)lj.data_limb * n, lj.table, 0, 0, nullptr};
     };
 
     uint64_t nx[kPer];
