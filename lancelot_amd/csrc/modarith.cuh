@@ -79,6 +79,59 @@ __device__ __forceinline__ void mac128(U128 &acc, uint64_t a, uint64_t b) {
     acc.hi += hi + (acc.lo < lo);
 }
 
+// Lazy sum of products of residues below 2^61 with few carries.  The factors are split at bit 31
+// (a = a1 2^31 + a0 with a0 < 2^31, a1 < 2^30); the four partial products of a term go, by weight, into three
+// 64-bit words (ll: a0 b0 < 2^62, mid: a1 b0 + a0 b1 < 2^62, hh: a1 b1 < 2^60), each a 32 x 32 + 64 multiply-add with
+// no carry out.  Four terms fit (4 * 2^62 = 2^64) before the words have to be relieved (spill3), so a product costs 4
+// multiply-adds and a few additions instead of a 64 x 64 -> 128 product (6 multiplies) and a carry chain; the
+// 32 x 32 multiplies issue at a quarter of the rate of other vector instructions and dominate either way.
+struct Split31 {
+    uint32_t lo, hi;
+};
+
+__device__ __forceinline__ Split31 split31(uint64_t a) { return Split31{(uint32_t)a & 0x7fffffffu, (uint32_t)(a >> 31)}; }
+
+struct Lazy3 {
+    uint64_t ll, mid, hh;
+};
+
+// One term for two sums that share the factor a (the two key polynomials of an inner product): eight
+// v_mad_u64_u32 (32 x 32 + 64 -> 64; the carry out goes to a scalar pair that nobody reads, the sums stay below
+// 2^64).  Written out because the compiler emits a multiply with a zero addend followed by a 64-bit add for
+// `acc += (uint64_t)a * b`, and one statement because it separates inline-assembly statements by s_nop.
+__device__ __forceinline__ void mac3x2(Lazy3 &s, Lazy3 &t, Split31 a, Split31 b, Split31 c) {
+    uint64_t carry;
+    asm("v_mad_u64_u32 %0, %6, %7, %9, %0\n\t"
+        "v_mad_u64_u32 %1, %6, %8, %9, %1\n\t"
+        "v_mad_u64_u32 %2, %6, %8, %10, %2\n\t"
+        "v_mad_u64_u32 %3, %6, %7, %11, %3\n\t"
+        "v_mad_u64_u32 %4, %6, %8, %11, %4\n\t"
+        "v_mad_u64_u32 %5, %6, %8, %12, %5\n\t"
+        "v_mad_u64_u32 %1, %6, %7, %10, %1\n\t"
+        "v_mad_u64_u32 %4, %6, %7, %12, %4"
+        : "+v"(s.ll), "+v"(s.mid), "+v"(s.hh), "+v"(t.ll), "+v"(t.mid), "+v"(t.hh), "=&s"(carry)
+        : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi), "v"(c.lo), "v"(c.hi));
+}
+
+// After four terms the upper halves of the three words move into three counters of weight 2^32 (two additions and
+// a move per word: no carries between the words), which leaves room for four more terms; total3 puts the six words
+// together at the end.  Up to 64 terms (the counters stay below 2^37).
+__device__ __forceinline__ void spill3(Lazy3 &h, Lazy3 &s) {
+    h.ll += s.ll >> 32;
+    s.ll &= 0xffffffffu;
+    h.mid += s.mid >> 32;
+    s.mid &= 0xffffffffu;
+    h.hh += s.hh >> 32;
+    s.hh &= 0xffffffffu;
+}
+
+__device__ __forceinline__ U128 total3(const Lazy3 &h, const Lazy3 &s) {
+    typedef unsigned __int128 u128;
+    const u128 t = ((u128)s.ll + ((u128)h.ll << 32)) + (((u128)s.mid + ((u128)h.mid << 32)) << 31) +
+                   (((u128)s.hh + ((u128)h.hh << 32)) << 62);
+    return U128{(uint64_t)t, (uint64_t)(t >> 64)};
+}
+
 // Cooley-Tukey butterfly, inputs in [0, 4q), outputs in [0, 4q).
 __device__ __forceinline__ void ct_butterfly(uint64_t &x, uint64_t &y, Shoup tw, uint64_t q) {
     uint64_t q2 = q << 1;

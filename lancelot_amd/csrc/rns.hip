@@ -436,13 +436,19 @@ struct HoistArgs {
 
 // Hoisted rotations in one launch: grid (N / 256, (L + K) + L [+ L], ceil(items / I)); a thread serves the same
 // coefficient of I consecutive items, so that a key word is loaded once for all of them.
-// rows t < L + K:  out[p][t] = sum_s sum_d sigma_s(y_d)[t] * evk_{s,d}[p][t]  (n_steps * beta <= 64 products, summed in
-//                  128 bits and reduced once); the automorphism is the gather index of the load of y.
+// rows t < L + K:  out[p][t] = sum_s sum_d sigma_s(y_d)[t] * evk_{s,d}[p][t]  (n_steps * beta <= 64 products, summed
+//                  lazily as split 31-bit partial products, see Lazy3, and reduced once); the automorphism is the
+//                  gather index of the load of y.  The kernel is bound by its 32 x 32 multiplies (quarter rate).
 // rows L + K + t:  c0_out[t] = sum_s sigma_s(c0)[t]  (+ c0[t] with_self)
 // rows L + K + L + t (with_self only): c1 is copied to the output, so that the ModDown that follows adds onto
 //                  the input ciphertext: ct_out = ct_in + sum_s rot_s(ct_in)
-template <int I>
+// LOCAL: every step's Galois element is 1 modulo 2^(log_n - 7) (steps that are multiples of N / 512), so the
+// automorphism permutes inside each aligned block of 256 NTT-order words: a workgroup stages its block of every item
+// and digit in LDS once (I * beta <= kHoistLocalTiles) and gathers from there, instead of one global gather per step.
+constexpr int kHoistLocalTiles = 16;
+template <int I, bool LOCAL>
 __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
+    __shared__ uint64_t ybuf[LOCAL ? kHoistLocalTiles * kThreads : 1];
     const uint32_t LK = p.L + p.K;
     const uint32_t j = blockIdx.x * kThreads + threadIdx.x;
     const uint32_t item0 = blockIdx.z * I;
@@ -473,23 +479,51 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     const size_t key_off = ((size_t)table << p.log_n) + j;
     const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
     const size_t digit = (size_t)LK << p.log_n;
-    U128 a0[I], a1[I];
+    Lazy3 s0[I], s1[I], h0[I], h1[I];
 #pragma unroll
-    for (int it = 0; it < I; it++) a0[it] = a1[it] = U128{0, 0};
-    for (uint32_t s = 0; s < p.n_steps; s++) {
-        const uint32_t src = galois_index(j, p.elts[s], p.log_n);
-        for (uint32_t d = 0; d < p.beta; d++) {
-            const uint64_t *k = p.evk.p[s * p.beta + d];
-            const uint64_t k0 = k[key_off], k1 = k[key_off + key_poly];
-            uint64_t v[I];
+    for (int it = 0; it < I; it++) s0[it] = s1[it] = h0[it] = h1[it] = Lazy3{0, 0, 0};
+    if (LOCAL) {
+        for (uint32_t d = 0; d < p.beta; d++)
 #pragma unroll
-            for (int it = 0; it < I; it++) v[it] = (uint32_t)it < count ? y[it * y_item + d * digit + src] : 0;
+            for (int it = 0; it < I; it++)
+                ybuf[(it * p.beta + d) * kThreads + threadIdx.x] = (uint32_t)it < count ? y[it * y_item + d * digit + j] : 0;
+        __syncthreads();
+    }
+    // term e = step e / beta, digit e mod beta; the operands of term e + 1 are requested before term e is
+    // multiplied, so that a wave does not wait for memory once per term
+    const uint32_t n_terms = p.n_steps * p.beta;
+    auto fetch = [&](uint32_t e, uint64_t &k0, uint64_t &k1, uint64_t(&v)[I]) {
+        const uint32_t st = e / p.beta, d = e - st * p.beta;
+        const uint32_t src = galois_index(j, p.elts[st], p.log_n);
+        const uint64_t *k = p.evk.p[e];
+        k0 = k[key_off];
+        k1 = k[key_off + key_poly];
+#pragma unroll
+        for (int it = 0; it < I; it++)
+            v[it] = LOCAL ? ybuf[(it * p.beta + d) * kThreads + (src & (kThreads - 1))]
+                          : ((uint32_t)it < count ? y[it * y_item + d * digit + src] : 0);
+    };
+    uint64_t k0, k1, v[I];
+    fetch(0, k0, k1, v);
+    for (uint32_t e = 0; e < n_terms; e++) {
+        uint64_t nk0, nk1, nv[I];
+        fetch(e + 1 < n_terms ? e + 1 : e, nk0, nk1, nv);
+        const Split31 ks0 = split31(k0), ks1 = split31(k1);
+#pragma unroll
+        for (int it = 0; it < I; it++) {
+            mac3x2(s0[it], s1[it], split31(v[it]), ks0, ks1);
+        }
+        if ((e & 3) == 3) {
 #pragma unroll
             for (int it = 0; it < I; it++) {
-                mac128(a0[it], v[it], k0);
-                mac128(a1[it], v[it], k1);
+                spill3(h0[it], s0[it]);
+                spill3(h1[it], s1[it]);
             }
         }
+        k0 = nk0;
+        k1 = nk1;
+#pragma unroll
+        for (int it = 0; it < I; it++) v[it] = nv[it];
     }
     const uint64_t q = p.moduli[table], r0 = p.barrett[2 * table], r1 = p.barrett[2 * table + 1];
     const size_t o = ((size_t)t << p.log_n) + j;
@@ -498,8 +532,9 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     for (int it = 0; it < I; it++) {
         if ((uint32_t)it >= count) break;
         uint64_t *out = p.out + (item0 + it) * ((size_t)2 * LK << p.log_n);
-        uint64_t o0 = barrett128(a0[it].lo, a0[it].hi, q, r0, r1);
-        uint64_t o1 = barrett128(a1[it].lo, a1[it].hi, q, r0, r1);
+        const U128 a0 = total3(h0[it], s0[it]), a1 = total3(h1[it], s1[it]);
+        uint64_t o0 = barrett128(a0.lo, a0.hi, q, r0, r1);
+        uint64_t o1 = barrett128(a1.lo, a1.hi, q, r0, r1);
         if (p.accumulate) {
             o0 = add_mod(o0, out[o], q);
             o1 = add_mod(o1, out[o + opoly], q);
@@ -858,14 +893,23 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
     p.items = items;
     const uint32_t rows = (L + K) + (with_self ? 2 : 1) * L;
     auto grid = [&](uint32_t per) { return dim3((1u << t.log_n) / kThreads, rows, (items + per - 1) / per); };
-    if (items >= 8)
-        hipLaunchKernelGGL(hoist_inner_kernel<8>, grid(8), dim3(kThreads), 0, s, p);
-    else if (items >= 4)
-        hipLaunchKernelGGL(hoist_inner_kernel<4>, grid(4), dim3(kThreads), 0, s, p);
-    else if (items >= 2)
-        hipLaunchKernelGGL(hoist_inner_kernel<2>, grid(2), dim3(kThreads), 0, s, p);
-    else
-        hipLaunchKernelGGL(hoist_inner_kernel<1>, grid(1), dim3(kThreads), 0, s, p);
+    // every automorphism of the launch stays inside the aligned 256-word blocks of the NTT order
+    bool local = t.log_n >= 8 && beta * 4 <= (uint32_t)kHoistLocalTiles;
+    for (uint32_t i = 0; i < n_steps && local; i++) local = t.log_n < 9 || ((elts[i] - 1) & ((1u << (t.log_n - 7)) - 1)) == 0;
+    static const bool no_local = [] { const char *e = getenv("CAHEL_HIP_NO_LOCAL_HOIST"); return e && e[0] == '1'; }();
+    if (no_local) local = false;
+#define HE_HOIST(I) \
+    if (local) hipLaunchKernelGGL((hoist_inner_kernel<I, true>), grid(I), dim3(kThreads), 0, s, p); \
+    else hipLaunchKernelGGL((hoist_inner_kernel<I, false>), grid(I), dim3(kThreads), 0, s, p)
+    // (8 items per thread halve the key traffic again but need 220 registers, 2 waves per SIMD: measured 20 % slower)
+    if (items >= 4) {
+        HE_HOIST(4);
+    } else if (items >= 2) {
+        HE_HOIST(2);
+    } else {
+        HE_HOIST(1);
+    }
+#undef HE_HOIST
     return hipGetLastError();
 }
 

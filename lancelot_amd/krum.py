@@ -105,9 +105,14 @@ def rotate_sum_plan(log_slots: int, config: KrumConfig):
     if config.hoisting_radix < 2 or log_slots <= 4:
         head = [list(range(1, 16))] if log_slots > 4 else []
         return head + [[2 ** k] for k in range(4 if head else 0, log_slots)]
-    rounds, block, slots = [], 1, 1 << log_slots
-    while block < slots:
-        radix = min(config.hoisting_radix, slots // block)
+    # The short round comes first: rounds whose steps are multiples of N / 512 permute the NTT order inside blocks of
+    # 256 words, which the hoisting kernel serves from LDS; the rounds before them gather from memory once per step,
+    # so those get the fewer steps.
+    log_radix = max(1, int(math.log2(config.hoisting_radix)))
+    n_rounds = -(-log_slots // log_radix)
+    rounds, block = [], 1
+    for r in range(n_rounds):
+        radix = 1 << (log_slots - (n_rounds - 1) * log_radix if r == 0 else log_radix)
         rounds.append([block * s for s in range(1, radix)])
         block *= radix
     return rounds

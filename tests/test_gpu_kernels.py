@@ -292,6 +292,39 @@ def test_hoisted_rotations_entry_point(oracle, capi, logn, bits, size_p, L, n_st
     assert lib.he_hoisted_rotations(h, L, din.ptr, flat, d_elts, n_steps, dout.ptr, ws.ptr, None) == -1   # even element
 
 
+@pytest.mark.parametrize("no_local", ["0", "1"])
+@pytest.mark.parametrize("logn,bits,size_p,L,items", [(11, [60, 40, 40, 60], 1, 2, 9), (12, [50, 50, 49, 50, 50, 50], 2, 4, 3),
+                                                       (9, [45, 40, 40, 50], 1, 2, 2)])
+def test_hoisted_rotations_with_block_local_steps(oracle, capi, monkeypatch, logn, bits, size_p, L, items, no_local):
+    """Steps that are multiples of N / 512 (Galois elements 1 modulo 2^(log N - 7)) permute the NTT order inside
+    aligned blocks of 256 words; the batch kernel then gathers from a copy of the block in LDS.  Against the oracle
+    item by item, with that path on and switched off, for groups of 8 + 1, 2 + 1 and 2 items."""
+    monkeypatch.setenv("CAHEL_HIP_NO_LOCAL_HOIST", no_local)
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    rng = np.random.default_rng(17)
+    lib, h = capi.lib(), ctx.he_handle()
+    beta = -(-L // size_p)
+    keys = [_evk(p, rng, capi) for _ in range(2)]
+    unit = max(1, p.n // 512)
+    steps = [unit * k for k in (1, 2, 3, 5)]
+    elts = [pow(5, s, 2 * p.n) for s in steps]
+    assert all((e - 1) % (1 << max(logn - 7, 2)) == 0 for e in elts)
+    n_steps = len(elts)
+    flat = capi.evk_array([keys[i % 2][1][d].ptr for i in range(n_steps) for d in range(beta)])
+    d_elts = (C.c_uint32 * n_steps)(*elts)
+    wsb = DeviceArray(capi, shape=(lib.he_keyswitch_batch_workspace_words(h, L, items),))
+    cts = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
+    din, dout = DeviceArray(capi, host=cts), DeviceArray(capi, shape=(items, 2, L, p.n))
+    for add_input in (0, 1):
+        capi.check(lib.he_hoisted_rotations_batch(h, L, items, din.ptr, flat, d_elts, n_steps, add_input, dout.ptr, wsb.ptr, None))
+        got = dout.numpy()
+        for k in range(items):
+            want = p.hoisting(cts[k], elts, [keys[i % 2][0] for i in range(n_steps)])
+            if add_input:
+                want = np.stack([p.add(want[b], cts[k][b]) for b in range(2)])
+            assert (got[k] == want).all(), (add_input, k)
+
+
 @pytest.mark.parametrize("logn,bits,size_p,L,items", [(11, [45, 40, 40, 50], 1, 3, 5), (11, [60, 40, 40, 60], 1, 2, 3),
                                                        (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5, 2),
                                                        (11, [50, 50, 49, 50, 50, 50], 2, 4, 3),

@@ -441,7 +441,7 @@ def test_batched_pair_distances_equal_the_pairwise_ciphertexts(oracle):
     assert len(cts[0]) == 2
     pairs = [(0, 1), (0, 2), (1, 2), (2, 0)]
     rounds = krum.rotate_sum_plan(11, cfg)
-    assert [len(r) for r in rounds] == [7, 7, 7, 3]
+    assert [len(r) for r in rounds] == [3, 7, 7, 7]   # the short round first, block-local rounds last
     c = state.cahel
     batch = c.pair_square_distances(state.context, cts, pairs, state.rlk, state.glk, rounds, cfg.scale)
     c._synchronize()
