@@ -143,6 +143,52 @@ def cpu_baseline():
                           "sample": "%d iterations" % iters1, "ms_per_op": 1e3 / v1}}
 
 
+def gpu_c1(capi, cahel, timer, steps=400):
+    """BASELINE.json configs[0] (the reference's own CPU-runnable case: N = 2^14, 4 limbs of 50 bits + 1 special
+    prime) on the GPU: one operation after the other on the null stream, and batches of 32 per call."""
+    lib = capi.lib()
+    n, L, K = 1 << 14, 4, 1
+    parms = cahel.params(cahel.scheme_type.ckks)
+    parms.set_poly_modulus_degree(n)
+    parms.set_coeff_modulus(cahel.coeff_modulus_create(n, [50] * (L + K)))
+    parms.set_special_modulus_size(K)
+    ctx = cahel.context(parms, True, cahel.sec_level_type.none)
+    ctx.set_seed(2025)
+    sk = cahel.secret_key(parms)
+    sk.gen_secretkey(ctx)
+    pk = cahel.public_key(ctx)
+    sk.gen_publickey(ctx, pk)
+    rlk = cahel.relin_key(ctx)
+    sk.gen_relinkey(ctx, rlk)
+    enc = cahel.ckks_encoder(ctx)
+    rng = np.random.default_rng(14)
+    x, y = rng.uniform(-1, 1, n // 2), rng.uniform(-1, 1, n // 2)
+    ct1 = pk.encrypt_asymmetric(ctx, enc.encode(ctx, x, SCALE))
+    ct2 = pk.encrypt_asymmetric(ctx, enc.encode(ctx, y, SCALE))
+    h = ctx.he_handle()
+    evk = capi.evk_array([rlk.digit_ptr(d) for d in range(rlk.digit_count())])
+    ws, res = Buf(capi, lib.he_multiply_relin_rescale_workspace_words(h, L)), Buf(capi, 2 * (L - 1) * n)
+    single = timer.time(lambda: capi.check(lib.he_multiply_relin_rescale(h, L, ct1.data_ptr(), ct2.data_ptr(), evk,
+                                                                         res.ptr, ws.ptr, None)), steps, 20)
+    B = 32
+    ba, bb = Buf(capi, B * 2 * L * n), Buf(capi, B * 2 * L * n)
+    for k in range(B):
+        capi.check(lib.he_memcpy_d2d(ba.at(k * 2 * L * n), ct1.data_ptr(), 8 * 2 * L * n, None))
+        capi.check(lib.he_memcpy_d2d(bb.at(k * 2 * L * n), ct2.data_ptr(), 8 * 2 * L * n, None))
+    bres, bws = Buf(capi, B * 2 * (L - 1) * n), Buf(capi, lib.he_multiply_relin_rescale_batch_workspace_words(h, L, B))
+    batch = timer.time(lambda: capi.check(lib.he_multiply_relin_rescale_batch(h, L, B, ba.ptr, bb.ptr, evk, bres.ptr,
+                                                                              bws.ptr, None)), max(1, steps // B), 3) / B
+    prod = cahel.ciphertext(ctx)
+    cahel.multiply_relin_rescale(ctx, ct1, ct2, rlk, prod)
+    got = np.empty((2, L - 1, n), dtype=np.uint64)
+    capi.check(lib.he_memcpy_d2h(got.ctypes.data, bres.at((B - 1) * 2 * (L - 1) * n), got.nbytes, None))
+    err = float(np.max(np.abs(np.array(enc.decode(ctx, sk.decrypt(ctx, prod))) - x * y)))
+    return {"workload": "BASELINE.json configs[0]: HMult+relinearize+rescale, N=2^14, 4 limbs of 50 bits + 1 special prime",
+            "single_stream": {"ms_per_step": single, "ops_per_s": 1e3 / single},
+            "batch": {"ms_per_step": batch, "ops_per_s": 1e3 / batch, "ops_per_call": B},
+            "batch_equals_single": bool((got == prod.to_numpy()).all()), "decrypt_max_abs_err_vs_xy": err}
+
+
 def krum_cpu_evaluate(updates, pairs_sampled=2):
     """The evaluate phase of the Krum round on the CPU checker: per pair sub, square and add over the chunks,
     relinearise, rescale, and the slot sum as 15 rotations (each a key switch) + additions, with Lancelot's
@@ -462,6 +508,7 @@ def main():
                              "value path (%s): " % path, B if path == "batch" else 1),
         "single_stream_roofline": roofline(single_ms, "single", "one operation after the other on one stream: ", 1),
         "ntt": ntt, "rotate": rotate,
+        "config_c1": gpu_c1(capi, cahel, timer),
     }
     if not args.no_krum:
         line["krum"] = krum_round(with_cpu=not args.no_cpu_baseline)
