@@ -1102,7 +1102,7 @@ int he_hoisted_rotations_batch(const he_context *ctx, uint32_t L, uint32_t items
         const uint32_t count = n_steps - first < per_launch ? n_steps - first : per_launch;
         HE_HIP(launch_hoist_inner(ctx->tables(), w.y, ct_in, evk + (size_t)first * lv->beta, galois_elts + first, count,
                                   w.cx, ct_out, L, ctx->size_p, ctx->size_q, lv->beta, first != 0, add_input != 0, items,
-                                  2 * (size_t)L * n, S(s)));
+                                  2 * (size_t)L * n, S(s), ctx->use_fp ? ctx->d_fp_consts : nullptr, ctx->fp_mask));
     }
     // out0 = [c0 +] sum sigma(c0) + ModDown(cx0), out1 = [c1 +] ModDown(cx1)
     return moddown_impl(ctx, L, w.cx, ct_out, 2 * items, add_input ? 0xffffffffu : 0x55555555u, w.tmp, s);

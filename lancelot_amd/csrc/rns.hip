@@ -432,6 +432,10 @@ struct HoistArgs {
     int accumulate, with_self;
     uint32_t items;
     size_t ct_item_stride;          // words between the ciphertexts of consecutive items (blockIdx.z), in and out
+    const double *fp_consts;        // [tables][4] of the FP64 back end
+    uint64_t fp_mask;               // bit t: the products of table t (a prime below 2^50) are formed in FP64
+    uint32_t rows, groups;          // grid: N / 256 blocks x rows x groups of items, as one dimension
+    int xcd_map;                    // workgroup order that keeps the sharers of a key block on one XCD
 };
 
 // Hoisted rotations in one launch: grid (N / 256, (L + K) + L [+ L], ceil(items / I)); a thread serves the same
@@ -450,20 +454,38 @@ template <int I, bool LOCAL>
 __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     __shared__ uint64_t ybuf[LOCAL ? kHoistLocalTiles * kThreads : 1];
     const uint32_t LK = p.L + p.K;
-    const uint32_t j = blockIdx.x * kThreads + threadIdx.x;
-    const uint32_t item0 = blockIdx.z * I;
+    // Workgroup -> (block of 256 coefficients bx, row by, group of items bz).  The workgroups that share key words
+    // (same block and row, every group) get linear ids 8 apart and consecutive in that sequence: the hardware deals
+    // consecutive ids round-robin to the 8 XCDs, so they run on one XCD at about the same time and all but the first
+    // find the keys in that XCD's L2 (p.xcd_map; otherwise the plain order).
+    uint32_t bx, by, bz;
+    {
+        const uint32_t nb = (1u << p.log_n) / kThreads, id = blockIdx.x;
+        if (p.xcd_map) {
+            const uint32_t s = id >> 3, pair = (s / p.groups) * 8 + (id & 7);
+            bz = s % p.groups;
+            bx = pair % nb;
+            by = pair / nb;
+        } else {
+            bx = id % nb;
+            by = (id / nb) % p.rows;
+            bz = id / (nb * p.rows);
+        }
+    }
+    const uint32_t j = bx * kThreads + threadIdx.x;
+    const uint32_t item0 = bz * I;
     const uint32_t count = p.items - item0 < (uint32_t)I ? p.items - item0 : (uint32_t)I;
     // (the argument struct stays untouched: a modified copy would move its tables to scratch memory)
-    if (blockIdx.y >= LK) {
+    if (by >= LK) {
         for (uint32_t it = 0; it < count; it++) {
             const uint64_t *c0 = p.c0 + (item0 + it) * p.ct_item_stride;
             uint64_t *c0_out = p.c0_out + (item0 + it) * p.ct_item_stride;
-            const size_t o = ((size_t)(blockIdx.y - LK) << p.log_n) + j;
-            if (blockIdx.y >= LK + p.L) {
+            const size_t o = ((size_t)(by - LK) << p.log_n) + j;
+            if (by >= LK + p.L) {
                 if (!p.accumulate) c0_out[o] = c0[o];
                 continue;
             }
-            const uint32_t t = blockIdx.y - LK;
+            const uint32_t t = by - LK;
             const uint64_t q = p.moduli[t];
             const uint64_t *in = c0 + ((size_t)t << p.log_n);
             uint64_t acc = p.accumulate ? c0_out[o] : (p.with_self ? in[j] : 0);
@@ -472,16 +494,13 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
         }
         return;
     }
-    const uint32_t t = blockIdx.y;
+    const uint32_t t = by;
     const size_t y_item = (size_t)p.beta * LK << p.log_n;
     const uint64_t *y = p.y + item0 * y_item + ((size_t)t << p.log_n);
     const uint32_t table = t < p.L ? t : p.size_q + (t - p.L);
     const size_t key_off = ((size_t)table << p.log_n) + j;
     const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
     const size_t digit = (size_t)LK << p.log_n;
-    Lazy3 s0[I], s1[I], h0[I], h1[I];
-#pragma unroll
-    for (int it = 0; it < I; it++) s0[it] = s1[it] = h0[it] = h1[it] = Lazy3{0, 0, 0};
     if (LOCAL) {
         for (uint32_t d = 0; d < p.beta; d++)
 #pragma unroll
@@ -505,6 +524,55 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     };
     uint64_t k0, k1, v[I];
     fetch(0, k0, k1, v);
+    const size_t o = ((size_t)t << p.log_n) + j;
+    const size_t opoly = (size_t)LK << p.log_n;
+    if (table < 64 && ((p.fp_mask >> table) & 1)) {
+        // a prime below 2^50: exact FP64 products (6 full-rate instructions instead of 4 quarter-rate multiply-adds),
+        // each below 0.875 q in magnitude, eight of them between two reductions
+        const FpMod m{p.fp_consts[4 * table], p.fp_consts[4 * table + 1]};
+        double f0[I], f1[I];
+#pragma unroll
+        for (int it = 0; it < I; it++) f0[it] = f1[it] = 0.0;
+        for (uint32_t e = 0; e < n_terms; e++) {
+            uint64_t nk0, nk1, nv[I];
+            fetch(e + 1 < n_terms ? e + 1 : e, nk0, nk1, nv);
+            const double w0 = fp_from_u64(k0), w1 = fp_from_u64(k1);
+            const FpTw t0{w0, w0 * m.qinv}, t1{w1, w1 * m.qinv};
+#pragma unroll
+            for (int it = 0; it < I; it++) {
+                const double x = fp_from_u64(v[it]);
+                f0[it] += fp_mulmod(x, t0, m);
+                f1[it] += fp_mulmod(x, t1, m);
+            }
+            if ((e & 7) == 7) {
+#pragma unroll
+                for (int it = 0; it < I; it++) {
+                    f0[it] = fp_reduce(f0[it], m);
+                    f1[it] = fp_reduce(f1[it], m);
+                }
+            }
+            k0 = nk0;
+            k1 = nk1;
+#pragma unroll
+            for (int it = 0; it < I; it++) v[it] = nv[it];
+        }
+#pragma unroll
+        for (int it = 0; it < I; it++) {
+            if ((uint32_t)it >= count) break;
+            uint64_t *out = p.out + (item0 + it) * ((size_t)2 * LK << p.log_n);
+            double o0 = f0[it], o1 = f1[it];
+            if (p.accumulate) {
+                o0 += fp_from_u64(out[o]);
+                o1 += fp_from_u64(out[o + opoly]);
+            }
+            out[o] = fp_to_u64(fp_canonical(o0, m));
+            out[o + opoly] = fp_to_u64(fp_canonical(o1, m));
+        }
+        return;
+    }
+    Lazy3 s0[I], s1[I], h0[I], h1[I];
+#pragma unroll
+    for (int it = 0; it < I; it++) s0[it] = s1[it] = h0[it] = h1[it] = Lazy3{0, 0, 0};
     for (uint32_t e = 0; e < n_terms; e++) {
         uint64_t nk0, nk1, nv[I];
         fetch(e + 1 < n_terms ? e + 1 : e, nk0, nk1, nv);
@@ -526,8 +594,6 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
         for (int it = 0; it < I; it++) v[it] = nv[it];
     }
     const uint64_t q = p.moduli[table], r0 = p.barrett[2 * table], r1 = p.barrett[2 * table + 1];
-    const size_t o = ((size_t)t << p.log_n) + j;
-    const size_t opoly = (size_t)LK << p.log_n;
 #pragma unroll
     for (int it = 0; it < I; it++) {
         if ((uint32_t)it >= count) break;
@@ -869,7 +935,7 @@ hipError_t launch_inner_product_fp(const Tables &t, const double *fp_consts, con
 hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
                               const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
                               uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, bool with_self, uint32_t items,
-                              size_t ct_item_stride, hipStream_t s) {
+                              size_t ct_item_stride, hipStream_t s, const double *fp_consts, uint64_t fp_mask) {
     if (n_steps == 0 || n_steps * beta > (uint32_t)kMaxDigits || items == 0 || items > 65535) return hipErrorInvalidValue;
     HoistArgs p;
     memset(&p, 0, sizeof(p));
@@ -891,18 +957,31 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
     p.with_self = with_self ? 1 : 0;
     p.ct_item_stride = ct_item_stride;
     p.items = items;
+    p.fp_consts = fp_consts;
+    p.fp_mask = fp_consts ? fp_mask : 0;
     const uint32_t rows = (L + K) + (with_self ? 2 : 1) * L;
-    auto grid = [&](uint32_t per) { return dim3((1u << t.log_n) / kThreads, rows, (items + per - 1) / per); };
+    const uint32_t nb = (1u << t.log_n) / kThreads;
+    p.rows = rows;
     // every automorphism of the launch stays inside the aligned 256-word blocks of the NTT order
     bool local = t.log_n >= 8 && beta * 4 <= (uint32_t)kHoistLocalTiles;
     for (uint32_t i = 0; i < n_steps && local; i++) local = t.log_n < 9 || ((elts[i] - 1) & ((1u << (t.log_n - 7)) - 1)) == 0;
     static const bool no_local = [] { const char *e = getenv("CAHEL_HIP_NO_LOCAL_HOIST"); return e && e[0] == '1'; }();
+    static const bool no_xcd = [] { const char *e = getenv("CAHEL_HIP_NO_XCD_MAP"); return e && e[0] == '1'; }();
     if (no_local) local = false;
+    const bool p_xcd_ok = !no_xcd && (nb * rows) % 8 == 0;
+    auto launch = [&](auto kernel, uint32_t per) {
+        p.groups = (items + per - 1) / per;
+        p.xcd_map = p_xcd_ok && p.groups > 1;
+        hipLaunchKernelGGL(kernel, dim3(nb * rows * p.groups), dim3(kThreads), 0, s, p);
+    };
 #define HE_HOIST(I) \
-    if (local) hipLaunchKernelGGL((hoist_inner_kernel<I, true>), grid(I), dim3(kThreads), 0, s, p); \
-    else hipLaunchKernelGGL((hoist_inner_kernel<I, false>), grid(I), dim3(kThreads), 0, s, p)
-    // (8 items per thread halve the key traffic again but need 220 registers, 2 waves per SIMD: measured 20 % slower)
-    if (items >= 4) {
+    if (local) launch(hoist_inner_kernel<I, true>, I); \
+    else launch(hoist_inner_kernel<I, false>, I)
+    // (more items per thread read the keys less often but need more registers: 5, 6 and 8 items at 3, 2 and 2 waves per
+    // SIMD measured 6 %, 5 to 20 % and 20 % slower than 4 items at 4 waves)
+    // With the keys shared through L2, gathers from memory are served better by twice the waves (2 items per thread:
+    // 452 against 498 us for 15 steps of 45 items at N = 2^16); the block-local form keeps 4 (389 against 500 us).
+    if (items >= 4 && (local || !p_xcd_ok)) {
         HE_HOIST(4);
     } else if (items >= 2) {
         HE_HOIST(2);
