@@ -94,6 +94,7 @@ struct he_context {
     bool fuse_rows = true;       // environment CAHEL_HIP_NO_FUSED_BCONV=1: conversion kernel, then the rows pass
     bool fuse_tensor = true;     // environment CAHEL_HIP_NO_FUSED_TENSOR=1: he_multiply_relin_rescale as tensor kernel + key switch
     bool single_limb_digits = false;  // K = 1 (environment CAHEL_HIP_NO_REDUCE_IN_NTT=1: keep the conversion kernels)
+    bool batch_fused_inner = true;  // environment CAHEL_HIP_NO_BATCH_FUSED_KS=1: a batch's inner product as a kernel of its own
     bool fp_inner = true;        // environment CAHEL_HIP_NO_FP_INNER=1: a batch's inner product on the integer kernel
     uint32_t *d_rot_group = nullptr;     // encoder: 5^j mod 2N
     double2 *d_ksi = nullptr;            // encoder: e^{2 pi i k / 2N}, k <= 2N
@@ -409,6 +410,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->fuse_tensor = !(nt && nt[0] == '1');
         const char *nr = getenv("CAHEL_HIP_NO_REDUCE_IN_NTT");
         ctx->single_limb_digits = ctx->size_p == 1 && !(nr && nr[0] == '1');
+        const char *nbf = getenv("CAHEL_HIP_NO_BATCH_FUSED_KS");
+        ctx->batch_fused_inner = !(nbf && nbf[0] == '1');
         const char *ni = getenv("CAHEL_HIP_NO_FP_INNER");
         ctx->fp_inner = !(ni && ni[0] == '1');
         ctx->fp_ok.assign(qp, 0);
@@ -967,7 +970,8 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
     const KsWorkspace w = ks_workspace(ctx, lv, L, items, ws);
     uint64_t *y = w.y, *cx = w.cx, *tmp = w.tmp;
     const uint64_t *src = c;
-    const bool fused_inner = items == 1 && ctx->fuse_inner && lv->batched && fp_for_level(ctx, L);
+    const bool fused_inner = ctx->fuse_inner && lv->batched && fp_for_level(ctx, L) &&
+                             (items == 1 || (ctx->batch_fused_inner && !tin));
     if (galois_elt && !fused_inner) {
         // sigma(c) is staged in the second half of the ModDown workspace, which ModUp leaves alone and ModDown
         // only touches after the inner product has read it (the fused path gathers sigma(c) where it reads c)
@@ -978,17 +982,19 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
     if (fused_inner) {
         // ModUp without the copy of a digit's own limbs, then the forward NTT fused with the inner product: the
         // transformed digits are never written (216 limb transfers less at L = 24, K = 8)
+        // (a batch: the items are the polynomials of the inverse transform and the items of everything after it)
         NttArgs inv = base_args(ctx, false);
         inv.in = src;
         inv.out = tmp;
-        inv.in_poly_stride = inv.out_poly_stride = L;
+        inv.in_poly_stride = items == 1 ? L : c_item_stride;
+        inv.out_poly_stride = L;
         inv.map = plain_map(L, 0);
         inv.epi_mode = NTT_EPI_MUL;
         inv.w = lv->d_part_hat_inv;
         inv.in_galois = galois_elt;
         // tin: c is the third polynomial of a tensor product that has not been formed yet; the blocks pass forms it
         if (tin) HE_HIP(launch_tensor_intt_blocks(inv, *tin, S(s)));
-        HE_HIP(launch_ntt_inverse(inv, 1, NTT_BACKEND_FP, S(s), tin != nullptr));
+        HE_HIP(launch_ntt_inverse(inv, items, NTT_BACKEND_FP, S(s), tin != nullptr));
         NttArgs fwd = base_args(ctx, true);
         fwd.in = y;
         fwd.out = y;
@@ -996,14 +1002,17 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         fwd.n_jobs = lv->n_modup_jobs;
         fwd.groups = lv->d_modup_groups;
         fwd.n_groups = lv->n_modup_groups;
+        fwd.items = items;
+        fwd.item_stride = (size_t)lv->beta * (L + ctx->size_p) * n;
         const bool rows_done = fuse_rows_ok(ctx, lv, L);
         if (rows_done) {
             BconvRows b{tmp, y, nullptr, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                        lv->beta, lv->modup_max_rows, 0, 1, 0, 0, 0, 0};
+                        lv->beta, lv->modup_max_rows, 0, items, (size_t)L * n, fwd.item_stride, 0, 0};
             HE_HIP(launch_bconv_rows(fwd, b, S(s)));
         } else {
             BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                         lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts, 1, 0, 0, 0};
+                         lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts, items, (size_t)L * n,
+                         fwd.item_stride, 0};
             HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
         }
         KsFuseArgs x;
@@ -1024,6 +1033,9 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         x.beta = lv->beta;
         x.fold_ct = fold_ct;
         x.fold_w = fold_w;
+        x.items = items;
+        x.own_item_stride = (size_t)c_item_stride * n;
+        x.fold_item_stride = 2 * (size_t)L * n;
         HE_HIP(launch_ntt_forward_inner(fwd, x, S(s), rows_done));
     } else {
         // a batch on the FP64 back end shares each key word among the items of a group and reads a digit's own limbs

@@ -273,6 +273,12 @@ struct KsFuseArgs {
     // transforms back to coefficients); fold_ct = nullptr leaves the inner product as it is
     const uint64_t *fold_ct;  // [2][L][N]
     const uint64_t *fold_w;   // Shoup pair of P^-1 mod q_{L-1}
+    // items > 1: that many inputs in one launch (no Galois element, no add_c0); item i's own limbs, output and fold_ct
+    // lie i * own_item_stride, i * 2 (L+K) N and i * fold_item_stride words further on, its lazy digits
+    // i * NttArgs::item_stride.  The workgroups of one (limb, tile) for all items are placed on one XCD next to each
+    // other, so that the key tile is read from memory by the first and from that XCD's L2 by the others.
+    uint32_t items;
+    size_t own_item_stride, fold_item_stride;
 };
 hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s, bool rows_done = false);
 

@@ -982,14 +982,33 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
     const uint32_t lr = a.log_n - 8;
     const uint32_t log_b = 31 - __builtin_clz(tile_elems >> 8);
     const uint32_t tiles_per_limb = 1u << (lr - log_b);
-    const uint32_t lb = logical_block();
-    const uint32_t t = lb / tiles_per_limb, tile = lb % tiles_per_limb;
+    const uint32_t LK = x.L + x.K;
     const size_t n = (size_t)1 << a.log_n;
+    uint32_t lb, item = 0;
+    if (x.items > 1) {
+        // hardware id -> XCD id & 7; inside an XCD the items of one (limb, tile) are consecutive
+        const uint32_t pairs = LK * tiles_per_limb, id = blockIdx.x;
+        if (pairs % 8 == 0) {
+            const uint32_t s = id >> 3;
+            item = s % x.items;
+            lb = (s / x.items) * 8 + (id & 7);
+        } else {
+            item = id / pairs;
+            lb = id - item * pairs;
+        }
+    } else {
+        lb = logical_block();
+    }
+    const uint32_t t = lb / tiles_per_limb, tile = lb % tiles_per_limb;
     const size_t off = (size_t)tile * tile_elems;
     const uint32_t blk0 = tile << log_b;
-    const uint32_t LK = x.L + x.K;
     const uint32_t table = t < x.L ? t : x.size_q + (t - x.L);
     const uint32_t own = t < x.L ? t / x.K : 0xffffffffu;
+    // (locals: a modified copy of the argument structs would move their pointer tables to scratch memory)
+    const uint64_t *own_base = x.own + item * x.own_item_stride;
+    const uint64_t *lazy_base = a.out + item * a.item_stride;
+    uint64_t *out_base = x.out + item * (2 * (size_t)LK * n);
+    const uint64_t *fold_base = x.fold_ct ? x.fold_ct + item * x.fold_item_stride : nullptr;
     double *ld = reinterpret_cast<double *>(lds);
     const FpCtx fc = fp_ctx(a, table);
     const FpMod m = fc.m;
@@ -1002,7 +1021,7 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
     const size_t key_off = ((size_t)role * x.size_qp + table) * n + off;
     double acc[kPer];
     if (own != 0xffffffffu) {
-        const uint64_t *src = x.own + (size_t)t * n;
+        const uint64_t *src = own_base + (size_t)t * n;
         const uint64_t *key = x.evk.p[own] + key_off;
 #pragma unroll
         for (int i = 0; i < kPer; i++) {
@@ -1026,7 +1045,7 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
         if (!role && a.rows_direct) {
             // the 16 words of the first register block (stride 16 inside a 256-block) straight from global memory:
             // 16 neighbouring threads read one 128-byte line per access
-            const uint64_t *src = a.out + ((size_t)d * LK + t) * n + off;  // lazy values left by the rows pass
+            const uint64_t *src = lazy_base + ((size_t)d * LK + t) * n + off;  // lazy values left by the rows pass
             double v[16];
 #pragma unroll
             for (int j = 0; j < 16; j++) v[j] = __longlong_as_double((long long)src[base0 + (j << 4)]);
@@ -1035,7 +1054,7 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
             for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
         } else if (!a.rows_direct) {
             if (!role) {
-                const uint64_t *src = a.out + ((size_t)d * LK + t) * n + off;
+                const uint64_t *src = lazy_base + ((size_t)d * LK + t) * n + off;
 #pragma unroll
                 for (int i = 0; i < kPer; i++) lds[skew(tid + i * half)] = src[tid + i * half];
             }
@@ -1083,9 +1102,9 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
             acc[i] += fp_mulmod(fp_from_u64(c0[x.own_galois ? galois_index(e, x.own_galois, a.log_n) : e]), pw, m);
         }
     }
-    uint64_t *o = x.out + ((size_t)role * LK + t) * n + off;
-    if (x.fold_ct && t == x.L - 1) {
-        const uint64_t *cl = x.fold_ct + ((size_t)role * x.L + t) * n + off;
+    uint64_t *o = out_base + ((size_t)role * LK + t) * n + off;
+    if (fold_base && t == x.L - 1) {
+        const uint64_t *cl = fold_base + ((size_t)role * x.L + t) * n + off;
         const double wd = fp_from_u64(x.fold_w[0]);
         const FpTw w{wd, wd * m.qinv};
 #pragma unroll
@@ -1398,13 +1417,16 @@ hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, h
 
 hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s, bool rows_done) {
     if (a.log_n < 9 || a.log_n > 16 || !a.jobs) return hipErrorInvalidValue;
+    const uint32_t items = x.items ? x.items : 1;
+    if (items > 1 && (x.own_galois || x.add_c0 || (a.items ? a.items : 1) != items)) return hipErrorInvalidValue;
     if (a.n_jobs && !rows_done) {
-        hipError_t e = launch_rows<true, NTT_BACKEND_FP>(a, a.n_jobs, s);
+        hipError_t e = launch_rows<true, NTT_BACKEND_FP>(a, a.n_jobs * items, s);
         if (e != hipSuccess) return e;
     }
     const uint32_t n = 1u << a.log_n;
     const uint32_t tile = n < 2048 ? n : 2048;
-    const dim3 grid((x.L + x.K) * (n / tile));
+    if ((uint64_t)(x.L + x.K) * (n / tile) * items > 0x7fffffffu) return hipErrorInvalidValue;
+    const dim3 grid((x.L + x.K) * (n / tile) * items);
     if (tile == 2048)
         hipLaunchKernelGGL(ntt_blocks_fp_inner_kernel<128>, grid, dim3(256), 0, s, a, x);
     else if (tile == 1024)
