@@ -52,10 +52,11 @@ PROFILE = {"single": {"traffic_limbs": 1128.5, "valu_wave_instr": 35.89e6,
                       "kernels": "tensor_intt_blocks_fp, ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp_inner, "
                                  "ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp with the rescale "
                                  "epilogue"},
-           "batch": {"traffic_limbs": 1066.6, "valu_wave_instr": 35.2e6,
+           "batch": {"traffic_limbs": 894.8, "valu_wave_instr": 35.7e6,
                      "kernels": "per call of 8 operations: tensor_fp, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, "
-                                "ntt_blocks_fp, inner_product_fp, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, "
-                                "ntt_blocks_fp with the rescale epilogue"}}
+                                "ntt_blocks_fp_inner (items of a tile on one XCD, key tile shared through L2), "
+                                "ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp with the rescale "
+                                "epilogue"}}
 
 
 def sync(capi):
@@ -393,6 +394,25 @@ def main():
     calls = max(1, -(-K_steps // B))
     batch_ms = timer.time(batch_call, calls, max(1, W // B)) / B
 
+    # (3b) the same batch calls dealt to two streams (each with its own operands, workspace and output): the tail of
+    # one call's kernels overlaps the head of the other's
+    batch_lanes = []
+    for k in range(min(2, args.lanes)):
+        la, lb = Buf(capi, B * 2 * L * n), Buf(capi, B * 2 * L * n)
+        capi.check(lib.he_memcpy_d2d(la.ptr, ba.ptr, 8 * B * 2 * L * n, None))
+        capi.check(lib.he_memcpy_d2d(lb.ptr, bb.ptr, 8 * B * 2 * L * n, None))
+        batch_lanes.append((lane_streams[k], la, lb, Buf(capi, B * 2 * (L - 1) * n),
+                            Buf(capi, lib.he_multiply_relin_rescale_batch_workspace_words(h, L, B))))
+
+    def batch_lane_call(i):
+        st, la, lb, lres, lws = batch_lanes[i % len(batch_lanes)]
+        capi.check(lib.he_multiply_relin_rescale_batch(h, L, B, la.ptr, lb.ptr, evk, lres.ptr, lws.ptr, st))
+
+    for i in range(2 * len(batch_lanes)):
+        batch_lane_call(i)
+    bs_ms, bs_blocks = timed_wall(batch_lane_call, max(2 * len(batch_lanes), calls))
+    bs_ms /= B
+
     # (4) the reference's own call sequence through pyCAHEL on the null stream
     prod = cahel.ciphertext(ctx)
 
@@ -408,7 +428,9 @@ def main():
     want = prod.to_numpy()
     got = np.empty((2, L - 1, n), dtype=np.uint64)
     same = True
-    for buf in [res] + [lres for _, lres in lane_bufs] + [type("B", (), {"ptr": bres.at(k * 2 * (L - 1) * n)}) for k in (0, B - 1)]:
+    views = [type("B", (), {"ptr": bres.at(k * 2 * (L - 1) * n)}) for k in (0, B - 1)]
+    views += [type("B", (), {"ptr": lane[3].at((B - 1) * 2 * (L - 1) * n)}) for lane in batch_lanes]
+    for buf in [res] + [lres for _, lres in lane_bufs] + views:
         capi.check(lib.he_memcpy_d2h(got.ctypes.data, buf.ptr, got.nbytes, None))
         same = same and bool((got == want).all())
     fused = cahel.ciphertext(ctx)
@@ -480,7 +502,7 @@ def main():
                          "fp64_issue_peak_lane_ops_per_s": rate.value, "issue_bound_ms": issue_ms,
                          "frac_of_issue_bound": issue_ms / ms_per_op}}
 
-    best_ms, path = min((streams_ms, "streams"), (batch_ms, "batch"))
+    best_ms, path = min((streams_ms, "streams"), (batch_ms, "batch"), (bs_ms, "batch_streams"))
     line = {
         "metric": "HMult+relin+rescale ops/s at N=2^16, L=24 (dnum=3, 8 special primes)",
         "value": 1e3 / best_ms, "unit": "ops/s", "n_gpus": 1, "steps": K_steps, "warmup": W,
@@ -491,8 +513,9 @@ def main():
         "timing": "median of %d blocks of %d steps each" % (BLOCKS, K_steps),
         "config": {"workload": "HMult+relinearize+rescale, N=2^16, L=24 limbs of 50 bits, K=8, dnum=3, scale 2^40, "
                                "two fresh ciphertexts of 32768 uniform[-1,1] slots (BASELINE.json configs[2]); "
-                               "independent operations, the better of %d streams and batches of %d per call"
-                               % (args.lanes, B),
+                               "independent operations, the best of %d streams of single calls, batches of %d per "
+                               "call on one stream, and such batches dealt to %d streams"
+                               % (args.lanes, B, len(batch_lanes)),
                    "value_path": path, "lanes": args.lanes, "batch": B},
         "hmult_frac_of_hbm_roofline": frac(best_ms),
         "hmult_algorithmic_bytes": alg_bytes,
@@ -500,12 +523,14 @@ def main():
                     "blocks_ms": streams_blocks},
         "batch": {"ms_per_step": batch_ms, "ops_per_s": 1e3 / batch_ms, "frac_of_hbm_roofline": frac(batch_ms),
                   "ops_per_call": B},
+        "batch_streams": {"ms_per_step": bs_ms, "ops_per_s": 1e3 / bs_ms, "frac_of_hbm_roofline": frac(bs_ms),
+                          "ops_per_call": B, "streams": len(batch_lanes), "blocks_ms": [b / B for b in bs_blocks]},
         "single_stream": {"ms_per_step": single_ms, "ops_per_s": 1e3 / single_ms, "frac_of_hbm_roofline": frac(single_ms)},
         "api_path": {"calls": "pyCAHEL multiply, relinearize_inplace, rescale_to_next_inplace on the null stream",
                      "ms_per_step": api_ms, "ops_per_s": 1e3 / api_ms, "frac_of_hbm_roofline": frac(api_ms)},
         "check": {"all_paths_equal_the_evaluator": same, "decrypt_max_abs_err_vs_xy": max_err},
-        "roofline": roofline(best_ms, "batch" if path == "batch" else "single",
-                             "value path (%s): " % path, B if path == "batch" else 1),
+        "roofline": roofline(best_ms, "single" if path == "streams" else "batch",
+                             "value path (%s): " % path, 1 if path == "streams" else B),
         "single_stream_roofline": roofline(single_ms, "single", "one operation after the other on one stream: ", 1),
         "ntt": ntt, "rotate": rotate,
         "config_c1": gpu_c1(capi, cahel, timer),
