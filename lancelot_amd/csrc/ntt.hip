@@ -974,8 +974,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 // The key tiles are fetched before the butterflies start, so that they travel meanwhile; the digit that owns
 // limb t contributes the input itself.
 template <uint32_t T>
-__global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, KsFuseArgs x) {
-    __shared__ uint64_t lds[16 * T + T];
+__global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(2))) void ntt_blocks_fp_inner_kernel(NttArgs a, KsFuseArgs x) {
+    constexpr uint32_t kInnerTile = 16 * T + T;   // words of one skewed tile
+    __shared__ uint64_t lds[2 * kInnerTile];
     constexpr uint32_t half = T, tile_elems = half << 4;
     const uint32_t role = threadIdx.x >= half ? 1u : 0u;       // which key polynomial this thread accumulates
     const uint32_t tid = threadIdx.x - role * half;
@@ -1035,61 +1036,87 @@ __global__ __launch_bounds__(2 * T) void ntt_blocks_fp_inner_kernel(NttArgs a, K
         for (int i = 0; i < kPer; i++) acc[i] = 0.0;
     }
 
+    // The other digits two at a time: the threads of role 0 transform the first one's tile, those of role 1 the
+    // second one's (each into its own LDS tile, the same sequence of steps at the same time), then every thread
+    // multiplies both tiles by its key polynomial.  With the transforms on one role only, half of the workgroup's
+    // waves (and the SIMDs they sit on) would idle during the butterflies.
     uint32_t terms = 1;
-    for (uint32_t d = 0; d < x.beta; d++) {
-        if (d == own) continue;
-        const uint64_t *key = x.evk.p[d] + key_off;
-        uint64_t pk[kPer];
+    auto skip_own = [&](uint32_t d) { return d == own ? d + 1 : d; };
+    for (uint32_t da = skip_own(0); da < x.beta;) {
+        const uint32_t db = skip_own(da + 1);
+        const bool two = db < x.beta;
+        const uint32_t mine = role ? db : da;
+        const bool work = role ? two : true;
+        // key words of the first digit are requested before the butterflies, those of the second after them (they
+        // arrive while the first tile is multiplied): both sets up front would not fit the register file
+        uint64_t pka[kPer], pkb[kPer];
+        const uint64_t *ka = x.evk.p[da] + key_off, *kb = x.evk.p[two ? db : da] + key_off;
 #pragma unroll
-        for (int i = 0; i < kPer; i++) pk[i] = key[tid + i * half];
-        if (!role && a.rows_direct) {
+        for (int i = 0; i < kPer; i++) pka[i] = ka[tid + i * half];
+        double *ldm = ld + role * kInnerTile;
+        uint64_t *ldsm = lds + role * kInnerTile;
+        const uint64_t *src = lazy_base + ((size_t)mine * LK + t) * n + off;  // lazy values left by the rows pass
+        if (work && a.rows_direct) {
             // the 16 words of the first register block (stride 16 inside a 256-block) straight from global memory:
             // 16 neighbouring threads read one 128-byte line per access
-            const uint64_t *src = lazy_base + ((size_t)d * LK + t) * n + off;  // lazy values left by the rows pass
             double v[16];
 #pragma unroll
             for (int j = 0; j < 16; j++) v[j] = __longlong_as_double((long long)src[base0 + (j << 4)]);
             fp_ct_block<4, true>(v, fc.tw, idx0, m);
 #pragma unroll
-            for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
+            for (int j = 0; j < 16; j++) ldm[skew(base0 + (j << 4))] = v[j];
         } else if (!a.rows_direct) {
-            if (!role) {
-                const uint64_t *src = lazy_base + ((size_t)d * LK + t) * n + off;
+            if (work) {
 #pragma unroll
-                for (int i = 0; i < kPer; i++) lds[skew(tid + i * half)] = src[tid + i * half];
+                for (int i = 0; i < kPer; i++) ldsm[skew(tid + i * half)] = src[tid + i * half];
             }
             lds_barrier();
-            if (!role) {
+            if (work) {
                 double v[16];
 #pragma unroll
-                for (int j = 0; j < 16; j++) v[j] = ld[skew(base0 + (j << 4))];
+                for (int j = 0; j < 16; j++) v[j] = ldm[skew(base0 + (j << 4))];
                 fp_ct_block<4, true>(v, fc.tw, idx0, m);
 #pragma unroll
-                for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
+                for (int j = 0; j < 16; j++) ldm[skew(base0 + (j << 4))] = v[j];
             }
         }
         lds_barrier();
-        if (!role) {
+        if (work) {
             double v[16];
 #pragma unroll
-            for (int j = 0; j < 16; j++) v[j] = ld[skew(base1 + j)];
+            for (int j = 0; j < 16; j++) v[j] = ldm[skew(base1 + j)];
             fp_ct_block<4, true>(v, fc.tw, idx1, m);
 #pragma unroll
-            for (int j = 0; j < 16; j++) ld[skew(base1 + j)] = v[j];
+            for (int j = 0; j < 16; j++) ldm[skew(base1 + j)] = v[j];
         }
+#pragma unroll
+        for (int i = 0; i < kPer; i++) pkb[i] = kb[tid + i * half];
         lds_barrier();
         // every term is below 0.7 q, so eight of them fit between two reductions of the accumulators
 #pragma unroll
         for (int i = 0; i < kPer; i++) {
             const double y = fp_reduce(ld[skew(tid + i * half)], m);
-            const double w = fp_from_u64(pk[i]);
+            const double w = fp_from_u64(pka[i]);
             acc[i] += fp_mulmod(y, FpTw{w, w * m.qinv}, m);
         }
         if ((++terms & 7) == 0) {
 #pragma unroll
             for (int i = 0; i < kPer; i++) acc[i] = fp_reduce(acc[i], m);
         }
-        lds_barrier();  // every read of this tile is done before the next one overwrites it
+        if (two) {
+#pragma unroll
+            for (int i = 0; i < kPer; i++) {
+                const double y = fp_reduce(ld[kInnerTile + skew(tid + i * half)], m);
+                const double w = fp_from_u64(pkb[i]);
+                acc[i] += fp_mulmod(y, FpTw{w, w * m.qinv}, m);
+            }
+            if ((++terms & 7) == 0) {
+#pragma unroll
+                for (int i = 0; i < kPer; i++) acc[i] = fp_reduce(acc[i], m);
+            }
+        }
+        lds_barrier();  // every read of these tiles is done before the next pair overwrites them
+        da = skip_own(db + 1);
     }
     if (x.add_c0 && !role && t < x.L) {
         // a rotation: polynomial 0 gains P sigma(c0), which ModDown's division by P turns into sigma(c0)
