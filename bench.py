@@ -48,7 +48,7 @@ BLOCKS = 5
 # `--only batch`), per operation: L2-miss traffic in limbs of 8 N bytes (FETCH_SIZE scaled by 2, WRITE_SIZE by 1: the
 # factors a copy of known size gives) and SQ_INSTS_VALU summed over the kernels.  Constants of the profile, not
 # measured in this run.
-PROFILE = {"single": {"traffic_limbs": 1128.5, "valu_wave_instr": 35.89e6,
+PROFILE = {"single": {"traffic_limbs": 1122.3, "valu_wave_instr": 35.96e6,
                       "kernels": "tensor_intt_blocks_fp, ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp_inner, "
                                  "ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp with the rescale "
                                  "epilogue"},
