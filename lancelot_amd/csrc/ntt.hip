@@ -998,7 +998,9 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(2))) void
             lb = id - item * pairs;
         }
     } else {
-        lb = logical_block();
+        // plain order, last limb first: the special limbs have one digit more to transform than the others, so their
+        // workgroups start first and are spread over all XCDs (a tile's twiddles are its own: nothing to share)
+        lb = gridDim.x - 1 - blockIdx.x;
     }
     const uint32_t t = lb / tiles_per_limb, tile = lb % tiles_per_limb;
     const size_t off = (size_t)tile * tile_elems;
