@@ -1,10 +1,12 @@
 """Full-size configurations on the GPU.
 
-C1 (N = 2^14, 4 + 1 primes of 50 bits) is small enough for the CPU oracle: HMult + relinearise + rescale is compared
-limb for limb.  At the benchmark sizes (N = 2^16, L = 24, K = 8 and Lancelot's [60, 40, 40, 60] chain) the oracle
-would take minutes, so the checks are properties that do not depend on the size: commutativity of the product
-(bit-exact), decryption of a size-3 ciphertext against its relinearisation, rotation = roll of the slots,
-rotate-and-sum = sum of all slots, and the encrypted Krum distances against the float64 closed form.
+C1 (N = 2^14, 4 + 1 primes of 50 bits): HMult + relinearise + rescale through pyCAHEL is compared with the oracle limb
+for limb, keys and ciphertexts included.  At the benchmark shape (N = 2^16, L = 24, K = 8) the C-ABI entry points
+that `bench.py` times (one product per call, a batch, a rotation) are compared with the oracle limb for limb on
+random residues; the scheme-level checks there and on Lancelot's [60, 40, 40, 60] chain are properties that do not
+depend on the size: commutativity of the product (bit-exact), decryption of a size-3 ciphertext against its
+relinearisation, rotation = roll of the slots, rotate-and-sum = sum of all slots, and the encrypted Krum distances
+against the float64 closed form.
 """
 import numpy as np
 import pytest
@@ -63,6 +65,50 @@ def test_c1_hmult_relin_rescale_bit_exact(oracle):
     assert (pt.to_numpy() == ks.decrypt(want, O.gauss_cdt())).all()
     got = np.array(enc.decode(ctx, pt))
     assert np.max(np.abs(got - x * y)) < 1e-2           # scale 2^40 after a 50-bit rescale: about 2^30 left
+
+
+@pytest.mark.parametrize("inner", ["fused", "fp_kernel"])
+def test_c2_benchmark_shape_entry_points_bit_exact(oracle, monkeypatch, inner):
+    """N = 2^16, L = 24, K = 8 (dnum = 3), 50-bit primes, random residues: he_multiply_relin_rescale, its batch form
+    (3 products; with the inner product inside the blocks pass and as the FP64 kernel of its own) and he_rotate
+    against the oracle's tensor / relinearise / rescale and apply_galois, every limb."""
+    from gpu_util import DeviceArray, make_pair, rand_limbs
+    from lancelot_amd import capi
+    monkeypatch.setenv("CAHEL_HIP_NO_BATCH_FUSED_KS", "0" if inner == "fused" else "1")
+    cahel, parms, ctx, p = make_pair(oracle, 16, [50] * 32, 8)
+    lib, h = capi.lib(), ctx.he_handle()
+    rng = np.random.default_rng(4242)
+    n, L, K = p.n, 24, 8
+    host_evk = [rand_limbs(p, rng, range(L + K), n_polys=2) for _ in range(L // K)]
+    dev_evk = [DeviceArray(capi, host=k) for k in host_evk]
+    ptrs = capi.evk_array([d.ptr for d in dev_evk])
+    items = 3
+    a = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
+    b = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
+    want = [p.rescale(p.relinearize(p.tensor(a[k], b[k]), host_evk)) for k in range(items)]
+    da, db = DeviceArray(capi, host=a), DeviceArray(capi, host=b)
+    # one product per call (items 0 and 2, the second a square)
+    ws = DeviceArray(capi, shape=(lib.he_multiply_relin_rescale_workspace_words(h, L),))
+    out = DeviceArray(capi, shape=(2, L - 1, n))
+    capi.check(lib.he_multiply_relin_rescale(h, L, da.ptr, db.ptr, ptrs, out.ptr, ws.ptr, None))
+    assert (out.numpy() == want[0]).all()
+    last = da.ptr + 8 * (items - 1) * 2 * L * n
+    capi.check(lib.he_multiply_relin_rescale(h, L, last, last, ptrs, out.ptr, ws.ptr, None))
+    assert (out.numpy() == p.rescale(p.relinearize(p.tensor(a[items - 1], a[items - 1]), host_evk))).all()
+    # the batch
+    bws = DeviceArray(capi, shape=(lib.he_multiply_relin_rescale_batch_workspace_words(h, L, items),))
+    bout = DeviceArray(capi, shape=(items, 2, L - 1, n))
+    capi.check(lib.he_multiply_relin_rescale_batch(h, L, items, da.ptr, db.ptr, ptrs, bout.ptr, bws.ptr, None))
+    got = bout.numpy()
+    for k in range(items):
+        assert (got[k] == want[k]).all(), k
+    # a rotation (the key plays the Galois key of the element)
+    elt = pow(5, 7, 2 * n)
+    rws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    rout = DeviceArray(capi, shape=(2, L, n))
+    capi.check(lib.he_rotate(h, L, da.ptr, ptrs, rout.ptr, elt, rws.ptr, None))
+    assert (rout.numpy() == p.apply_galois(a[0], elt, host_evk)).all()
+    assert (da.numpy() == a).all() and (db.numpy() == b).all()
 
 
 @pytest.fixture(scope="module")
