@@ -294,7 +294,12 @@ def main():
     parms.set_coeff_modulus(cahel.coeff_modulus_create(n, [BITS] * (SIZE_Q + SIZE_P)))
     parms.set_special_modulus_size(SIZE_P)
     steps_pow2 = [1 << k for k in range(15)]
-    parms.set_galois_elts(cahel.get_elts_from_steps(steps_pow2 if args.only in ("all", "rotate") else [1], n))
+    # the same slot sum as four hoisted rounds (`hoisting` of the reference's API): steps 1..7, then 8, 128 and 2048
+    # times 1..15
+    hoist_rounds = [[m * k for k in range(1, r)] for m, r in ((1, 8), (8, 16), (128, 16), (2048, 16))]
+    all_steps = sorted(set(steps_pow2) | {s for rnd in hoist_rounds for s in rnd})
+    parms.set_galois_elts(cahel.get_elts_from_steps(all_steps if args.only == "all" else
+                                                    (steps_pow2 if args.only == "rotate" else [1]), n))
     ctx = cahel.context(parms, True, cahel.sec_level_type.tc128)
     ctx.set_seed(2025)
     sk = cahel.secret_key(parms)
@@ -470,11 +475,22 @@ def main():
 
     ras_ms = timer.time(rotate_and_sum, 5, warmup=1)
     total = np.array(enc.decode(ctx, sk.decrypt(ctx, rotate_and_sum())))
+
+    def hoisted_sum():
+        acc = ct1.copy()
+        for steps in hoist_rounds:
+            cahel.add_inplace(ctx, acc, cahel.hoisting(ctx, acc, glk, steps))
+        return acc
+
+    hs_ms = timer.time(hoisted_sum, 5, warmup=1)
+    total_h = np.array(enc.decode(ctx, sk.decrypt(ctx, hoisted_sum())))
     rotate = {"one_rotation_ms": rot_ms, "rotate_and_sum_15_ms": ras_ms,
               "one_rotation_GBps": 288 * limb_bytes / (rot_ms * 1e-3) / 1e9,
               "one_rotation_frac_of_hbm_roofline": 288 * limb_bytes / (rot_ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
               "rotate_and_sum_GBps": 15 * 432 * limb_bytes / (ras_ms * 1e-3) / 1e9,
-              "slot_sum_rel_err": float(np.max(np.abs(total - x.sum())) / abs(x.sum()))}
+              "slot_sum_rel_err": float(np.max(np.abs(total - x.sum())) / abs(x.sum())),
+              "slot_sum_4_hoisted_rounds_ms": hs_ms,
+              "slot_sum_hoisted_rel_err": float(np.max(np.abs(total_h - x.sum())) / abs(x.sum()))}
 
     alg_bytes = 334 * limb_bytes
 
