@@ -105,6 +105,8 @@ struct he_context {
     bool fuse_inner = true;      // environment CAHEL_HIP_NO_FUSED_KS=1: separate NTT and inner-product kernels
     uint64_t fp_mask = 0;        // bit t: table t has a prime below 2^50
     bool mixed_ok = false;       // mixed launches allowed (at most 64 tables; CAHEL_HIP_NO_MIXED=1 switches them off)
+    int one_pass = 1;            // environment CAHEL_HIP_NO_ONE_PASS=1: plain transforms at N <= 2^14 as rows pass + blocks pass;
+                                 // CAHEL_HIP_FORCE_ONE_PASS=1: the whole-limb kernel also where two launches are faster
     int rows_direct = 1;         // environment CAHEL_HIP_ROWS_VIA_LDS=1: every register block of the rows pass (and of the
                                  // fused inner-product kernel) takes its operands from LDS
     std::vector<Level> levels;   // indexed by L
@@ -157,6 +159,7 @@ NttArgs base_args(const he_context *ctx, bool forward) {
     a.epi_b_mask = 0xffffffffu;
     a.fp_mask = ctx->fp_mask;
     a.rows_direct = ctx->rows_direct;
+    a.one_pass = ctx->one_pass;
     return a;
 }
 
@@ -404,6 +407,8 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->mixed_ok = qp <= 64 && !(nx && nx[0] == '1');
         const char *rv = getenv("CAHEL_HIP_ROWS_VIA_LDS");
         ctx->rows_direct = !(rv && rv[0] == '1');
+        const char *no1 = getenv("CAHEL_HIP_NO_ONE_PASS"), *f1 = getenv("CAHEL_HIP_FORCE_ONE_PASS");
+        ctx->one_pass = (no1 && no1[0] == '1') ? 0 : ((f1 && f1[0] == '1') ? 2 : 1);
         const char *nb = getenv("CAHEL_HIP_NO_FUSED_BCONV");
         ctx->fuse_rows = !(nb && nb[0] == '1');
         const char *nt = getenv("CAHEL_HIP_NO_FUSED_TENSOR");

@@ -69,6 +69,7 @@ struct NttArgs {
     const double *tw_fp;      // [tables][N] twiddles as exact doubles for the FP64 back end (primes below 2^50)
     const double *fp_consts;  // [tables][4]: q, 1/q, N^-1 mod q, (N^-1 mod q)/q
     uint64_t fp_mask;         // bit t: table t has a prime below 2^50 (read by the mixed back end only)
+    int one_pass;             // N <= 2^14, FP64 back end, plain transforms: one kernel with the limb resident in LDS
     int rows_direct;          // N = 2^16: rows pass with its outer half-pass on registers (one LDS exchange); fused
                               // inner-product kernel: first register block straight from global memory
     const uint64_t *moduli;   // [tables]

@@ -506,6 +506,130 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------------
+// Whole-limb transform for N <= 2^14 (FP64 back end, plain forward / inverse with the optional inverse scaling):
+// one workgroup of N / 16 threads per limb keeps the limb in LDS (at most 136 KiB of the CU's 160) between its
+// register blocks, so the limb crosses memory once in each direction instead of twice, in one launch instead of two.
+// Forward: the first block (stages 0..3, words t + j N/16) comes straight from the coalesced load; the blocks after
+// it exchange through LDS (skewed by a word per 16); the last block's results return to LDS for a coalesced store of
+// canonical residues.  Inverse: the mirror image, the last block (words t + j N/16) is scaled and stored from
+// registers.  LOGN = 4 NB4 + REM: NB4 blocks of four stages and one of REM stages at the fine end.
+// ---------------------------------------------------------------------------------------------------
+template <int LOGN, bool FWD>
+__global__ __launch_bounds__((1 << LOGN) / 16) void ntt_limb_fp_kernel(NttArgs a) {
+    constexpr uint32_t N = 1u << LOGN, T = N / 16;
+    constexpr int NB4 = LOGN / 4, REM = LOGN % 4, PER = 16 >> REM;
+    static_assert(LOGN >= 9 && LOGN <= 14, "a limb of at most 2^14 words");
+    __shared__ double ld[N + N / 16];
+    const Job job = decode_job(a, blockIdx.x);
+    const FpCtx c = fp_ctx(a, job.table);
+    const FpMod m = c.m;
+    const uint32_t t = threadIdx.x;
+    double v[16];
+    // block k (stages 4k .. 4k+3) of thread t: words base + (j << low), twiddle index (1 << 4k) + upper
+    auto geom = [&](int k, uint32_t &base, uint32_t &low, uint32_t &idx) {
+        low = (uint32_t)(LOGN - 4 * (k + 1));
+        const uint32_t upper = t >> low;
+        base = (upper << (low + 4)) | (t & ((1u << low) - 1));
+        idx = (1u << (4 * k)) + upper;
+    };
+    if (FWD) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[j] = fp_from_u64(job.in[t + T * j]);
+        fp_ct_block<4, false>(v, c.tw, 1u, m);
+#pragma unroll
+        for (int j = 0; j < 16; j++) ld[skew(t + T * j)] = v[j];
+        lds_barrier();
+#pragma unroll
+        for (int k = 1; k < NB4; k++) {
+            uint32_t base, low, idx;
+            geom(k, base, low, idx);
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[skew(base + ((uint32_t)j << low))];
+            fp_ct_block<4, true>(v, c.tw, idx, m);
+#pragma unroll
+            for (int j = 0; j < 16; j++) ld[skew(base + ((uint32_t)j << low))] = v[j];
+            lds_barrier();
+        }
+        if constexpr (REM > 0) {
+#pragma unroll
+            for (int gi = 0; gi < PER; gi++) {
+                const uint32_t g = t * PER + gi, base = g << REM;
+                double w[1 << REM];
+#pragma unroll
+                for (int j = 0; j < (1 << REM); j++) w[j] = ld[skew(base + j)];
+                fp_ct_block<(REM > 0 ? REM : 1), true>(w, c.tw, (1u << (4 * NB4)) + g, m);
+#pragma unroll
+                for (int j = 0; j < (1 << REM); j++) ld[skew(base + j)] = w[j];
+            }
+            lds_barrier();
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) job.out[t + T * j] = fp_to_u64(fp_canonical(ld[skew(t + T * j)], m));
+    } else {
+#pragma unroll
+        for (int j = 0; j < 16; j++) ld[skew(t + T * j)] = fp_from_u64(job.in[t + T * j]);
+        lds_barrier();
+        if constexpr (REM > 0) {
+#pragma unroll
+            for (int gi = 0; gi < PER; gi++) {
+                const uint32_t g = t * PER + gi, base = g << REM;
+                double w[1 << REM];
+#pragma unroll
+                for (int j = 0; j < (1 << REM); j++) w[j] = ld[skew(base + j)];
+                fp_gs_block<(REM > 0 ? REM : 1), false>(w, c.tw, (1u << (4 * NB4)) + g, m);
+#pragma unroll
+                for (int j = 0; j < (1 << REM); j++) ld[skew(base + j)] = w[j];
+            }
+            lds_barrier();
+        }
+#pragma unroll
+        for (int k = NB4 - 1; k >= 0; k--) {
+            uint32_t base, low, idx;
+            geom(k, base, low, idx);
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = ld[skew(base + ((uint32_t)j << low))];
+            if (REM == 0 && k == NB4 - 1)
+                fp_gs_block<4, false>(v, c.tw, idx, m);   // canonical inputs
+            else
+                fp_gs_block<4, true>(v, c.tw, idx, m);
+            if (k > 0) {
+#pragma unroll
+                for (int j = 0; j < 16; j++) ld[skew(base + ((uint32_t)j << low))] = v[j];
+                lds_barrier();
+            }
+        }
+        // block 0: base = t, low = log2(T): the coalesced store pattern
+        const FpTw scale = inverse_scale(a, job, m);
+#pragma unroll
+        for (int j = 0; j < 16; j++) job.out[t + T * j] = fp_to_u64(fp_canonical(fp_mulmod(v[j], scale, m), m));
+    }
+}
+
+template <bool FWD>
+hipError_t launch_limb_fp(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
+    switch (a.log_n) {
+#define HE_CASE(LOGN) \
+    case LOGN: hipLaunchKernelGGL((ntt_limb_fp_kernel<LOGN, FWD>), dim3(n_jobs), dim3((1u << LOGN) / 16), 0, s, a); break;
+        HE_CASE(9) HE_CASE(10) HE_CASE(11) HE_CASE(12) HE_CASE(13) HE_CASE(14)
+#undef HE_CASE
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// The launches that the whole-limb kernel covers and wins.  A limb is one workgroup on one CU: up to N = 2^12 that is
+// faster than two launches whatever the number of limbs (10-12 us against 15-16 us for a forward + inverse pair);
+// a limb of 2^13 or 2^14 words takes one CU 9 or 17 us, so there the kernel pays only when the launch has enough limbs
+// to occupy the chip (measured break-even: 64 and 192 limbs; at 256 limbs 23 against 34 us and 50 against 60 us).
+// a.one_pass = 2 forces it (tests).
+inline bool one_pass_ok(const NttArgs &a, int backend, bool forward, uint32_t n_jobs) {
+    if (!a.one_pass || backend != NTT_BACKEND_FP || a.log_n > 14 || a.jobs || a.pro_mode != NTT_PLAIN || a.in_galois ||
+        !(a.epi_mode == NTT_PLAIN || (!forward && a.epi_mode == NTT_EPI_MUL)))
+        return false;
+    return a.one_pass == 2 || a.log_n <= 12 || n_jobs >= (a.log_n == 13 ? 64u : 192u);
+}
+
+// ---------------------------------------------------------------------------------------------------
 // Base conversion fused with the rows pass of the forward transform that follows it (FP64 back end, N >= 2^12).
 //
 // Both operate on the same set of coefficients: a tile of all 2^LD rows x C columns of the limb's (N / 256) x 256
@@ -1434,6 +1558,7 @@ hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, h
     if (a.log_n < 9 || a.log_n > 16 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
+    if (!rows_done && one_pass_ok(a, backend, true, n_jobs)) return launch_limb_fp<true>(a, n_jobs, s);
     hipError_t e = rows_done                    ? hipSuccess
                    : backend == NTT_BACKEND_MIXED ? launch_rows<true, NTT_BACKEND_MIXED>(a, n_jobs, s)
                    : backend                    ? launch_rows<true, NTT_BACKEND_FP>(a, n_jobs, s)
@@ -1481,6 +1606,7 @@ hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, h
     if (a.log_n < 9 || a.log_n > 16 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
+    if (!blocks_done && one_pass_ok(a, backend, false, n_jobs)) return launch_limb_fp<false>(a, n_jobs, s);
     hipError_t e = blocks_done                    ? hipSuccess
                    : backend == NTT_BACKEND_MIXED ? launch_blocks<false, NTT_BACKEND_MIXED>(a, n_polys, s)
                    : backend                    ? launch_blocks<false, NTT_BACKEND_FP>(a, n_polys, s)

@@ -49,9 +49,17 @@ def test_tables_match_oracle(small):
 
 # [60, 50, 35, 59]: a prime above 2^50 keeps the launch on the integer back end; [50, 49, 35, 50]: all below
 # 2^50, the FP64 back end
+@pytest.mark.parametrize("one_pass", ["default", "off", "forced"])
 @pytest.mark.parametrize("bits", [[60, 50, 35, 59], [50, 49, 35, 50]])
 @pytest.mark.parametrize("logn", [9, 10, 11, 12, 13, 14, 15, 16])
-def test_ntt_all_sizes(oracle, capi, logn, bits):
+def test_ntt_all_sizes(oracle, capi, monkeypatch, logn, bits, one_pass):
+    """Forward and inverse against the oracle at every degree; up to N = 2^14 with all primes below 2^50 the plain
+    transform can be one kernel with the limb resident in LDS (by default where it is the faster form: N <= 2^12, or
+    many limbs), and is rows pass + blocks pass otherwise."""
+    if one_pass != "default" and (logn > 14 or bits[0] == 60):
+        pytest.skip("the switches only change N <= 2^14 on the FP64 back end")
+    monkeypatch.setenv("CAHEL_HIP_NO_ONE_PASS", "1" if one_pass == "off" else "0")
+    monkeypatch.setenv("CAHEL_HIP_FORCE_ONE_PASS", "1" if one_pass == "forced" else "0")
     cahel, parms, ctx, p = make_pair(oracle, logn, bits, 1)
     rng = np.random.default_rng(logn)
     h = ctx.he_handle()
