@@ -1112,14 +1112,16 @@ int he_hoisted_rotations_batch(const he_context *ctx, uint32_t L, uint32_t items
     }
     const size_t n = ctx->n();
     const KsWorkspace w = ks_workspace(ctx, lv, L, items, ws);
-    if (int rc = modup_impl(ctx, L, ct_in + (size_t)L * n, 2 * L, items, w.y, w.tmp, s)) return rc;
+    // (the digits' own limbs are not copied into y: the kernel reads them from c1 where they are)
+    const bool skip_own = lv->batched;
+    if (int rc = modup_impl(ctx, L, ct_in + (size_t)L * n, 2 * L, items, w.y, w.tmp, s, skip_own)) return rc;
     // as many steps per launch as the 128-bit accumulator and the pointer table allow
     const uint32_t per_launch = (uint32_t)kMaxDigits / lv->beta;
     for (uint32_t first = 0; first < n_steps; first += per_launch) {
         const uint32_t count = n_steps - first < per_launch ? n_steps - first : per_launch;
         HE_HIP(launch_hoist_inner(ctx->tables(), w.y, ct_in, evk + (size_t)first * lv->beta, galois_elts + first, count,
                                   w.cx, ct_out, L, ctx->size_p, ctx->size_q, lv->beta, first != 0, add_input != 0, items,
-                                  2 * (size_t)L * n, S(s), ctx->use_fp ? ctx->d_fp_consts : nullptr, ctx->fp_mask));
+                                  2 * (size_t)L * n, S(s), ctx->use_fp ? ctx->d_fp_consts : nullptr, ctx->fp_mask, skip_own));
     }
     // out0 = [c0 +] sum sigma(c0) + ModDown(cx0), out1 = [c1 +] ModDown(cx1)
     return moddown_impl(ctx, L, w.cx, ct_out, 2 * items, add_input ? 0xffffffffu : 0x55555555u, w.tmp, s);

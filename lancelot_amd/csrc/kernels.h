@@ -249,11 +249,13 @@ hipError_t launch_inner_product_fp(const Tables &t, const double *fp_consts, con
 // of the L limbs after c0 (c1), so that ModDown can add onto the input ciphertext.  items: that many inputs,
 // y and out dense, the ciphertexts ct_item_stride words apart.  evk: n_steps * beta HOST-side device pointers, step-major; n_steps * beta <=
 // kMaxDigits per launch.  fp_consts / fp_mask: rows whose table has its bit set (a prime below 2^50) form their
-// products in exact FP64 arithmetic; the results are the same canonical residues.
+// products in exact FP64 arithmetic; the results are the same canonical residues.  own_from_ct: y holds no copy of the
+// digits' own limbs (ModUp skipped it); they are read from c1 of the input ciphertext, which follows c0's L limbs.
 hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
                               const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
                               uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, bool with_self, uint32_t items,
-                              size_t ct_item_stride, hipStream_t s, const double *fp_consts = nullptr, uint64_t fp_mask = 0);
+                              size_t ct_item_stride, hipStream_t s, const double *fp_consts = nullptr, uint64_t fp_mask = 0,
+                              bool own_from_ct = false);
 
 // Forward NTT of ModUp's converted limbs fused with the key-switch inner product (FP64 back end only).
 // `a` describes the converted limbs as launch_ntt_forward's job list does (a.out = the beta x (L+K) x N digit

@@ -434,6 +434,7 @@ struct HoistArgs {
     size_t ct_item_stride;          // words between the ciphertexts of consecutive items (blockIdx.z), in and out
     const double *fp_consts;        // [tables][4] of the FP64 back end
     uint64_t fp_mask;               // bit t: the products of table t (a prime below 2^50) are formed in FP64
+    int own_from_ct;                // a digit's own limbs are read from c1 of the input (c0 + L limbs), not from y
     uint32_t rows, groups;          // grid: N / 256 blocks x rows x groups of items, as one dimension
     int xcd_map;                    // workgroup order that keeps the sharers of a key block on one XCD
 };
@@ -501,11 +502,17 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     const size_t key_off = ((size_t)table << p.log_n) + j;
     const size_t key_poly = (size_t)(p.size_q + p.K) << p.log_n;
     const size_t digit = (size_t)LK << p.log_n;
+    // the digit that owns limb t: its "lifted" limb is the input's c1 itself
+    const uint32_t own = (p.own_from_ct && t < p.L) ? t / p.K : 0xffffffffu;
+    const uint64_t *c1 = p.c0 + item0 * p.ct_item_stride + ((size_t)(p.L + t) << p.log_n);
+    auto word = [&](uint32_t d, int it, uint32_t at) {
+        return d == own ? c1[it * p.ct_item_stride + at] : y[it * y_item + d * digit + at];
+    };
     if (LOCAL) {
         for (uint32_t d = 0; d < p.beta; d++)
 #pragma unroll
             for (int it = 0; it < I; it++)
-                ybuf[(it * p.beta + d) * kThreads + threadIdx.x] = (uint32_t)it < count ? y[it * y_item + d * digit + j] : 0;
+                ybuf[(it * p.beta + d) * kThreads + threadIdx.x] = (uint32_t)it < count ? word(d, it, j) : 0;
         __syncthreads();
     }
     // term e = step e / beta, digit e mod beta; the operands of term e + 1 are requested before term e is
@@ -520,7 +527,7 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
 #pragma unroll
         for (int it = 0; it < I; it++)
             v[it] = LOCAL ? ybuf[(it * p.beta + d) * kThreads + (src & (kThreads - 1))]
-                          : ((uint32_t)it < count ? y[it * y_item + d * digit + src] : 0);
+                          : ((uint32_t)it < count ? word(d, it, src) : 0);
     };
     uint64_t k0, k1, v[I];
     fetch(0, k0, k1, v);
@@ -935,7 +942,8 @@ hipError_t launch_inner_product_fp(const Tables &t, const double *fp_consts, con
 hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
                               const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
                               uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, bool with_self, uint32_t items,
-                              size_t ct_item_stride, hipStream_t s, const double *fp_consts, uint64_t fp_mask) {
+                              size_t ct_item_stride, hipStream_t s, const double *fp_consts, uint64_t fp_mask,
+                              bool own_from_ct) {
     if (n_steps == 0 || n_steps * beta > (uint32_t)kMaxDigits || items == 0 || items > 65535) return hipErrorInvalidValue;
     HoistArgs p;
     memset(&p, 0, sizeof(p));
@@ -959,6 +967,7 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
     p.items = items;
     p.fp_consts = fp_consts;
     p.fp_mask = fp_consts ? fp_mask : 0;
+    p.own_from_ct = own_from_ct ? 1 : 0;
     const uint32_t rows = (L + K) + (with_self ? 2 : 1) * L;
     const uint32_t nb = (1u << t.log_n) / kThreads;
     p.rows = rows;
