@@ -833,16 +833,39 @@ void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
         const uint32_t limb = __builtin_amdgcn_readfirstlane(mlimb[rl]);
         const double *tws = twl[r % 3];
         double *tile_ld = ld[WAVE_B ? (r & 1) : 0];
-        double v[P];
+        // sum_k x_k M_k as an exact pair (hi, lo) before any reduction, four operations per term instead of the seven of
+        // a modular product and an addition.  hi runs in [2^103, 2^104), where doubles are the multiples of 2^51: the
+        // fused multiply-add t = fl(x w + hi) rounds the exact sum to such a multiple (eight products below 2^100 keep
+        // it under 2^104), t - hi is exact, x w - (t - hi) is the rounding error, an integer of at most 2^50 in
+        // magnitude that the second fused multiply-add returns exactly, and eight of those sum exactly (<= 2^53).
+        // The value is (hi - 2^103) + lo; it is reduced once per output word.
+        double hi[P], lo[P];
 #pragma unroll
-        for (int i = 0; i < P; i++) v[i] = p.b.mdr ? fp_reduce(rr[i], mod) : 0.0;
-        // every product is reduced to |r| <= 0.75 m: the sums stay exact integers below 7 m < 2^53
+        for (int i = 0; i < P; i++) {
+            hi[i] = 0x1p103;
+            lo[i] = 0.0;
+        }
 #pragma unroll
         for (int k = 0; k < 8; k++) {
-            const bool on = (uint32_t)k < d.n_in;
-            const FpTw w{on ? uniform_f64(mrow[rl][2 * k]) : 0.0, on ? uniform_f64(mrow[rl][2 * k + 1]) : 0.0};
+            const double w = (uint32_t)k < d.n_in ? uniform_f64(mrow[rl][2 * k]) : 0.0;
 #pragma unroll
-            for (int i = 0; i < P; i++) v[i] += fp_mulmod(xv[k][i], w, mod);
+            for (int i = 0; i < P; i++) {
+                const double t = __builtin_fma(xv[k][i], w, hi[i]);
+                const double step = t - hi[i];
+                lo[i] += __builtin_fma(xv[k][i], w, -step);
+                hi[i] = t;
+            }
+        }
+        // (hi - 2^103) / 2^51 is an integer below 2^52; times c = 2^51 mod m it is congruent to the high part.  The
+        // modular product takes it as it is: for |x| < 2^52 the quotient estimate is off by at most 1.5 |x| 2^-52 + 1,
+        // so |x c - k m| <= 2.5 m < 2^53 and every step stays exact.  v <= 3.5 m; the first block reduces it.
+        const double c51 = fp_reduce(0x1p51, mod);
+        const FpTw w51{c51, c51 * mod.qinv};
+        double v[P];
+#pragma unroll
+        for (int i = 0; i < P; i++) {
+            v[i] = fp_mulmod((hi[i] - 0x1p103) * 0x1p-51, w51, mod) + fp_reduce(lo[i], mod);
+            if (p.b.mdr) v[i] += fp_reduce(rr[i], mod);
         }
         // the first log2(P) stages pair rows that differ in their top bits: this thread's own P words
         fp_ct_block<LOGP, true>(v, tws, 1u, mod);

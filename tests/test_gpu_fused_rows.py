@@ -54,6 +54,14 @@ def test_entry_points_with_fused_conversion(oracle, capi, monkeypatch, logn, bit
         ws = DeviceArray(capi, shape=(2 * L, n))
         capi.check(lib.he_modup(h, L, dc.ptr, dy.ptr, ws.ptr, None))
         assert (dy.numpy() == p.modup(c)).all(), ("modup", L)
+        # the largest and smallest sums of the conversion: every coefficient of every limb q - 1 (then 1) in
+        # coefficient form, which is what the conversion sees after the inverse transform
+        for fill in ("max", "one"):
+            coeff = np.stack([np.full(n, (p.moduli[t] - 1) if fill == "max" else 1, dtype=np.uint64) for t in range(L)])
+            cc = p.ntt_fwd(coeff.copy(), list(range(L)))
+            capi.check(lib.he_memcpy_h2d(dc.ptr, np.ascontiguousarray(cc).ctypes.data, cc.nbytes, None))
+            capi.check(lib.he_modup(h, L, dc.ptr, dy.ptr, ws.ptr, None))
+            assert (dy.numpy() == p.modup(cc)).all(), ("modup", fill, L)
         # ModDown of 1, 2, 3 and 6 polynomials, overwriting and adding
         for n_polys in (1, 2, 3, 6):
             cx = np.stack([rand_limbs(p, rng, tables) for _ in range(n_polys)])
