@@ -709,7 +709,9 @@ __device__ __forceinline__ double uniform_f64(double v) {
     return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
 }
 
-constexpr uint32_t kFuseMaxRows = 8;   // output limbs per workgroup, at most
+// output limbs per workgroup, at most.  The workgroup's first kFuseMaxRows * 18 threads fetch the rows' constants
+// (one word each), so the cap is tied to the smallest workgroup of the kernel (256 threads).
+constexpr uint32_t kFuseMaxRows = 12;
 
 // P = coefficients per thread.  8: 256 threads, two waves per SIMD.  (4, with 512 threads and four waves per SIMD,
 // compiles but measured 1.7 times slower at N = 2^16: the inputs' registers spill, and a tile needs twice the LDS
@@ -730,6 +732,7 @@ void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
     __shared__ double mrow[kFuseMaxRows][18];
     __shared__ uint32_t mlimb[kFuseMaxRows], mtable[kFuseMaxRows];
     static_assert(LD >= 4 && LD <= 8 && (P == 8 || P == 4), "N from 2^12 to 2^16");
+    static_assert(kFuseMaxRows * 18 <= kFuseWords / P, "one thread per constant of the group's rows");
     constexpr int LOGC = kFuseLog - LD, LOGP = P == 8 ? 3 : 2;
     constexpr uint32_t T = kFuseWords / P;
     constexpr uint32_t C = 1u << LOGC, tiles_per_limb = 256u >> LOGC, row_step = T >> LOGC;
@@ -1552,16 +1555,20 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
 
 hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s) {
     if (a.log_n < 12 || a.log_n > 16 || !b.mat_fp || b.n_units == 0) return hipErrorInvalidValue;
-    static const uint32_t target = [] {
+    // 0: by the number of items.  One operation needs the workgroups of 3 rows each to fill the chip; from 4 items on
+    // there are enough of them at 12 rows, and a workgroup's inputs and set-up serve four times as many rows
+    // (8 items at N = 2^16: 1.046 -> 1.012 ms per call; one item: 0.181 -> 0.193 ms at 8 rows).
+    static const uint32_t forced = [] {
         const char *e = getenv("CAHEL_HIP_FUSE_ROWS");
-        const int v = e ? atoi(e) : 3;
-        return (uint32_t)(v >= 1 && v <= (int)kFuseMaxRows ? v : 3);
+        const int v = e ? atoi(e) : 0;
+        return (uint32_t)(v >= 1 && v <= (int)kFuseMaxRows ? v : 0);
     }();
+    const uint32_t items = b.items ? b.items : 1;
+    const uint32_t target = forced ? forced : items >= 4 ? kFuseMaxRows : 3;
     const uint32_t rows = b.mdr ? b.max_rows - 1 : b.max_rows;
     if (rows == 0) return hipErrorInvalidValue;
     BconvRowsK p{b, (rows + target - 1) / target, 0, target};
     p.copy_groups = b.copy_base ? (b.max_copy + target - 1) / target : 0;
-    const uint32_t items = b.items ? b.items : 1;
     const int ld = (int)a.log_n - 8;
     const uint32_t tiles = 256u >> (kFuseLog - ld);
     const uint64_t wgs = (uint64_t)b.n_units * items * tiles * (p.compute_groups + p.copy_groups);
