@@ -270,15 +270,21 @@ __device__ __forceinline__ FpTw load_fptw(const double *table, size_t idx, FpMod
     return FpTw{w, w * m.qinv};
 }
 
-// Forward block on lazy signed doubles.  REDUCE_FIRST brings every input back to |v| <= q/2; from there
+// Forward block on lazy signed doubles.  REDUCE_FIRST = 1 brings every input back to |v| <= q/2; from there
 // (or from canonical inputs) the bound grows by 1.375 b + 0.5 per stage: 5.3 q after four stages, 7.1 q from
 // canonical inputs, always below 8 q < 2^53.
-template <int LOGR, bool REDUCE_FIRST>
+// REDUCE_FIRST = 2 reduces only the inputs that the first stage adds and subtracts; those that it multiplies go into
+// the modular product as they are (its result is at most (1/2 + 0.375 b) 2^50 for an input of b 2^50).  In units of
+// 2^50, for every q below 2^50: the first stage ends at 1 + 0.375 b and each later one at 1.375 b' + 0.5, which
+// is 5.92 after three stages from inputs of 4, 7.28 after three more, 5.63 after two more: for a chain of blocks of
+// at most 3, 3 and 2 stages whose first inputs are at most 4 x 2^50, and whose consumer reduces first.
+template <int LOGR, int REDUCE_FIRST>
 __device__ __forceinline__ void fp_ct_block(double *v, const double *table, uint32_t idx, FpMod m) {
     constexpr int R = 1 << LOGR;
+    static_assert(REDUCE_FIRST != 2 || LOGR <= 3, "bounds of the partial reduction are derived for blocks of at most 3 stages");
     if (REDUCE_FIRST) {
 #pragma unroll
-        for (int j = 0; j < R; j++) v[j] = fp_reduce(v[j], m);
+        for (int j = 0; j < (REDUCE_FIRST == 2 ? R / 2 : R); j++) v[j] = fp_reduce(v[j], m);
     }
 #pragma unroll
     for (int l = 0; l < LOGR; l++) {

@@ -677,7 +677,7 @@ __device__ __forceinline__ void fuse_block(double *ld, const double *twl, uint32
         double v[R];
 #pragma unroll
         for (int j = 0; j < R; j++) v[j] = ld[skew8(base + ((uint32_t)j << low_bits))];
-        fp_ct_block<LOGR, true>(v, twl, (1u << s0) + upper, m);
+        fp_ct_block<LOGR, 2>(v, twl, (1u << s0) + upper, m);
 #pragma unroll
         for (int j = 0; j < R; j++) {
             const uint32_t e = base + ((uint32_t)j << low_bits);
@@ -861,17 +861,19 @@ void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
         }
         // (hi - 2^103) / 2^51 is an integer below 2^52; times c = 2^51 mod m it is congruent to the high part.  The
         // modular product takes it as it is: for |x| < 2^52 the quotient estimate is off by at most 1.5 |x| 2^-52 + 1,
-        // so |x c - k m| <= 2.5 m < 2^53 and every step stays exact.  v <= 3.5 m; the first block reduces it.
+        // so |x c - k m| <= 2.5 m < 2^53 and every step stays exact.  With the rescale term (canonical for the dropped
+        // prime, below 2^50, added as it is) |v| <= 3 m + 2^50 <= 4 x 2^50: the bound that the register blocks of
+        // this pass start from (they reduce only what they do not multiply, see fp_ct_block).
         const double c51 = fp_reduce(0x1p51, mod);
         const FpTw w51{c51, c51 * mod.qinv};
         double v[P];
 #pragma unroll
         for (int i = 0; i < P; i++) {
             v[i] = fp_mulmod((hi[i] - 0x1p103) * 0x1p-51, w51, mod) + fp_reduce(lo[i], mod);
-            if (p.b.mdr) v[i] += fp_reduce(rr[i], mod);
+            if (p.b.mdr) v[i] += rr[i];
         }
         // the first log2(P) stages pair rows that differ in their top bits: this thread's own P words
-        fp_ct_block<LOGP, true>(v, tws, 1u, mod);
+        fp_ct_block<LOGP, 2>(v, tws, 1u, mod);
 #pragma unroll
         for (int i = 0; i < P; i++) tile_ld[skew8(e0 + T * i)] = v[i];
         uint64_t *dst = out + ((size_t)limb << a.log_n);
@@ -882,7 +884,7 @@ void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
             const uint32_t base = ((32 * u + wave) << LOGC) + col;
 #pragma unroll
             for (int j = 0; j < 8; j++) v[j] = tile_ld[skew8(base + ((uint32_t)(4 * j) << LOGC))];
-            fp_ct_block<3, true>(v, tws, 8u + u, mod);
+            fp_ct_block<3, 2>(v, tws, 8u + u, mod);
 #pragma unroll
             for (int j = 0; j < 8; j++) tile_ld[skew8(base + ((uint32_t)(4 * j) << LOGC))] = v[j];
             // the twiddles of the next limb become visible with the same barrier (their buffer was last read two
