@@ -273,6 +273,7 @@ def main():
                     help="streams that the timed operations are dealt to (three and the null stream fill the four "
                          "hardware queues of a process)")
     ap.add_argument("--batch", type=int, default=8, help="operations per he_multiply_relin_rescale_batch call")
+    ap.add_argument("--batch-streams", type=int, default=2, help="streams that the batch calls are dealt to")
     ap.add_argument("--no-krum", action="store_true", help="skip the encrypted Krum round (BASELINE.json configs[4])")
     ap.add_argument("--only", choices=["all", "step", "batch", "rotate", "ntt", "krum"], default="all",
                     help="step / rotate / ntt: run just that workload on the null stream (for rocprofv3)")
@@ -402,7 +403,7 @@ def main():
     # (3b) the same batch calls dealt to two streams (each with its own operands, workspace and output): the tail of
     # one call's kernels overlaps the head of the other's
     batch_lanes = []
-    for k in range(min(2, args.lanes)):
+    for k in range(min(args.batch_streams, len(lane_streams))):
         la, lb = Buf(capi, B * 2 * L * n), Buf(capi, B * 2 * L * n)
         capi.check(lib.he_memcpy_d2d(la.ptr, ba.ptr, 8 * B * 2 * L * n, None))
         capi.check(lib.he_memcpy_d2d(lb.ptr, bb.ptr, 8 * B * 2 * L * n, None))

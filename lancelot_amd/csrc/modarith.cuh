@@ -42,19 +42,18 @@ __device__ __forceinline__ uint64_t sub_mod(uint64_t a, uint64_t b, uint64_t q) 
 
 __device__ __forceinline__ uint64_t neg_mod(uint64_t a, uint64_t q) { return a ? q - a : 0; }
 
-// 128-bit value (hi:lo) mod q with ratio = floor(2^128 / q) = (r1:r0).
+// 128-bit value (hi:lo) mod q with ratio = floor(2^128 / q) = (r1:r0), q < 2^62.  r1 = floor(2^64 / q), so
+// w = 2^64 mod q = 2^64 - r1 q, and r0 = floor(2^128 / q) - r1 2^64 = floor(w 2^64 / q) is the Shoup quotient of w:
+// hi w - floor(hi r0 / 2^64) q lies in [0, 2q) for every hi below 2^64, and lo - floor(lo r1 / 2^64) q in [0, 2q).
+// Two high and three low 64-bit products (w comes from scalar operands) where the plain Barrett reduction of the
+// 128-bit value takes four and four.
 __device__ __forceinline__ uint64_t barrett128(uint64_t lo, uint64_t hi, uint64_t q, uint64_t r0, uint64_t r1) {
-    uint64_t carry = mulhi64(lo, r0);
-    uint64_t t_lo = lo * r1;
-    uint64_t t_hi = mulhi64(lo, r1);
-    uint64_t tmp = t_lo + carry;
-    uint64_t quo = t_hi + (tmp < t_lo);
-    uint64_t u_lo = hi * r0;
-    uint64_t u_hi = mulhi64(hi, r0);
-    uint64_t tmp2 = tmp + u_lo;
-    quo += u_hi + (tmp2 < tmp);
-    quo += hi * r1;
-    uint64_t r = lo - quo * q;
+    const uint64_t w = 0 - r1 * q;
+    const uint64_t a = hi * w - mulhi64(hi, r0) * q;
+    const uint64_t b = lo - mulhi64(lo, r1) * q;
+    const uint64_t q2 = q << 1;
+    uint64_t r = a + b;
+    r = r >= q2 ? r - q2 : r;
     return r >= q ? r - q : r;
 }
 
@@ -79,17 +78,19 @@ __device__ __forceinline__ void mac128(U128 &acc, uint64_t a, uint64_t b) {
     acc.hi += hi + (acc.lo < lo);
 }
 
-// Lazy sum of products of residues below 2^61 with few carries.  The factors are split at bit 31
-// (a = a1 2^31 + a0 with a0 < 2^31, a1 < 2^30); the four partial products of a term go, by weight, into three
-// 64-bit words (ll: a0 b0 < 2^62, mid: a1 b0 + a0 b1 < 2^62, hh: a1 b1 < 2^60), each a 32 x 32 + 64 multiply-add with
-// no carry out.  Four terms fit (4 * 2^62 = 2^64) before the words have to be relieved (spill3), so a product costs 4
-// multiply-adds and a few additions instead of a 64 x 64 -> 128 product (6 multiplies) and a carry chain; the
-// 32 x 32 multiplies issue at a quarter of the rate of other vector instructions and dominate either way.
-struct Split31 {
+// Lazy sum of products of residues below 2^61 with few carries.  The factors are split at bit 30
+// (a = a1 2^30 + a0 with a0 < 2^30, a1 < 2^31); the four partial products of a term go, by weight, into three
+// 64-bit words (ll: a0 b0 < 2^60, mid: a1 b0 + a0 b1 < 2^62, hh: a1 b1 < 2^62), each a 32 x 32 + 64 multiply-add with
+// no carry out.  Four terms fit (4 * 2^62 = 2^64) before the words have to be relieved (spill3), eight when the
+// residues are below 2^60 (a1 < 2^30: mid < 2^61, hh < 2^60), so a product costs 4 multiply-adds and a few
+// additions instead of a 64 x 64 -> 128 product (6 multiplies) and a carry chain.  (Measured on gfx950: every
+// 32-bit multiply, v_mad_u64_u32 included, issues at the rate of an FP64 fused multiply-add, half the rate of a
+// 32-bit addition.)
+struct Split30 {
     uint32_t lo, hi;
 };
 
-__device__ __forceinline__ Split31 split31(uint64_t a) { return Split31{(uint32_t)a & 0x7fffffffu, (uint32_t)(a >> 31)}; }
+__device__ __forceinline__ Split30 split30(uint64_t a) { return Split30{(uint32_t)a & 0x3fffffffu, (uint32_t)(a >> 30)}; }
 
 struct Lazy3 {
     uint64_t ll, mid, hh;
@@ -99,7 +100,7 @@ struct Lazy3 {
 // v_mad_u64_u32 (32 x 32 + 64 -> 64; the carry out goes to a scalar pair that nobody reads, the sums stay below
 // 2^64).  Written out because the compiler emits a multiply with a zero addend followed by a 64-bit add for
 // `acc += (uint64_t)a * b`, and one statement because it separates inline-assembly statements by s_nop.
-__device__ __forceinline__ void mac3x2(Lazy3 &s, Lazy3 &t, Split31 a, Split31 b, Split31 c) {
+__device__ __forceinline__ void mac3x2(Lazy3 &s, Lazy3 &t, Split30 a, Split30 b, Split30 c) {
     uint64_t carry;
     asm("v_mad_u64_u32 %0, %6, %7, %9, %0\n\t"
         "v_mad_u64_u32 %1, %6, %8, %9, %1\n\t"
@@ -113,8 +114,8 @@ __device__ __forceinline__ void mac3x2(Lazy3 &s, Lazy3 &t, Split31 a, Split31 b,
         : "v"(a.lo), "v"(a.hi), "v"(b.lo), "v"(b.hi), "v"(c.lo), "v"(c.hi));
 }
 
-// After four terms the upper halves of the three words move into three counters of weight 2^32 (two additions and
-// a move per word: no carries between the words), which leaves room for four more terms; total3 puts the six words
+// The upper halves of the three words move into three counters of weight 2^32 (two additions and a move per word:
+// no carries between the words), which leaves room for the next four (eight) terms; total3 puts the six words
 // together at the end.  Up to 64 terms (the counters stay below 2^37).
 __device__ __forceinline__ void spill3(Lazy3 &h, Lazy3 &s) {
     h.ll += s.ll >> 32;
@@ -127,8 +128,8 @@ __device__ __forceinline__ void spill3(Lazy3 &h, Lazy3 &s) {
 
 __device__ __forceinline__ U128 total3(const Lazy3 &h, const Lazy3 &s) {
     typedef unsigned __int128 u128;
-    const u128 t = ((u128)s.ll + ((u128)h.ll << 32)) + (((u128)s.mid + ((u128)h.mid << 32)) << 31) +
-                   (((u128)s.hh + ((u128)h.hh << 32)) << 62);
+    const u128 t = ((u128)s.ll + ((u128)h.ll << 32)) + (((u128)s.mid + ((u128)h.mid << 32)) << 30) +
+                   (((u128)s.hh + ((u128)h.hh << 32)) << 60);
     return U128{(uint64_t)t, (uint64_t)(t >> 64)};
 }
 

@@ -442,8 +442,8 @@ struct HoistArgs {
 // Hoisted rotations in one launch: grid (N / 256, (L + K) + L [+ L], ceil(items / I)); a thread serves the same
 // coefficient of I consecutive items, so that a key word is loaded once for all of them.
 // rows t < L + K:  out[p][t] = sum_s sum_d sigma_s(y_d)[t] * evk_{s,d}[p][t]  (n_steps * beta <= 64 products, summed
-//                  lazily as split 31-bit partial products, see Lazy3, and reduced once); the automorphism is the
-//                  gather index of the load of y.  The kernel is bound by its 32 x 32 multiplies (quarter rate).
+//                  lazily as partial products of factors split at bit 30, see Lazy3, and reduced once); the automorphism is the
+//                  gather index of the load of y.  The kernel is bound by instruction issue (its multiply-adds).
 // rows L + K + t:  c0_out[t] = sum_s sigma_s(c0)[t]  (+ c0[t] with_self)
 // rows L + K + L + t (with_self only): c1 is copied to the output, so that the ModDown that follows adds onto
 //                  the input ciphertext: ct_out = ct_in + sum_s rot_s(ct_in)
@@ -478,21 +478,36 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     const uint32_t count = p.items - item0 < (uint32_t)I ? p.items - item0 : (uint32_t)I;
     // (the argument struct stays untouched: a modified copy would move its tables to scratch memory)
     if (by >= LK) {
-        for (uint32_t it = 0; it < count; it++) {
-            const uint64_t *c0 = p.c0 + (item0 + it) * p.ct_item_stride;
-            uint64_t *c0_out = p.c0_out + (item0 + it) * p.ct_item_stride;
-            const size_t o = ((size_t)(by - LK) << p.log_n) + j;
-            if (by >= LK + p.L) {
-                if (!p.accumulate) c0_out[o] = c0[o];
-                continue;
-            }
-            const uint32_t t = by - LK;
-            const uint64_t q = p.moduli[t];
-            const uint64_t *in = c0 + ((size_t)t << p.log_n);
-            uint64_t acc = p.accumulate ? c0_out[o] : (p.with_self ? in[j] : 0);
-            for (uint32_t s = 0; s < p.n_steps; s++) acc = add_mod(acc, in[galois_index(j, p.elts[s], p.log_n)], q);
-            c0_out[o] = acc;
+        const size_t o = ((size_t)(by - LK) << p.log_n) + j;
+        if (by >= LK + p.L) {
+            if (!p.accumulate)
+                for (uint32_t it = 0; it < count; it++)
+                    p.c0_out[(item0 + it) * p.ct_item_stride + o] = p.c0[(item0 + it) * p.ct_item_stride + o];
+            return;
         }
+        // the gathers of a step are independent of the running sums: one index per step for all items, and the
+        // loads of several steps in flight (a loop of one dependent load after the other ran longer than the rows
+        // that multiply)
+        const uint32_t t = by - LK;
+        const uint64_t q = p.moduli[t];
+        const uint64_t *in = p.c0 + item0 * p.ct_item_stride + ((size_t)t << p.log_n);
+        uint64_t *c0_out = p.c0_out + item0 * p.ct_item_stride + o;
+        uint64_t acc[I];
+#pragma unroll
+        for (int it = 0; it < I; it++)
+            acc[it] = (uint32_t)it >= count ? 0 : p.accumulate ? c0_out[it * p.ct_item_stride] : p.with_self ? in[it * p.ct_item_stride + j] : 0;
+#pragma unroll 4
+        for (uint32_t s = 0; s < p.n_steps; s++) {
+            const uint32_t g = galois_index(j, p.elts[s], p.log_n);
+            uint64_t w[I];
+#pragma unroll
+            for (int it = 0; it < I; it++) w[it] = (uint32_t)it < count ? in[it * p.ct_item_stride + g] : 0;
+#pragma unroll
+            for (int it = 0; it < I; it++) acc[it] = add_mod(acc[it], w[it], q);
+        }
+#pragma unroll
+        for (int it = 0; it < I; it++)
+            if ((uint32_t)it < count) c0_out[it * p.ct_item_stride] = acc[it];
         return;
     }
     const uint32_t t = by;
@@ -508,6 +523,7 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     auto word = [&](uint32_t d, int it, uint32_t at) {
         return d == own ? c1[it * p.ct_item_stride + at] : y[it * y_item + d * digit + at];
     };
+    const uint32_t n_terms = p.n_steps * p.beta;
     if (LOCAL) {
         for (uint32_t d = 0; d < p.beta; d++)
 #pragma unroll
@@ -517,10 +533,12 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     }
     // term e = step e / beta, digit e mod beta; the operands of term e + 1 are requested before term e is
     // multiplied, so that a wave does not wait for memory once per term
-    const uint32_t n_terms = p.n_steps * p.beta;
+    // (the gather index belongs to the step: it is formed for a step's first digit and kept for the others; the last
+    // iteration's repeated request is for the term just served)
+    uint32_t src = 0;
     auto fetch = [&](uint32_t e, uint64_t &k0, uint64_t &k1, uint64_t(&v)[I]) {
         const uint32_t st = e / p.beta, d = e - st * p.beta;
-        const uint32_t src = galois_index(j, p.elts[st], p.log_n);
+        if (d == 0 || e == 0) src = galois_index(j, p.elts[st], p.log_n);
         const uint64_t *k = p.evk.p[e];
         k0 = k[key_off];
         k1 = k[key_off + key_poly];
@@ -534,35 +552,65 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     const size_t o = ((size_t)t << p.log_n) + j;
     const size_t opoly = (size_t)LK << p.log_n;
     if (table < 64 && ((p.fp_mask >> table) & 1)) {
-        // a prime below 2^50: exact FP64 products (6 full-rate instructions instead of 4 quarter-rate multiply-adds),
-        // each below 0.875 q in magnitude, eight of them between two reductions
+        // a prime below 2^50: the sum of the products as an exact pair (hi, lo) before any reduction, four FP64
+        // operations per product.  hi runs in [2^B, 2^(B+1)), where doubles are the multiples of 2^(B-52): the fused
+        // multiply-add t = fl(x w + hi) rounds the exact sum to such a multiple, t - hi is exact, x w - (t - hi) is the
+        // rounding error, an integer of at most 2^(B-53) in magnitude that the second fused multiply-add returns
+        // exactly.  B = 103 takes 8 products below 2^100 between two folds (8 errors sum exactly, <= 2^53); when
+        // n_terms q^2 <= 2^100 a smaller B takes all of them (at most 64) in one go.
         const FpMod m{p.fp_consts[4 * table], p.fp_consts[4 * table + 1]};
-        double f0[I], f1[I];
+        const uint32_t qbits = 64 - __builtin_clzll(p.moduli[table]);              // q < 2^qbits
+        const uint32_t tbits = 32 - __builtin_clz(n_terms);                        // n_terms < 2^tbits
+        const bool one_go = 2 * qbits + tbits <= 100;
+        const uint32_t B = !one_go ? 103 : 2 * qbits + tbits < 60 ? 60 : 2 * qbits + tbits;   // (any B up to 100 serves small primes)
+        const uint32_t period = one_go ? n_terms : 8;
+        const double base = __hiloint2double((int)((1023 + B) << 20), 0);
+        const double down = __hiloint2double((int)((1023 + 52 - B) << 20), 0);     // 2^-(B-52)
+        const double cB = fp_reduce(__hiloint2double((int)((1023 + B - 52) << 20), 0), m);
+        const FpTw wB{cB, cB * m.qinv};
+        double hi0[I], lo0[I], hi1[I], lo1[I], f0[I], f1[I];
 #pragma unroll
-        for (int it = 0; it < I; it++) f0[it] = f1[it] = 0.0;
+        for (int it = 0; it < I; it++) {
+            hi0[it] = hi1[it] = base;
+            lo0[it] = lo1[it] = f0[it] = f1[it] = 0.0;
+        }
+        // (hi - 2^B) / 2^(B-52) is an integer below 2^52; times 2^(B-52) mod q it is congruent to the high part, and the
+        // modular product takes it as it is (result at most 2.5 q in magnitude)
+        auto fold = [&]() {
+#pragma unroll
+            for (int it = 0; it < I; it++) {
+                f0[it] = fp_reduce(f0[it] + fp_mulmod((hi0[it] - base) * down, wB, m) + fp_reduce(lo0[it], m), m);
+                f1[it] = fp_reduce(f1[it] + fp_mulmod((hi1[it] - base) * down, wB, m) + fp_reduce(lo1[it], m), m);
+                hi0[it] = hi1[it] = base;
+                lo0[it] = lo1[it] = 0.0;
+            }
+        };
+        uint32_t pending = 0;
         for (uint32_t e = 0; e < n_terms; e++) {
             uint64_t nk0, nk1, nv[I];
             fetch(e + 1 < n_terms ? e + 1 : e, nk0, nk1, nv);
+            asm volatile("" ::: "memory");       // (a compiler barrier: without it the loads, whose values are first used in the
+            __builtin_amdgcn_sched_barrier(0);   //  next iteration, sink to the end of this one and every term waits for its operands)
             const double w0 = fp_from_u64(k0), w1 = fp_from_u64(k1);
-            const FpTw t0{w0, w0 * m.qinv}, t1{w1, w1 * m.qinv};
 #pragma unroll
             for (int it = 0; it < I; it++) {
                 const double x = fp_from_u64(v[it]);
-                f0[it] += fp_mulmod(x, t0, m);
-                f1[it] += fp_mulmod(x, t1, m);
+                const double t0 = __builtin_fma(x, w0, hi0[it]), t1 = __builtin_fma(x, w1, hi1[it]);
+                lo0[it] += __builtin_fma(x, w0, -(t0 - hi0[it]));
+                lo1[it] += __builtin_fma(x, w1, -(t1 - hi1[it]));
+                hi0[it] = t0;
+                hi1[it] = t1;
             }
-            if ((e & 7) == 7) {
-#pragma unroll
-                for (int it = 0; it < I; it++) {
-                    f0[it] = fp_reduce(f0[it], m);
-                    f1[it] = fp_reduce(f1[it], m);
-                }
+            if (++pending == period) {
+                fold();
+                pending = 0;
             }
             k0 = nk0;
             k1 = nk1;
 #pragma unroll
             for (int it = 0; it < I; it++) v[it] = nv[it];
         }
+        if (pending) fold();
 #pragma unroll
         for (int it = 0; it < I; it++) {
             if ((uint32_t)it >= count) break;
@@ -578,17 +626,21 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
         return;
     }
     Lazy3 s0[I], s1[I], h0[I], h1[I];
+    // the words are relieved every 8 terms for a prime below 2^60, every 4 otherwise (see Lazy3)
+    const uint32_t spill_mask = (p.moduli[table] >> 60) ? 3u : 7u;
 #pragma unroll
     for (int it = 0; it < I; it++) s0[it] = s1[it] = h0[it] = h1[it] = Lazy3{0, 0, 0};
     for (uint32_t e = 0; e < n_terms; e++) {
         uint64_t nk0, nk1, nv[I];
         fetch(e + 1 < n_terms ? e + 1 : e, nk0, nk1, nv);
-        const Split31 ks0 = split31(k0), ks1 = split31(k1);
+        asm volatile("" ::: "memory");       // (a compiler barrier: without it the loads, whose values are first used in the
+            __builtin_amdgcn_sched_barrier(0);   //  next iteration, sink to the end of this one and every term waits for its operands)
+        const Split30 ks0 = split30(k0), ks1 = split30(k1);
 #pragma unroll
         for (int it = 0; it < I; it++) {
-            mac3x2(s0[it], s1[it], split31(v[it]), ks0, ks1);
+            mac3x2(s0[it], s1[it], split30(v[it]), ks0, ks1);
         }
-        if ((e & 3) == 3) {
+        if ((e & spill_mask) == spill_mask) {
 #pragma unroll
             for (int it = 0; it < I; it++) {
                 spill3(h0[it], s0[it]);
