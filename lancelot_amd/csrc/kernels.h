@@ -81,6 +81,8 @@ struct NttArgs {
     uint32_t items;           // list mode: the whole list is applied to `items` buffers (0 = 1) ...
     size_t item_stride;       // ... that lie item_stride words apart
     uint32_t batch, n_polys;  // filled in by the launcher
+    uint32_t unit_filter;     // blocks pass of a mixed launch run as two kernels (filled in by the launcher): 1 = only the
+                              // units whose prime is below 2^50, 2 = only the others, 0 = every unit
     uint32_t log_n;
     LimbMap map;
     int pro_mode;

@@ -970,6 +970,7 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
     const bool has_addend = EPI && (a.epi_mode == NTT_EPI_SUB_MUL_ADD || fma_mode);
 
     Job job = decode_job(a, g.unit.j0);
+    if (a.unit_filter == 1 && !((a.fp_mask >> job.table) & 1)) return;   // (the whole workgroup: a unit has one prime)
     const FpCtx fc = fp_ctx(a, job.table);
     const FpMod m = fc.m;
 
@@ -1384,6 +1385,7 @@ __device__ __forceinline__ void ntt_blocks_int_body(const NttArgs &a, uint64_t *
     const bool epi = FWD && (a.epi_mode == NTT_EPI_SUB_MUL || a.epi_mode == NTT_EPI_SUB_MUL_ADD || fma_mode);
     const bool has_addend = FWD && (a.epi_mode == NTT_EPI_SUB_MUL_ADD || fma_mode);
 
+    if (a.unit_filter == 2 && ((a.fp_mask >> decode_job(a, g.unit.j0).table) & 1)) return;
     for (uint32_t b = 0; b < g.unit.count; b++) {
         const Job job = decode_job(a, g.unit.j0 + b * g.unit.jstride);
         const IntCtx ic = int_ctx(a, job.table);
@@ -1523,6 +1525,8 @@ BlocksPlan plan_blocks(const NttArgs &a, uint32_t n_polys) {
     return p;
 }
 
+constexpr uint32_t kSplitMixedGrid = 1024;   // workgroups from which a mixed blocks pass runs as two kernels
+
 template <bool FWD, int FP>
 hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
     const BlocksPlan p = plan_blocks(a, n_polys);
@@ -1533,6 +1537,24 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
     // the Galois gather of an inverse pass's input lives in instantiations of its own
     const bool gal = !FWD && a.in_galois != 0 && !a.jobs;
     const dim3 grid(p.grid), block(p.threads);
+    if (FP == NTT_BACKEND_MIXED && p.grid >= kSplitMixedGrid) {
+        // A large mixed launch runs as two kernels over the same grid, each leaving the other's units at once: the
+        // integer body then has its own three waves per SIMD (the mixed kernel is compiled for the FP64 body's
+        // registers: two), which its unpipelined load -> butterflies -> store sequence needs.
+        a.unit_filter = 1;
+        if (gal)
+            hipLaunchKernelGGL((ntt_blocks_fp_kernel<false, false, true>), grid, block, 0, s, a);
+        else if (epi)
+            hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, FWD, false>), grid, block, 0, s, a);
+        else
+            hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, false, false>), grid, block, 0, s, a);
+        a.unit_filter = 2;
+        if (gal)
+            hipLaunchKernelGGL((ntt_blocks_int_kernel<false, true>), grid, block, 0, s, a);
+        else
+            hipLaunchKernelGGL((ntt_blocks_int_kernel<FWD, false>), grid, block, 0, s, a);
+        return hipGetLastError();
+    }
     if (gal) {
         if (FP == NTT_BACKEND_MIXED)
             hipLaunchKernelGGL((ntt_blocks_mixed_kernel<false, false, true>), grid, block, 0, s, a);
