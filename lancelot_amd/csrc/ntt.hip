@@ -709,9 +709,9 @@ __device__ __forceinline__ double uniform_f64(double v) {
     return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
 }
 
-// output limbs per workgroup, at most.  The workgroup's first kFuseMaxRows * 18 threads fetch the rows' constants
-// (one word each), so the cap is tied to the smallest workgroup of the kernel (256 threads).
-constexpr uint32_t kFuseMaxRows = 12;
+// output limbs per workgroup, at most (the LDS arrays of the rows' constants have this many entries; their loader
+// strides over the workgroup, whatever its size)
+constexpr uint32_t kFuseMaxRows = 24;
 
 // P = coefficients per thread.  8: 256 threads, two waves per SIMD.  (4, with 512 threads and four waves per SIMD,
 // compiles but measured 1.7 times slower at N = 2^16: the inputs' registers spill, and a tile needs twice the LDS
@@ -732,7 +732,6 @@ void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
     __shared__ double mrow[kFuseMaxRows][18];
     __shared__ uint32_t mlimb[kFuseMaxRows], mtable[kFuseMaxRows];
     static_assert(LD >= 4 && LD <= 8 && (P == 8 || P == 4), "N from 2^12 to 2^16");
-    static_assert(kFuseMaxRows * 18 <= kFuseWords / P, "one thread per constant of the group's rows");
     constexpr int LOGC = kFuseLog - LD, LOGP = P == 8 ? 3 : 2;
     constexpr uint32_t T = kFuseWords / P;
     constexpr uint32_t C = 1u << LOGC, tiles_per_limb = 256u >> LOGC, row_step = T >> LOGC;
@@ -778,8 +777,8 @@ void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
     // The constants of this group's output limbs (matrix row, modulus, output limb, table) go to LDS once, and are
     // read back into scalar registers limb by limb: a scalar load per limb would stall the workgroup for a cache miss.
     const double *mat = p.b.mat_fp + 2 * d.mat_off;
-    if (threadIdx.x < (r_end - r_begin) * 18) {
-        const uint32_t rl = threadIdx.x / 18, c = threadIdx.x - rl * 18, r = r_begin + rl;
+    for (uint32_t w = threadIdx.x; w < (r_end - r_begin) * 18; w += T) {
+        const uint32_t rl = w / 18, c = w - rl * 18, r = r_begin + rl;
         const uint32_t table = p.b.out_table[d.map_off + r];
         // (the matrices are padded: 8 pairs can be fetched whatever the row's length)
         mrow[rl][c] = c < 16 ? mat[2 * (size_t)r * d.n_in + c] : a.fp_consts[4 * (size_t)table + (c - 16)];
@@ -1579,22 +1578,40 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
 
 hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s) {
     if (a.log_n < 12 || a.log_n > 16 || !b.mat_fp || b.n_units == 0) return hipErrorInvalidValue;
-    // 0: by the number of items.  One operation needs the workgroups of 3 rows each to fill the chip; from 4 items on
-    // there are enough of them at 12 rows, and a workgroup's inputs and set-up serve four times as many rows
-    // (8 items at N = 2^16: 1.046 -> 1.012 ms per call; one item: 0.181 -> 0.193 ms at 8 rows).
     static const uint32_t forced = [] {
         const char *e = getenv("CAHEL_HIP_FUSE_ROWS");
         const int v = e ? atoi(e) : 0;
         return (uint32_t)(v >= 1 && v <= (int)kFuseMaxRows ? v : 0);
     }();
     const uint32_t items = b.items ? b.items : 1;
-    const uint32_t target = forced ? forced : items >= 4 ? kFuseMaxRows : 3;
-    const uint32_t rows = b.mdr ? b.max_rows - 1 : b.max_rows;
-    if (rows == 0) return hipErrorInvalidValue;
-    BconvRowsK p{b, (rows + target - 1) / target, 0, target};
-    p.copy_groups = b.copy_base ? (b.max_copy + target - 1) / target : 0;
     const int ld = (int)a.log_n - 8;
     const uint32_t tiles = 256u >> (kFuseLog - ld);
+    const uint32_t rows = b.mdr ? b.max_rows - 1 : b.max_rows;
+    if (rows == 0) return hipErrorInvalidValue;
+    // Output limbs per workgroup.  The kernel is bound by instruction issue, so a CU's time is the number of workgroups
+    // it is dealt times a workgroup's work: r rows plus about 1.5 rows' worth of fetching and converting its 8 x 8 block
+    // of inputs and setting up.  Few rows per workgroup pay that overhead often, many leave CUs with one workgroup more
+    // than others; the count that minimises ceil(workgroups / CUs) x (r + 1.5) matches the measured order at N = 2^16
+    // (one operation: 3 and 6 equal, 4 and 8 slower; 8 operations: 207, 179, 168 us at 3, 8, 12 rows).
+    uint32_t target = forced;
+    if (!target) {
+        static const uint32_t cus = [] {
+            int dev = 0, n = 0;
+            if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+            return (uint32_t)n;
+        }();
+        uint64_t best = ~0ull;
+        for (uint32_t r = 1; r <= kFuseMaxRows && r <= rows; r++) {
+            const uint64_t wgs = (uint64_t)b.n_units * items * tiles * ((rows + r - 1) / r);
+            const uint64_t cost = ((wgs + cus - 1) / cus) * (2 * r + 3);
+            if (cost < best) {
+                best = cost;
+                target = r;
+            }
+        }
+    }
+    BconvRowsK p{b, (rows + target - 1) / target, 0, target};
+    p.copy_groups = b.copy_base ? (b.max_copy + target - 1) / target : 0;
     const uint64_t wgs = (uint64_t)b.n_units * items * tiles * (p.compute_groups + p.copy_groups);
     if (wgs > 0x7fffffffu) return hipErrorInvalidValue;
     const dim3 grid((uint32_t)wgs);

@@ -70,8 +70,9 @@ def test_c1_hmult_relin_rescale_bit_exact(oracle):
 @pytest.mark.parametrize("inner", ["fused", "fp_kernel"])
 def test_c2_benchmark_shape_entry_points_bit_exact(oracle, monkeypatch, inner):
     """N = 2^16, L = 24, K = 8 (dnum = 3), 50-bit primes, random residues: he_multiply_relin_rescale, its batch form
-    (4 products, from which on the fused conversion kernel forms 12 output limbs per workgroup instead of 3; with the
-    inner product inside the blocks pass and as the FP64 kernel of its own) and he_rotate
+    (8 products, as `bench.py` issues them: the fused conversion kernel then forms all 24 or 23 output limbs of a
+    unit in one workgroup, where one product per call takes 5 or 6; with the inner product inside the blocks pass and
+    as the FP64 kernel of its own) and he_rotate
     against the oracle's tensor / relinearise / rescale and apply_galois, every limb."""
     from gpu_util import DeviceArray, make_pair, rand_limbs
     from lancelot_amd import capi
@@ -83,7 +84,7 @@ def test_c2_benchmark_shape_entry_points_bit_exact(oracle, monkeypatch, inner):
     host_evk = [rand_limbs(p, rng, range(L + K), n_polys=2) for _ in range(L // K)]
     dev_evk = [DeviceArray(capi, host=k) for k in host_evk]
     ptrs = capi.evk_array([d.ptr for d in dev_evk])
-    items = 4
+    items = 8
     a = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
     b = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
     want = [p.rescale(p.relinearize(p.tensor(a[k], b[k]), host_evk)) for k in range(items)]
