@@ -333,6 +333,38 @@ def test_hoisted_rotations_with_block_local_steps(oracle, capi, monkeypatch, log
             assert (got[k] == want).all(), (add_input, k)
 
 
+@pytest.mark.parametrize("local", [False, True])
+@pytest.mark.parametrize("bits,L", [([60, 60, 60, 60, 60], 4), ([50, 49, 50, 50, 50], 4), ([60, 40, 60, 40, 60], 4)])
+def test_hoisted_rotations_largest_residues(oracle, capi, bits, L, local):
+    """Every residue of the inputs and of the keys is q - 1 and the launch has the most products it accepts (16 steps x
+    4 digits = 64 per output word): the lazy sums of the hoisting kernel (three 64-bit words relieved every 8 terms for
+    the 60-bit primes, the exact FP64 pair for those below 2^50) and its final 128-bit reduction at their bounds.
+    5 items: a group of 4 and a remainder.  Against the oracle, item by item."""
+    logn, size_p, items, n_steps = 11, 1, 5, 16
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
+    lib, h = capi.lib(), ctx.he_handle()
+    beta = -(-L // size_p)
+    assert n_steps * beta == 64
+    top = lambda tidx, n_polys: np.stack([np.stack([np.full(p.n, p.moduli[t] - 1, dtype=np.uint64) for t in tidx])] * n_polys)
+    host_key = [top(range(p.size_qp), 2) for _ in range(beta)]
+    dev_key = [DeviceArray(capi, host=k) for k in host_key]
+    unit = p.n // 512
+    steps = [unit * (k + 1) for k in range(n_steps)] if local else [k + 1 for k in range(n_steps)]
+    elts = [pow(5, s, 2 * p.n) for s in steps]
+    flat = capi.evk_array([dev_key[d].ptr for _ in range(n_steps) for d in range(beta)])
+    d_elts = (C.c_uint32 * n_steps)(*elts)
+    wsb = DeviceArray(capi, shape=(lib.he_keyswitch_batch_workspace_words(h, L, items),))
+    ct = top(range(L), 2)
+    cts = np.stack([ct] * items)
+    din, dout = DeviceArray(capi, host=cts), DeviceArray(capi, shape=(items, 2, L, p.n))
+    capi.check(lib.he_hoisted_rotations_batch(h, L, items, din.ptr, flat, d_elts, n_steps, 1, dout.ptr, wsb.ptr, None))
+    want = p.hoisting(ct, elts, [host_key] * n_steps)
+    want = np.stack([p.add(want[b], ct[b]) for b in range(2)])
+    got = dout.numpy()
+    for k in range(items):
+        assert (got[k] == want).all(), k
+
+
 @pytest.mark.parametrize("logn,bits,size_p,L,items", [(11, [45, 40, 40, 50], 1, 3, 5), (11, [60, 40, 40, 60], 1, 2, 3),
                                                        (12, [60, 40, 50, 45, 30, 59, 60, 60], 2, 5, 2),
                                                        (11, [50, 50, 49, 50, 50, 50], 2, 4, 3),
@@ -577,6 +609,30 @@ def _evk(p, rng, capi):
     host = [rand_limbs(p, rng, range(p.size_qp), n_polys=2) for _ in range(dnum)]
     dev = [DeviceArray(capi, host=k) for k in host]
     return host, dev, capi.evk_array([d.ptr for d in dev])
+
+
+@pytest.mark.parametrize("bits", [[60] * 9, [50] * 9, [60, 40] * 4 + [60]])
+def test_inner_product_largest_residues(oracle, capi, bits):
+    """he_ks_inner_product with every digit word and every key word equal to q - 1 (8 digits of one limb each): the
+    128-bit sums of the integer kernel and their reduction, and the FP64 kernel's, at their bounds; plain and
+    accumulating onto a result that is q - 1 everywhere."""
+    cahel, parms, ctx, p = make_pair(oracle, 11, bits, 1)
+    lib, h = capi.lib(), ctx.he_handle()
+    L, K, n = 8, 1, p.n
+    tidx = [p.table_index(L, t) for t in range(L + K)]
+    row = np.stack([np.full(n, p.moduli[t] - 1, dtype=np.uint64) for t in tidx])
+    y = np.stack([row] * L)
+    host_evk = [np.stack([np.stack([np.full(n, p.moduli[t] - 1, dtype=np.uint64) for t in range(p.size_qp)])] * 2) for _ in range(L)]
+    dev_evk = [DeviceArray(capi, host=k) for k in host_evk]
+    ptrs = capi.evk_array([d.ptr for d in dev_evk])
+    dy = DeviceArray(capi, host=y)
+    dcx = DeviceArray(capi, host=np.stack([row, row]))
+    cx = p.inner_prod(y, host_evk)
+    capi.check(lib.he_ks_inner_product(h, L, dy.ptr, ptrs, dcx.ptr, 0, 1, None))
+    assert (dcx.numpy() == np.stack([p._add_tidx(row, cx[b], tidx) for b in range(2)])).all()
+    capi.check(lib.he_ks_inner_product(h, L, dy.ptr, ptrs, dcx.ptr, 0, 0, None))
+    assert (dcx.numpy() == cx).all()
+    assert (cx == (L % np.array([p.moduli[t] for t in tidx], dtype=np.uint64))[None, :, None]).all()   # 8 x (q - 1)^2 = 8 mod q
 
 
 @pytest.mark.parametrize("L", [6, 5, 4, 3, 1])
