@@ -59,6 +59,23 @@ PROFILE = {"single": {"traffic_limbs": 1120.2, "valu_wave_instr": 33.41e6,
                                 "epilogue"}}
 
 
+def issue_rates(capi):
+    """he_probe_issue_rate for every kind at 2, 4 and 8 waves per SIMD of every CU: 10^12 lane-operations per second
+    (multiply-adds for the matrix kinds)."""
+    cus = 256   # MI355X
+    kinds = ["v_fma_f64", "v_mad_u64_u32", "v_mul_lo_u32", "v_add_u32", "v_mfma_f64_16x16x4_f64",
+             "v_mfma_f64_16x16x4_f64 + v_fma_f64 (equal work on each, sum of both)"]
+    out = {"unit": "1e12 lane-operations per second", "compute_units": cus, "waves_per_simd": [2, 4, 8], "rates": {}}
+    for kind, name in enumerate(kinds):
+        row = []
+        for waves in out["waves_per_simd"]:
+            rate = C.c_double()
+            capi.check(capi.lib().he_probe_issue_rate(kind, cus * waves, 2000, C.byref(rate), None))
+            row.append(round(rate.value / 1e12, 2))
+        out["rates"][name] = row
+    return out
+
+
 def sync(capi):
     capi.check(capi.lib().he_stream_synchronize(None), "sync")
 
@@ -275,8 +292,9 @@ def main():
     ap.add_argument("--batch", type=int, default=8, help="operations per he_multiply_relin_rescale_batch call")
     ap.add_argument("--batch-streams", type=int, default=2, help="streams that the batch calls are dealt to")
     ap.add_argument("--no-krum", action="store_true", help="skip the encrypted Krum round (BASELINE.json configs[4])")
-    ap.add_argument("--only", choices=["all", "step", "batch", "rotate", "ntt", "krum"], default="all",
-                    help="step / rotate / ntt: run just that workload on the null stream (for rocprofv3)")
+    ap.add_argument("--only", choices=["all", "step", "batch", "rotate", "ntt", "krum", "probe"], default="all",
+                    help="step / rotate / ntt: run just that workload on the null stream (for rocprofv3); probe: the "
+                         "issue rates of the instruction kinds that the kernels' bounds are argued with")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -288,6 +306,9 @@ def main():
 
     if args.only == "krum":
         print(json.dumps(krum_round()))
+        return
+    if args.only == "probe":
+        print(json.dumps(issue_rates(capi)))
         return
     n = 1 << LOG_N
     parms = cahel.params(cahel.scheme_type.ckks)

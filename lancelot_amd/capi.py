@@ -36,6 +36,7 @@ SIGNATURES = {
     "he_stream_wait_event": (C.c_int, [vp, vp]),
     "he_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
     "he_probe_fp64_issue_rate": (C.c_int, [u32, u32, C.POINTER(C.c_double), vp]),
+    "he_probe_issue_rate": (C.c_int, [u32, u32, u32, C.POINTER(C.c_double), vp]),
     "he_context_create": (C.c_int, [vp, C.POINTER(vp)]),
     "he_context_set_level": (C.c_int, [vp, vp]),
     "he_context_destroy": (C.c_int, [vp]),

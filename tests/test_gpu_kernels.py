@@ -886,3 +886,23 @@ def test_ckks_encode_bad_arguments(small, capi):
     for slots, count in ((3, 2), (p.n, 4), (8, 9), (1, 1)):
         assert lib.he_ckks_encode(h, buf.ptr, None, count, slots, 2.0 ** 30, p.size_q, out.ptr, buf.ptr, None) == -1
     assert lib.he_ckks_decode(h, out.ptr, p.size_q + 1, 8, 2.0 ** 30, buf.ptr, buf.ptr, None) == -1
+
+
+def test_issue_rate_probe(capi):
+    """he_probe_issue_rate: every kind returns a rate, an unknown kind and empty launches are refused, and the
+    ordering that the design notes rely on holds (a 32-bit addition issues faster than an FP64 multiply-add or a
+    32-bit multiply; the FP64 matrix instruction interleaved with FP64 vector multiply-adds does not reach the sum
+    of the two alone)."""
+    lib, r = capi.lib(), C.c_double()
+    assert lib.he_probe_issue_rate(6, 256, 10, C.byref(r), None) == -1
+    assert lib.he_probe_issue_rate(0, 0, 10, C.byref(r), None) == -1
+    assert lib.he_probe_issue_rate(0, 256, 0, C.byref(r), None) == -1
+    assert lib.he_probe_issue_rate(0, 256, 10, None, None) == -1
+    rate = []
+    for kind in range(6):
+        capi.check(lib.he_probe_issue_rate(kind, 1024, 500, C.byref(r), None))
+        rate.append(r.value)
+    assert all(v > 5e12 for v in rate), rate
+    fma, mad, mul, add, mfma, both = rate
+    assert add > 1.5 * fma and add > 1.5 * mad and add > 1.5 * mul, rate
+    assert both < 0.75 * (fma + mfma), rate
