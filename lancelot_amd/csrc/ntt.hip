@@ -1592,7 +1592,9 @@ hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s
     // it is dealt times a workgroup's work: r rows plus about 1.5 rows' worth of fetching and converting its 8 x 8 block
     // of inputs and setting up.  Few rows per workgroup pay that overhead often, many leave CUs with one workgroup more
     // than others; the count that minimises ceil(workgroups / CUs) x (r + 1.5) matches the measured order at N = 2^16
-    // (one operation: 3 and 6 equal, 4 and 8 slower; 8 operations: 207, 179, 168 us at 3, 8, 12 rows).
+    // (one operation: 3 and 6 equal, 4 and 8 slower; 8 operations: 207, 179, 168 us at 3, 8, 12 rows).  A CU with a
+    // single workgroup has one wave per SIMD and nothing to cover its waits with (ModDown of one operation: 24.2 us in
+    // 256 workgroups of 6 rows against 22.5 us in 512 of 3), so fewer than two per CU count as two.
     uint32_t target = forced;
     if (!target) {
         static const uint32_t cus = [] {
@@ -1603,7 +1605,8 @@ hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s
         uint64_t best = ~0ull;
         for (uint32_t r = 1; r <= kFuseMaxRows && r <= rows; r++) {
             const uint64_t wgs = (uint64_t)b.n_units * items * tiles * ((rows + r - 1) / r);
-            const uint64_t cost = ((wgs + cus - 1) / cus) * (2 * r + 3);
+            const uint64_t per_cu = (wgs + cus - 1) / cus;
+            const uint64_t cost = (per_cu < 2 ? 2 : per_cu) * (2 * r + 3);
             if (cost < best) {
                 best = cost;
                 target = r;
