@@ -463,7 +463,16 @@ __global__ __launch_bounds__(kThreads) void hoist_inner_kernel(HoistArgs p) {
     {
         const uint32_t nb = (1u << p.log_n) / kThreads, id = blockIdx.x;
         if (p.xcd_map) {
-            const uint32_t s = id >> 3, pair = (s / p.groups) * 8 + (id & 7);
+            // xcd_map 2 (gathers from memory, N >= 2^15): an XCD also takes the 16 blocks of an aligned 4,096-word
+            // stretch of one row one after the other, so that the words which the steps' gathers bring into its L2 (a
+            // step of 8 k permutes inside such stretches) are found there by the neighbouring workgroups; the stretches
+            // of every row are dealt to the XCDs in turn, heavy rows first everywhere
+            const uint32_t s = id >> 3;
+            uint32_t pair = (s / p.groups) * 8 + (id & 7);
+            if (p.xcd_map == 2) {
+                const uint32_t q = s / p.groups, u = (q >> 4) * 8 + (id & 7), stretches = nb >> 4;
+                pair = (u / stretches) * nb + (u % stretches) * 16 + (q & 15);
+            }
             bz = s % p.groups;
             bx = pair % nb;
             by = pair / nb;
@@ -1026,13 +1035,18 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
     // every automorphism of the launch stays inside the aligned 256-word blocks of the NTT order
     bool local = t.log_n >= 8 && beta * 4 <= (uint32_t)kHoistLocalTiles;
     for (uint32_t i = 0; i < n_steps && local; i++) local = t.log_n < 9 || ((elts[i] - 1) & ((1u << (t.log_n - 7)) - 1)) == 0;
-    static const bool no_local = [] { const char *e = getenv("CAHEL_HIP_NO_LOCAL_HOIST"); return e && e[0] == '1'; }();
-    static const bool no_xcd = [] { const char *e = getenv("CAHEL_HIP_NO_XCD_MAP"); return e && e[0] == '1'; }();
+    // (read at every launch, so that a test can compare the paths inside one process)
+    auto env_on = [](const char *name) { const char *e = getenv(name); return e && e[0] == '1'; };
+    const bool no_local = env_on("CAHEL_HIP_NO_LOCAL_HOIST"), no_xcd = env_on("CAHEL_HIP_NO_XCD_MAP"),
+               no_contig = env_on("CAHEL_HIP_NO_XCD_CONTIG");
     if (no_local) local = false;
+    // ... or inside the aligned stretches of 4,096 words (steps that are multiples of N / 8192)
+    bool stretch_local = t.log_n >= 12;
+    for (uint32_t i = 0; i < n_steps && stretch_local; i++) stretch_local = ((elts[i] - 1) & ((1u << (t.log_n - 11)) - 1)) == 0;
     const bool p_xcd_ok = !no_xcd && (nb * rows) % 8 == 0;
     auto launch = [&](auto kernel, uint32_t per) {
         p.groups = (items + per - 1) / per;
-        p.xcd_map = p_xcd_ok && p.groups > 1;
+        p.xcd_map = p_xcd_ok && p.groups > 1 ? (local || no_contig || !stretch_local || nb < 128 || (nb >> 4) % 8 != 0 ? 1 : 2) : 0;
         hipLaunchKernelGGL(kernel, dim3(nb * rows * p.groups), dim3(kThreads), 0, s, p);
     };
 #define HE_HOIST(I) \

@@ -247,3 +247,36 @@ def test_c5_krum_round_full_shape():
     assert np.max(np.abs(dist[off] - want[off]) / want[off]) < 2e-5
     assert chosen == krum.krum_select(want) and chosen not in (8, 9)
     assert timings["total"] > 0
+
+
+@pytest.mark.parametrize("switch", ["", "CAHEL_HIP_NO_XCD_CONTIG", "CAHEL_HIP_NO_XCD_MAP"])
+def test_hoisted_rotations_batch_workgroup_orders(oracle, monkeypatch, switch):
+    """N = 2^15, Lancelot's chain, 5 ciphertexts, steps 4, 8, 12 and 20 (multiples of N / 8192 but not of N / 512: the
+    automorphisms stay inside aligned stretches of 4,096 words, so the launch gathers from memory and takes the workgroup
+    order in which an XCD walks through such a stretch): against the oracle's hoisting item by item, with that order,
+    with the plain XCD-aware one and with the plain one."""
+    import ctypes as C
+    from gpu_util import DeviceArray, make_pair, rand_limbs
+    from lancelot_amd import capi
+    if switch:
+        monkeypatch.setenv(switch, "1")
+    cahel, parms, ctx, p = make_pair(oracle, 15, [60, 40, 40, 60], 1)
+    lib, h = capi.lib(), ctx.he_handle()
+    rng = np.random.default_rng(31)
+    L, items, steps = 2, 5, [4, 8, 12, 20]
+    beta = L
+    elts = [pow(5, s, 2 * p.n) for s in steps]
+    assert all((e - 1) % 16 == 0 and (e - 1) % 256 != 0 for e in elts)
+    host_keys = [[rand_limbs(p, rng, range(p.size_qp), n_polys=2) for _ in range(beta)] for _ in range(2)]
+    dev_keys = [[DeviceArray(capi, host=k) for k in ks] for ks in host_keys]
+    flat = capi.evk_array([dev_keys[i % 2][d].ptr for i in range(len(steps)) for d in range(beta)])
+    d_elts = (C.c_uint32 * len(steps))(*elts)
+    wsb = DeviceArray(capi, shape=(lib.he_keyswitch_batch_workspace_words(h, L, items),))
+    cts = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
+    din, dout = DeviceArray(capi, host=cts), DeviceArray(capi, shape=(items, 2, L, p.n))
+    capi.check(lib.he_hoisted_rotations_batch(h, L, items, din.ptr, flat, d_elts, len(steps), 1, dout.ptr, wsb.ptr, None))
+    got = dout.numpy()
+    for k in range(items):
+        want = p.hoisting(cts[k], elts, [host_keys[i % 2] for i in range(len(steps))])
+        want = np.stack([p.add(want[b], cts[k][b]) for b in range(2)])
+        assert (got[k] == want).all(), k
