@@ -1172,7 +1172,11 @@ int ksr_impl(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *
     HE_HIP(launch_ntt_inverse(inv, polys, backend_for(ctx, inv.map), S(s)));
     // (3) delta = P -> Ql conversion of the special limbs
     const bool fused = fuse_rows_ok(ctx, lv, L);
-    if (fused) {
+    // one special prime: the conversion is the reduction of its coefficients modulo every q_j, which the prologue of (4)
+    // does where it reads them (no conversion kernel, no delta in memory before the transform)
+    const bool k1 = ctx->single_limb_digits && !fused;
+    if (k1) {
+    } else if (fused) {
         // with the prologue of (4) and the rows pass of its transform
         BconvRows b{cx, delta, nullptr, ctx->d_phat_pinv_fp, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
                     items, 2 * (size_t)LK * n, 2 * (size_t)L * n, 0, 1};
@@ -1201,6 +1205,11 @@ int ksr_impl(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *
     fwd.pro2_poly_stride = L;
     fwd.pro_w = ctx->d_pinv_mod_q;
     fwd.pro_last = L - 1;
+    if (k1) {
+        fwd.pro_src2 = cx + (size_t)L * n;
+        fwd.pro2_poly_stride = LK;
+        fwd.pro_k1 = 1;
+    }
     fwd.epi_mode = NTT_EPI_FMA_SUB_MUL;
     fwd.epi_a = cx;
     fwd.epi_a_poly_stride = LK;

@@ -101,6 +101,9 @@ struct NttArgs {
     const uint64_t *pro_src2; // NTT_PRO_MODDOWN_RESCALE: second source, limb (poly) at pro_src2 + poly * pro2_poly_stride * N
     uint32_t pro2_poly_stride;
     uint32_t pro_last;        // NTT_PRO_MODDOWN_RESCALE: table (and index into pro_w) of the limb that is dropped
+    int pro_k1;               // NTT_PRO_MODDOWN_RESCALE with one special prime: the P -> Q conversion is the reduction of
+                              // that prime's coefficients, so pro_src2 is the special limb itself (any residue below 2^61)
+                              // and both delta_j and delta_last are its Barrett reductions; `in` is not read
     const uint64_t *w;        // [limbs][2] Shoup constants indexed by limb i of the map
     uint64_t *epi_dst;        // destination of the forward epilogues
     uint32_t epi_dst_poly_stride;

@@ -232,12 +232,16 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
                 const FpMod ml = fp_ctx(a, a.pro_last).m;
                 const double wd = fp_from_u64(a.pro_w[2 * job.limb]), wl = fp_from_u64(a.pro_w[2 * a.pro_last]);
                 const FpTw w{wd, wd * c.m.qinv}, wlast{wl, wl * ml.qinv};
+                const uint64_t qj = a.moduli[job.table], rj = a.barrett[2 * job.table + 1];
+                const uint64_t qlast = a.moduli[a.pro_last], rlast = a.barrett[2 * a.pro_last + 1];
 #pragma unroll
                 for (int j = 0; j < 16; j++) {
+                    const uint64_t ds = dsrc[glob(e_far(j))];
+                    const uint64_t dl = a.pro_k1 ? barrett64(ds, qlast, rlast) : ds;
+                    const uint64_t dj = a.pro_k1 ? barrett64(ds, qj, rj) : job.in[glob(e_far(j))];
                     // coefficient of the dropped limb of the ModDown result, canonical mod q_last
-                    const double r = fp_canonical(
-                        fp_from_u64(tsrc[glob(e_far(j))]) - fp_mulmod(fp_from_u64(dsrc[glob(e_far(j))]), wlast, ml), ml);
-                    v[j] = fp_mulmod(fp_from_u64(job.in[glob(e_far(j))]), w, c.m) + fp_reduce(r, c.m);
+                    const double r = fp_canonical(fp_from_u64(tsrc[glob(e_far(j))]) - fp_mulmod(fp_from_u64(dl), wlast, ml), ml);
+                    v[j] = fp_mulmod(fp_from_u64(dj), w, c.m) + fp_reduce(r, c.m);
                 }
             } else if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE) {
                 // one source limb for every limb: it may exceed this limb's prime, so reduce first
@@ -305,10 +309,14 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
             const uint64_t *dsrc = a.pro_src2 + ((size_t)job.poly * a.pro2_poly_stride << a.log_n);
             const uint64_t ql = a.moduli[a.pro_last];
             const Shoup w = load_shoup(a.pro_w, job.limb), wlast = load_shoup(a.pro_w, a.pro_last);
+            const uint64_t rlast = a.barrett[2 * a.pro_last + 1];
 #pragma unroll
             for (int j = 0; j < 16; j++) {
-                const uint64_t r = sub_mod(tsrc[glob(e_far(j))], mul_shoup(dsrc[glob(e_far(j))], wlast, ql), ql);
-                v[j] = add_mod(mul_shoup(job.in[glob(e_far(j))], w, q), barrett64(r, q, r1), q);
+                const uint64_t ds = dsrc[glob(e_far(j))];
+                const uint64_t dl = a.pro_k1 ? barrett64(ds, ql, rlast) : ds;
+                const uint64_t dj = a.pro_k1 ? barrett64(ds, q, r1) : job.in[glob(e_far(j))];
+                const uint64_t r = sub_mod(tsrc[glob(e_far(j))], mul_shoup(dl, wlast, ql), ql);
+                v[j] = add_mod(mul_shoup(dj, w, q), barrett64(r, q, r1), q);
             }
         } else {
 #pragma unroll
@@ -386,12 +394,17 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
                 const FpMod ml = fp_ctx(a, a.pro_last).m;
                 const double wd = fp_from_u64(a.pro_w[2 * job.limb]), wl = fp_from_u64(a.pro_w[2 * a.pro_last]);
                 const FpTw w{wd, wd * c.m.qinv}, wlast{wl, wl * ml.qinv};
+                const uint64_t qj = a.moduli[job.table], rj = a.barrett[2 * job.table + 1];
+                const uint64_t qlast = a.moduli[a.pro_last], rlast = a.barrett[2 * a.pro_last + 1];
                 for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
                     uint32_t row = e >> LOGC, col = e & (C - 1);
                     const size_t g = (size_t)row * 256 + col0 + col;
+                    const uint64_t ds = dsrc[g];
+                    const uint64_t dl = a.pro_k1 ? barrett64(ds, qlast, rlast) : ds;
+                    const uint64_t dj = a.pro_k1 ? barrett64(ds, qj, rj) : src[g];
                     // coefficient of the dropped limb of the ModDown result, canonical mod q_last
-                    const double r = fp_canonical(fp_from_u64(bsrc[g]) - fp_mulmod(fp_from_u64(dsrc[g]), wlast, ml), ml);
-                    ld[skew(e)] = fp_mulmod(fp_from_u64(src[g]), w, c.m) + fp_reduce(r, c.m);
+                    const double r = fp_canonical(fp_from_u64(bsrc[g]) - fp_mulmod(fp_from_u64(dl), wlast, ml), ml);
+                    ld[skew(e)] = fp_mulmod(fp_from_u64(dj), w, c.m) + fp_reduce(r, c.m);
                 }
             } else if (a.pro_mode == NTT_PRO_SOURCE_REDUCE) {
                 const uint64_t q = a.moduli[job.table], r1 = a.barrett[2 * job.table + 1];
@@ -457,11 +470,15 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
         const uint64_t *dsrc = a.pro_src2 + ((size_t)job.poly * a.pro2_poly_stride << a.log_n);
         const uint64_t ql = a.moduli[a.pro_last];
         const Shoup w = load_shoup(a.pro_w, job.limb), wlast = load_shoup(a.pro_w, a.pro_last);
+        const uint64_t rlast = a.barrett[2 * a.pro_last + 1];
         for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
             uint32_t row = e >> LOGC, col = e & (C - 1);
             const size_t g = (size_t)row * 256 + col0 + col;
-            const uint64_t r = sub_mod(tsrc[g], mul_shoup(dsrc[g], wlast, ql), ql);
-            lds[skew(e)] = add_mod(mul_shoup(job.in[g], w, q), barrett64(r, q, r1), q);
+            const uint64_t ds = dsrc[g];
+            const uint64_t dl = a.pro_k1 ? barrett64(ds, ql, rlast) : ds;
+            const uint64_t dj = a.pro_k1 ? barrett64(ds, q, r1) : job.in[g];
+            const uint64_t r = sub_mod(tsrc[g], mul_shoup(dl, wlast, ql), ql);
+            lds[skew(e)] = add_mod(mul_shoup(dj, w, q), barrett64(r, q, r1), q);
         }
     } else {
         for (uint32_t e = threadIdx.x; e < tile_elems; e += kRowThreads) {
