@@ -1048,7 +1048,10 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         const bool fp_batch = items > 1 && ctx->fp_inner && lv->batched && fp_for_level(ctx, L) && n >= 512 &&
                               !galois_elt && !add_c0;
         if (tin) return HE_E_INVALID_ARGUMENT;
-        if (int rc = modup_impl(ctx, L, src, galois_elt ? L : c_item_stride, items, y, tmp, s, fp_batch)) return rc;
+        // (batched levels: neither kernel needs the copy of a digit's own limbs into y)
+        const bool skip_own = fp_batch || lv->batched;
+        const uint32_t src_stride = galois_elt ? L : c_item_stride;
+        if (int rc = modup_impl(ctx, L, src, src_stride, items, y, tmp, s, skip_own)) return rc;
         EvkPtrs ptrs;
         memset(&ptrs, 0, sizeof(ptrs));
         for (uint32_t d = 0; d < lv->beta; d++) {
@@ -1062,7 +1065,8 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
             return HE_OK;
         }
         HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, cx, L, ctx->size_p, ctx->size_q, lv->beta, 0, false,
-                                    fold_ct, fold_w, items, 2 * (size_t)L * n, S(s), add_c0, galois_elt, ctx->d_p_mod_q));
+                                    fold_ct, fold_w, items, 2 * (size_t)L * n, S(s), add_c0, galois_elt, ctx->d_p_mod_q,
+                                    skip_own ? src : nullptr, (size_t)src_stride * n));
     }
     return HE_OK;
 }

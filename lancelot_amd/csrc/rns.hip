@@ -374,6 +374,8 @@ struct InnerArgs {
     size_t y_item_stride, out_item_stride, fold_item_stride;   // blockIdx.z = item (words between items)
     const uint64_t *add_c0, *p_mod_q;
     uint32_t add_elt;
+    const uint64_t *own;            // optional: the key-switch input [L][N]; a digit's own limbs are read from it (their
+    size_t own_item_stride;         // slots in y were left unwritten), items own_item_stride words apart
 };
 
 // grid: (N / 256, L + K, items).  Streams beta digit limbs of y and 2 beta key limbs, writes (or accumulates) the
@@ -390,9 +392,11 @@ __global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
     // (the argument struct stays untouched: a modified copy would move its pointer table to scratch memory)
     const uint64_t *y = p.y + blockIdx.z * p.y_item_stride;
     uint64_t *out = p.out + blockIdx.z * p.out_item_stride;
+    const uint64_t *own = p.own ? p.own + blockIdx.z * p.own_item_stride + ((size_t)t << p.log_n) : nullptr;
+    const uint32_t own_d = (own && t < p.L) ? t / p.K : 0xffffffffu;
     U128 a0{0, 0}, a1{0, 0};
     for (uint32_t d = 0; d < p.beta; d++) {
-        const uint64_t v = y[(((size_t)d * LK + t) << p.log_n) + src];
+        const uint64_t v = d == own_d ? own[src] : y[(((size_t)d * LK + t) << p.log_n) + src];
         const uint64_t *k = p.evk.p[d];
         mac128(a0, v, k[key_off]);
         mac128(a1, v, k[key_off + key_poly]);
@@ -892,11 +896,12 @@ hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_
 hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
                                 const uint64_t *fold_ct, const uint64_t *fold_w, uint32_t items, size_t fold_item_stride,
-                                hipStream_t s, const uint64_t *add_c0, uint32_t add_elt, const uint64_t *p_mod_q) {
+                                hipStream_t s, const uint64_t *add_c0, uint32_t add_elt, const uint64_t *p_mod_q,
+                                const uint64_t *own, size_t own_item_stride) {
     const size_t n = (size_t)1 << t.log_n;
     InnerArgs p{y, out, t.moduli, t.barrett, evk, L, K, size_q, beta, t.log_n, galois_elt, accumulate ? 1 : 0,
                 fold_ct, fold_w, (size_t)beta * (L + K) * n, 2 * (size_t)(L + K) * n, fold_item_stride,
-                add_c0, p_mod_q, add_elt};
+                add_c0, p_mod_q, add_elt, own, own_item_stride};
     if (items == 0 || items > 65535 || (add_c0 && (items != 1 || !p_mod_q))) return hipErrorInvalidValue;
     hipLaunchKernelGGL(inner_product_kernel, dim3((1u << t.log_n) / kThreads, L + K, items), dim3(kThreads), 0, s, p);
     return hipGetLastError();
