@@ -96,6 +96,26 @@ __global__ __launch_bounds__(kThreads) void encode_load_kernel(const double *re,
     if (i < slots) v[i] = i < count ? double2{re[i], im ? im[i] : 0.0} : double2{0.0, 0.0};
 }
 
+// The largest magnitude of an item's coefficients (the bit patterns of non-negative doubles order like the values):
+// reduced over the wave, then over the workgroup, one atomic per workgroup.  Atomics on one address are served one
+// after the other: one per thread took most of the rounding kernel's time, one per wave still half of it.  Every
+// thread of the workgroup calls this.
+__device__ __forceinline__ void block_max_to(unsigned long long *dst, unsigned long long m) {
+    __shared__ unsigned long long wave_max[kThreads / 64];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        const unsigned long long o = __shfl_xor(m, d);
+        m = o > m ? o : m;
+    }
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < kThreads / 64; w++) m = wave_max[w] > m ? wave_max[w] : m;
+        if (m) atomicMax(dst, m);
+    }
+}
+
 // coefficient c of the plaintext: real parts fill the first half, imaginary parts the second, `gap` apart;
 // value i comes from position bitrev(i) of the transformed vector
 __global__ __launch_bounds__(kThreads) void encode_round_kernel(const double2 *v, uint32_t log_slots, uint32_t gap,
@@ -112,9 +132,35 @@ __global__ __launch_bounds__(kThreads) void encode_round_kernel(const double2 *v
         const uint32_t i = k / gap;
         const double2 z = v[__brev(i) >> (32 - log_slots)];
         val = round((imag ? z.y : z.x) * fix);
-        atomicMax(max_bits, (unsigned long long)__double_as_longlong(fabs(val)));
     }
     coeffs[c] = val;
+    block_max_to(max_bits, (unsigned long long)__double_as_longlong(fabs(val)));
+}
+
+// The same for full packing (gap = 1, at least 256 slots): the bit reversal as a tiled transpose through LDS, so that
+// both the reads of the transformed vector and the writes of the coefficients touch whole cache lines (with one thread
+// per coefficient every lane of a wave reads a line of its own).  Slot i = (top 4 bits | middle | low 4 bits); a
+// workgroup takes one value of the middle bits: thread (x, y) reads the slot with low bits y and top bits brev4(x),
+// which sits at position (brev4(y) | brev(middle) | x) of the vector (consecutive in x), and writes the slot with low
+// bits x and top bits brev4(y) (consecutive in x), real part to coefficient i, imaginary part to coefficient N/2 + i.
+__global__ __launch_bounds__(kThreads) void encode_round_tiled_kernel(const double2 *v, uint32_t log_slots, uint32_t half,
+                                                                      double fix, double *coeffs, unsigned long long *max_bits) {
+    __shared__ double2 tile[16][17];
+    const uint32_t x = threadIdx.x & 15, y = threadIdx.x >> 4, mid = blockIdx.x, mid_bits = log_slots - 8;
+    v += (size_t)blockIdx.y << log_slots;
+    coeffs += (size_t)blockIdx.y * 2 * half;
+    max_bits += blockIdx.y;
+    const uint32_t rmid = mid_bits ? __brev(mid) >> (32 - mid_bits) : 0;
+    const uint32_t brev4_y = __brev(y) >> 28;
+    tile[y][x] = v[(brev4_y << (log_slots - 4)) | (rmid << 4) | x];
+    __syncthreads();
+    const double2 z = tile[x][y];
+    const uint32_t i = (brev4_y << (log_slots - 4)) | (mid << 4) | x;
+    const double re = round(z.x * fix), im = round(z.y * fix);
+    coeffs[i] = re;
+    coeffs[half + i] = im;
+    const double big = fabs(re) > fabs(im) ? fabs(re) : fabs(im);
+    block_max_to(max_bits, (unsigned long long)__double_as_longlong(big));
 }
 
 constexpr int kMaxComposeLimbs = 64;
@@ -202,8 +248,12 @@ hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double
                        reinterpret_cast<unsigned long long *>(max_bits), value_stride);
     hipError_t e = run_fft<true>(v, slots, items, t, s);
     if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(encode_round_kernel, blocks(n), dim3(kThreads), 0, s, v, log_slots, (n / 2) / slots, n / 2,
-                       scale / (double)slots, coeffs, reinterpret_cast<unsigned long long *>(max_bits));
+    if (slots == n / 2 && log_slots >= 8)
+        hipLaunchKernelGGL(encode_round_tiled_kernel, dim3(slots / kThreads, items), dim3(kThreads), 0, s, v, log_slots, n / 2,
+                           scale / (double)slots, coeffs, reinterpret_cast<unsigned long long *>(max_bits));
+    else
+        hipLaunchKernelGGL(encode_round_kernel, blocks(n), dim3(kThreads), 0, s, v, log_slots, (n / 2) / slots, n / 2,
+                           scale / (double)slots, coeffs, reinterpret_cast<unsigned long long *>(max_bits));
     return hipGetLastError();
 }
 

@@ -78,11 +78,12 @@ std::vector<CAHELGPUCiphertext> CAHELGPUCKKSEncoder::encode_encrypt_many(const C
     check_status(he_encrypt_batch(h, L, (uint32_t)items, pk.pk_.data(), context.prng_key(), context.next_stream(3 * items),
                                   batch.get(), ews.get(), st),
                  "he_encrypt_batch");
+    // one ciphertext object per message, each a slice of the batch (no copies)
     std::vector<CAHELGPUCiphertext> out(items);
+    auto shared = std::make_shared<DeviceBuffer>(std::move(batch));
     for (std::size_t k = 0; k < items; k++) {
         CAHELGPUCiphertext &ct = out[k];
-        ct.data_.allocate(words);
-        check_status(he_memcpy_d2d(ct.data(), batch.get() + k * words, words * sizeof(uint64_t), st), "copy");
+        ct.data_ = DeviceBuffer::slice(shared, k * words, words);
         ct.size_ = 2;
         ct.coeff_modulus_size_ = L;
         ct.poly_modulus_degree_ = n;

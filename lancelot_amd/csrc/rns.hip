@@ -724,6 +724,10 @@ struct SampleArgs {
 
 // ternary / error / gauss: one thread = one ChaCha block = 16 (ternary) or 8 coefficients, the same
 // signed value written to every limb.  uniform: one thread = one block = 4 residues of one limb.
+// KIND is a template parameter so that the loops over the block's words unroll and the words stay in registers (with
+// a run-time count the array lived in scratch memory); a thread's 16 or 8 consecutive output words leave as 16-byte
+// stores.
+template <int KIND>
 __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
     const uint32_t n = 1u << p.log_n;
     const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
@@ -731,41 +735,51 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
     const uint64_t stream = p.stream + (uint64_t)blockIdx.y * p.stream_stride;
     uint64_t *out = p.out + blockIdx.y * p.out_item_stride;
     uint32_t w[16];
-    if (p.kind == SAMPLE_UNIFORM) {
+    if (KIND == SAMPLE_UNIFORM) {
         const uint32_t per_limb = n / 4;
         if (b >= per_limb * p.map.limbs) return;
         const uint32_t limb = b / per_limb, blk = b % per_limb;
         const uint32_t table = map_table(p.map, limb);
         const uint64_t q = p.moduli[table], r0 = p.barrett[2 * table], r1 = p.barrett[2 * table + 1];
         chacha20_block(p.key, b, stream, w);
+        uint64_t r[4];
+#pragma unroll
         for (int e = 0; e < 4; e++) {
             uint64_t lo = ((uint64_t)w[4 * e + 1] << 32) | w[4 * e];
             uint64_t hi = ((uint64_t)w[4 * e + 3] << 32) | w[4 * e + 2];
-            out[((size_t)limb << p.log_n) + 4 * blk + e] = barrett128(lo, hi, q, r0, r1);
+            r[e] = barrett128(lo, hi, q, r0, r1);
         }
+        ulonglong2 *dst = reinterpret_cast<ulonglong2 *>(out + ((size_t)limb << p.log_n) + 4 * blk);
+        dst[0] = ulonglong2{r[0], r[1]};
+        dst[1] = ulonglong2{r[2], r[3]};
         return;
     }
-    const uint32_t per_block = p.kind == SAMPLE_TERNARY ? 16 : 8;
+    constexpr int per_block = KIND == SAMPLE_TERNARY ? 16 : 8;
     if (b >= n / per_block) return;
     chacha20_block(p.key, b, stream, w);
-    for (uint32_t e = 0; e < per_block; e++) {
-        int v;
-        if (p.kind == SAMPLE_TERNARY) {
-            v = (int)(((uint64_t)w[e] * 3) >> 32) - 1;
-        } else if (p.kind == SAMPLE_ERROR) {
-            v = __popc(w[2 * e] & 0x1FFFFFu) - __popc(w[2 * e + 1] & 0x1FFFFFu);
+    int v[per_block];
+#pragma unroll
+    for (int e = 0; e < per_block; e++) {
+        if (KIND == SAMPLE_TERNARY) {
+            v[e] = (int)(((uint64_t)w[e] * 3) >> 32) - 1;
+        } else if (KIND == SAMPLE_ERROR) {
+            v[e] = __popc(w[2 * e] & 0x1FFFFFu) - __popc(w[2 * e + 1] & 0x1FFFFFu);
         } else {
             uint64_t u = ((uint64_t)w[2 * e + 1] << 32) | w[2 * e];
             const bool neg = u >> 63;
             u &= 0x7FFFFFFFFFFFFFFFull;
             uint32_t mag = 0;
             while (mag < p.cdt_len && u >= p.cdt[mag]) mag++;
-            v = neg ? -(int)mag : (int)mag;
+            v[e] = neg ? -(int)mag : (int)mag;
         }
-        for (uint32_t limb = 0; limb < p.map.limbs; limb++) {
-            const uint64_t q = p.moduli[map_table(p.map, limb)];
-            out[((size_t)limb << p.log_n) + per_block * b + e] = v < 0 ? q - (uint64_t)(-v) : (uint64_t)v;
-        }
+    }
+    for (uint32_t limb = 0; limb < p.map.limbs; limb++) {
+        const uint64_t q = p.moduli[map_table(p.map, limb)];
+        ulonglong2 *dst = reinterpret_cast<ulonglong2 *>(out + ((size_t)limb << p.log_n) + (size_t)per_block * b);
+#pragma unroll
+        for (int e = 0; e < per_block; e += 2)
+            dst[e / 2] = ulonglong2{v[e] < 0 ? q - (uint64_t)(-v[e]) : (uint64_t)v[e],
+                                    v[e + 1] < 0 ? q - (uint64_t)(-v[e + 1]) : (uint64_t)v[e + 1]};
     }
 }
 
@@ -1078,8 +1092,17 @@ hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stre
     if (items == 0 || items > 65535) return hipErrorInvalidValue;
     const uint32_t n = 1u << t.log_n;
     uint32_t blocks = kind == SAMPLE_UNIFORM ? (n / 4) * map.limbs : (kind == SAMPLE_TERNARY ? n / 16 : n / 8);
+    // (a thread's words leave as 16-byte stores)
+    if ((reinterpret_cast<uintptr_t>(out) & 15) || (out_item_stride & 1)) return hipErrorInvalidValue;
     SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind, stream_stride, out_item_stride};
-    hipLaunchKernelGGL(sample_kernel, dim3((blocks + kThreads - 1) / kThreads, items), dim3(kThreads), 0, s, p);
+    const dim3 grid((blocks + kThreads - 1) / kThreads, items);
+    switch (kind) {
+        case SAMPLE_UNIFORM: hipLaunchKernelGGL(sample_kernel<SAMPLE_UNIFORM>, grid, dim3(kThreads), 0, s, p); break;
+        case SAMPLE_TERNARY: hipLaunchKernelGGL(sample_kernel<SAMPLE_TERNARY>, grid, dim3(kThreads), 0, s, p); break;
+        case SAMPLE_ERROR: hipLaunchKernelGGL(sample_kernel<SAMPLE_ERROR>, grid, dim3(kThreads), 0, s, p); break;
+        case SAMPLE_GAUSS: hipLaunchKernelGGL(sample_kernel<SAMPLE_GAUSS>, grid, dim3(kThreads), 0, s, p); break;
+        default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 
