@@ -367,7 +367,8 @@ int he_decrypt_decode_batch(const he_context *ctx, const uint64_t *const *d_cts,
 
 /* ---- samplers (replace sample_ternary_poly / sample_error_poly / sample_uniform_poly, src/prng.cu:143-242,
  *      and the OpenFHE Gaussian of src/secretkey.cu:632-649) ----
- * ChaCha20 block function keyed by key[8]; `stream_id` selects an independent stream.  out: [limbs][N],
+ * ChaCha20 block function keyed by key[8]; `stream_id` selects an independent stream.  out: [limbs][N], 16-byte
+ * aligned (HE_E_INVALID_ARGUMENT otherwise: the words leave as 16-byte stores),
  * limb i mod table first_table+i (i < split) / tail_table + i - split.
  * kind: 0 ternary {-1,0,1}; 1 centred binomial (21 - 21 bits); 2 uniform residues; 3 discrete Gaussian by
  * the cumulative table cdt[cdt_len] (DEVICE pointer, cdt[i] = floor(2^63 P(|X| <= i))). */

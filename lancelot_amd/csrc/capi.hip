@@ -1406,7 +1406,7 @@ static int sample_impl(const he_context *ctx, int kind, const uint32_t key[8], u
                        uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail, const uint64_t *cdt,
                        uint32_t cdt_len, uint32_t items, he_stream s) {
     if (!ctx || !key || !out || kind < 0 || kind > 3 || (kind == SAMPLE_GAUSS && (!cdt || !cdt_len)) || items == 0 ||
-        items > 16384)
+        items > 16384 || (reinterpret_cast<uintptr_t>(out) & 15))
         return HE_E_INVALID_ARGUMENT;
     if (int rc = check_map(ctx, limbs, first, split, tail)) return rc;
     ChaChaKey k;

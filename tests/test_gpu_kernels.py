@@ -906,3 +906,13 @@ def test_issue_rate_probe(capi):
     fma, mad, mul, add, mfma, both = rate
     assert add > 1.5 * fma and add > 1.5 * mad and add > 1.5 * mul, rate
     assert both < 0.75 * (fma + mfma), rate
+
+
+def test_sampler_refuses_a_misaligned_output(small, capi):
+    """The sampler stores 16 bytes at a time: an output pointer that is only 8-byte aligned is refused."""
+    cahel, parms, ctx, p = small
+    lib, h = capi.lib(), ctx.he_handle()
+    buf = DeviceArray(capi, shape=(2 * p.n + 2,))
+    key = (C.c_uint32 * 8)(*range(8))
+    assert lib.he_sample(h, 0, key, 7, buf.ptr + 8, 2, 0, 2, 0, None, 0, None) == -1
+    capi.check(lib.he_sample(h, 0, key, 7, buf.ptr + 16, 2, 0, 2, 0, None, 0, None))
