@@ -167,11 +167,15 @@ constexpr int kMaxComposeLimbs = 64;
 
 // Garner's mixed-radix composition of one coefficient, centred around zero, as a double divided by the scale.
 // thread s < slots: real part of value s, else imaginary part of value s - slots; stored at position bitrev.
-__global__ __launch_bounds__(kThreads) void decode_compose_kernel(const uint64_t *res, uint32_t limbs, uint32_t log_n,
+// LIMBS > 0: the number of limbs at compile time (the digits then stay in registers; with a run-time count the array
+// lives in scratch memory), 0: any number up to kMaxComposeLimbs.
+template <int LIMBS>
+__global__ __launch_bounds__(kThreads) void decode_compose_kernel(const uint64_t *res, uint32_t limbs_rt, uint32_t log_n,
                                                                   uint32_t log_slots, uint32_t gap, double inv_scale,
                                                                   const uint64_t *moduli, const uint64_t *barrett,
                                                                   const uint64_t *garner_inv, uint32_t garner_stride,
                                                                   double2 *v) {
+    const uint32_t limbs = LIMBS ? (uint32_t)LIMBS : limbs_rt;
     const uint32_t s = blockIdx.x * kThreads + threadIdx.x;
     const uint32_t slots = 1u << log_slots, half = 1u << (log_n - 1);
     if (s >= 2 * slots) return;
@@ -180,10 +184,12 @@ __global__ __launch_bounds__(kThreads) void decode_compose_kernel(const uint64_t
     const bool imag = s >= slots;
     const uint32_t i0 = imag ? s - slots : s;
     const size_t coeff = (imag ? half : 0) + (size_t)i0 * gap;
-    uint64_t d[kMaxComposeLimbs];
+    uint64_t d[LIMBS ? LIMBS : kMaxComposeLimbs];
+#pragma unroll
     for (uint32_t i = 0; i < limbs; i++) {
         const uint64_t q = moduli[i], r0 = barrett[2 * i], r1 = barrett[2 * i + 1];
         uint64_t t = res[((size_t)i << log_n) + coeff];
+#pragma unroll
         for (uint32_t j = 0; j < i; j++) {
             const uint64_t dj = barrett64(d[j], q, r1);
             t = mul_mod(sub_mod(t, dj, q), garner_inv[(size_t)i * garner_stride + j], q, r0, r1);
@@ -191,24 +197,37 @@ __global__ __launch_bounds__(kThreads) void decode_compose_kernel(const uint64_t
         d[i] = t;
     }
     // negative iff the digits, read from the top, exceed those of (Q - 1) / 2, whose digits are (q_i - 1) / 2
-    bool negative = false;
-    for (uint32_t i = limbs; i-- > 0;) {
+    // (written without early exits so that the loops unroll: `decided` / `carry` play the part of the breaks)
+    bool negative = false, decided = false;
+#pragma unroll
+    for (uint32_t k = 0; k < limbs; k++) {
+        const uint32_t i = limbs - 1 - k;
         const uint64_t h = (moduli[i] - 1) >> 1;
-        if (d[i] != h) {
+        if (!decided && d[i] != h) {
             negative = d[i] > h;
-            break;
+            decided = true;
         }
     }
     if (negative) {
         // Q - v = (Q - 1 - v) + 1: digit-wise complement, then increment
-        for (uint32_t i = 0; i < limbs; i++) d[i] = moduli[i] - 1 - d[i];
+        bool carry = true;
+#pragma unroll
         for (uint32_t i = 0; i < limbs; i++) {
-            if (++d[i] < moduli[i]) break;
-            d[i] = 0;
+            uint64_t x = moduli[i] - 1 - d[i];
+            if (carry) {
+                x++;
+                carry = x >= moduli[i];
+                if (carry) x = 0;
+            }
+            d[i] = x;
         }
     }
     double acc = 0.0;
-    for (uint32_t i = limbs; i-- > 0;) acc = acc * (double)moduli[i] + (double)d[i];
+#pragma unroll
+    for (uint32_t k = 0; k < limbs; k++) {
+        const uint32_t i = limbs - 1 - k;
+        acc = acc * (double)moduli[i] + (double)d[i];
+    }
     const double val = (negative ? -acc : acc) * inv_scale;
     double *slot = reinterpret_cast<double *>(&v[__brev(i0) >> (32 - log_slots)]);
     slot[imag ? 1 : 0] = val;
@@ -262,9 +281,18 @@ hipError_t launch_ckks_decode(const FftTables &t, const Tables &tab, const uint6
                               double2 *v, uint32_t items, hipStream_t s) {
     const uint32_t n = 1u << t.log_n, log_slots = 31 - __builtin_clz(slots);
     if (limbs == 0 || limbs > (uint32_t)kMaxComposeLimbs || items == 0 || items > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(decode_compose_kernel, dim3((2 * slots + kThreads - 1) / kThreads, items), dim3(kThreads), 0, s, res,
-                       limbs, t.log_n, log_slots, (n / 2) / slots, 1.0 / scale, tab.moduli, tab.barrett, garner_inv,
-                       garner_stride, v);
+    const dim3 grid((2 * slots + kThreads - 1) / kThreads, items);
+#define HE_COMPOSE(L)                                                                                                     \
+    hipLaunchKernelGGL(decode_compose_kernel<L>, grid, dim3(kThreads), 0, s, res, limbs, t.log_n, log_slots, (n / 2) / slots, \
+                       1.0 / scale, tab.moduli, tab.barrett, garner_inv, garner_stride, v)
+    switch (limbs) {
+        case 1: HE_COMPOSE(1); break;
+        case 2: HE_COMPOSE(2); break;
+        case 3: HE_COMPOSE(3); break;
+        case 4: HE_COMPOSE(4); break;
+        default: HE_COMPOSE(0); break;
+    }
+#undef HE_COMPOSE
     return run_fft<false>(v, slots, items, t, s);
 }
 
