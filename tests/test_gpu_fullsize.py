@@ -64,7 +64,12 @@ def test_c1_hmult_relin_rescale_bit_exact(oracle):
     pt = sk.decrypt(ctx, cx)
     assert (pt.to_numpy() == ks.decrypt(want, O.gauss_cdt())).all()
     got = np.array(enc.decode(ctx, pt))
-    assert np.max(np.abs(got - x * y)) < 1e-2           # scale 2^40 after a 50-bit rescale: about 2^30 left
+    # 2^30 of scale left.  The reference's rescale floors (src/rns.cu:507-570: no rounding offset), which leaves a mean
+    # of 1/2 on every coefficient of both polynomials; through c1 * s that is (1/2) (1 + X + ... + X^(N-1)) s, whose
+    # value in the slot nearest to X = 1 is about N / pi * sqrt(2 N / 3) / scale = 5e-4 here for a typical secret
+    # (measured with this seed: 9.8e-5 in slot 0, 1.3e-6 in the median slot)
+    assert np.max(np.abs(got - x * y)) < 3e-4
+    assert np.median(np.abs(got - x * y)) < 5e-6
 
 
 @pytest.mark.parametrize("inner", ["fused", "fp_kernel"])
@@ -160,7 +165,10 @@ def test_c3_hmult_properties(bench_world):
     c.rescale_to_next_inplace(ctx, xy)
     assert xy.chain_index() == 2
     got = _decode(w, xy)
-    assert np.max(np.abs(got - w["x"] * w["y"])) < 1e-2                       # about 2^30 of scale left
+    # about 2^30 of scale left; the floor-style rescale's bias in the slots nearest to X = 1 is about
+    # N / pi * sqrt(2 N / 3) / scale = 4e-3 at this degree (measured 3.1e-3 in slot 0, 5.1e-6 in the median slot)
+    assert np.max(np.abs(got - w["x"] * w["y"])) < 5e-3
+    assert np.median(np.abs(got - w["x"] * w["y"])) < 2e-5
     # the same product through the fused call
     fused = c.ciphertext(ctx)
     c.multiply(ctx, w["cx"], w["cy"], fused)
@@ -225,7 +233,7 @@ def test_c4_rotations(bench_world):
         c.add_inplace(ctx, acc, tmp)
     total = _decode(w, acc)
     want = float(np.sum(w["x"]))
-    assert np.max(np.abs(total - want)) < 2.0 ** -10 * max(1.0, abs(want))
+    assert np.max(np.abs(total - want)) < 1e-5 * max(1.0, abs(want))       # measured 3.7e-6
     # hoisted rotations of one ciphertext: sum of the rotated copies
     hoisted = c.hoisting(ctx, w["cx"], w["glk"], [1, 2, 4])
     ref = sum(np.roll(base, -s) for s in (1, 2, 4))
@@ -280,3 +288,171 @@ def test_hoisted_rotations_batch_workgroup_orders(oracle, monkeypatch, switch):
         want = p.hoisting(cts[k], elts, [host_keys[i % 2] for i in range(len(steps))])
         want = np.stack([p.add(want[b], cts[k][b]) for b in range(2)])
         assert (got[k] == want).all(), k
+
+
+@pytest.mark.parametrize("kind", ["gather", "block_local"])
+def test_hoisted_rotations_benchmark_shape(oracle, kind):
+    """he_hoisted_rotations and he_hoisted_rotations_batch (3 ciphertexts, with and without the input added) at
+    N = 2^16, L = 24, K = 8 (three digits): a step set that gathers from memory (1, 2, 3, 5) and one whose automorphisms
+    stay inside 256-word blocks (multiples of N / 512 = 128), two random keys alternating between the steps, every limb
+    against the oracle's hoisting (src/evaluate.cu:2412-2629)."""
+    import ctypes as C
+    from gpu_util import DeviceArray, make_pair, rand_limbs
+    from lancelot_amd import capi
+    cahel, parms, ctx, p = make_pair(oracle, 16, [50] * 32, 8)
+    lib, h = capi.lib(), ctx.he_handle()
+    rng = np.random.default_rng(1816)
+    L, K, items = 24, 8, 3
+    beta = L // K
+    steps = [1, 2, 3, 5] if kind == "gather" else [128 * k for k in (1, 2, 3, 5)]
+    elts = [pow(5, s, 2 * p.n) for s in steps]
+    assert all(((e - 1) % 512 == 0) == (kind == "block_local") for e in elts)
+    host_keys = [[rand_limbs(p, rng, range(L + K), n_polys=2) for _ in range(beta)] for _ in range(2)]
+    dev_keys = [[DeviceArray(capi, host=k) for k in ks] for ks in host_keys]
+    flat = capi.evk_array([dev_keys[i % 2][d].ptr for i in range(len(steps)) for d in range(beta)])
+    d_elts = (C.c_uint32 * len(steps))(*elts)
+    cts = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
+    want = [p.hoisting(cts[k], elts, [host_keys[i % 2] for i in range(len(steps))]) for k in range(items)]
+    din = DeviceArray(capi, host=cts)
+    ws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+    out = DeviceArray(capi, shape=(2, L, p.n))
+    capi.check(lib.he_hoisted_rotations(h, L, din.at(2 * L * p.n), flat, d_elts, len(steps), out.ptr, ws.ptr, None))
+    assert (out.numpy() == want[1]).all()
+    wsb = DeviceArray(capi, shape=(lib.he_keyswitch_batch_workspace_words(h, L, items),))
+    dout = DeviceArray(capi, shape=(items, 2, L, p.n))
+    for add_input in (0, 1):
+        capi.check(lib.he_hoisted_rotations_batch(h, L, items, din.ptr, flat, d_elts, len(steps), add_input, dout.ptr,
+                                                  wsb.ptr, None))
+        got = dout.numpy()
+        for k in range(items):
+            w = want[k] if not add_input else np.stack([p.add(want[k][b], cts[k][b]) for b in range(2)])
+            assert (got[k] == w).all(), (add_input, k)
+    assert (din.numpy() == cts).all()
+
+
+def _centred_distance(a, b, q):
+    d = (a.astype(np.int64) - b.astype(np.int64)) % q
+    return np.minimum(d, q - d)
+
+
+@pytest.mark.parametrize("bits,size_p", [([50] * 32, 8), ([60, 40, 40, 60], 1)])
+@pytest.mark.parametrize("slots", [32768, 256])
+def test_encoder_at_full_degree(oracle, bits, size_p, slots):
+    """he_ckks_encode / he_ckks_decode and their batch forms (he_ckks_encode_batch, he_decrypt_decode_batch) at
+    N = 2^16 with all 32,768 slots (the special FFT then has stages wider than a workgroup's LDS tile) and with a
+    sparse slot count, on 24 limbs (the general Garner composition) and on Lancelot's 3 limbs (the one templated on
+    the limb count): encoded coefficients within one unit of the oracle's encoder, decoded values within 2^-20 of its
+    decoder and of the message (src/ckks.cu:104-209, 292-465)."""
+    import ctypes as C
+    from gpu_util import DeviceArray, make_pair
+    from lancelot_amd import capi
+    cahel, parms, ctx, p = make_pair(oracle, 16, bits, size_p)
+    lib, h = capi.lib(), ctx.he_handle()
+    limbs, n, items = p.size_q, p.n, 3
+    count = slots - 5
+    scale = 2.0 ** 40
+    rng = np.random.default_rng(slots + limbs)
+    z = rng.uniform(-1, 1, (items, count)) + 1j * rng.uniform(-1, 1, (items, count))
+    o_enc = oracle.Encoder(p)
+    want = [o_enc.encode(z[k], scale, limbs, slots) for k in range(items)]
+    want_coeff = [p.ntt_inv(w.copy()) for w in want]
+    re = DeviceArray(capi, host=np.ascontiguousarray(z.real))
+    im = DeviceArray(capi, host=np.ascontiguousarray(z.imag))
+    ws = DeviceArray(capi, shape=(lib.he_ckks_workspace_words(h, limbs),))
+    out = DeviceArray(capi, shape=(limbs, n))
+    capi.check(lib.he_ckks_encode(h, re.ptr, im.ptr, count, slots, scale, limbs, out.ptr, ws.ptr, None))
+    got = out.numpy()
+    got_coeff = p.ntt_inv(got.copy())
+    for i in range(limbs):
+        assert _centred_distance(got_coeff[i], want_coeff[0][i], p.moduli[i]).max() <= 1, i
+    q0 = p.moduli[0]
+    centred = np.where(got_coeff[0] > q0 // 2, got_coeff[0].astype(np.int64) - q0, got_coeff[0].astype(np.int64))
+    assert ws.numpy().view(np.float64)[0] == np.abs(centred).max()
+    dec = DeviceArray(capi, shape=(2 * slots,), dtype=np.float64)
+    capi.check(lib.he_ckks_decode(h, out.ptr, limbs, slots, scale, dec.ptr, ws.ptr, None))
+    v = dec.numpy().reshape(slots, 2)
+    got_z = v[:, 0] + 1j * v[:, 1]
+    padded = np.zeros((items, slots), dtype=np.complex128)
+    padded[:, :count] = z
+    assert np.max(np.abs(got_z - o_enc.decode(got, scale, slots))) < REL
+    assert np.max(np.abs(got_z - padded[0])) < REL
+    # the batch forms: three messages into polynomial 0 of three ciphertexts, whose polynomial 1 is zero, so that
+    # decryption returns the plaintext whatever the key
+    wsb = DeviceArray(capi, shape=(lib.he_ckks_encode_batch_workspace_words(h, items),))
+    cts = DeviceArray(capi, host=np.zeros((items, 2, limbs, n), dtype=np.uint64))
+    capi.check(lib.he_ckks_encode_batch(h, re.ptr, im.ptr, count, slots, scale, limbs, items, count, cts.ptr,
+                                        2 * limbs, wsb.ptr, None))
+    got_cts = cts.numpy()
+    assert (got_cts[0, 0] == got).all()                       # the batch's first item equals the single call
+    assert not got_cts[:, 1].any()
+    for k in range(items):
+        coeff = p.ntt_inv(got_cts[k, 0].copy())
+        for i in range(limbs):
+            assert _centred_distance(coeff[i], want_coeff[k][i], p.moduli[i]).max() <= 1, (k, i)
+    table = np.array([cts.at(k * 2 * limbs * n) for k in range(items)], dtype=np.uint64)
+    d_table = DeviceArray(capi, host=table)
+    sk = DeviceArray(capi, host=np.ones((limbs, n), dtype=np.uint64))
+    take = min(slots, 300)
+    dws = DeviceArray(capi, shape=(lib.he_decrypt_decode_batch_workspace_words(h, limbs, slots, items),))
+    dout = DeviceArray(capi, shape=(items, take, 2), dtype=np.float64)
+    capi.check(lib.he_decrypt_decode_batch(h, d_table.ptr, items, limbs, sk.ptr, None, slots, scale, take, dout.ptr,
+                                           dws.ptr, None))
+    vals = dout.numpy()
+    for k in range(items):
+        got_k = vals[k, :, 0] + 1j * vals[k, :, 1]
+        assert np.max(np.abs(got_k - o_enc.decode(got_cts[k, 0], scale, slots)[:take])) < REL, k
+        assert np.max(np.abs(got_k - padded[k, :take])) < REL, k
+
+
+def test_c5_pair_distances_against_the_oracle():
+    """C5 at its real shape (N = 2^16, chain [60, 40, 40, 60], one special prime, 2 chunks per client): for three of the
+    pairs, the ciphertext that pair_square_distances returns against the oracle's sub -> square -> add -> relinearise
+    -> rescale -> hoisted rounds on the same ciphertexts and the same seeded keys, every limb
+    (lancelot-main-GPU/utils/byzantine_fl.py:173-321)."""
+    from lancelot_amd import krum
+    from oracle import ckks_oracle as O
+    rng = np.random.default_rng(2025)
+    updates = [rng.normal(0.0, 0.01, 62006).astype(np.float32) for _ in range(4)]
+    updates[3] = updates[3] * 10
+    cfg = krum.KrumConfig(seed=77, reproducible=True)
+    state = krum.gpu_init(cfg)
+    c, ctx = state.cahel, state.context
+    n = 1 << cfg.log_n
+    mods = O.coeff_modulus_create(n, list(cfg.modulus_bits))
+    p = O.Params(cfg.log_n, mods, cfg.special_modulus_size)
+    ks = O.KeySet(p, seed=cfg.seed)
+    ks.gen_secret()
+    ks.gen_public()
+    o_rlk = ks.gen_relin()
+    rounds = krum.rotate_sum_plan(cfg.log_n - 1, cfg)
+    steps = sorted({s for r in rounds for s in r})
+    elts = list(c.get_elts_from_steps(steps, n))
+    o_glk = {e: ks.gen_galois(e) for e in elts}
+    for d in range(state.rlk.digit_count()):
+        assert (state.rlk.digit_to_numpy(d) == o_rlk[d]).all()
+    assert state.glk.key_count() == len(elts)
+    for i in (0, len(elts) // 2, len(elts) - 1):
+        for d in range(state.rlk.digit_count()):
+            assert (state.glk.key(i).digit_to_numpy(d) == o_glk[elts[i]][d]).all()
+    cts = krum.encrypt_updates(state, krum.split_updates(updates, state.slots))
+    assert len(cts[0]) == 2
+    pairs = [(0, 1), (1, 3), (2, 3)]
+    got = c.pair_square_distances(ctx, cts, pairs, state.rlk, state.glk, rounds, cfg.scale, 0)
+    c._synchronize()
+    host = [[ct.to_numpy() for ct in row] for row in cts]
+    for (i, j), ct in zip(pairs, got):
+        acc = None
+        for a, b in zip(host[i], host[j]):
+            sq = p.square(np.stack([p.sub(b[k], a[k]) for k in range(2)]))
+            acc = sq if acc is None else np.stack([p.add(acc[k], sq[k]) for k in range(3)])
+        r = p.rescale(p.relinearize(acc, o_rlk))
+        for rnd in rounds:
+            es = [elts[steps.index(s)] for s in rnd]
+            hs = p.hoisting(r, es, [o_glk[e] for e in es])
+            r = np.stack([p.add(r[k], hs[k]) for k in range(2)])
+        assert (ct.to_numpy() == r).all(), (i, j)
+    # and the decrypted distances, which are what the round reports
+    values = state.sk.decrypt_decode_many(ctx, got, state.slots, 1)[:, 0]
+    want = krum.plain_distance_matrix(updates)
+    for (i, j), v in zip(pairs, values):
+        assert abs(v - want[i, j]) / want[i, j] < 2e-5
