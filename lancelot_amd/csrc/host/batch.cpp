@@ -118,7 +118,7 @@ std::vector<CAHELGPUCiphertext> pair_square_distances(
     auto shared = std::make_shared<DeviceBuffer>(std::move(acc));
     for (uint32_t k = 0; k < items; k++) {
         CAHELGPUCiphertext &ct = out[k];
-        ct.data_ = DeviceBuffer::slice(shared, k * words, words);
+        ct.adopt(DeviceBuffer::slice(shared, k * words, words));
         ct.size_ = 2;
         ct.coeff_modulus_size_ = L1;
         ct.poly_modulus_degree_ = n;

@@ -189,6 +189,7 @@ PYBIND11_MODULE(pyCAHEL, m) {
     py::class_<CAHELGPURelinKey>(m, "relin_key")
         .def(py::init<CAHELGPUContext &>())
         .def("digit_count", [](const CAHELGPURelinKey &k) { return k.public_keys_.size(); })
+        .def("copy", [](const CAHELGPURelinKey &k) { return CAHELGPURelinKey(k); })
         .def("digit_ptr", [](const CAHELGPURelinKey &k, std::size_t d) {
             return reinterpret_cast<std::uintptr_t>(k.public_keys_.at(d).pk_.data());
         })
@@ -295,6 +296,8 @@ PYBIND11_MODULE(pyCAHEL, m) {
         .def("coeff_modulus_size", &CAHELGPUCiphertext::coeff_modulus_size)
         .def("data_ptr", [](const CAHELGPUCiphertext &c) { return reinterpret_cast<std::uintptr_t>(c.data()); })
         .def("copy", [](const CAHELGPUCiphertext &c) { return CAHELGPUCiphertext(c); })
+        // True between a relinearize_inplace whose key switch was deferred and the first use of the data
+        .def("_has_pending_key_switch", &CAHELGPUCiphertext::has_pending_key_switch)
         .def("to_numpy", [](const CAHELGPUCiphertext &c) {
             return to_host(c.data(), {(py::ssize_t)c.size(), (py::ssize_t)c.coeff_modulus_size(),
                                       (py::ssize_t)c.poly_modulus_degree()});

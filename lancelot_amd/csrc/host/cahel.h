@@ -92,6 +92,11 @@ public:
     // returns nothing to the pool itself (batched evaluations hand out their results this way); a copy of a slice
     // is an ordinary buffer of its own
     static DeviceBuffer slice(std::shared_ptr<DeviceBuffer> parent, std::size_t offset, std::size_t words);
+    // Turns the buffer into the only slice of a shared owner of its block, so that others can keep the block alive
+    // past this object (owner()); the words stay where they are.  Not safe against concurrent use of this object.
+    void make_shared();
+    // the shared owner of the block, or null for a plain buffer
+    const std::shared_ptr<DeviceBuffer> &owner() const { return parent_; }
     uint64_t *get() const { return ptr_; }
     std::size_t words() const { return words_; }
     static void trim_pool();  // return every cached block to the driver
@@ -216,6 +221,17 @@ public:
     cahel::parms_id_type parms_id_ = cahel::parms_id_zero;
 };
 
+// A relinearize_inplace that has not run yet: the ciphertext still holds the three polynomials of the product and
+// counts as two.  rescale_to_next consumes it together with the rescale in one device call (ModDown and the rescale
+// then share one inverse and one forward transform); every other use of the ciphertext's data runs the key switch
+// first, so nothing outside this layer can tell the difference except by the clock.
+struct PendingKeySwitch {
+    he_context *handle = nullptr;
+    uint32_t limbs = 0;                                          // L of the level the product lives at
+    std::vector<const uint64_t *> key_ptrs;                      // the relinearisation key's digits
+    std::vector<std::shared_ptr<cahel::DeviceBuffer>> key_owners;  // keep those blocks alive until the switch has run
+};
+
 // include/ciphertext.h: size_ polynomials, layout [poly][limb][coeff].
 class CAHELGPUCiphertext {
 public:
@@ -230,7 +246,18 @@ public:
     // keeps the leading min(old, new) words (include/ciphertext.h:303-333)
     void resize(const CAHELGPUContext &context, std::size_t chain_index, std::size_t size);
     void resize(std::size_t size, std::size_t coeff_modulus_size, std::size_t poly_modulus_degree);
-    uint64_t *data() const { return data_.get(); }
+    uint64_t *data() const {
+        if (pending_) settle();
+        return data_.get();
+    }
+    // runs a deferred relinearisation (on the current lane); a no-op otherwise
+    void settle() const;
+    bool has_pending_key_switch() const { return static_cast<bool>(pending_); }
+    // takes over a freshly computed block (whatever was deferred on the old one is dropped with it)
+    void adopt(cahel::DeviceBuffer &&block) {
+        pending_.reset();
+        data_ = std::move(block);
+    }
     std::size_t size() const { return size_; }
     std::size_t &chain_index() { return chain_index_; }
     std::size_t chain_index() const { return chain_index_; }
@@ -256,6 +283,8 @@ public:
     // the 64 seed bytes that close a ciphertext record (the reference keeps them on the device and fills them only
     // when asked to save the seed, include/ciphertext.h:31, 205-213); kept here so that a record survives a round trip
     std::array<std::uint8_t, 64> prng_seed_{};
+    // set by relinearize_inplace when it defers its key switch; data_ then holds size_ + 1 polynomials
+    mutable std::shared_ptr<PendingKeySwitch> pending_;
 };
 
 // include/secretkey.h:20-108: a key-level ciphertext (-(a s + e), a)

@@ -152,6 +152,15 @@ DeviceBuffer DeviceBuffer::slice(std::shared_ptr<DeviceBuffer> parent, std::size
     return v;
 }
 
+void DeviceBuffer::make_shared() {
+    if (!ptr_ || parent_) return;
+    auto owner = std::make_shared<DeviceBuffer>();
+    owner->ptr_ = ptr_;
+    owner->words_ = words_;
+    owner->lane_ = lane_;
+    parent_ = std::move(owner);
+}
+
 DeviceBuffer::DeviceBuffer(const DeviceBuffer &o) {
     allocate(o.words_);
     if (words_) check_status(he_memcpy_d2d(ptr_, o.ptr_, words_ * sizeof(uint64_t), current_stream()), "device copy failed");
@@ -244,6 +253,8 @@ void CAHELGPUPlaintext::resize(std::size_t coeff_modulus_size, std::size_t poly_
 
 CAHELGPUCiphertext &CAHELGPUCiphertext::operator=(const CAHELGPUCiphertext &o) {
     if (this == &o) return *this;
+    o.settle();
+    pending_.reset();
     data_.assign(o.data_, o.size_ * o.coeff_modulus_size_ * o.poly_modulus_degree_);
     size_ = o.size_;
     chain_index_ = o.chain_index_;
@@ -257,7 +268,23 @@ CAHELGPUCiphertext &CAHELGPUCiphertext::operator=(const CAHELGPUCiphertext &o) {
     return *this;
 }
 
+void CAHELGPUCiphertext::settle() const {
+    if (!pending_) return;
+    // (two host threads may read one ciphertext; only one of them runs the switch)
+    static std::mutex mu;
+    std::lock_guard<std::mutex> g(mu);
+    if (!pending_) return;
+    const PendingKeySwitch &p = *pending_;
+    const std::size_t poly = (std::size_t)p.limbs * poly_modulus_degree_;
+    DeviceBuffer ws(he_keyswitch_workspace_words(p.handle, p.limbs));
+    check_status(he_keyswitch(p.handle, p.limbs, data_.get() + 2 * poly, p.key_ptrs.data(), data_.get(), 0, ws.get(),
+                              current_stream()),
+                 "he_keyswitch");
+    pending_.reset();
+}
+
 void CAHELGPUCiphertext::resize(std::size_t size, std::size_t coeff_modulus_size, std::size_t poly_modulus_degree) {
+    settle();
     const std::size_t old_words = size_ * coeff_modulus_size_ * poly_modulus_degree_;
     const std::size_t new_words = size * coeff_modulus_size * poly_modulus_degree;
     // a block that is large enough stays: the leading words are the ones to keep anyway

@@ -83,7 +83,7 @@ std::vector<CAHELGPUCiphertext> CAHELGPUCKKSEncoder::encode_encrypt_many(const C
     auto shared = std::make_shared<DeviceBuffer>(std::move(batch));
     for (std::size_t k = 0; k < items; k++) {
         CAHELGPUCiphertext &ct = out[k];
-        ct.data_ = DeviceBuffer::slice(shared, k * words, words);
+        ct.adopt(DeviceBuffer::slice(shared, k * words, words));
         ct.size_ = 2;
         ct.coeff_modulus_size_ = L;
         ct.poly_modulus_degree_ = n;

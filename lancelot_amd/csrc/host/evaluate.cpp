@@ -174,7 +174,8 @@ static void multiply_into(const CAHELGPUContext &context, const CAHELGPUCipherte
                      "he_tensor");
     const bool asym = encrypted1.is_asymmetric_;
     const auto id = encrypted1.parms_id();
-    destination.data_ = std::move(product);
+    destination.prng_seed_ = encrypted1.prng_seed_;   // the reference's `destination = encrypted1` carries it along
+    destination.adopt(std::move(product));
     destination.size_ = dest_size;
     destination.coeff_modulus_size_ = L;
     destination.poly_modulus_degree_ = n;
@@ -242,12 +243,36 @@ void switch_key_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encr
                  "he_keyswitch");
 }
 
+// The key switch itself is deferred when the key's blocks can be kept alive (keys made by gen_relinkey or load):
+// callers run rescale_to_next_inplace right after (lancelot-main-GPU/utils/byzantine_fl.py:254-256), and that call
+// then does both in one device call (he_keyswitch_rescale, the same limbs); any other use of the ciphertext runs the
+// switch first (CAHELGPUCiphertext::settle).  Every check is made here, as in the reference.
 void relinearize_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, const CAHELGPURelinKey &relin_keys) {
     if (encrypted.size() != 3) throw std::invalid_argument("destination_size must be 3");
     if (!encrypted.is_ntt_form()) throw std::invalid_argument("CKKS encrypted must be in NTT form");
     const std::size_t poly = encrypted.coeff_modulus_size() * encrypted.poly_modulus_degree();
-    switch_key_inplace(context, encrypted, encrypted.data() + 2 * poly, relin_keys, true);
-    encrypted.resize(2, encrypted.coeff_modulus_size(), encrypted.poly_modulus_degree());
+    const uint32_t L = (uint32_t)encrypted.coeff_modulus_size();
+    const std::size_t beta = context.size_p() ? (L + context.size_p() - 1) / context.size_p() : 0;
+    bool defer = relin_keys.parms_id() == context.key_parms_id() && context.using_keyswitching() &&
+                 encrypted.chain_index() != 0 && relin_keys.public_keys_.size() >= beta;
+    for (std::size_t d = 0; defer && d < beta; d++) defer = static_cast<bool>(relin_keys.public_keys_[d].pk_.data_.owner());
+    if (!defer) {
+        // (also every argument error: switch_key_inplace throws it)
+        switch_key_inplace(context, encrypted, encrypted.data() + 2 * poly, relin_keys, true);
+        encrypted.resize(2, encrypted.coeff_modulus_size(), encrypted.poly_modulus_degree());
+        return;
+    }
+    (void)encrypted.data();   // (a size-3 ciphertext has nothing deferred; this keeps the invariant in one place)
+    auto pending = std::make_shared<PendingKeySwitch>();
+    pending->handle = context.handle();
+    pending->limbs = L;
+    for (std::size_t d = 0; d < beta; d++) {
+        const DeviceBuffer &block = relin_keys.public_keys_[d].pk_.data_;
+        pending->key_ptrs.push_back(block.get());
+        pending->key_owners.push_back(block.owner());
+    }
+    encrypted.size_ = 2;
+    encrypted.pending_ = std::move(pending);
 }
 
 // relinearize_inplace followed by rescale_to_next_inplace in one device call (he_keyswitch_rescale): the same limbs,
@@ -274,7 +299,7 @@ void relinearize_rescale_inplace(const CAHELGPUContext &context, CAHELGPUCiphert
                                       encrypted.data(), out.get(), 0, ws.get(), context.stream()),
                  "he_keyswitch_rescale");
     const double scale = encrypted.scale() / static_cast<double>(context.key_modulus()[L - 1].value());
-    encrypted.data_ = std::move(out);
+    encrypted.adopt(std::move(out));
     encrypted.size_ = 2;
     encrypted.coeff_modulus_size_ = L - 1;
     encrypted.poly_modulus_degree_ = n;
@@ -316,7 +341,8 @@ void multiply_relin_rescale(const CAHELGPUContext &context, const CAHELGPUCipher
                  "he_multiply_relin_rescale");
     destination.is_ntt_form() = true;
     destination.is_asymmetric_ = encrypted1.is_asymmetric_;
-    destination.data_ = std::move(out);
+    destination.prng_seed_ = encrypted1.prng_seed_;
+    destination.adopt(std::move(out));
     destination.size_ = 2;
     destination.coeff_modulus_size_ = L - 1;
     destination.poly_modulus_degree_ = n;
@@ -382,7 +408,7 @@ void mod_switch_to_next(const CAHELGPUContext &context, const CAHELGPUCiphertext
                      "copy");
     const double scale = encrypted.scale();
     const bool asym = encrypted.is_asymmetric_;
-    destination.data_ = std::move(fresh);
+    destination.adopt(std::move(fresh));
     destination.size_ = size;
     destination.coeff_modulus_size_ = next_limbs;
     destination.poly_modulus_degree_ = n;
@@ -417,12 +443,22 @@ void rescale_to_next(const CAHELGPUContext &context, const CAHELGPUCiphertext &e
     if (chain == context.max_chain_index()) throw std::invalid_argument("end of modulus switching chain reached");
     const std::size_t n = context.poly_degree(), size = encrypted.size();
     const uint32_t L = (uint32_t)encrypted.coeff_modulus_size();
-    DeviceBuffer out(size * (L - 1) * n), ws(size * n);
-    check_status(he_rescale(context.handle(), encrypted.data(), out.get(), (uint32_t)size, L, ws.get(), context.stream()),
-                 "he_rescale");
+    DeviceBuffer out(size * (L - 1) * n);
+    if (const std::shared_ptr<PendingKeySwitch> pending = encrypted.pending_) {
+        // a relinearisation is still due: both in one call, from the three polynomials that the block still holds
+        const uint64_t *raw = encrypted.data_.get();
+        DeviceBuffer ws(he_keyswitch_workspace_words(context.handle(), L));
+        check_status(he_keyswitch_rescale(context.handle(), L, raw + 2 * (std::size_t)L * n, pending->key_ptrs.data(), raw,
+                                          out.get(), 0, ws.get(), context.stream()),
+                     "he_keyswitch_rescale");
+    } else {
+        DeviceBuffer ws(size * n);
+        check_status(he_rescale(context.handle(), encrypted.data(), out.get(), (uint32_t)size, L, ws.get(), context.stream()),
+                     "he_rescale");
+    }
     const double scale = encrypted.scale() / static_cast<double>(context.key_modulus()[L - 1].value());
     const bool asym = encrypted.is_asymmetric_;
-    destination.data_ = std::move(out);
+    destination.adopt(std::move(out));
     destination.size_ = size;
     destination.coeff_modulus_size_ = L - 1;
     destination.poly_modulus_degree_ = n;
@@ -475,7 +511,7 @@ static void apply_galois_into(const CAHELGPUContext &context, const CAHELGPUCiph
         destination.is_ntt_form_ = encrypted.is_ntt_form_;
         destination.is_asymmetric_ = encrypted.is_asymmetric_;
     }
-    destination.data_ = std::move(rotated);
+    destination.adopt(std::move(rotated));
 }
 
 void apply_galois_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &encrypted, std::size_t galois_elt_index,
@@ -611,7 +647,7 @@ static void hoisting_into(const CAHELGPUContext &context, const CAHELGPUCipherte
         destination.is_ntt_form_ = ct.is_ntt_form_;
         destination.is_asymmetric_ = ct.is_asymmetric_;
     }
-    destination.data_ = std::move(sum);
+    destination.adopt(std::move(sum));
 }
 
 void hoisting_inplace(const CAHELGPUContext &context, CAHELGPUCiphertext &ct, const CAHELGPUGaloisKey &glk,

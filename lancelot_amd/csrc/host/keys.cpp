@@ -113,6 +113,8 @@ void CAHELGPUSecretKey::generate_one_kswitch_key(const CAHELGPUContext &context,
                                        (uint32_t)alpha, context.stream()),
                      "he_add_p_multiple");
     }
+    // shared ownership of the digits' blocks: a deferred relinearisation keeps them alive (relinearize_inplace)
+    for (auto &pk : relin_key.public_keys_) pk.pk_.data_.make_shared();
     relin_key.gen_flag_ = true;
     relin_key.parms_id_ = context.key_parms_id();
 }

@@ -227,7 +227,10 @@ void CAHELGPURelinKey::load(const CAHELGPUContext &context, std::istream &stream
     const std::size_t dnum = context.size_p() ? context.size_q() / context.size_p() : 0;
     if (count != dnum) throw std::invalid_argument("key count does not match the number of digits");
     std::vector<CAHELGPUPublicKey> fresh((std::size_t)count);
-    for (auto &pk : fresh) pk.load(context, stream);
+    for (auto &pk : fresh) {
+        pk.load(context, stream);
+        pk.pk_.data_.make_shared();   // as generate_one_kswitch_key leaves them
+    }
     public_keys_ = std::move(fresh);
     pk_num_ = (std::size_t)count;
     gen_flag_ = generated;

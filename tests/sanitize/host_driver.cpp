@@ -113,6 +113,71 @@ int main(int argc, char **argv) {
         copy.resize(3, copy.coeff_modulus_size(), n);
         REQUIRE(std::memcmp(copy.data(), cipher.data(), 2 * context.limbs_at(2) * n * 8) == 0);
     }
+    // ---- device blocks: slices, shared owners, and a key switch that is deferred past its key's lifetime ----
+    {
+        auto parent = std::make_shared<DeviceBuffer>(4 * n);
+        for (std::size_t i = 0; i < 4 * n; i++) parent->get()[i] = i;
+        DeviceBuffer s1 = DeviceBuffer::slice(parent, n, n), s2 = DeviceBuffer::slice(parent, 3 * n, n);
+        parent.reset();                       // the slices keep the block
+        REQUIRE(s1.get()[0] == n && s2.get()[n - 1] == 4 * n - 1);
+        REQUIRE(refuses([&] { DeviceBuffer::slice(s1.owner(), 4 * n, 1); }));
+        DeviceBuffer own(n);
+        for (std::size_t i = 0; i < n; i++) own.get()[i] = 7 * i;
+        s1 = own;                             // copy-assign into a slice of the same size: the words land in the parent's block
+        REQUIRE(s1.get()[5] == 35 && s1.owner());
+        DeviceBuffer big(2 * n);
+        for (std::size_t i = 0; i < 2 * n; i++) big.get()[i] = i + 1;
+        s1.assign(big, 2 * n);                // larger than the slice: it takes a block of its own
+        REQUIRE(s1.words() == 2 * n && !s1.owner() && s1.get()[2 * n - 1] == 2 * n);
+        { DeviceBuffer last = std::move(s2); }   // the last slice to go frees the parent's block
+        // a ciphertext whose block is a slice: growing it past the slice moves it to a block of its own
+        auto batch = std::make_shared<DeviceBuffer>(4 * context.limbs_at(2) * n);
+        for (std::size_t i = 0; i < batch->words(); i++) batch->get()[i] = 3 * i;
+        CAHELGPUCiphertext part(context);
+        part.adopt(DeviceBuffer::slice(batch, 2 * context.limbs_at(2) * n, 2 * context.limbs_at(2) * n));
+        part.size_ = 2;
+        part.coeff_modulus_size_ = context.limbs_at(2);
+        part.poly_modulus_degree_ = n;
+        batch.reset();
+        const uint64_t first = part.data()[0];
+        part.resize(3, part.coeff_modulus_size(), n);
+        REQUIRE(part.data()[0] == first && !part.data_.owner());
+        // make_shared keeps the words in place; owners outlive the object that made them
+        DeviceBuffer key(2 * context.size_qp() * n);
+        for (std::size_t i = 0; i < key.words(); i++) key.get()[i] = i ^ 0x55;
+        const uint64_t *where = key.get();
+        key.make_shared();
+        REQUIRE(key.get() == where && key.owner() && key.owner().use_count() == 1);
+        // a relinearisation deferred on `three` (as relinearize_inplace leaves it) while its key object goes away
+        const std::size_t L2 = context.limbs_at(2);
+        CAHELGPUCiphertext three(context);
+        three.resize(context, 2, 3);
+        for (std::size_t i = 0; i < 3 * L2 * n; i++) three.data()[i] = i;
+        auto pending = std::make_shared<PendingKeySwitch>();
+        pending->handle = context.handle();
+        pending->limbs = (uint32_t)L2;
+        std::vector<DeviceBuffer> digits((L2 + context.size_p() - 1) / context.size_p());
+        for (auto &d : digits) {
+            d.allocate(2 * context.size_qp() * n);
+            std::memset(d.get(), 1, d.words() * 8);
+            d.make_shared();
+            pending->key_ptrs.push_back(d.get());
+            pending->key_owners.push_back(d.owner());
+        }
+        three.size_ = 2;
+        three.pending_ = pending;
+        pending.reset();
+        digits.clear();                       // the key is gone; the owners in the pending switch keep its blocks
+        DeviceBuffer::trim_pool();
+        REQUIRE(three.has_pending_key_switch() && three.size() == 2);
+        CAHELGPUCiphertext after = three;     // a copy runs the switch on the source first
+        REQUIRE(!three.has_pending_key_switch() && !after.has_pending_key_switch());
+        REQUIRE(three.data()[0] == 1 && after.data()[1] == 2 && after.size() == 2);   // the mock adds one to (c0, c1)
+        three.pending_ = std::make_shared<PendingKeySwitch>();   // overwritten as a whole: nothing runs
+        three.adopt(DeviceBuffer(2 * L2 * n));
+        REQUIRE(!three.has_pending_key_switch());
+    }
+
     // a record of another level, a truncated one and one with a wrong degree are refused
     REQUIRE(refuses([&] {
         std::string bad = ctrec.substr(0, ctrec.size() / 2);

@@ -1,6 +1,6 @@
-// Host-memory stand-in for the eleven C-ABI entry points that the host layer's table construction and record
-// parsing call (he_malloc .. he_context_destroy), so that those CPU code paths can run under AddressSanitizer and
-// UndefinedBehaviorSanitizer without a GPU.  Test infrastructure: "device" memory is malloc'ed host memory, copies
+// Host-memory stand-in for the C-ABI entry points that the host layer's table construction, record parsing and
+// containers call (he_malloc .. he_context_destroy, and he_keyswitch for a deferred relinearisation), so that those
+// CPU code paths can run under AddressSanitizer and UndefinedBehaviorSanitizer without a GPU.  Test infrastructure: "device" memory is malloc'ed host memory, copies
 // are memcpy, a context is an opaque token.  Nothing here computes.
 #include <cstdlib>
 #include <cstring>
@@ -83,6 +83,24 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
 
 int he_context_destroy(he_context *ctx) {
     delete ctx;
+    return HE_OK;
+}
+
+size_t he_keyswitch_workspace_words(const he_context *ctx, uint32_t L) { return ctx ? (size_t)L << ctx->log_n : 0; }
+
+// Touches what the real call reads and writes (every word of c, of the beta key digits and of ct, and the
+// workspace), so that a stale pointer shows up as a sanitizer report; marks ct so that the caller can tell it ran.
+int he_keyswitch(const he_context *ctx, uint32_t L, const uint64_t *c, const uint64_t *const *evk, uint64_t *ct,
+                 uint32_t, uint64_t *workspace, he_stream) {
+    if (!ctx || !c || !evk || !ct || !workspace || L == 0 || L > ctx->size_q || ctx->size_p == 0) return HE_E_INVALID_ARGUMENT;
+    const size_t n = (size_t)1 << ctx->log_n, qp = (size_t)ctx->size_q + ctx->size_p;
+    const uint32_t beta = (L + ctx->size_p - 1) / ctx->size_p;
+    uint64_t sum = 0;
+    for (size_t i = 0; i < (size_t)L * n; i++) sum += c[i];
+    for (uint32_t d = 0; d < beta; d++)
+        for (size_t i = 0; i < 2 * qp * n; i += 97) sum += evk[d][i];
+    for (size_t i = 0; i < (size_t)L * n; i++) workspace[i] = sum;
+    for (size_t i = 0; i < 2 * (size_t)L * n; i++) ct[i] += 1;
     return HE_OK;
 }
 

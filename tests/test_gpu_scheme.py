@@ -140,6 +140,80 @@ def test_encrypt_multiply_relin_rescale_bit_exact(world):
     assert (cx.to_numpy() == o_r).all()
 
 
+def test_deferred_relinearisation_is_invisible(world):
+    """relinearize_inplace defers its key switch so that a rescale_to_next right after it does both in one device call
+    (the reference's callers run the two back to back, lancelot-main-GPU/utils/byzantine_fl.py:254-256).  Whatever is
+    done with the ciphertext between or instead of the two calls, the limbs are the oracle's: rescale at once, a read in
+    between, a copy, an addition, a rescale into another object, a key that is dropped before the switch has run, and a
+    destination that still had a switch pending."""
+    w = world
+    c, ctx, p = w["cahel"], w["ctx"], w["p"]
+    rng = np.random.default_rng(33)
+    x, y = rng.uniform(-1, 1, p.n // 2), rng.uniform(-1, 1, p.n // 2)
+    _, _, cx, o_cx = _encrypt_both(w, x)
+    _, _, cy, o_cy = _encrypt_both(w, y)
+    o_t = p.tensor(o_cx, o_cy)
+    o_r = p.relinearize(o_t, w["o_rlk"])
+    o_s = p.rescale(o_r)
+
+    def product():
+        prod = c.ciphertext(ctx)
+        c.multiply(ctx, cx, cy, prod)
+        c.relinearize_inplace(ctx, prod, w["rlk"])
+        assert prod.size() == 2 and prod._has_pending_key_switch()
+        return prod
+
+    a = product()                                   # the reference's sequence, nothing in between
+    c.rescale_to_next_inplace(ctx, a)
+    assert not a._has_pending_key_switch() and a.chain_index() == 2 and (a.to_numpy() == o_s).all()
+    b = product()                                   # a read in between
+    assert (b.to_numpy() == o_r).all() and not b._has_pending_key_switch()
+    c.rescale_to_next_inplace(ctx, b)
+    assert (b.to_numpy() == o_s).all()
+    d = product()                                   # a copy, then the original goes on
+    e = d.copy()
+    assert (e.to_numpy() == o_r).all() and not e._has_pending_key_switch()
+    c.rescale_to_next_inplace(ctx, d)
+    assert (d.to_numpy() == o_s).all()
+    f = product()                                   # an addition
+    c.add_inplace(ctx, f, e)
+    assert (f.to_numpy() == np.stack([p.add(o_r[k], o_r[k]) for k in range(2)])).all()
+    g, h = product(), c.ciphertext(ctx)             # rescale into another object; the source is still the relinearised product
+    c.rescale_to_next(ctx, g, h)
+    assert (h.to_numpy() == o_s).all() and h.chain_index() == 2 and g.chain_index() == 1
+    assert (g.to_numpy() == o_r).all()
+    with pytest.raises(ValueError, match="destination_size must be 3"):
+        c.relinearize_inplace(ctx, product(), w["rlk"])
+    # a second key, dropped while its switch is pending
+    rlk2 = c.relin_key(ctx)
+    w["sk"].gen_relinkey(ctx, rlk2)
+    o_rlk2 = w["ks"].gen_relin()
+    i = c.ciphertext(ctx)
+    c.multiply(ctx, cx, cy, i)
+    c.relinearize_inplace(ctx, i, rlk2)
+    del rlk2
+    c._trim_pool()
+    junk = [c.ciphertext(ctx) for _ in range(3)]
+    for ct in junk:
+        c.multiply(ctx, cy, cy, ct)                 # allocations that would reuse the key's blocks had they been freed
+    c.rescale_to_next_inplace(ctx, i)
+    assert (i.to_numpy() == p.rescale(p.relinearize(o_t, o_rlk2))).all()
+    # a destination with a switch pending is overwritten as a whole
+    j = product()
+    c.multiply(ctx, cx, cy, j)
+    assert j.size() == 3 and not j._has_pending_key_switch() and (j.to_numpy() == o_t).all()
+    k = product()
+    c.sub(ctx, cx, cy, k)
+    assert (k.to_numpy() == np.stack([p.sub(o_cx[b], o_cy[b]) for b in range(2)])).all()
+    # a copy of a key owns plain blocks: the switch runs at once, same limbs
+    m = c.ciphertext(ctx)
+    c.multiply(ctx, cx, cy, m)
+    c.relinearize_inplace(ctx, m, w["rlk"].copy())
+    assert not m._has_pending_key_switch()
+    c.rescale_to_next_inplace(ctx, m)
+    assert (m.to_numpy() == o_s).all()
+
+
 def test_add_sub_negate_plain_ops(world):
     w = world
     c, ctx, p = w["cahel"], w["ctx"], w["p"]
