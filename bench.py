@@ -70,7 +70,7 @@ def issue_rates(capi):
         row = []
         for waves in out["waves_per_simd"]:
             rate = C.c_double()
-            capi.check(capi.lib().he_probe_issue_rate(kind, cus * waves, 2000, C.byref(rate), None))
+            capi.check(capi.probe_lib().he_probe_issue_rate(kind, cus * waves, 2000, C.byref(rate), None))
             row.append(round(rate.value / 1e12, 2))
         out["rates"][name] = row
     return out
@@ -472,7 +472,7 @@ def main():
 
     # measured FP64 issue rate of this GPU (8 waves per SIMD of independent multiply-add chains)
     rate = C.c_double()
-    capi.check(lib.he_probe_fp64_issue_rate(2048, 2000, C.byref(rate), None))
+    capi.check(capi.probe_lib().he_probe_fp64_issue_rate(2048, 2000, C.byref(rate), None))
 
     # config "NTT alone": 24 limbs x 2 polynomials, forward + inverse
     f = timer.time(lambda: capi.check(lib.he_ntt_forward(h, two.ptr, 2, L, L, 0, L, 0, None)), 100)

@@ -10,7 +10,10 @@
  *     negative HE_E_* code for invalid arguments; nothing throws across this boundary
  *   - all polynomial pointers are DEVICE pointers to uint64_t residues in [0, q), layout
  *     [poly][limb][coeff] with the coefficient index fastest (include/ciphertext.h:303-333); outputs
- *     are always canonical residues
+ *     are always canonical residues, and inputs (ciphertexts, keys, plaintexts) must be: a word of q or more
+ *     (every q is below 2^61) gives undefined limbs, not an error
+ *   - pointers need the 8-byte alignment of their words; buffers that hipMalloc / he_malloc return, and limbs
+ *     inside them, are 16-byte aligned, which the kernels use where they can (he_sample requires it)
  *   - "L" is the number of data limbs of the level, K = size_p special limbs; limb t of a Ql u P buffer
  *     uses modulus table t for t < L and size_q + (t - L) otherwise (src/ntt/ntt_modup.cu:404-406)
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); calls are asynchronous on it
@@ -67,28 +70,6 @@ int he_event_synchronize(he_event event);
 /* Work enqueued on `stream` after this call starts only when `event` (recorded on another stream) has completed. */
 int he_stream_wait_event(he_stream stream, he_event event);
 int he_event_elapsed_ms(he_event start, he_event stop, float *ms);
-
-/* Measures the issue rate of full-rate FP64 vector instructions on this GPU (lane-operations per second, 8
- * independent fused multiply-add chains per lane over `blocks` workgroups of 256 lanes, `iters` x 64 operations per
- * lane): the peak that the VALU roofline of the FP64 back end is priced against.  Measurement support; allocates a
- * 64-byte buffer and two events for the duration of the call.  No counterpart in the reference. */
-int he_probe_fp64_issue_rate(uint32_t blocks, uint32_t iters, double *lane_ops_per_second, he_stream stream);
-
-/* The same measurement for the other instruction kinds that the kernels' bounds are argued with (`kind` below): 8
- * independent chains per lane, `iters` x 64 operations per lane; the result counts lane-operations (multiply-adds for
- * the matrix kinds: one v_mfma_f64_16x16x4_f64 is 1,024 of them per wave, i.e. 16 per lane; HE_PROBE_MFMA_F64_WITH_FMA
- * issues as many multiply-adds on the matrix instruction as on v_fma_f64 and reports their sum, so a result equal to
- * either kind alone means that the two do not run side by side).  Measurement support, as above.  No counterpart in
- * the reference. */
-enum {
-    HE_PROBE_FMA_F64 = 0,           /* v_fma_f64 */
-    HE_PROBE_MAD_U64_U32 = 1,       /* v_mad_u64_u32: 32 x 32 + 64 -> 64 */
-    HE_PROBE_MUL_LO_U32 = 2,        /* v_mul_lo_u32 */
-    HE_PROBE_ADD_U32 = 3,           /* v_add_u32 */
-    HE_PROBE_MFMA_F64 = 4,          /* v_mfma_f64_16x16x4_f64 alone */
-    HE_PROBE_MFMA_F64_WITH_FMA = 5  /* the matrix instruction interleaved with v_fma_f64, equal work on each */
-};
-int he_probe_issue_rate(uint32_t kind, uint32_t blocks, uint32_t iters, double *lane_ops_per_second, he_stream stream);
 
 /* ---- parameter tables ---- */
 
@@ -301,7 +282,9 @@ int he_multiply_relin_rescale(const he_context *ctx, uint32_t L, const uint64_t 
 
 /* he_multiply_relin_rescale over `items` independent products with one launch per stage: ct1, ct2 [items][2][L][N]
  * -> out [items][2][L-1][N] (ct2 == ct1 squares every item), all with the same relinearisation key.  The limbs are
- * those of `items` separate calls.  No counterpart in the reference, which multiplies one pair per call.
+ * those of `items` separate calls.  Contexts with more than 8 special primes are not served (HE_E_UNSUPPORTED: the
+ * batched base conversion holds at most 8 input limbs per thread); call he_multiply_relin_rescale per item there.
+ * No counterpart in the reference, which multiplies one pair per call.
  * workspace: he_multiply_relin_rescale_batch_workspace_words words. */
 size_t he_multiply_relin_rescale_batch_workspace_words(const he_context *ctx, uint32_t L, uint32_t items);
 int he_multiply_relin_rescale_batch(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *ct1,

@@ -1,6 +1,7 @@
 """Builds the native parts of the package in-tree.
 
   libcahel_hip.so   HIP kernels + C-ABI (include/cahel_hip.h), compiled with hipcc for gfx950
+  libcahel_probe.so issue-rate micro-benchmarks for bench.py (include/cahel_probe.h), hipcc for gfx950
   pyCAHEL*.so       C++ host layer + pybind11 binding (g++), linked against libcahel_hip.so
 
 Run as `python -m lancelot_amd.build`.  Nothing here needs a GPU: hipcc cross-compiles.
@@ -21,6 +22,7 @@ HOST = os.path.join(CSRC, "host")
 OBJ = os.path.join(PKG, "build")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 LIB = os.path.join(PKG, "libcahel_hip.so")
+PROBE_LIB = os.path.join(PKG, "libcahel_probe.so")
 
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-ffp-contract=off",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -44,6 +46,15 @@ def build_hip(verbose: bool = False) -> str:
     if verbose:
         print("built", LIB)
     return LIB
+
+
+def build_probe(verbose: bool = False) -> str:
+    """The measurement library that bench.py loads beside the engine (not linked into it)."""
+    sources = sorted(glob.glob(os.path.join(CSRC, "probe", "*.hip")))
+    _run([HIPCC, *HIP_FLAGS, "-shared", "-o", PROBE_LIB, *sources])
+    if verbose:
+        print("built", PROBE_LIB)
+    return PROBE_LIB
 
 
 def module_path() -> str:
@@ -71,6 +82,7 @@ def build_host(verbose: bool = False) -> str:
 
 def build_all(verbose: bool = False):
     build_hip(verbose)
+    build_probe(verbose)
     build_host(verbose)
 
 

@@ -35,8 +35,6 @@ SIGNATURES = {
     "he_event_synchronize": (C.c_int, [vp]),
     "he_stream_wait_event": (C.c_int, [vp, vp]),
     "he_event_elapsed_ms": (C.c_int, [vp, vp, C.POINTER(C.c_float)]),
-    "he_probe_fp64_issue_rate": (C.c_int, [u32, u32, C.POINTER(C.c_double), vp]),
-    "he_probe_issue_rate": (C.c_int, [u32, u32, u32, C.POINTER(C.c_double), vp]),
     "he_context_create": (C.c_int, [vp, C.POINTER(vp)]),
     "he_context_set_level": (C.c_int, [vp, vp]),
     "he_context_destroy": (C.c_int, [vp]),
@@ -84,7 +82,15 @@ SIGNATURES = {
     "he_decrypt_decode_batch": (C.c_int, [vp, vp, u32, u32, vp, vp, u32, C.c_double, u32, vp, vp, vp]),
 }
 
+# the measurement library beside it (include/cahel_probe.h)
+PROBE_LIB_PATH = os.path.join(_PKG, "libcahel_probe.so")
+PROBE_SIGNATURES = {
+    "he_probe_fp64_issue_rate": (C.c_int, [u32, u32, C.POINTER(C.c_double), vp]),
+    "he_probe_issue_rate": (C.c_int, [u32, u32, u32, C.POINTER(C.c_double), vp]),
+}
+
 _lib = None
+_probe_lib = None
 
 
 def lib():
@@ -99,6 +105,20 @@ def lib():
             fn.restype = res
             fn.argtypes = args
     return _lib
+
+
+def probe_lib():
+    """Loads libcahel_probe.so (issue-rate micro-benchmarks for bench.py); raises if it has not been built."""
+    global _probe_lib
+    if _probe_lib is None:
+        if not os.path.exists(PROBE_LIB_PATH):
+            raise RuntimeError("libcahel_probe.so is missing: run `python -m lancelot_amd.build`")
+        _probe_lib = C.CDLL(PROBE_LIB_PATH)
+        for name, (res, args) in PROBE_SIGNATURES.items():
+            fn = getattr(_probe_lib, name)
+            fn.restype = res
+            fn.argtypes = args
+    return _probe_lib
 
 
 def check(rc: int, what: str = "libcahel_hip"):

@@ -95,7 +95,6 @@ struct he_context {
     bool fuse_tensor = true;     // environment CAHEL_HIP_NO_FUSED_TENSOR=1: he_multiply_relin_rescale as tensor kernel + key switch
     bool single_limb_digits = false;  // K = 1 (environment CAHEL_HIP_NO_REDUCE_IN_NTT=1: keep the conversion kernels)
     bool batch_fused_inner = true;  // environment CAHEL_HIP_NO_BATCH_FUSED_KS=1: a batch's inner product as a kernel of its own
-    bool fp_inner = true;        // environment CAHEL_HIP_NO_FP_INNER=1: a batch's inner product on the integer kernel
     uint32_t *d_rot_group = nullptr;     // encoder: 5^j mod 2N
     double2 *d_ksi = nullptr;            // encoder: e^{2 pi i k / 2N}, k <= 2N
     uint64_t *d_garner_inv = nullptr;    // decoder: [size_q][size_q], q_j^-1 mod q_i for j < i
@@ -107,8 +106,7 @@ struct he_context {
     bool mixed_ok = false;       // mixed launches allowed (at most 64 tables; CAHEL_HIP_NO_MIXED=1 switches them off)
     int one_pass = 1;            // environment CAHEL_HIP_NO_ONE_PASS=1: plain transforms at N <= 2^14 as rows pass + blocks pass;
                                  // CAHEL_HIP_FORCE_ONE_PASS=1: the whole-limb kernel also where two launches are faster
-    int rows_direct = 1;         // environment CAHEL_HIP_ROWS_VIA_LDS=1: every register block of the rows pass (and of the
-                                 // fused inner-product kernel) takes its operands from LDS
+    Tuning tune;                 // the device's size and the switches that the launchers would otherwise read per launch
     std::vector<Level> levels;   // indexed by L
     std::vector<void *> owned;
 
@@ -158,7 +156,6 @@ NttArgs base_args(const he_context *ctx, bool forward) {
     a.log_n = ctx->log_n;
     a.epi_b_mask = 0xffffffffu;
     a.fp_mask = ctx->fp_mask;
-    a.rows_direct = ctx->rows_direct;
     a.one_pass = ctx->one_pass;
     return a;
 }
@@ -405,8 +402,6 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->fuse_inner = !(nf && nf[0] == '1');
         const char *nx = getenv("CAHEL_HIP_NO_MIXED");
         ctx->mixed_ok = qp <= 64 && !(nx && nx[0] == '1');
-        const char *rv = getenv("CAHEL_HIP_ROWS_VIA_LDS");
-        ctx->rows_direct = !(rv && rv[0] == '1');
         const char *no1 = getenv("CAHEL_HIP_NO_ONE_PASS"), *f1 = getenv("CAHEL_HIP_FORCE_ONE_PASS");
         ctx->one_pass = (no1 && no1[0] == '1') ? 0 : ((f1 && f1[0] == '1') ? 2 : 1);
         const char *nb = getenv("CAHEL_HIP_NO_FUSED_BCONV");
@@ -417,8 +412,20 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->single_limb_digits = ctx->size_p == 1 && !(nr && nr[0] == '1');
         const char *nbf = getenv("CAHEL_HIP_NO_BATCH_FUSED_KS");
         ctx->batch_fused_inner = !(nbf && nbf[0] == '1');
-        const char *ni = getenv("CAHEL_HIP_NO_FP_INNER");
-        ctx->fp_inner = !(ni && ni[0] == '1');
+        auto env_on = [](const char *name) { const char *e = getenv(name); return e && e[0] == '1'; };
+        auto env_count = [](const char *name, int lo, int hi, int otherwise) {
+            const char *e = getenv(name);
+            const int v = e ? atoi(e) : otherwise;
+            return (uint32_t)(v >= lo && v <= hi ? v : otherwise);
+        };
+        ctx->tune.hoist_no_local = env_on("CAHEL_HIP_NO_LOCAL_HOIST");
+        ctx->tune.hoist_no_xcd = env_on("CAHEL_HIP_NO_XCD_MAP");
+        ctx->tune.hoist_no_contig = env_on("CAHEL_HIP_NO_XCD_CONTIG");
+        ctx->tune.fuse_rows_forced = env_count("CAHEL_HIP_FUSE_ROWS", 1, 24, 0);
+        ctx->tune.bconv_rows = env_count("CAHEL_HIP_BCONV_ROWS", 1, 64, 6);
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, ctx->device) == hipSuccess && cus > 0)
+            ctx->tune.cus = (uint32_t)cus;
         ctx->fp_ok.assign(qp, 0);
         std::vector<double> psi_fp(qp * n, 0.0), ipsi_fp(qp * n, 0.0), consts(4 * qp, 0.0);
         for (size_t t = 0; t < qp; t++) {
@@ -795,12 +802,12 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
         BconvRows b{ws, out, c, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                     lv->beta, lv->modup_max_rows, copy_rows,
                     items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n, 0};
-        HE_HIP(launch_bconv_rows(base_args(ctx, true), b, S(s)));
+        HE_HIP(launch_bconv_rows(base_args(ctx, true), b, ctx->tune, S(s)));
     } else if (lv->batched) {
         BconvBatch b{ws, out, c, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                      lv->beta, lv->modup_max_rows, copy_rows, lv->d_mats_fp, ctx->d_fp_consts,
                      items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n};
-        HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+        HE_HIP(launch_bconv_batched(ctx->tables(), b, ctx->tune, S(s)));
     }
     for (uint32_t d = 0; d < lv->beta && !lv->batched && !reduce_in_ntt; d++) {
         const Digit &g = lv->digits[d];
@@ -888,12 +895,12 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
         if (fused) {
             BconvRows b{cx, ws, nullptr, ctx->d_phat_mod_q_fp, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, units, L, 0,
                         items, (size_t)units * LK * n, (size_t)units * L * n, 0, 0};
-            HE_HIP(launch_bconv_rows(base_args(ctx, true), b, S(s)));
+            HE_HIP(launch_bconv_rows(base_args(ctx, true), b, ctx->tune, S(s)));
         } else {
             BconvBatch b{cx, ws, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, units, L, 0,
                          fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts,
                          items, (size_t)units * LK * n, (size_t)units * L * n, 0};
-            HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+            HE_HIP(launch_bconv_batched(ctx->tables(), b, ctx->tune, S(s)));
         }
     }
     for (uint32_t p = 0; p < n_polys && !batched && !reduce_in_ntt; p++) {
@@ -1013,12 +1020,12 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         if (rows_done) {
             BconvRows b{tmp, y, nullptr, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                         lv->beta, lv->modup_max_rows, 0, items, (size_t)L * n, fwd.item_stride, 0, 0};
-            HE_HIP(launch_bconv_rows(fwd, b, S(s)));
+            HE_HIP(launch_bconv_rows(fwd, b, ctx->tune, S(s)));
         } else {
             BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                          lv->beta, lv->modup_max_rows, 0, lv->d_mats_fp, ctx->d_fp_consts, items, (size_t)L * n,
                          fwd.item_stride, 0};
-            HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+            HE_HIP(launch_bconv_batched(ctx->tables(), b, ctx->tune, S(s)));
         }
         KsFuseArgs x;
         memset(&x, 0, sizeof(x));
@@ -1045,8 +1052,11 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
     } else {
         // a batch on the FP64 back end shares each key word among the items of a group and reads a digit's own limbs
         // where they are
-        const bool fp_batch = items > 1 && ctx->fp_inner && lv->batched && fp_for_level(ctx, L) && n >= 512 &&
-                              !galois_elt && !add_c0;
+        // (its kernel moves two words per access: operands that are only 8-byte aligned take the integer kernel)
+        auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+        bool fp_batch = items > 1 && lv->batched && fp_for_level(ctx, L) && n >= 512 && !galois_elt && !add_c0 &&
+                        aligned16(src) && aligned16(cx) && aligned16(y) && aligned16(fold_ct);
+        for (uint32_t d = 0; d < lv->beta && fp_batch; d++) fp_batch = aligned16(evk[d]);
         if (tin) return HE_E_INVALID_ARGUMENT;
         // (batched levels: neither kernel needs the copy of a digit's own limbs into y)
         const bool skip_own = fp_batch || lv->batched;
@@ -1123,7 +1133,7 @@ int he_hoisted_rotations_batch(const he_context *ctx, uint32_t L, uint32_t items
     const uint32_t per_launch = (uint32_t)kMaxDigits / lv->beta;
     for (uint32_t first = 0; first < n_steps; first += per_launch) {
         const uint32_t count = n_steps - first < per_launch ? n_steps - first : per_launch;
-        HE_HIP(launch_hoist_inner(ctx->tables(), w.y, ct_in, evk + (size_t)first * lv->beta, galois_elts + first, count,
+        HE_HIP(launch_hoist_inner(ctx->tables(), ctx->tune, w.y, ct_in, evk + (size_t)first * lv->beta, galois_elts + first, count,
                                   w.cx, ct_out, L, ctx->size_p, ctx->size_q, lv->beta, first != 0, add_input != 0, items,
                                   2 * (size_t)L * n, S(s), ctx->use_fp ? ctx->d_fp_consts : nullptr, ctx->fp_mask, skip_own));
     }
@@ -1184,12 +1194,12 @@ int ksr_impl(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *
         // with the prologue of (4) and the rows pass of its transform
         BconvRows b{cx, delta, nullptr, ctx->d_phat_pinv_fp, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
                     items, 2 * (size_t)LK * n, 2 * (size_t)L * n, 0, 1};
-        HE_HIP(launch_bconv_rows(base_args(ctx, true), b, S(s)));
+        HE_HIP(launch_bconv_rows(base_args(ctx, true), b, ctx->tune, S(s)));
     } else if (lv->batched) {
         BconvBatch b{cx, delta, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
                      fp_for_level(ctx, L) ? ctx->d_phat_mod_q_fp : nullptr, ctx->d_fp_consts,
                      items, 2 * (size_t)LK * n, 2 * (size_t)L * n, 0};
-        HE_HIP(launch_bconv_batched(ctx->tables(), b, S(s)));
+        HE_HIP(launch_bconv_batched(ctx->tables(), b, ctx->tune, S(s)));
     } else {
         for (uint32_t p = 0; p < 2; p++) {
             BconvArgs b{cx + ((size_t)p * LK + L) * n, delta + (size_t)p * L * n, ctx->d_phat_mod_q, ctx->d_iota,

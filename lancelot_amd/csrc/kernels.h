@@ -6,6 +6,17 @@
 
 namespace he {
 
+// Launch choices that the context fixes once, when it is created (the device's size and the environment switches
+// that select bit-identical alternates): the launchers read nothing from the environment themselves.
+struct Tuning {
+    uint32_t cus = 256;              // compute units of the context's device
+    uint32_t fuse_rows_forced = 0;   // CAHEL_HIP_FUSE_ROWS: output limbs per workgroup of bconv_rows_fp_kernel, 0 = chosen per launch
+    uint32_t bconv_rows = 6;         // CAHEL_HIP_BCONV_ROWS: output rows per workgroup of the batched base conversion
+    bool hoist_no_local = false;     // CAHEL_HIP_NO_LOCAL_HOIST=1
+    bool hoist_no_xcd = false;       // CAHEL_HIP_NO_XCD_MAP=1
+    bool hoist_no_contig = false;    // CAHEL_HIP_NO_XCD_CONTIG=1
+};
+
 // One limb-sized NTT job given explicitly: which limb of the buffer, which modulus table.
 struct LimbJob {
     uint32_t data_limb;
@@ -70,8 +81,6 @@ struct NttArgs {
     const double *fp_consts;  // [tables][4]: q, 1/q, N^-1 mod q, (N^-1 mod q)/q
     uint64_t fp_mask;         // bit t: table t has a prime below 2^50 (read by the mixed back end only)
     int one_pass;             // N <= 2^14, FP64 back end, plain transforms: one kernel with the limb resident in LDS
-    int rows_direct;          // N = 2^16: rows pass with its outer half-pass on registers (one LDS exchange); fused
-                              // inner-product kernel: first register block straight from global memory
     const uint64_t *moduli;   // [tables]
     const uint64_t *barrett;  // [tables][2]
     const LimbJob *jobs;      // explicit list (then in/out limbs are absolute, no prologue/epilogue)
@@ -205,7 +214,7 @@ struct BconvBatch {
     uint32_t items;
     size_t x_item_stride, out_item_stride, copy_item_stride;
 };
-hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s);
+hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, const Tuning &tune, hipStream_t s);
 
 // Base conversion fused with the rows pass of the forward transform of its output limbs (FP64 back end, N >= 2^12,
 // n_in <= 8): the units of a BconvBatch, with the results left as the lazy words that the blocks pass continues on.
@@ -225,7 +234,7 @@ struct BconvRows {
     int mdr;
 };
 // `a` supplies the FP64 twiddles and constants of a forward transform (base_args)
-hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s);
+hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, const Tuning &tune, hipStream_t s);
 
 constexpr int kMaxDigits = 64;
 struct EvkPtrs {
@@ -256,7 +265,7 @@ hipError_t launch_inner_product_fp(const Tables &t, const double *fp_consts, con
 // kMaxDigits per launch.  fp_consts / fp_mask: rows whose table has its bit set (a prime below 2^50) form their
 // products in exact FP64 arithmetic; the results are the same canonical residues.  own_from_ct: y holds no copy of the
 // digits' own limbs (ModUp skipped it); they are read from c1 of the input ciphertext, which follows c0's L limbs.
-hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
+hipError_t launch_hoist_inner(const Tables &t, const Tuning &tune, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
                               const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
                               uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, bool with_self, uint32_t items,
                               size_t ct_item_stride, hipStream_t s, const double *fp_consts = nullptr, uint64_t fp_mask = 0,

@@ -374,10 +374,8 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     const Job job = decode_job(a, lb / tiles_per_limb);
     const uint32_t col0 = (lb % tiles_per_limb) << LOGC;
     if constexpr (LD >= 4 && tile_elems == 16 * kRowThreads) {
-        if (a.rows_direct) {
-            rows_direct<LD, FWD, BE, LOGC>(a, job, col0, lds);
-            return;
-        }
+        rows_direct<LD, FWD, BE, LOGC>(a, job, col0, lds);
+        return;
     }
     double *ld = reinterpret_cast<double *>(lds);
 
@@ -1225,9 +1223,8 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(2))) void
 #pragma unroll
         for (int i = 0; i < kPer; i++) pka[i] = ka[tid + i * half];
         double *ldm = ld + role * kInnerTile;
-        uint64_t *ldsm = lds + role * kInnerTile;
         const uint64_t *src = lazy_base + ((size_t)mine * LK + t) * n + off;  // lazy values left by the rows pass
-        if (work && a.rows_direct) {
+        if (work) {
             // the 16 words of the first register block (stride 16 inside a 256-block) straight from global memory:
             // 16 neighbouring threads read one 128-byte line per access
             double v[16];
@@ -1236,20 +1233,6 @@ __global__ __launch_bounds__(2 * T) __attribute__((amdgpu_waves_per_eu(2))) void
             fp_ct_block<4, true>(v, fc.tw, idx0, m);
 #pragma unroll
             for (int j = 0; j < 16; j++) ldm[skew(base0 + (j << 4))] = v[j];
-        } else if (!a.rows_direct) {
-            if (work) {
-#pragma unroll
-                for (int i = 0; i < kPer; i++) ldsm[skew(tid + i * half)] = src[tid + i * half];
-            }
-            lds_barrier();
-            if (work) {
-                double v[16];
-#pragma unroll
-                for (int j = 0; j < 16; j++) v[j] = ldm[skew(base0 + (j << 4))];
-                fp_ct_block<4, true>(v, fc.tw, idx0, m);
-#pragma unroll
-                for (int j = 0; j < 16; j++) ldm[skew(base0 + (j << 4))] = v[j];
-            }
         }
         lds_barrier();
         if (work) {
@@ -1593,13 +1576,9 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
 
 }  // namespace
 
-hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s) {
+hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, const Tuning &tune, hipStream_t s) {
     if (a.log_n < 12 || a.log_n > 16 || !b.mat_fp || b.n_units == 0) return hipErrorInvalidValue;
-    static const uint32_t forced = [] {
-        const char *e = getenv("CAHEL_HIP_FUSE_ROWS");
-        const int v = e ? atoi(e) : 0;
-        return (uint32_t)(v >= 1 && v <= (int)kFuseMaxRows ? v : 0);
-    }();
+    const uint32_t forced = tune.fuse_rows_forced <= kFuseMaxRows ? tune.fuse_rows_forced : 0;
     const uint32_t items = b.items ? b.items : 1;
     const int ld = (int)a.log_n - 8;
     const uint32_t tiles = 256u >> (kFuseLog - ld);
@@ -1614,11 +1593,7 @@ hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, hipStream_t s
     // 256 workgroups of 6 rows against 22.5 us in 512 of 3), so fewer than two per CU count as two.
     uint32_t target = forced;
     if (!target) {
-        static const uint32_t cus = [] {
-            int dev = 0, n = 0;
-            if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
-            return (uint32_t)n;
-        }();
+        const uint32_t cus = tune.cus ? tune.cus : 256;
         uint64_t best = ~0ull;
         for (uint32_t r = 1; r <= kFuseMaxRows && r <= rows; r++) {
             const uint64_t wgs = (uint64_t)b.n_units * items * tiles * ((rows + r - 1) / r);

@@ -1,9 +1,11 @@
 // Issue-rate probe for the VALU roofline: the FP64 back end spends its time in v_fma_f64 / v_mul_f64 / v_add_f64 /
 // v_rndne_f64, all of which issue at the rate this kernel measures (8 independent fused multiply-add chains per
 // lane, enough waves to fill every SIMD).  bench.py prices the instruction counts of the step's kernels against it.
+// Built as a library of its own (libcahel_probe.so, include/cahel_probe.h): measurement support, not part of the
+// engine's C-ABI.
 #include <hip/hip_runtime.h>
 
-#include "../../include/cahel_hip.h"
+#include "../../../include/cahel_probe.h"
 
 namespace {
 
@@ -88,11 +90,11 @@ void launch_issue_probe_kind(uint32_t kind, uint32_t blocks, uint64_t *sink, uin
 
 }  // namespace
 
-extern "C" int he_probe_issue_rate(uint32_t kind, uint32_t blocks, uint32_t iters, double *lane_ops_per_second, he_stream stream) {
+extern "C" int he_probe_issue_rate(uint32_t kind, uint32_t blocks, uint32_t iters, double *lane_ops_per_second, void *stream) {
     if (!lane_ops_per_second || blocks == 0 || iters == 0 || blocks > 65535 || kind > HE_PROBE_MFMA_F64_WITH_FMA)
         return HE_E_INVALID_ARGUMENT;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipEvent_t e0, e1;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
     uint64_t *sink = nullptr;
     hipError_t e = hipMalloc(&sink, 64);
     if (e != hipSuccess) return (int)e;
@@ -109,8 +111,8 @@ extern "C" int he_probe_issue_rate(uint32_t kind, uint32_t blocks, uint32_t iter
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     float ms = 0.f;
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
     (void)hipFree(sink);
     if (e != hipSuccess) return (int)e;
     // per lane and iteration: 64 vector operations; the matrix kinds add 4 instructions of 1,024 multiply-adds per wave,
@@ -120,10 +122,10 @@ extern "C" int he_probe_issue_rate(uint32_t kind, uint32_t blocks, uint32_t iter
     return HE_OK;
 }
 
-extern "C" int he_probe_fp64_issue_rate(uint32_t blocks, uint32_t iters, double *lane_ops_per_second, he_stream stream) {
+extern "C" int he_probe_fp64_issue_rate(uint32_t blocks, uint32_t iters, double *lane_ops_per_second, void *stream) {
     if (!lane_ops_per_second || blocks == 0 || iters == 0 || blocks > 65535) return HE_E_INVALID_ARGUMENT;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    hipEvent_t e0, e1;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
     double *sink = nullptr;
     hipError_t e = hipMalloc(&sink, 64);
     if (e != hipSuccess) return (int)e;
@@ -140,8 +142,8 @@ extern "C" int he_probe_fp64_issue_rate(uint32_t blocks, uint32_t iters, double 
     if (e == hipSuccess) e = hipEventSynchronize(e1);
     float ms = 0.f;
     if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    (void)hipEventDestroy(e0);
-    (void)hipEventDestroy(e1);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
     (void)hipFree(sink);
     if (e != hipSuccess) return (int)e;
     *lane_ops_per_second = (double)blocks * 256.0 * iters * 64.0 / ((double)ms * 1e-3);

@@ -886,13 +886,9 @@ hipError_t launch_bconv(const Tables &t, const BconvArgs &a, hipStream_t s) {
     return hipGetLastError();
 }
 
-hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, hipStream_t s) {
+hipError_t launch_bconv_batched(const Tables &t, const BconvBatch &b, const Tuning &tune, hipStream_t s) {
     if (b.n_units == 0) return hipSuccess;
-    static const uint32_t target = [] {
-        const char *e = getenv("CAHEL_HIP_BCONV_ROWS");
-        const int v = e ? atoi(e) : 6;
-        return (uint32_t)(v >= 1 && v <= 64 ? v : 6);
-    }();
+    const uint32_t target = tune.bconv_rows >= 1 && tune.bconv_rows <= 64 ? tune.bconv_rows : 6;
     const uint32_t cg = (b.max_rows + target - 1) / target;
     const uint32_t rows_per = (b.max_rows + cg - 1) / cg;
     const uint32_t kg = (b.max_copy + rows_per - 1) / rows_per;
@@ -1019,7 +1015,7 @@ hipError_t launch_inner_product_fp(const Tables &t, const double *fp_consts, con
     return hipGetLastError();
 }
 
-hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
+hipError_t launch_hoist_inner(const Tables &t, const Tuning &tune, const uint64_t *y, const uint64_t *c0, const uint64_t *const *evk,
                               const uint32_t *elts, uint32_t n_steps, uint64_t *out, uint64_t *c0_out, uint32_t L,
                               uint32_t K, uint32_t size_q, uint32_t beta, bool accumulate, bool with_self, uint32_t items,
                               size_t ct_item_stride, hipStream_t s, const double *fp_consts, uint64_t fp_mask,
@@ -1054,10 +1050,7 @@ hipError_t launch_hoist_inner(const Tables &t, const uint64_t *y, const uint64_t
     // every automorphism of the launch stays inside the aligned 256-word blocks of the NTT order
     bool local = t.log_n >= 8 && beta * 4 <= (uint32_t)kHoistLocalTiles;
     for (uint32_t i = 0; i < n_steps && local; i++) local = t.log_n < 9 || ((elts[i] - 1) & ((1u << (t.log_n - 7)) - 1)) == 0;
-    // (read at every launch, so that a test can compare the paths inside one process)
-    auto env_on = [](const char *name) { const char *e = getenv(name); return e && e[0] == '1'; };
-    const bool no_local = env_on("CAHEL_HIP_NO_LOCAL_HOIST"), no_xcd = env_on("CAHEL_HIP_NO_XCD_MAP"),
-               no_contig = env_on("CAHEL_HIP_NO_XCD_CONTIG");
+    const bool no_local = tune.hoist_no_local, no_xcd = tune.hoist_no_xcd, no_contig = tune.hoist_no_contig;
     if (no_local) local = false;
     // ... or inside the aligned stretches of 4,096 words (steps that are multiples of N / 8192)
     bool stretch_local = t.log_n >= 12;

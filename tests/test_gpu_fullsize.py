@@ -178,15 +178,13 @@ def test_c3_hmult_properties(bench_world):
 
 
 def test_c3_fused_and_separate_kernels_agree(monkeypatch):
-    """At N = 2^16, L = 24, K = 8 the key switch with its fast paths (inner product inside the blocks pass of
-    ModUp's transform; rows pass with its outer half on registers) and without them (the separate kernels and the
-    rows pass through LDS, which are the ones that the small-size tests pin to the oracle) must give the same
-    limbs."""
+    """At N = 2^16, L = 24, K = 8 the key switch with the inner product inside the blocks pass of ModUp's transform
+    and with the separate kernels (he_modup + he_ks_inner_product, which the small-size tests pin to the oracle one
+    by one) must give the same limbs."""
     from lancelot_amd import capi
     outs = []
-    for no_fuse, via_lds in (("0", "0"), ("0", "1"), ("1", "1")):
+    for no_fuse in ("0", "1"):
         monkeypatch.setenv("CAHEL_HIP_NO_FUSED_KS", no_fuse)
-        monkeypatch.setenv("CAHEL_HIP_ROWS_VIA_LDS", via_lds)
         cahel, parms, ctx, mods = _context(16, [50] * 32, 8)
         lib, h = capi.lib(), ctx.he_handle()
         n, L, qp = 1 << 16, 24, 32
@@ -212,7 +210,7 @@ def test_c3_fused_and_separate_kernels_agree(monkeypatch):
         for ptr in d_evk + [d_c, d_ct, ws.value]:
             lib.he_free(ptr)
         outs.append(out)
-    assert (outs[0] == outs[2]).all() and (outs[1] == outs[2]).all()
+    assert (outs[0] == outs[1]).all()
 
 
 def test_c4_rotations(bench_world):

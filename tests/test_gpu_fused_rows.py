@@ -144,14 +144,13 @@ def test_multiply_relin_rescale_entry_point(oracle, capi, monkeypatch, logn, bit
                                                        (16, [50, 49, 50, 50, 50, 50], 2, 4, 2),
                                                        (12, [50, 49, 48, 50, 47, 50, 50, 50], 2, 5, 9),
                                                        (12, [50, 49, 48, 50, 47, 50, 50, 50], 2, 6, 7)])
-@pytest.mark.parametrize("inner", ["fused", "fp_kernel", "int_kernel"])
+@pytest.mark.parametrize("inner", ["fused", "fp_kernel"])
 def test_multiply_relin_rescale_batch_equals_single_calls(oracle, capi, monkeypatch, logn, bits, size_p, L, items, inner):
     """The batch entry point against the oracle item by item.  With every prime below 2^50 its inner product runs
     inside the blocks pass of ModUp's forward transform, the items of one tile next to each other on one XCD
     ("fused"); switched off, it is the FP64 kernel that shares key words among up to 8 items (groups of 2, 4 and 8,
-    full and partial), and with that switched off too, or with larger primes, the integer kernel."""
+    full and partial); with larger primes (the second parameter set) the integer kernel."""
     monkeypatch.setenv("CAHEL_HIP_NO_BATCH_FUSED_KS", "0" if inner == "fused" else "1")
-    monkeypatch.setenv("CAHEL_HIP_NO_FP_INNER", "1" if inner == "int_kernel" else "0")
     cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
     rng = np.random.default_rng(300 + logn)
     lib, h = capi.lib(), ctx.he_handle()

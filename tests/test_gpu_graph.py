@@ -33,24 +33,41 @@ def test_entry_points_under_stream_capture(oracle, logn, bits, size_p, L):
     want_prod = p.rescale(p.relinearize(p.tensor(a, b), host_evk[:beta]))
     want_rot = p.apply_galois(a, elt, host_evk[:beta])
 
+    # he_rescale_static: the entry point that takes no workspace (its scratch belongs to the library's device image)
+    stat = DeviceArray(capi, shape=(2, L - 1, n))
+    want_stat = p.rescale(a)
+
     st = C.c_void_p()
     capi.check(lib.he_stream_create(C.byref(st)))
     graph, gexec = C.c_void_p(), C.c_void_p()
-    assert hip.hipStreamBeginCapture(st, 0) == 0            # hipStreamCaptureModeGlobal
-    capi.check(lib.he_multiply_relin_rescale(h, L, da.ptr, db.ptr, ptrs, prod.ptr, ws.ptr, st))
-    capi.check(lib.he_rotate(h, L, da.ptr, ptrs, rot.ptr, elt, rws.ptr, st))
-    assert hip.hipStreamEndCapture(st, C.byref(graph)) == 0
-    assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
-    scratch = DeviceArray(capi, shape=(2, L - 1, n))
-    for replay in range(3):
-        # clear the outputs, run other work of the library eagerly, then replay
-        capi.check(lib.he_memset_zero(prod.ptr, 8 * 2 * (L - 1) * n, None))
-        capi.check(lib.he_memset_zero(rot.ptr, 8 * 2 * L * n, None))
-        capi.check(lib.he_multiply_relin_rescale(h, L, db.ptr, db.ptr, ptrs, scratch.ptr, ws.ptr, None))
-        capi.check(lib.he_stream_synchronize(None))
-        assert hip.hipGraphLaunch(gexec, st) == 0
-        capi.check(lib.he_stream_synchronize(st))
-        assert (prod.numpy() == want_prod).all(), replay
-        assert (rot.numpy() == want_rot).all(), replay
-    assert hip.hipGraphExecDestroy(gexec) == 0
-    assert hip.hipGraphDestroy(graph) == 0
+    try:
+        assert hip.hipStreamBeginCapture(st, 0) == 0            # hipStreamCaptureModeGlobal
+        try:
+            rcs = [lib.he_multiply_relin_rescale(h, L, da.ptr, db.ptr, ptrs, prod.ptr, ws.ptr, st),
+                   lib.he_rotate(h, L, da.ptr, ptrs, rot.ptr, elt, rws.ptr, st),
+                   lib.he_rescale_static(h, da.ptr, stat.ptr, 2, L, st)]
+        finally:
+            # always leave capture mode: a stream left capturing would fail every later call of the process
+            end = hip.hipStreamEndCapture(st, C.byref(graph))
+        assert rcs == [0, 0, 0] and end == 0
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, C.c_size_t(0)) == 0
+        scratch = DeviceArray(capi, shape=(2, L - 1, n))
+        for replay in range(3):
+            # clear the outputs, run other work of the library eagerly, then replay
+            capi.check(lib.he_memset_zero(prod.ptr, 8 * 2 * (L - 1) * n, None))
+            capi.check(lib.he_memset_zero(rot.ptr, 8 * 2 * L * n, None))
+            capi.check(lib.he_memset_zero(stat.ptr, 8 * 2 * (L - 1) * n, None))
+            capi.check(lib.he_multiply_relin_rescale(h, L, db.ptr, db.ptr, ptrs, scratch.ptr, ws.ptr, None))
+            capi.check(lib.he_rescale_static(h, db.ptr, scratch.ptr, 2, L, None))
+            capi.check(lib.he_stream_synchronize(None))
+            assert hip.hipGraphLaunch(gexec, st) == 0
+            capi.check(lib.he_stream_synchronize(st))
+            assert (prod.numpy() == want_prod).all(), replay
+            assert (rot.numpy() == want_rot).all(), replay
+            assert (stat.numpy() == want_stat).all(), replay
+    finally:
+        if gexec:
+            hip.hipGraphExecDestroy(gexec)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        capi.check(lib.he_stream_destroy(st))

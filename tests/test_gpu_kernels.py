@@ -186,12 +186,10 @@ def test_mixed_back_end_agrees_with_the_integer_one(oracle, capi, monkeypatch, l
                                                  (11, [45, 40, 40, 50], 1, 3), (9, [40, 40, 45, 45], 2, 2)])
 def test_fused_and_separate_key_switch_agree(oracle, capi, monkeypatch, logn, bits, size_p, L):
     """he_keyswitch with the inner product inside the forward NTT (the default for primes below 2^50) and, forced
-    by the environment, with the separate kernels, each with the rows pass on registers and through LDS: all equal
-    the oracle, with and without a Galois element, with a partial last digit (L = 3 over two special primes, L = 5
-    over three), and at the smallest degree."""
-    for no_fuse, via_lds in (("0", "0"), ("0", "1"), ("1", "0"), ("1", "1")):
+    by the environment, with the separate kernels: both equal the oracle, with and without a Galois element, with a
+    partial last digit (L = 3 over two special primes, L = 5 over three), and at the smallest degree."""
+    for no_fuse in ("0", "1"):
         monkeypatch.setenv("CAHEL_HIP_NO_FUSED_KS", no_fuse)
-        monkeypatch.setenv("CAHEL_HIP_ROWS_VIA_LDS", via_lds)
         cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
         rng = np.random.default_rng(12)
         lib, h = capi.lib(), ctx.he_handle()
@@ -204,7 +202,7 @@ def test_fused_and_separate_key_switch_agree(oracle, capi, monkeypatch, logn, bi
             capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, elt, ws.ptr, None))
             ks = p.key_switch(p.galois_ntt(c, elt) if elt else c, host_evk)
             want = np.stack([p.add(ct[b], ks[b]) for b in range(2)])
-            assert (dct.numpy() == want).all(), (no_fuse, via_lds, elt)
+            assert (dct.numpy() == want).all(), (no_fuse, elt)
 
 
 @pytest.mark.parametrize("logn,bits,size_p,L", [(13, [50, 50, 49, 50, 50, 50], 2, 4), (13, [50, 50, 49, 50, 50, 50], 2, 3),
@@ -892,8 +890,8 @@ def test_issue_rate_probe(capi):
     """he_probe_issue_rate: every kind returns a rate, an unknown kind and empty launches are refused, and the
     ordering that the design notes rely on holds (a 32-bit addition issues faster than an FP64 multiply-add or a
     32-bit multiply; the FP64 matrix instruction interleaved with FP64 vector multiply-adds does not reach the sum
-    of the two alone)."""
-    lib, r = capi.lib(), C.c_double()
+    of the two alone).  The probes live in a library of their own, beside the engine's."""
+    lib, r = capi.probe_lib(), C.c_double()
     assert lib.he_probe_issue_rate(6, 256, 10, C.byref(r), None) == -1
     assert lib.he_probe_issue_rate(0, 0, 10, C.byref(r), None) == -1
     assert lib.he_probe_issue_rate(0, 256, 0, C.byref(r), None) == -1

@@ -27,6 +27,12 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
     assert declared == set(capi.SIGNATURES), declared ^ set(capi.SIGNATURES)
     assert lib.he_error_string(0) == b"success" and lib.he_error_string(-3).startswith(b"tables of this level")
+    # the measurement library is a shared object of its own: its names are not part of the engine's interface
+    probe_header = open(os.path.join(ROOT, "include", "cahel_probe.h")).read()
+    probes = set(re.findall(r"\b(he_probe_[a-z0-9_]+)\s*\(", probe_header))
+    assert probes == set(capi.PROBE_SIGNATURES) and not probes & declared
+    for name in sorted(probes):
+        assert hasattr(capi.probe_lib(), name) and not hasattr(lib, name), name
 
 
 def test_pycahel_exports_the_reference_names(cahel):
