@@ -21,10 +21,14 @@ Extra objects on the line:
   roofline      the timed step on one stream against the HBM roofline: algorithmic bytes of the step / its duration
                 (HIP events on the stream the kernels run on), with the VALU bound beside it (`valu`: wave
                 instructions of the step's kernels from the committed counter profile, priced against the FP64
-                issue rate that he_probe_fp64_issue_rate measures in this run)
+                issue rate that he_probe_fp64_issue_rate measures in this run); `frac` prices the 334 limbs of
+                one operation (inputs, key, output), `frac_amortised_key` the bytes a launch of several operations
+                has to move (the key once per launch)
   ntt           config "batched forward + inverse NTT, 24 limbs x 2 polynomials": GB/s of limb data
   rotate        one rotation with key switch; rotate-and-sum over 15 steps
-  krum          the encrypted Krum round at its real shape, with the CPU checker's time for the same evaluate phase
+  krum          the encrypted Krum round at its real shape, with the CPU checker's time for the same evaluate phase,
+                and the distance phase driven call for call as lancelot-main-GPU's byzantine_fl.py does
+                (`reference_call_sequence`: 55 pairs, operands encoded and encrypted again for every pair)
   cpu_baseline  the CPU checker (oracle/, OpenMP) on the same HMult+relin+rescale workload, bounded sample; and at
                 BASELINE.json configs[0] (N = 2^14, 4 + 1 primes)
 """
@@ -150,8 +154,9 @@ def cpu_hmult(log_n, size_q, size_p, seconds_budget):
 
 
 def cpu_baseline():
-    v, iters, threads = cpu_hmult(LOG_N, SIZE_Q, SIZE_P, 10.0)
-    v1, iters1, _ = cpu_hmult(14, 4, 1, 4.0)
+    # bounded samples (3 s + 2 s), so that most of a default run is GPU work
+    v, iters, threads = cpu_hmult(LOG_N, SIZE_Q, SIZE_P, 3.0)
+    v1, iters1, _ = cpu_hmult(14, 4, 1, 2.0)
     return {"value": v, "unit": "HMult+relin+rescale ops/s", "cores": threads, "kind": "port",
             "sample": "%d iterations of the same workload (N=2^16, L=24, K=8, dnum=3, random residues) on "
                       "oracle/ckks_oracle.c with OpenMP" % iters,
@@ -248,7 +253,8 @@ def krum_cpu_evaluate(updates, pairs_sampled=2):
             % (pairs_sampled, per_pair, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))}
 
 
-def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60), sum_drop_levels=0, with_cpu=False):
+def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60), sum_drop_levels=0, with_cpu=False,
+               with_reference_sequence=False):
     """One encrypted Krum round at its real shape (10 clients x 62,006 parameters, N = 2^16, moduli
     [60, 40, 40, 60], one special prime): seconds per phase and the error against the float64 closed form."""
     from lancelot_amd import krum
@@ -281,6 +287,22 @@ def krum_round(seed: int = 2025, modulus_bits=(60, 40, 40, 60), sum_drop_levels=
     if with_cpu:
         out["cpu_baseline"] = krum_cpu_evaluate(updates)
         out["cpu_baseline"]["gpu_evaluate_s"] = timings["evaluate"]
+    if with_reference_sequence:
+        # the same distances the way the unchanged caller computes them (lancelot-main-GPU/utils/byzantine_fl.py:173-321,
+        # 466-514): 55 pairs, every pair encodes and encrypts its operands again, one pyCAHEL call per operation
+        del state
+        ref_state = krum.gpu_init(krum.KrumConfig(seed=seed, modulus_bits=tuple(modulus_bits), hoisting_radix=0,
+                                                  batched=False, lanes=0))
+        krum.reference_call_sequence(ref_state, updates[:2])        # warm-up: 3 pairs
+        ref_dist, ref_t = krum.reference_call_sequence(ref_state, updates)
+        out["reference_call_sequence"] = {
+            "calls": "GPU_computing_distance_cipher as byzantine_fl.py issues it: 55 pairs (i <= j), per pair 2 encryptions "
+                     "of zero + encode and encrypt of both operands per chunk, sub / square_inplace / add_inplace, "
+                     "relinearize_inplace + rescale_to_next_inplace, hoisting(1..15) + add_inplace, 11 x (rotate_vector + "
+                     "add_inplace); every call on the null stream, the phases timed with a synchronisation after each",
+            "seconds": ref_t, "chosen": krum.krum_select(ref_dist),
+            "max_rel_err_vs_float64": float(np.max(np.abs(ref_dist[off] - plain[off]) / plain[off])),
+            "batched_driver_distance_phase_s": timings["encode"] + timings["evaluate"]}
     return out
 
 
@@ -296,9 +318,11 @@ def main():
     ap.add_argument("--batch", type=int, default=8, help="operations per he_multiply_relin_rescale_batch call")
     ap.add_argument("--batch-streams", type=int, default=2, help="streams that the batch calls are dealt to")
     ap.add_argument("--no-krum", action="store_true", help="skip the encrypted Krum round (BASELINE.json configs[4])")
-    ap.add_argument("--only", choices=["all", "step", "batch", "rotate", "ntt", "krum", "probe"], default="all",
-                    help="step / rotate / ntt: run just that workload on the null stream (for rocprofv3); probe: the "
-                         "issue rates of the instruction kinds that the kernels' bounds are argued with")
+    ap.add_argument("--only", choices=["all", "step", "batch", "batch_streams", "rotate", "ntt", "krum", "krum_reference", "probe"], default="all",
+                    help="step / batch / rotate / ntt: run just that workload on the null stream (for rocprofv3); "
+                         "batch_streams: the batch calls dealt to --batch-streams streams, as `value` issues them; "
+                         "krum_reference: the Krum round plus the distance phase by the reference's own call sequence; "
+                         "probe: the issue rates of the instruction kinds that the kernels' bounds are argued with")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -310,6 +334,9 @@ def main():
 
     if args.only == "krum":
         print(json.dumps(krum_round()))
+        return
+    if args.only == "krum_reference":
+        print(json.dumps(krum_round(with_reference_sequence=True)))
         return
     if args.only == "probe":
         print(json.dumps(issue_rates(capi)))
@@ -375,6 +402,46 @@ def main():
     def batch_call():
         capi.check(lib.he_multiply_relin_rescale_batch(h, L, B, ba.ptr, bb.ptr, evk, bres.ptr, bws.ptr, None))
 
+    def make_batch_lanes(streams):
+        """Per stream: its own operands, output and workspace for he_multiply_relin_rescale_batch."""
+        lanes = []
+        for st in streams:
+            la, lb = Buf(capi, B * 2 * L * n), Buf(capi, B * 2 * L * n)
+            capi.check(lib.he_memcpy_d2d(la.ptr, ba.ptr, 8 * B * 2 * L * n, None))
+            capi.check(lib.he_memcpy_d2d(lb.ptr, bb.ptr, 8 * B * 2 * L * n, None))
+            lanes.append((st, la, lb, Buf(capi, B * 2 * (L - 1) * n),
+                          Buf(capi, lib.he_multiply_relin_rescale_batch_workspace_words(h, L, B))))
+        return lanes
+
+    if args.only == "batch_streams":
+        # what `value` times, alone (for rocprofv3): batch calls dealt round-robin to the streams
+        streams = []
+        for _ in range(args.batch_streams):
+            st = C.c_void_p()
+            capi.check(lib.he_stream_create(C.byref(st)))
+            streams.append(st)
+        lanes = make_batch_lanes(streams)
+        capi.check(lib.he_memcpy_d2d(ws.ptr, ws.at(48 * n), 8 * 48 * n, None))
+        sync(capi)
+
+        def issue(i):
+            st, la, lb, lres, lws = lanes[i % len(lanes)]
+            capi.check(lib.he_multiply_relin_rescale_batch(h, L, B, la.ptr, lb.ptr, evk, lres.ptr, lws.ptr, st))
+
+        calls = max(2 * len(lanes), -(-K_steps // B))
+        for i in range(2 * len(lanes)):
+            issue(i)
+        for st in streams:
+            capi.check(lib.he_stream_synchronize(st))
+        t0 = time.perf_counter()
+        for i in range(calls):
+            issue(i)
+        for st in streams:
+            capi.check(lib.he_stream_synchronize(st))
+        ms = (time.perf_counter() - t0) * 1e3 / calls
+        print(json.dumps({"only": args.only, "ms_per_call": ms, "ms_per_operation": ms / B, "calls": calls,
+                          "operations_per_call": B, "streams": len(lanes), "calibration_copy_bytes": 8 * 48 * n}))
+        return
     if args.only in ("step", "batch", "rotate", "ntt"):
         fn = {"step": step, "batch": batch_call, "rotate": one_rot,
               "ntt": lambda: (capi.check(lib.he_ntt_forward(h, two.ptr, 2, L, L, 0, L, 0, None)),
@@ -421,19 +488,14 @@ def main():
         lane_step(i % args.lanes)
     streams_ms, streams_blocks = timed_wall(lambda i: lane_step(i % args.lanes), K_steps)
 
-    # (3) `batch` operations per call, one launch per stage for all of them
-    calls = max(1, -(-K_steps // B))
+    # (3) `batch` operations per call, one launch per stage for all of them.  A timed block holds at least 20 calls
+    # whatever --steps says: a block of a few calls would be a few milliseconds of GPU time
+    calls = max(20, -(-K_steps // B))
     batch_ms = timer.time(batch_call, calls, max(1, W // B)) / B
 
     # (3b) the same batch calls dealt to two streams (each with its own operands, workspace and output): the tail of
     # one call's kernels overlaps the head of the other's
-    batch_lanes = []
-    for k in range(min(args.batch_streams, len(lane_streams))):
-        la, lb = Buf(capi, B * 2 * L * n), Buf(capi, B * 2 * L * n)
-        capi.check(lib.he_memcpy_d2d(la.ptr, ba.ptr, 8 * B * 2 * L * n, None))
-        capi.check(lib.he_memcpy_d2d(lb.ptr, bb.ptr, 8 * B * 2 * L * n, None))
-        batch_lanes.append((lane_streams[k], la, lb, Buf(capi, B * 2 * (L - 1) * n),
-                            Buf(capi, lib.he_multiply_relin_rescale_batch_workspace_words(h, L, B))))
+    batch_lanes = make_batch_lanes(lane_streams[:min(args.batch_streams, len(lane_streams))])
 
     def batch_lane_call(i):
         st, la, lb, lres, lws = batch_lanes[i % len(batch_lanes)]
@@ -441,7 +503,8 @@ def main():
 
     for i in range(2 * len(batch_lanes)):
         batch_lane_call(i)
-    bs_ms, bs_blocks = timed_wall(batch_lane_call, max(2 * len(batch_lanes), calls))
+    bs_calls = max(20, 2 * len(batch_lanes), calls)
+    bs_ms, bs_blocks = timed_wall(batch_lane_call, bs_calls)
     bs_ms /= B
 
     # (4) the reference's own call sequence through pyCAHEL on the null stream
@@ -531,7 +594,11 @@ def main():
         floor_ms = 920 * limb_bytes / 6.0e12 * 1e3
         return {"bound": "hbm", "kernel": what + prof["kernels"],
                 "achieved": alg_bytes / (ms_per_op * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": frac(ms_per_op), "ms_per_launch": ms_per_op * ops_per_launch,
+                "frac": frac(ms_per_op),
+                # the same with the bytes that a launch has to move: the key is read once per launch, not per operation
+                "frac_amortised_key": (96 + 46 + 192.0 / ops_per_launch) * limb_bytes / (ms_per_op * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                "compulsory_bytes_per_launch": int((96 + 46) * limb_bytes * ops_per_launch + 192 * limb_bytes),
+                "ms_per_launch": ms_per_op * ops_per_launch,
                 "operations_per_launch": ops_per_launch,
                 "algorithmic_bytes_per_launch": alg_bytes * ops_per_launch,
                 "traffic": int(prof["traffic_limbs"] * limb_bytes * ops_per_launch),
@@ -552,7 +619,9 @@ def main():
         "dtype": "u64", "data": "synthetic",
         "arithmetic": "64-bit residues; every stage in exact FP64 (primes below 2^50) with canonical 64-bit results; "
                       "every output bit-identical to the integer oracle",
-        "timing": "median of %d blocks of %d steps each" % (BLOCKS, K_steps),
+        "timing": "median of %d timed blocks after %d warm-up steps; a block is %d steps for the single-call paths, %d "
+                  "calls of %d operations for `batch` and %d such calls for `batch_streams` (`value`), whatever --steps says"
+                  % (BLOCKS, W, K_steps, calls, B, bs_calls),
         "config": {"workload": "HMult+relinearize+rescale, N=2^16, L=24 limbs of 50 bits, K=8, dnum=3, scale 2^40, "
                                "two fresh ciphertexts of 32768 uniform[-1,1] slots (BASELINE.json configs[2]); "
                                "independent operations, the best of %d streams of single calls, batches of %d per "
@@ -578,7 +647,7 @@ def main():
         "config_c1": gpu_c1(capi, cahel, timer),
     }
     if not args.no_krum:
-        line["krum"] = krum_round(with_cpu=not args.no_cpu_baseline)
+        line["krum"] = krum_round(with_cpu=not args.no_cpu_baseline, with_reference_sequence=True)
         # The same round with two settings that Lancelot's driver does not use (its own are the ones above): primes
         # below 2^50 (exact FP64 butterflies instead of 64-bit integer ones), and the slot sum one level further down
         # (mod_switch_to_next after the rescale: its key switches run over one limb instead of two).  The two do not

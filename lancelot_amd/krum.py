@@ -207,6 +207,81 @@ def pair_distance(state: KrumState, cts_i, cts_j):
     return acc
 
 
+def reference_call_sequence(state: KrumState, updates):
+    """The distance phase exactly as lancelot-main-GPU/utils/byzantine_fl.py drives the library, call for call, on the
+    null stream: GPU_computing_distance_cipher (:466-514) runs GPU_compute_pair_distance (:173-321) for the 55 pairs
+    i <= j, and every pair encodes and encrypts both operands again, chunk by chunk, besides two encryptions of zero
+    (one of them unused on the lazy-relinearisation branch that the file takes); then sub, square_inplace, add_inplace
+    onto the squared zero, relinearize_inplace, rescale_to_next_inplace, set_scale, hoisting of steps 1..15 +
+    add_inplace, and one rotate_vector + add_inplace per doubling from 2^4 on.  `state` must come from a KrumConfig
+    with hoisting_radix = 0 (that key set).  Returns (decrypted distance matrix, seconds per phase)."""
+    c, ctx, cfg = state.cahel, state.context, state.config
+    enc, pk, scale = state.encoder, state.pk, cfg.scale
+    log_slots = int(math.log2(state.slots))
+    chunks = split_updates(updates, state.slots)
+    n_clients = len(chunks)
+    spent = {"encode": 0.0, "encrypt": 0.0, "square_accumulate": 0.0, "relinearize_rescale": 0.0, "rotate_and_sum": 0.0}
+    zero = np.zeros(state.slots)
+
+    def lap(key, t0):
+        _sync(c)                      # the reference's timers bracket asynchronous calls; these wait for the work
+        now = time.perf_counter()
+        spent[key] += now - t0
+        return now
+
+    def pair(msg1, msg2):
+        t = time.perf_counter()
+        tmp = c.ciphertext(ctx)
+        pt_tmp1 = enc.encode(ctx, zero, scale)
+        t = lap("encode", t)
+        tmp1 = pk.encrypt_asymmetric(ctx, pt_tmp1)
+        c.mod_switch_to_inplace(ctx, tmp1, 2)
+        t = lap("encrypt", t)
+        pt_zero = enc.encode(ctx, zero, scale)
+        t = lap("encode", t)
+        acc = pk.encrypt_asymmetric(ctx, pt_zero)
+        t = lap("encrypt", t)
+        c.square_inplace(ctx, acc)
+        t = lap("square_accumulate", t)
+        for x1, x2 in zip(msg1, msg2):
+            pt1 = enc.encode(ctx, x1, scale)
+            pt2 = enc.encode(ctx, x2, scale)
+            t = lap("encode", t)
+            ct1 = pk.encrypt_asymmetric(ctx, pt1)
+            ct2 = pk.encrypt_asymmetric(ctx, pt2)
+            t = lap("encrypt", t)
+            c.sub(ctx, ct2, ct1, tmp)
+            c.square_inplace(ctx, tmp)
+            c.add_inplace(ctx, acc, tmp)
+            t = lap("square_accumulate", t)
+        c.relinearize_inplace(ctx, acc, state.rlk)
+        c.rescale_to_next_inplace(ctx, acc)
+        acc.set_scale(scale)
+        t = lap("relinearize_rescale", t)
+        rot = c.ciphertext(ctx)
+        hoisted = c.hoisting(ctx, acc, state.glk, list(range(1, 16)))
+        c.add_inplace(ctx, acc, hoisted)
+        for k in range(4, log_slots):
+            c.rotate_vector(ctx, acc, 2 ** k, state.glk, rot)
+            c.add_inplace(ctx, acc, rot)
+        lap("rotate_and_sum", t)
+        return acc
+
+    _sync(c)
+    t0 = time.perf_counter()
+    enc_dist = [[None] * n_clients for _ in range(n_clients)]
+    for i in range(n_clients):
+        for j in range(i, n_clients):
+            enc_dist[i][j] = enc_dist[j][i] = pair(chunks[i], chunks[j])
+    _sync(c)
+    timings = dict(spent, distance_phase=time.perf_counter() - t0, pairs=n_clients * (n_clients + 1) // 2)
+    dist = np.zeros((n_clients, n_clients))
+    for i in range(n_clients):
+        for j in range(i + 1, n_clients):
+            dist[i, j] = dist[j, i] = state.encoder.decode_array(ctx, state.sk.decrypt(ctx, enc_dist[i][j]), 1)[0]
+    return dist, timings
+
+
 def _map_lanes(state: KrumState, items, fn):
     """[fn(item) for item in items], the items dealt round-robin to `lanes` host threads, each issuing on its own
     lane (stream) of the host layer (the evaluator, decrypt and decode calls release the interpreter lock);
