@@ -149,11 +149,12 @@ int he_tensor(const he_context *ctx, const uint64_t *ct1, const uint64_t *ct2, u
 /* Squaring variant; replaces tensor_square_2x2_rns_poly (src/polymath.cu:568-612). */
 int he_tensor_square(const he_context *ctx, const uint64_t *ct, uint64_t *out, uint32_t L, he_stream stream);
 
-/* General tensor product of a size-`size1` and a size-`size2` ciphertext (1 <= sizes <= 3): ct1 [size1][L][N],
+/* General tensor product of a size-`size1` and a size-`size2` ciphertext (1 <= sizes <= 16): ct1 [size1][L][N],
  * ct2 [size2][L][N] -> out [size1 + size2 - 1][L][N], out_j = sum over a + b = j of ct1_a * ct2_b (dyadic products,
  * summed in 128 bits, one reduction).  out may be ct1's buffer when that has room for the result; it must not
- * overlap ct2 otherwise.  Sizes above 3 return HE_E_UNSUPPORTED (the operands are held in registers; the reference
- * allocates them per thread with device-side new[] and accepts any size).
+ * overlap ct2 otherwise.  Sizes up to 3 x 3 keep their operands in registers; larger ones read them where they are
+ * needed.  Sizes above 16 return HE_E_UNSUPPORTED (the reference allocates its operands per thread with device-side
+ * new[] and accepts any size).
  * Replaces tensor_prod_mxn_rns_poly (src/polymath.cu:614-672). */
 int he_tensor_mxn(const he_context *ctx, const uint64_t *ct1, uint32_t size1, const uint64_t *ct2, uint32_t size2,
                   uint64_t *out, uint32_t L, he_stream stream);

@@ -698,7 +698,7 @@ int he_tensor_mxn(const he_context *ctx, const uint64_t *ct1, uint32_t size1, co
                   uint64_t *out, uint32_t L, he_stream s) {
     if (!ctx || !ct1 || !ct2 || !out || L == 0 || L > ctx->size_qp) return HE_E_INVALID_ARGUMENT;
     if (size1 == 0 || size2 == 0) return HE_E_INVALID_ARGUMENT;
-    if (size1 > 3 || size2 > 3) return HE_E_UNSUPPORTED;
+    if (size1 > 16 || size2 > 16) return HE_E_UNSUPPORTED;
     HE_HIP(launch_tensor_mxn(ctx->tables(), ct1, size1, ct2, size2, out, L, S(s)));
     return HE_OK;
 }

@@ -154,9 +154,9 @@ static void multiply_into(const CAHELGPUContext &context, const CAHELGPUCipherte
         throw std::invalid_argument("encrypted1 or encrypted2 must be in NTT form");
     const std::size_t size1 = encrypted1.size(), size2 = encrypted2.size();
     if (size1 < 2 || size2 < 2) throw std::invalid_argument("ciphertext size must be at least 2");
-    // the reference takes operands of any size (src/evaluate.cu:474-488: tensor_prod_mxn_rns_poly); here a size-3
-    // operand is the largest (what a multiplication without relinearisation leaves)
-    if (size1 > 3 || size2 > 3) throw std::invalid_argument("ciphertext multiplication takes operands of size 2 or 3");
+    // the reference takes operands of any size (src/evaluate.cu:474-488: tensor_prod_mxn_rns_poly); here up to 16
+    // polynomials each (he_tensor_mxn)
+    if (size1 > 16 || size2 > 16) throw std::invalid_argument("ciphertext multiplication takes operands of at most 16 polynomials");
     const std::size_t dest_size = size1 + size2 - 1;
     const uint32_t L = (uint32_t)encrypted1.coeff_modulus_size();
     const std::size_t chain = encrypted1.chain_index(), n = encrypted1.poly_modulus_degree();

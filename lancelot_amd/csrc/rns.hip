@@ -186,6 +186,23 @@ __global__ __launch_bounds__(kThreads) void tensor_mxn_kernel(TensorArgs p) {
     for (int j = 0; j < S1 + S2 - 1; j++) p.out[idx + poly * j] = o[j];
 }
 
+// The same product for operands of any size (run-time sizes, up to 16 polynomials each): nothing is kept in registers,
+// the operands are read where they are needed (a coefficient's S1 + S2 words stay in the first-level cache), at most
+// 16 products of 61-bit factors are summed in 128 bits per output.  Outputs are formed from the last to the first, so
+// that out may be ct1's buffer: output j overwrites word j of ct1, which only the outputs from j on read.
+__global__ __launch_bounds__(kThreads) void tensor_any_kernel(TensorArgs p, uint32_t s1, uint32_t s2) {
+    const uint32_t limb = blockIdx.y;
+    const uint64_t q = p.moduli[limb], r0 = p.barrett[2 * limb], r1 = p.barrett[2 * limb + 1];
+    const size_t poly = (size_t)p.L << p.log_n;
+    const size_t idx = ((size_t)limb << p.log_n) + blockIdx.x * kThreads + threadIdx.x;
+    for (uint32_t j = s1 + s2 - 1; j-- > 0;) {
+        const uint32_t a_first = j >= s2 ? j - (s2 - 1) : 0, a_last = j < s1 ? j : s1 - 1;
+        U128 acc{0, 0};
+        for (uint32_t a = a_first; a <= a_last; a++) mac128(acc, p.ct1[idx + poly * a], p.ct2[idx + poly * (j - a)]);
+        p.out[idx + poly * j] = barrett128(acc.lo, acc.hi, q, r0, r1);
+    }
+}
+
 // grid: (N / 256, limbs, items).  out[item][limb] = c0 + c1 * s (+ noise[item][limb]) for the ciphertext cts[item]
 __global__ __launch_bounds__(kThreads) void decrypt_gather_kernel(const uint64_t *const *cts, const uint64_t *sk,
                                                                   const uint64_t *noise, uint64_t *out,
@@ -843,7 +860,10 @@ hipError_t launch_tensor_mxn(const Tables &t, const uint64_t *ct1, uint32_t s1, 
 #define HE_CASE(A, B) \
     if (s1 == A && s2 == B) hipLaunchKernelGGL((tensor_mxn_kernel<A, B>), grid, dim3(kThreads), 0, s, p); else
     HE_CASE(1, 1) HE_CASE(1, 2) HE_CASE(1, 3) HE_CASE(2, 1) HE_CASE(2, 2) HE_CASE(2, 3) HE_CASE(3, 1) HE_CASE(3, 2)
-    HE_CASE(3, 3) return hipErrorInvalidValue;
+    HE_CASE(3, 3) {
+        if (s1 == 0 || s2 == 0 || s1 > 16 || s2 > 16) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(tensor_any_kernel, grid, dim3(kThreads), 0, s, p, s1, s2);
+    }
 #undef HE_CASE
     return hipGetLastError();
 }

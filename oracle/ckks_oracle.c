@@ -287,7 +287,7 @@ void orc_tensor_mxn(const orc_params *p, const uint64_t *ct1, uint32_t s1, const
         uint64_t q = p->mod[l];
         const uint64_t *r = p->ratio + 2 * (size_t)l;
         for (size_t i = (size_t)l * n; i < (size_t)(l + 1) * n; i++) {
-            uint64_t c1[8], c2[8], o[16];
+            uint64_t c1[16], c2[16], o[32];
             for (uint32_t a = 0; a < s1; a++) c1[a] = ct1[i + poly * a];
             for (uint32_t b = 0; b < s2; b++) c2[b] = ct2[i + poly * b];
             for (uint32_t j = 0; j < res; j++) {

@@ -343,7 +343,9 @@ class Params:
         return out
 
     def tensor_mxn(self, ct1: np.ndarray, ct2: np.ndarray) -> np.ndarray:
-        """(s1,L,N) x (s2,L,N) -> (s1+s2-1,L,N), sizes up to 8 (src/polymath.cu:614-672)."""
+        """(s1,L,N) x (s2,L,N) -> (s1+s2-1,L,N), sizes up to 16 (src/polymath.cu:614-672)."""
+        if not (1 <= ct1.shape[0] <= 16 and 1 <= ct2.shape[0] <= 16):
+            raise ValueError("tensor_mxn takes 1 to 16 polynomials per operand")
         s1, L = ct1.shape[0], ct1.shape[1]
         s2 = ct2.shape[0]
         out = np.empty((s1 + s2 - 1, L, self.n), dtype=np.uint64)

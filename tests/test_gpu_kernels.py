@@ -545,10 +545,11 @@ def test_tensor_and_square(small, capi):
         assert (dbuf.numpy() == p.tensor(a, b)).all()
 
 
-@pytest.mark.parametrize("s1,s2", [(2, 3), (3, 2), (3, 3), (2, 2), (1, 2)])
+@pytest.mark.parametrize("s1,s2", [(2, 3), (3, 2), (3, 3), (2, 2), (1, 2), (4, 2), (3, 5), (5, 5), (16, 16), (1, 9)])
 def test_tensor_mxn(small, capi, s1, s2):
-    """he_tensor_mxn against the oracle for every operand size up to 3 x 3, out of place and into the first operand's
-    buffer, with edge residues; sizes beyond 3 are refused."""
+    """he_tensor_mxn against the oracle for operand sizes up to 3 x 3 (operands in registers) and beyond (the
+    general kernel, up to 16 x 16: sixteen products of the largest residues in one 128-bit sum), out of place and
+    into the first operand's buffer, with edge residues; sizes beyond 16 are refused."""
     cahel, parms, ctx, p = small
     rng = np.random.default_rng(70 + 10 * s1 + s2)
     L = 5
@@ -570,7 +571,7 @@ def test_tensor_mxn(small, capi, s1, s2):
     dbig = DeviceArray(capi, host=big)
     capi.check(lib.he_tensor_mxn(h, dbig.ptr, s1, db.ptr, s2, dbig.ptr, L, None))
     assert (dbig.numpy() == want).all()
-    assert lib.he_tensor_mxn(h, da.ptr, 4, db.ptr, s2, dout.ptr, L, None) == -2
+    assert lib.he_tensor_mxn(h, da.ptr, 17, db.ptr, s2, dout.ptr, L, None) == -2
     assert lib.he_tensor_mxn(h, da.ptr, 0, db.ptr, s2, dout.ptr, L, None) == -1
 
 

@@ -360,7 +360,8 @@ def test_encrypt_symmetric_bit_exact_and_round_trip(world):
 def test_multiply_with_size_three_operands(world):
     """multiply / square of ciphertexts that were not relinearised (size 3): the general tensor product of
     src/evaluate.cu:474-488, 531-545.  Limbs against the oracle, and the size-5 results decrypt (c0 + c1 s + ... +
-    c4 s^4) to the product of the slots.  As in the reference, operands of different sizes are refused
+    c4 s^4) to the product of the slots; a size-5 operand squares to 9 polynomials.  As in the reference, operands of
+    different sizes are refused
     (src/evaluate.cu:369-370)."""
     w = world
     c, ctx, p = w["cahel"], w["ctx"], w["p"]
@@ -391,10 +392,14 @@ def test_multiply_with_size_three_operands(world):
         assert xy.size() == 5 and (xy.to_numpy() == p.tensor_mxn(o_xy, o_xy)).all()
         got = np.array(w["enc"].decode(ctx, w["sk"].decrypt(ctx, xy)))
         assert np.max(np.abs(got - (x * y) ** 2)) < 1e-3
+        # and once more: 5 x 5 polynomials take the general kernel (operands read in place), 9 come back
+        o_xy2 = p.tensor_mxn(o_xy, o_xy)
+        c.square_inplace(ctx, xy)
+        assert xy.size() == 9 and (xy.to_numpy() == p.tensor_mxn(o_xy2, o_xy2)).all()
+        got = np.array(w["enc"].decode(ctx, w["sk"].decrypt(ctx, xy)))
+        assert np.max(np.abs(got - (x * y) ** 4)) < 1e-2
     finally:
         w["sk"].set_noise_flooding(True)
-    with pytest.raises(ValueError, match="operands of size 2 or 3"):
-        c.square_inplace(ctx, xy)
 
 
 def test_error_behaviour(world):

@@ -263,7 +263,7 @@ def test_tensor_and_square_bigint(small):
             assert [int(s[k][i][j]) for k in range(3)] == [a0 * a0 % q, 2 * a0 * a1 % q, a1 * a1 % q]
 
 
-@pytest.mark.parametrize("s1,s2", [(2, 2), (2, 3), (3, 2), (3, 3), (1, 3)])
+@pytest.mark.parametrize("s1,s2", [(2, 2), (2, 3), (3, 2), (3, 3), (1, 3), (4, 2), (5, 5), (16, 16)])
 def test_tensor_mxn_is_the_convolution_of_the_operands(small, s1, s2):
     """orc_tensor_mxn against Python integers: polynomial j of the product is the sum of ct1_a ct2_b over a + b = j
     (the ciphertexts multiplied as polynomials in the secret key), coefficient by coefficient and limb by limb, with
