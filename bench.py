@@ -323,7 +323,12 @@ def main():
                          "batch_streams: the batch calls dealt to --batch-streams streams, as `value` issues them; "
                          "krum_reference: the Krum round plus the distance phase by the reference's own call sequence; "
                          "probe: the issue rates of the instruction kinds that the kernels' bounds are argued with")
+    ap.add_argument("--prime-bits", type=int, default=BITS,
+                    help="with --only ntt: size of the 32 primes (50: the benchmark's, FP64 back end; 51 to 60: the "
+                         "integer back end; the context is then built without the security check)")
     args = ap.parse_args()
+    if args.prime_bits != BITS and args.only != "ntt":
+        sys.exit("--prime-bits applies to --only ntt")
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
@@ -344,7 +349,7 @@ def main():
     n = 1 << LOG_N
     parms = cahel.params(cahel.scheme_type.ckks)
     parms.set_poly_modulus_degree(n)
-    parms.set_coeff_modulus(cahel.coeff_modulus_create(n, [BITS] * (SIZE_Q + SIZE_P)))
+    parms.set_coeff_modulus(cahel.coeff_modulus_create(n, [args.prime_bits] * (SIZE_Q + SIZE_P)))
     parms.set_special_modulus_size(SIZE_P)
     steps_pow2 = [1 << k for k in range(15)]
     # the same slot sum as four hoisted rounds (`hoisting` of the reference's API): steps 1..7, then 8, 128 and 2048
@@ -353,7 +358,7 @@ def main():
     all_steps = sorted(set(steps_pow2) | {s for rnd in hoist_rounds for s in rnd})
     parms.set_galois_elts(cahel.get_elts_from_steps(all_steps if args.only == "all" else
                                                     (steps_pow2 if args.only == "rotate" else [1]), n))
-    ctx = cahel.context(parms, True, cahel.sec_level_type.tc128)
+    ctx = cahel.context(parms, True, cahel.sec_level_type.tc128 if args.prime_bits == BITS else cahel.sec_level_type.none)
     ctx.set_seed(2025)
     sk = cahel.secret_key(parms)
     sk.gen_secretkey(ctx)
