@@ -77,7 +77,7 @@ int he_event_elapsed_ms(he_event start, he_event stop, float *ms);
  * (include/gpucontext.h:53-136: DNTTTable, DModulus) and the level-independent part of DRNSTool::init
  * (src/rns.cu:9-67).  All arrays are HOST pointers, copied during he_context_create. */
 typedef struct {
-    uint32_t log_n;               /* N = 2^log_n, 9 <= log_n <= 16 */
+    uint32_t log_n;               /* N = 2^log_n, 9 <= log_n <= 17 */
     uint32_t size_q;              /* Q limbs at the key level */
     uint32_t size_p;              /* special limbs (alpha); may be 0 when no key switching is used */
     uint32_t reserved;

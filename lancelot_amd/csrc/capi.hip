@@ -198,7 +198,7 @@ bool fp_for_level(const he_context *ctx, uint32_t L) {
 
 // base conversion fused with the rows pass of the forward transform that follows it (launch_bconv_rows)
 bool fuse_rows_ok(const he_context *ctx, const Level *lv, uint32_t L) {
-    return ctx->fuse_rows && lv && lv->batched && ctx->log_n >= 12 && fp_for_level(ctx, L);
+    return ctx->fuse_rows && lv && lv->batched && ctx->log_n >= 12 && ctx->log_n <= 16 && fp_for_level(ctx, L);
 }
 
 int check_map(const he_context *ctx, uint32_t limbs, uint32_t first, uint32_t split, uint32_t tail) {
@@ -331,7 +331,7 @@ int he_event_elapsed_ms(he_event start, he_event stop, float *ms) {
 
 int he_context_create(const he_context_desc *d, he_context **out) {
     if (!d || !out || !d->moduli || !d->barrett || !d->psi || !d->ipsi_div2) return HE_E_INVALID_ARGUMENT;
-    if (d->log_n < 9 || d->log_n > 16) return HE_E_UNSUPPORTED;
+    if (d->log_n < 9 || d->log_n > 17) return HE_E_UNSUPPORTED;
     if (d->size_q == 0 || d->size_q + d->size_p > 256) return HE_E_INVALID_ARGUMENT;
     if (d->size_p && (!d->p_mod_q || !d->pinv_mod_q || !d->phat_inv_mod_p || !d->phat_mod_q)) return HE_E_INVALID_ARGUMENT;
     for (uint32_t i = 0; i < d->size_q + d->size_p; i++)

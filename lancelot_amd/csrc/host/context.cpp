@@ -349,7 +349,7 @@ CAHELGPUContext::CAHELGPUContext(const EncryptionParameters &params, bool expand
     n_ = params.poly_modulus_degree();
     log_n_ = power_of_two(n_);
     if (log_n_ < 0) throw std::invalid_argument("invalid poly_modulus_degree");
-    if (log_n_ < 9 || log_n_ > 16) throw std::invalid_argument("poly_modulus_degree must be between 2^9 and 2^16");
+    if (log_n_ < 9 || log_n_ > 17) throw std::invalid_argument("poly_modulus_degree must be between 2^9 and 2^17");
     const auto &mods = params.coeff_modulus();
     if (mods.empty() || mods.size() > 64) throw std::invalid_argument("parameter generate failed");
     std::size_t size_qp = mods.size();

@@ -337,8 +337,8 @@ __device__ __forceinline__ void fp_ct_block(double *v, const double *table, uint
 }
 
 // Inverse block (no halving: the factor 1/N is applied once at the end of the transform).  Sums double
-// per stage, so after two stages the sum outputs are reduced again; outputs stay at or below 5 q (8 q from
-// canonical inputs without REDUCE_FIRST), which is below 2^53.
+// per stage, so in blocks of four or five stages the sum outputs are reduced again after every second stage (not
+// after the last); outputs stay at or below 5 q (8 q from canonical inputs without REDUCE_FIRST), which is below 2^53.
 template <int LOGR, bool REDUCE_FIRST>
 __device__ __forceinline__ void fp_gs_block(double *v, const double *table, uint32_t idx, FpMod m) {
     constexpr int R = 1 << LOGR;
@@ -359,7 +359,7 @@ __device__ __forceinline__ void fp_gs_block(double *v, const double *table, uint
                 v[2 * b * half + j + half] = fp_mulmod(x - y, tw, m);
             }
         }
-        if (LOGR == 4 && l == 2) {
+        if (LOGR >= 4 && l > 0 && ((LOGR - l) & 1) == 0) {
 #pragma unroll
             for (int b = 0; b < (1 << l); b++)
 #pragma unroll
@@ -426,7 +426,7 @@ __device__ __forceinline__ void fp_gs_block_tw(double *v, const double *tw, FpMo
                 v[2 * b * half + j + half] = fp_mulmod(x - y, t, m);
             }
         }
-        if (LOGR == 4 && l == 2) {
+        if (LOGR >= 4 && l > 0 && ((LOGR - l) & 1) == 0) {
 #pragma unroll
             for (int b = 0; b < (1 << l); b++)
 #pragma unroll

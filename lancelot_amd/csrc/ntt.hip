@@ -373,7 +373,9 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     const uint32_t lb = logical_block();
     const Job job = decode_job(a, lb / tiles_per_limb);
     const uint32_t col0 = (lb % tiles_per_limb) << LOGC;
-    if constexpr (LD >= 4 && tile_elems == 16 * kRowThreads) {
+    // (N = 2^17, 512 rows: the inner block would be five stages, 32 words a thread; that degree takes the tile
+    // through LDS between its blocks, below)
+    if constexpr (LD >= 4 && LD <= 8 && tile_elems == 16 * kRowThreads) {
         rows_direct<LD, FWD, BE, LOGC>(a, job, col0, lds);
         return;
     }
@@ -1488,7 +1490,7 @@ hipError_t launch_rows(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
         else                                                                                          \
             hipLaunchKernelGGL((ntt_rows_kernel<LD, FWD, FP, 12>), grid(LD, 12), dim3(256), 0, s, a); \
         break;
-        HE_CASE(1) HE_CASE(2) HE_CASE(3) HE_CASE(4) HE_CASE2(5) HE_CASE2(6) HE_CASE2(7) HE_CASE2(8)
+        HE_CASE(1) HE_CASE(2) HE_CASE(3) HE_CASE(4) HE_CASE2(5) HE_CASE2(6) HE_CASE2(7) HE_CASE2(8) HE_CASE(9)
 #undef HE_CASE
 #undef HE_CASE2
         default:
@@ -1621,7 +1623,7 @@ hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, const Tuning 
 }
 
 hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool rows_done) {
-    if (a.log_n < 9 || a.log_n > 16 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
+    if (a.log_n < 9 || a.log_n > 17 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
     if (!rows_done && one_pass_ok(a, backend, true, n_jobs)) return launch_limb_fp<true>(a, n_jobs, s);
@@ -1636,7 +1638,7 @@ hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, h
 }
 
 hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipStream_t s, bool rows_done) {
-    if (a.log_n < 9 || a.log_n > 16 || !a.jobs) return hipErrorInvalidValue;
+    if (a.log_n < 9 || a.log_n > 17 || !a.jobs) return hipErrorInvalidValue;
     const uint32_t items = x.items ? x.items : 1;
     if (items > 1 && (x.own_galois || x.add_c0 || (a.items ? a.items : 1) != items)) return hipErrorInvalidValue;
     if (a.n_jobs && !rows_done) {
@@ -1657,7 +1659,7 @@ hipError_t launch_ntt_forward_inner(const NttArgs &a, const KsFuseArgs &x, hipSt
 }
 
 hipError_t launch_tensor_intt_blocks(NttArgs a, const TensorFuse &x, hipStream_t s) {
-    if (a.log_n < 9 || a.log_n > 16 || a.jobs || a.map.limbs != x.L || x.L == 0) return hipErrorInvalidValue;
+    if (a.log_n < 9 || a.log_n > 17 || a.jobs || a.map.limbs != x.L || x.L == 0) return hipErrorInvalidValue;
     const BlocksPlan p = plan_blocks(a, 1);
     a.batch = 1;
     a.n_polys = 1;
@@ -1669,7 +1671,7 @@ hipError_t launch_tensor_intt_blocks(NttArgs a, const TensorFuse &x, hipStream_t
 }
 
 hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool blocks_done) {
-    if (a.log_n < 9 || a.log_n > 16 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
+    if (a.log_n < 9 || a.log_n > 17 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
     if (!blocks_done && one_pass_ok(a, backend, false, n_jobs)) return launch_limb_fp<false>(a, n_jobs, s);

@@ -454,3 +454,104 @@ def test_c5_pair_distances_against_the_oracle():
     want = krum.plain_distance_matrix(updates)
     for (i, j), v in zip(pairs, values):
         assert abs(v - want[i, j]) / want[i, j] < 2e-5
+
+
+@pytest.mark.parametrize("bits,size_p,L", [([50, 49, 50, 50, 50, 50], 2, 4), ([50, 49, 50, 50, 50, 50], 2, 3),
+                                            ([60, 40, 40, 60], 1, 3)])
+@pytest.mark.parametrize("no_fuse", ["0", "1"])
+def test_largest_degree_entry_points_bit_exact(oracle, monkeypatch, bits, size_p, L, no_fuse):
+    """N = 2^17, the largest degree of the reference's parameter tables (include/util/hestdparms.h): the rows pass has
+    512 rows there (a register block of five stages), the base conversions run as kernels of their own.  he_keyswitch,
+    he_keyswitch_rescale, he_multiply_relin_rescale, he_rotate and he_hoisted_rotations against the oracle, every
+    limb, on the FP64 and the mixed back end, with the inner product inside the forward transform and as a kernel of
+    its own, with a partial last digit."""
+    import ctypes as C
+    from gpu_util import DeviceArray, make_pair, rand_limbs
+    from lancelot_amd import capi
+    monkeypatch.setenv("CAHEL_HIP_NO_FUSED_KS", no_fuse)
+    cahel, parms, ctx, p = make_pair(oracle, 17, bits, size_p)
+    lib, h = capi.lib(), ctx.he_handle()
+    rng = np.random.default_rng(1700 + L)
+    n = p.n
+    beta = -(-L // size_p)
+    host_evk = [rand_limbs(p, rng, range(p.size_qp), n_polys=2) for _ in range(p.size_q // size_p)]
+    dev_evk = [DeviceArray(capi, host=k) for k in host_evk]
+    ptrs = capi.evk_array([d.ptr for d in dev_evk])
+    a, b = rand_limbs(p, rng, range(L), n_polys=2), rand_limbs(p, rng, range(L), n_polys=2)
+    da, db = DeviceArray(capi, host=a), DeviceArray(capi, host=b)
+    ws = DeviceArray(capi, shape=(lib.he_multiply_relin_rescale_workspace_words(h, L),))
+    # key switch of b[1] onto a, with and without the rescale
+    ks = p.key_switch(b[1], host_evk[:beta])
+    want_ks = np.stack([p.add(a[k], ks[k]) for k in range(2)])
+    dct = DeviceArray(capi, host=a)
+    capi.check(lib.he_keyswitch(h, L, db.at(L * n), ptrs, dct.ptr, 0, ws.ptr, None))
+    assert (dct.numpy() == want_ks).all()
+    out = DeviceArray(capi, shape=(2, L - 1, n))
+    capi.check(lib.he_keyswitch_rescale(h, L, db.at(L * n), ptrs, da.ptr, out.ptr, 0, ws.ptr, None))
+    assert (out.numpy() == p.rescale(want_ks)).all()
+    # the whole product
+    capi.check(lib.he_multiply_relin_rescale(h, L, da.ptr, db.ptr, ptrs, out.ptr, ws.ptr, None))
+    assert (out.numpy() == p.rescale(p.relinearize(p.tensor(a, b), host_evk[:beta]))).all()
+    # a rotation and a hoisted sum of three
+    elt = pow(5, 3, 2 * n)
+    rot = DeviceArray(capi, shape=(2, L, n))
+    capi.check(lib.he_rotate(h, L, da.ptr, ptrs, rot.ptr, elt, ws.ptr, None))
+    assert (rot.numpy() == p.apply_galois(a, elt, host_evk[:beta])).all()
+    steps = [1, 256, 777]
+    elts = [pow(5, s, 2 * n) for s in steps]
+    flat = capi.evk_array([dev_evk[d].ptr for _ in steps for d in range(beta)])
+    d_elts = (C.c_uint32 * len(steps))(*elts)
+    capi.check(lib.he_hoisted_rotations(h, L, da.ptr, flat, d_elts, len(steps), rot.ptr, ws.ptr, None))
+    assert (rot.numpy() == p.hoisting(a, elts, [host_evk[:beta]] * len(steps))).all()
+    assert (da.numpy() == a).all() and (db.numpy() == b).all()
+
+
+def test_largest_degree_scheme_flow(oracle):
+    """N = 2^17 through pyCAHEL: keys, encryption of 65,536 slots, multiply + relinearize_inplace + rescale, a rotation
+    and the decryption against the oracle limb for limb (same seeded randomness), decoded slots against the plain
+    product."""
+    O = oracle
+    from gpu_util import make_pair
+    logn, bits = 17, [50, 40, 40, 50, 50]
+    cahel, parms, ctx, p = make_pair(O, logn, bits, 1, seed=17)
+    # (make_pair builds the context without Galois elements: one of its own here)
+    parms.set_galois_elts(cahel.get_elts_from_steps([5], p.n))
+    ctx = cahel.context(parms, True, cahel.sec_level_type.tc128)
+    ctx.set_seed(17)
+    ks = O.KeySet(p, seed=17)
+    sk = cahel.secret_key(parms)
+    sk.gen_secretkey(ctx)
+    ks.gen_secret()
+    pk = cahel.public_key(ctx)
+    sk.gen_publickey(ctx, pk)
+    o_pk = ks.gen_public()
+    rlk = cahel.relin_key(ctx)
+    sk.gen_relinkey(ctx, rlk)
+    o_rlk = ks.gen_relin()
+    glk = cahel.galois_key(ctx)
+    sk.create_galois_keys(ctx, glk)
+    elt = cahel.get_elts_from_steps([5], p.n)[0]
+    o_glk = ks.gen_galois(elt)
+    enc = cahel.ckks_encoder(ctx)
+    assert enc.slot_count() == 65536
+    rng = np.random.default_rng(17)
+    x, y = rng.uniform(-1, 1, p.n // 2), rng.uniform(-1, 1, p.n // 2)
+    px, py = enc.encode(ctx, x, 2.0 ** 40), enc.encode(ctx, y, 2.0 ** 40)
+    cx, cy = pk.encrypt_asymmetric(ctx, px), pk.encrypt_asymmetric(ctx, py)
+    o_cx = ks.encrypt_asymmetric(o_pk, px.to_numpy())
+    o_cy = ks.encrypt_asymmetric(o_pk, py.to_numpy())
+    assert (cx.to_numpy() == o_cx).all() and (cy.to_numpy() == o_cy).all()
+    prod = cahel.ciphertext(ctx)
+    cahel.multiply(ctx, cx, cy, prod)
+    cahel.relinearize_inplace(ctx, prod, rlk)
+    cahel.rescale_to_next_inplace(ctx, prod)
+    want = p.rescale(p.relinearize(p.tensor(o_cx, o_cy), o_rlk))
+    assert (prod.to_numpy() == want).all()
+    rot = cahel.ciphertext(ctx)
+    cahel.rotate_vector(ctx, prod, 5, glk, rot)
+    assert (rot.to_numpy() == p.apply_galois(want, elt, o_glk)).all()
+    pt = sk.decrypt(ctx, rot)
+    assert (pt.to_numpy() == ks.decrypt(p.apply_galois(want, elt, o_glk), O.gauss_cdt())).all()
+    got = np.array(enc.decode(ctx, pt))
+    err = np.abs(got - np.roll(x * y, -5))
+    assert np.median(err) < 1e-4 and np.max(err) < 2e-2      # 2^30 of scale left; the floor-rescale bias in the first slots

@@ -51,7 +51,7 @@ def test_tables_match_oracle(small):
 # 2^50, the FP64 back end
 @pytest.mark.parametrize("one_pass", ["default", "off", "forced"])
 @pytest.mark.parametrize("bits", [[60, 50, 35, 59], [50, 49, 35, 50]])
-@pytest.mark.parametrize("logn", [9, 10, 11, 12, 13, 14, 15, 16])
+@pytest.mark.parametrize("logn", [9, 10, 11, 12, 13, 14, 15, 16, 17])
 def test_ntt_all_sizes(oracle, capi, monkeypatch, logn, bits, one_pass):
     """Forward and inverse against the oracle at every degree; up to N = 2^14 with all primes below 2^50 the plain
     transform can be one kernel with the limb resident in LDS (by default where it is the faster form: N <= 2^12, or
