@@ -43,6 +43,7 @@ struct Level {
     uint32_t modup_max_rows = 0, modup_max_copy = 0;
     bool batched = false;
     double *d_mats_fp = nullptr;         // (M, M/m) pairs of the digit matrices, when every prime is below 2^50
+    int32_t *d_mx_up = nullptr;          // the same matrices as 7-bit digits for the int8 matrix cores (N = 2^16)
 };
 
 }  // namespace
@@ -110,6 +111,7 @@ struct he_context {
     std::vector<Level> levels;   // indexed by L
     std::vector<void *> owned;
 
+    int32_t *d_mx_down = nullptr, *d_mx_last = nullptr;   // the P -> Ql matrix (times P^-1) for the int8 matrix cores
     Tables tables() const { return Tables{d_moduli, d_barrett, log_n}; }
     size_t n() const { return (size_t)1 << log_n; }
 };
@@ -121,6 +123,43 @@ namespace {
         hipError_t _e = (expr);               \
         if (_e != hipSuccess) return (int)_e; \
     } while (0)
+
+// One record of BconvRows::mx_tab: up to four rows of a conversion matrix with at most 8 columns as 7-bit digits of
+// M[r][i] 2^(8 j) mod q_r, laid out as the A operands of v_mfma_i32_16x16x64_i8, and the offsets that undo the shift of
+// the input bytes by 128.  entry(rr, i) / modulus(rr): row rr of the record (rr < rows).  term = +1 / -1: byte 7 of limb i
+// carries byte i of a number that is added / subtracted (digits of +-2^(8 i) mod q_r there), see BconvRows::mx_last.
+template <typename Entry, typename Modulus>
+void mx_record(std::vector<int32_t> &tab, uint32_t rows, uint32_t n_in, int term, Entry entry, Modulus modulus) {
+    const size_t base = tab.size();
+    tab.resize(base + 4 * kMxRecord, 0);
+    int8_t *amat = reinterpret_cast<int8_t *>(tab.data() + base);
+    double offs[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    uint64_t m8[64];
+    for (uint32_t rr = 0; rr < 4 && rr < rows; rr++) {
+        const uint64_t q = modulus(rr);
+        for (uint32_t i = 0; i < 8; i++) {
+            uint64_t v = i < n_in ? entry(rr, i) % q : 0;
+            for (uint32_t j = 0; j < 7; j++) {
+                m8[8 * i + j] = v;
+                v = (uint64_t)(((unsigned __int128)v << 8) % q);
+            }
+            const uint64_t pw = (uint64_t)((((unsigned __int128)1) << (8 * i)) % q);
+            m8[8 * i + 7] = (term == 0 || i == 7) ? 0 : term > 0 ? pw : (q - pw) % q;
+        }
+        for (uint32_t h = 0; h < 2; h++)
+            for (uint32_t e = 0; e < 4; e++) {
+                // row 4 rr + e of the instruction: lanes 16 kg + (4 rr + e) supply k = 16 kg .. 16 kg + 15
+                int64_t sum = 0;
+                for (uint32_t k = 0; k < 64; k++) {
+                    const int8_t digit = (int8_t)((m8[k] >> (7 * (4 * h + e))) & 127);
+                    amat[((size_t)h * 64 + 16 * (k / 16) + 4 * rr + e) * 16 + k % 16] = digit;
+                    sum += digit;
+                }
+                offs[2 * rr + h] += (double)((128 * sum) << (7 * e));
+            }
+    }
+    memcpy(tab.data() + base + 4 * 128, offs, sizeof(offs));
+}
 
 template <typename T>
 int upload(he_context *ctx, T **dst, const T *src, size_t count) {
@@ -421,6 +460,7 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->tune.hoist_no_local = env_on("CAHEL_HIP_NO_LOCAL_HOIST");
         ctx->tune.hoist_no_xcd = env_on("CAHEL_HIP_NO_XCD_MAP");
         ctx->tune.hoist_no_contig = env_on("CAHEL_HIP_NO_XCD_CONTIG");
+        ctx->tune.no_matrix_bconv = env_on("CAHEL_HIP_NO_MATRIX_BCONV");
         ctx->tune.fuse_rows_forced = env_count("CAHEL_HIP_FUSE_ROWS", 1, 24, 0);
         ctx->tune.bconv_rows = env_count("CAHEL_HIP_BCONV_ROWS", 1, 64, 6);
         int cus = 0;
@@ -465,6 +505,22 @@ int he_context_create(const he_context_desc *d, he_context **out) {
                     pfp[2 * (jq * d->size_p + k) + 1] = (double)v / (double)q;
                 }
             if (!rc) rc = upload(ctx, &ctx->d_phat_pinv_fp, pfp.data(), pfp.size());
+            if (!rc && d->log_n == 16 && d->size_p <= 8) {
+                // the same matrix for the int8 matrix cores: rows in groups of four with the bytes of the rescale term,
+                // and every row alone (the row of the limb that a level drops)
+                std::vector<int32_t> grp, single;
+                auto entry = [&](size_t jq, uint32_t k) {
+                    return (uint64_t)((unsigned __int128)d->phat_mod_q[jq * d->size_p + k] * d->pinv_mod_q[2 * jq] % d->moduli[jq]);
+                };
+                for (uint32_t r0 = 0; r0 < d->size_q; r0 += 4)
+                    mx_record(grp, d->size_q - r0, d->size_p, 1, [&](uint32_t rr, uint32_t k) { return entry(r0 + rr, k); },
+                              [&](uint32_t rr) { return d->moduli[r0 + rr]; });
+                for (uint32_t r = 0; r < d->size_q; r++)
+                    mx_record(single, 4, d->size_p, 0, [&](uint32_t, uint32_t k) { return entry(r, k); },
+                              [&](uint32_t) { return d->moduli[r]; });
+                rc = upload(ctx, &ctx->d_mx_down, grp.data(), grp.size());
+                if (!rc) rc = upload(ctx, &ctx->d_mx_last, single.data(), single.size());
+            }
         }
         if (!rc) rc = upload(ctx, &ctx->d_psi_fp, psi_fp.data(), psi_fp.size());
         if (!rc) rc = upload(ctx, &ctx->d_ipsi_fp, ipsi_fp.data(), ipsi_fp.size());
@@ -563,8 +619,7 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
                 bd.n_in = K;
                 bd.n_out = L;
             }
-            rc = upload(ctx, &lv.d_modup_descs, up.data(), up.size());
-            if (!rc) rc = upload(ctx, &lv.d_moddown_descs, down.data(), down.size());
+            rc = upload(ctx, &lv.d_moddown_descs, down.data(), down.size());
             if (!rc) rc = upload(ctx, &lv.d_modup_limb, limb_all.data(), limb_all.size());
             if (!rc) rc = upload(ctx, &lv.d_modup_table, table_all.data(), table_all.size());
             if (rc) return rc;
@@ -585,7 +640,26 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
                 }
                 rc = upload(ctx, &lv.d_mats_fp, mfp.data(), mfp.size());
                 if (rc) return rc;
+                if (ctx->log_n == 16) {
+                    // the digit matrices for the int8 matrix cores (BconvRows::mx_tab), one record per four output rows
+                    std::vector<int32_t> tab;
+                    for (uint32_t dg = 0; dg < beta; dg++) {
+                        const Digit &g = lv.digits[dg];
+                        up[dg].mx_off = (uint32_t)(tab.size() / (4 * kMxRecord));
+                        for (uint32_t r0 = 0; r0 < g.n_out; r0 += 4)
+                            mx_record(tab, g.n_out - r0, g.size, 0,
+                                      [&](uint32_t rr, uint32_t i) { return d->digit_mats[g.mat_off + (size_t)(r0 + rr) * g.size + i]; },
+                                      [&](uint32_t rr) {
+                                          const uint32_t r = r0 + rr;
+                                          return ctx->h_moduli[table_of(ctx, L, r < g.start ? r : r + g.size)];
+                                      });
+                    }
+                    rc = upload(ctx, &lv.d_mx_up, tab.data(), tab.size());
+                    if (rc) return rc;
+                }
             }
+            rc = upload(ctx, &lv.d_modup_descs, up.data(), up.size());
+            if (rc) return rc;
         }
         // limbs with the same modulus sit together so that one set of workgroups can share the twiddle table
         std::stable_sort(jobs.begin(), jobs.end(), [](const LimbJob &x, const LimbJob &y) { return x.table < y.table; });
@@ -801,7 +875,7 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     } else if (fused) {
         BconvRows b{ws, out, c, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
                     lv->beta, lv->modup_max_rows, copy_rows,
-                    items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n, 0};
+                    items, (size_t)L * n, (size_t)lv->beta * LK * n, (size_t)c_item_stride * n, 0, lv->d_mx_up};
         HE_HIP(launch_bconv_rows(base_args(ctx, true), b, ctx->tune, S(s)));
     } else if (lv->batched) {
         BconvBatch b{ws, out, c, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
@@ -1019,7 +1093,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         const bool rows_done = fuse_rows_ok(ctx, lv, L);
         if (rows_done) {
             BconvRows b{tmp, y, nullptr, lv->d_mats_fp, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
-                        lv->beta, lv->modup_max_rows, 0, items, (size_t)L * n, fwd.item_stride, 0, 0};
+                        lv->beta, lv->modup_max_rows, 0, items, (size_t)L * n, fwd.item_stride, 0, 0, lv->d_mx_up};
             HE_HIP(launch_bconv_rows(fwd, b, ctx->tune, S(s)));
         } else {
             BconvBatch b{tmp, y, src, lv->d_mats, lv->d_modup_limb, lv->d_modup_table, lv->d_modup_descs,
@@ -1193,7 +1267,8 @@ int ksr_impl(const he_context *ctx, uint32_t L, uint32_t items, const uint64_t *
     } else if (fused) {
         // with the prologue of (4) and the rows pass of its transform
         BconvRows b{cx, delta, nullptr, ctx->d_phat_pinv_fp, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,
-                    items, 2 * (size_t)LK * n, 2 * (size_t)L * n, 0, 1};
+                    items, 2 * (size_t)LK * n, 2 * (size_t)L * n, 0, 1, ctx->d_mx_down,
+                    ctx->d_mx_last ? ctx->d_mx_last + (size_t)(L - 1) * 4 * kMxRecord : nullptr};
         HE_HIP(launch_bconv_rows(base_args(ctx, true), b, ctx->tune, S(s)));
     } else if (lv->batched) {
         BconvBatch b{cx, delta, nullptr, ctx->d_phat_mod_q, ctx->d_iota, ctx->d_iota, lv->d_moddown_descs, 2, L, 0,

@@ -15,6 +15,7 @@ struct Tuning {
     bool hoist_no_local = false;     // CAHEL_HIP_NO_LOCAL_HOIST=1
     bool hoist_no_xcd = false;       // CAHEL_HIP_NO_XCD_MAP=1
     bool hoist_no_contig = false;    // CAHEL_HIP_NO_XCD_CONTIG=1
+    bool no_matrix_bconv = false;    // CAHEL_HIP_NO_MATRIX_BCONV=1: the fused base conversion stays on the FP64 vector units
 };
 
 // One limb-sized NTT job given explicitly: which limb of the buffer, which modulus table.
@@ -194,7 +195,7 @@ struct BconvDesc {
     uint32_t map_off;    // offset into out_limb / out_table
     uint32_t n_in, n_out;
     uint32_t copy_first, copy_count;  // limbs copied from copy_base (same limb index in the unit's output)
-    uint32_t pad;
+    uint32_t mx_off;     // first record of this unit in BconvRows::mx_tab (one record per four output rows)
 };
 struct BconvBatch {
     const uint64_t *x_base;
@@ -232,7 +233,20 @@ struct BconvRows {
     // merged ModDown + rescale: the last row of every unit's matrix is the limb that is dropped; the other output
     // limbs receive sum_i x_i M[j][i] + ((t - sum_i x_i M[last][i] mod q_last) mod q_j), t = the limb before x
     int mdr;
+    // The unit's matrices for the int8 matrix cores (N = 2^16), or nullptr.  M_ij = M[r][i] 2^(8 j) mod q_r in eight
+    // digits of 7 bits: sum_i x_i M[r][i] = sum over the bytes x_ij of x_i of x_ij M_ij (mod q_r), a 64-term product per
+    // digit with the bytes as they lie in memory.  One record of kMxRecord 16-byte words per group of four output rows:
+    // [half h = digits 4 h .. 4 h + 3][lane]: the lane's 16 bytes of the A operand (row 4 rr + e of the instruction is
+    // digit 4 h + e of output row rr; k = 8 limb + byte), then 8 doubles: for each row rr the offsets of its low and
+    // high digit groups, 128 x sum_e 2^(7 e) x (sum of the row of digit 4 h + e): the bytes enter as x - 128.
+    const void *mx_tab;
+    // mdr: the record of the dropped limb's row, alone and repeated in the four row slots of its record (every lane then
+    // holds the row's sums for its coefficient).  Byte 7 of input limb i is free (the residues are below 2^50): the kernel
+    // stores byte i of r = (t - sum_i x_i M[last][i]) mod q_last there, and the records of mx_tab multiply it by the
+    // digits of 2^(8 i) mod q_r.
+    const void *mx_last;
 };
+constexpr uint32_t kMxRecord = 144;
 // `a` supplies the FP64 twiddles and constants of a forward transform (base_args)
 hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, const Tuning &tune, hipStream_t s);
 

@@ -679,8 +679,9 @@ struct BconvRowsK {
 // register block of LOGR stages on the groups of a tile that lives in LDS (tile index bits: [upper][LOGR bits][low_bits]);
 // P words per thread; twl: entries 0..255 of the limb's twiddle table, in LDS; LAST: the results go to global memory
 // (lazy signed doubles for the blocks pass), else back to LDS
-template <int LD, int P, int LOGR, bool LAST>
+template <int LD, int P, int LOGR, bool LAST, bool SWZ = false>
 __device__ __forceinline__ void fuse_block(double *ld, const double *twl, uint32_t s0, FpMod m, uint64_t *dst, uint32_t col0) {
+    auto slot = [](uint32_t e) { return SWZ ? e ^ ((((e >> 5) ^ (e >> 8)) & 3u) << 3) : skew8(e); };
     constexpr int LOGC = kFuseLog - LD;
     constexpr uint32_t C = 1u << LOGC, T = kFuseWords / P;
     constexpr int R = 1 << LOGR, PER = P >> LOGR;
@@ -693,7 +694,7 @@ __device__ __forceinline__ void fuse_block(double *ld, const double *twl, uint32
         const uint32_t base = (upper << (low_bits + LOGR)) | (g & low_mask);
         double v[R];
 #pragma unroll
-        for (int j = 0; j < R; j++) v[j] = ld[skew8(base + ((uint32_t)j << low_bits))];
+        for (int j = 0; j < R; j++) v[j] = ld[slot(base + ((uint32_t)j << low_bits))];
         fp_ct_block<LOGR, 2>(v, twl, (1u << s0) + upper, m);
 #pragma unroll
         for (int j = 0; j < R; j++) {
@@ -701,7 +702,7 @@ __device__ __forceinline__ void fuse_block(double *ld, const double *twl, uint32
             if (LAST)
                 dst[(size_t)(e >> LOGC) * 256 + col0 + (e & (C - 1))] = (uint64_t)__double_as_longlong(v[j]);
             else
-                ld[skew8(e)] = v[j];
+                ld[slot(e)] = v[j];
         }
     }
 }
@@ -914,6 +915,267 @@ void bconv_rows_fp_kernel(NttArgs a, BconvRowsK p) {
             if (more && threadIdx.x < 256) twl[(r + 1) % 3][threadIdx.x] = tw_nxt;
             lds_barrier();  // every read of this tile is done before the next output limb overwrites it
         }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The same fusion at N = 2^16 with the matrix product of the conversion on the int8 matrix cores.
+//
+// sum_i x_i M[r][i] mod q_r is a 64-term integer product per 7-bit digit of the constants M_ij = M[r][i] 2^(8 j) mod q_r,
+// over the bytes x_ij of the inputs as they lie in memory (BconvRows::mx_tab).  One v_mfma_i32_16x16x64_i8 forms it for 16
+// coefficients, four output rows and four digits; two of them (digits 0..3, 4..7) leave the 8 digit sums S_e < 2^21 of
+// (row rr, coefficient c) in lane 16 rr + c, and
+//     sum_e S_e 2^(7 e) = lo + 2^28 hi,   lo = S_0 + 2^7 S_1 + 2^14 S_2 + 2^21 S_3 < 2^43,  hi likewise,
+// becomes the lazy residue (hi x (2^28 mod q)) mod q + lo with one modular product: 13 FP64-rate operations and two
+// matrix instructions per word against 44 operations for the eight exact multiply-adds on the vector units.
+//
+// Wave w of the workgroup owns the coefficients of rows w + 4 j + 32 i (j, i < 8) of the 256 x 8 tile, as in the kernel
+// above; lane (kg, c) keeps the words of input limbs 2 kg, 2 kg + 1 for coefficient c of each of 32 sets of 16
+// coefficients (set (g, i): (j, column) = (2 g + c / 8, c % 8), row w + 4 j + 32 i), which is at once the B operand of the
+// set.  Output rows go four at a time: lane (rr, c) receives row rr's words of every set, i.e. for each g the 8 words
+// i = 0..7 of one first register block, runs the block on them and stores them to row rr's tile in LDS.  The second block
+// (stages 3..5) stays inside the wave tile by tile, the third follows a workgroup barrier, as above.
+//
+// LDS index of tile word e = (row << 3) | column: bits 4..3 are XORed with bits 6..5 and bits 9..8.  The accesses of
+// a half-wave vary the column and either bit 5 (first block), bits 9..8 (second) or bits 6..5 (third) with bits 4..3
+// fixed, so they fall into distinct 8-byte banks; consecutive tiles start 16 words apart modulo 32, which separates the
+// two output rows that the lanes of a half-wave store in the first block.
+// ---------------------------------------------------------------------------------------------------
+typedef int v4i __attribute__((ext_vector_type(4)));
+constexpr uint32_t kMxStride = kFuseWords + 16;
+__device__ __forceinline__ uint32_t swz8(uint32_t e) { return e ^ ((((e >> 5) ^ (e >> 8)) & 3u) << 3); }
+
+template <bool MDR>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
+void bconv_rows_mx_kernel(NttArgs a, BconvRowsK p) {
+    __shared__ double tiles[4 * kMxStride];
+    __shared__ double twl[4][256];
+    __shared__ double rconst[2][4][4];         // per group parity and row: q, 1/q, and the two offsets of the digit sums
+    __shared__ uint32_t rlimb[2][4];
+    __shared__ uint32_t rtable[kFuseMaxRows + 4];
+    constexpr int LOGC = 3;
+    constexpr uint32_t tiles_per_limb = 32;
+
+    uint32_t lb = logical_block();
+    const uint32_t groups = p.compute_groups + p.copy_groups;
+    const uint32_t grp = lb % groups;
+    lb /= groups;
+    const uint32_t tile = lb % tiles_per_limb, uidx = lb / tiles_per_limb;
+    const uint32_t item = uidx / p.b.n_units;
+    const BconvDesc d = p.b.descs[uidx - item * p.b.n_units];
+    const uint32_t col0 = tile << LOGC;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6, kg = lane >> 4, cn = lane & 15;
+    uint64_t *out = p.b.out_base + item * p.b.out_item_stride + d.out_off;
+
+    if (grp >= p.compute_groups) {
+        // limbs that pass through unchanged (a digit's own limbs keep their NTT form)
+        const uint64_t *from = p.b.copy_base + item * p.b.copy_item_stride;
+        const uint32_t first = (grp - p.compute_groups) * p.rows_per;
+        const size_t g0 = (size_t)(threadIdx.x >> LOGC) * 256 + col0 + (threadIdx.x & 7);
+        for (uint32_t r = first; r < first + p.rows_per && r < d.copy_count; r++) {
+            const size_t limb = (size_t)(d.copy_first + r) << 16;
+            uint64_t w[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) w[i] = from[limb + g0 + (size_t)i * 32 * 256];
+#pragma unroll
+            for (int i = 0; i < 8; i++) out[limb + g0 + (size_t)i * 32 * 256] = w[i];
+        }
+        return;
+    }
+    const uint32_t n_rows = MDR ? d.n_out - 1 : d.n_out;
+    const uint32_t r_begin = grp * p.rows_per;
+    const uint32_t r_end = r_begin + p.rows_per < n_rows ? r_begin + p.rows_per : n_rows;
+    if (r_begin >= n_rows) return;
+
+    // the tables of this workgroup's rows (rows past the end repeat the last one; they are computed and not stored)
+    if (threadIdx.x < kFuseMaxRows + 4) {
+        const uint32_t r = r_begin + threadIdx.x < r_end ? r_begin + threadIdx.x : r_end - 1;
+        rtable[threadIdx.x] = p.b.out_table[d.map_off + r];
+    }
+    // the inputs: bytes 0..6 as signed numbers (x - 128), byte 7 (zero: the residues are below 2^50) stays zero
+    const uint64_t *x = p.b.x_base + item * p.b.x_item_stride + d.x_off;
+    const uint32_t l0 = 2 * kg < d.n_in ? 2 * kg : d.n_in - 1, l1 = 2 * kg + 1 < d.n_in ? 2 * kg + 1 : d.n_in - 1;
+    // (a uniform base and 32-bit byte offsets: one address register per load in flight instead of two)
+    const char *xbytes = reinterpret_cast<const char *>(x);
+    int xb[32][4];   // (scalars: the merged mode rewrites single bytes of them in place)
+    auto operand = [&](int s) { return v4i{xb[s][0], xb[s][1], xb[s][2], xb[s][3]}; };
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const uint32_t G = cn + 16 * g;
+        const uint32_t o = ((wave + 4 * (G >> 3)) * 256 + (G & 7) + col0) * 8;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t oi = o + (uint32_t)i * (32 * 256 * 8);
+            const uint64_t u0 = *reinterpret_cast<const uint64_t *>(xbytes + ((l0 << 19) + oi)) ^ 0x0080808080808080ull;
+            const uint64_t u1 = *reinterpret_cast<const uint64_t *>(xbytes + ((l1 << 19) + oi)) ^ 0x0080808080808080ull;
+            xb[8 * g + i][0] = (int)(uint32_t)u0;
+            xb[8 * g + i][1] = (int)(uint32_t)(u0 >> 32);
+            xb[8 * g + i][2] = (int)(uint32_t)u1;
+            xb[8 * g + i][3] = (int)(uint32_t)(u1 >> 32);
+        }
+    }
+    if (MDR) {
+        // merged ModDown + rescale: r = (t - sum_i x_i M[last][i]) mod q_last, canonical, is added to every output row;
+        // its bytes 0..6 go into byte 7 of the words of limbs 0..6, where the rows' records hold the digits of 2^(8 i).
+        // The record of the dropped row repeats it in all four row slots, so that every lane holds r of its coefficient.
+        // t, the limb before the unit's inputs, crosses LDS (the tiles are not in use yet): fetched per lane where it is
+        // needed, its 32 words would wait in registers beside the inputs.
+        {
+            const uint64_t *tsrc = x - ((size_t)1 << 16) + col0 + (size_t)(threadIdx.x >> LOGC) * 256 + (threadIdx.x & 7);
+            uint64_t *tl = reinterpret_cast<uint64_t *>(tiles);
+            uint64_t tw[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) tw[i] = tsrc[(size_t)i * 32 * 256];
+#pragma unroll
+            for (int i = 0; i < 8; i++) tl[threadIdx.x + 256 * i] = tw[i];   // tile word (row << 3) | column
+        }
+        lds_barrier();
+        const uint32_t ltable = p.b.out_table[d.map_off + d.n_out - 1];
+        const FpMod ml{a.fp_consts[4 * (size_t)ltable], a.fp_consts[4 * (size_t)ltable + 1]};
+        const v4i *lrec = reinterpret_cast<const v4i *>(p.b.mx_last);
+        const v4i la = lrec[lane], lh = lrec[64 + lane];
+        const double *loff = reinterpret_cast<const double *>(lrec + 128);
+        const double off_lo = loff[0], off_hi = loff[1];
+        const double c28 = fp_reduce(0x1p28, ml);
+        const FpTw w28{c28, c28 * ml.qinv};
+        const uint64_t *tl = reinterpret_cast<const uint64_t *>(tiles);
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const uint32_t G = cn + 16 * g;
+            const uint32_t e = ((wave + 4 * (G >> 3)) << LOGC) | (G & 7);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const v4i zero = {0, 0, 0, 0};
+                const v4i lo = __builtin_amdgcn_mfma_i32_16x16x64_i8(la, operand(8 * g + i), zero, 0, 0, 0);
+                const v4i hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(lh, operand(8 * g + i), zero, 0, 0, 0);
+                const int l01 = lo.x + lo.y * 128, l23 = lo.z + lo.w * 128;
+                const int h01 = hi.x + hi.y * 128, h23 = hi.z + hi.w * 128;
+                const double ld = __builtin_fma((double)l23, 16384.0, (double)l01) + off_lo;
+                const double hd = __builtin_fma((double)h23, 16384.0, (double)h01) + off_hi;
+                const double t = fp_from_u64(tl[e + ((uint32_t)(32 * i) << LOGC)]);
+                const uint64_t r = fp_to_u64(fp_canonical(t - (fp_mulmod(hd, w28, ml) + ld), ml));
+                const uint32_t b0 = (uint32_t)(r >> (16 * kg)) & 0xffu, b1 = (uint32_t)(r >> (16 * kg + 8)) & 0xffu;
+                // (in place: as a new value in the source, the compiler keeps the old and the new operand beside each other,
+                // 32 times four registers)
+                asm volatile("v_or_b32 %0, %0, %1" : "+v"(xb[8 * g + i][1]) : "v"((b0 ^ 0x80u) << 24));
+                asm volatile("v_or_b32 %0, %0, %1" : "+v"(xb[8 * g + i][3]) : "v"((b1 ^ 0x80u) << 24));
+            }
+        }
+        lds_barrier();   // the tiles are free again
+    }
+    const v4i *rec = reinterpret_cast<const v4i *>(p.b.mx_tab) + ((size_t)d.mx_off + (r_begin >> 2)) * kMxRecord;
+    lds_barrier();   // rtable
+
+    // Twiddles: entries 1..63 of a row's table serve the first two blocks, 64..255 the third.  Thread t fetches entry
+    // t % 64 of row t / 64 for the first part and entries 64 + t % 64 + 64 c (c < 3) of that row for the second.
+    const uint32_t trow = threadIdx.x >> 6, tcol = threadIdx.x & 63;
+    auto low_part = [&](uint32_t k) {   // group k of this workgroup: (entry tcol of row trow, that row's constants)
+        return a.tw_fp[((size_t)rtable[4 * k + trow] << 16) + tcol];
+    };
+    auto stage_consts = [&](uint32_t k, const v4i *rc) {
+        if (threadIdx.x < 16) {
+            const uint32_t rr = threadIdx.x >> 2, c = threadIdx.x & 3;
+            const double *off = reinterpret_cast<const double *>(rc + 128);
+            rconst[k & 1][rr][c] = c < 2 ? a.fp_consts[4 * (size_t)rtable[4 * k + rr] + c] : off[2 * rr + (c - 2)];
+        }
+        if (threadIdx.x >= 16 && threadIdx.x < 20) {
+            const uint32_t rr = threadIdx.x - 16;
+            const uint32_t r = r_begin + 4 * k + rr < r_end ? r_begin + 4 * k + rr : r_end - 1;
+            rlimb[k & 1][rr] = p.b.out_limb[d.map_off + r];
+        }
+    };
+    twl[trow][tcol] = low_part(0);
+    stage_consts(0, rec);
+    lds_barrier();
+
+    // a group's matrix digits (from L2: every workgroup of the unit reads the same ones); the next group's are requested
+    // as soon as the first block has issued its last product
+    v4i alo = rec[lane], ahi = rec[64 + lane];
+    uint32_t k = 0;
+    for (uint32_t r0 = r_begin; r0 < r_end; r0 += 4, rec += kMxRecord, k++) {
+        const uint32_t nr = r_end - r0 < 4 ? r_end - r0 : 4;
+        const bool more = r0 + 4 < r_end;
+        {
+            // first block, lane (rr, c) on row rr = kg
+            const FpMod mod{rconst[k & 1][kg][0], rconst[k & 1][kg][1]};
+            const double off_lo = rconst[k & 1][kg][2], off_hi = rconst[k & 1][kg][3];
+            const double c28 = fp_reduce(0x1p28, mod);
+            const FpTw w28{c28, c28 * mod.qinv};
+            const double *tws = twl[kg];
+            double *tile_ld = tiles + kg * kMxStride;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                // (opaque: computed once for the whole loop, the 32 store addresses would occupy registers through all of it)
+                uint32_t cn_ = cn;
+                asm volatile("" : "+v"(cn_));
+                const uint32_t G = cn_ + 16 * g;
+                const uint32_t z = swz8(((wave + 4 * (G >> 3)) << LOGC) | (G & 7));
+                double v[8];
+                // (the products of set i + 1 are issued before set i's are taken up: the matrix cores need 16 cycles each)
+                const v4i zero = {0, 0, 0, 0};
+                v4i lo_next = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, operand(8 * g), zero, 0, 0, 0);
+                v4i hi_next = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, operand(8 * g), zero, 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const v4i lo = lo_next, hi = hi_next;
+                    if (i < 7) {
+                        lo_next = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, operand(8 * g + i + 1), zero, 0, 0, 0);
+                        hi_next = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, operand(8 * g + i + 1), zero, 0, 0, 0);
+                    }
+                    // signed digit sums (the bytes entered as x - 128): |S| < 2^21, the pairs below 2^29, lo and hi exact
+                    const int l01 = lo.x + lo.y * 128, l23 = lo.z + lo.w * 128;
+                    const int h01 = hi.x + hi.y * 128, h23 = hi.z + hi.w * 128;
+                    const double ld = __builtin_fma((double)l23, 16384.0, (double)l01) + off_lo;
+                    const double hd = __builtin_fma((double)h23, 16384.0, (double)h01) + off_hi;
+                    // |v| <= (1/2 + 2^-8) q + 2^43: within the 4 x 2^50 that the register blocks of this pass start from
+                    v[i] = fp_mulmod(hd, w28, mod) + ld;
+                }
+                fp_ct_block<3, 2>(v, tws, 1u, mod);
+                // word i is 32 i rows further: bits 10..8 of the tile index, of which the slot takes bits 9..8 into bits 4..3
+#pragma unroll
+                for (int i = 0; i < 8; i++) tile_ld[z ^ (uint32_t)(((i & 3) << 3) | (i << 8))] = v[i];
+            }
+        }
+        if (more) {
+            alo = rec[kMxRecord + lane];
+            ahi = rec[kMxRecord + 64 + lane];
+        }
+        // the twiddles of the third block travel during the second
+        double tw_hi[3];
+#pragma unroll
+        for (int c = 0; c < 3; c++) tw_hi[c] = a.tw_fp[((size_t)rtable[4 * k + trow] << 16) + 64 + tcol + 64 * c];
+        // stages 3..5 inside the wave, tile by tile: lane (u, col) takes rows 32 u + 4 j + wave, which lanes of this wave wrote
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        for (uint32_t rr = 0; rr < nr; rr++) {
+            const FpMod mod{uniform_f64(rconst[k & 1][rr][0]), uniform_f64(rconst[k & 1][rr][1])};
+            double *tile_ld = tiles + rr * kMxStride;
+            const uint32_t u = lane >> 3;
+            const uint32_t base = ((32 * u + wave) << LOGC) + (lane & 7);
+            double v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) v[j] = tile_ld[swz8(base + ((uint32_t)(4 * j) << LOGC))];
+            fp_ct_block<3, 2>(v, twl[rr], 8u + u, mod);
+#pragma unroll
+            for (int j = 0; j < 8; j++) tile_ld[swz8(base + ((uint32_t)(4 * j) << LOGC))] = v[j];
+        }
+        // (the third block of the previous group, the last reader of these entries, ended before that group's last barrier)
+#pragma unroll
+        for (int c = 0; c < 3; c++) twl[trow][64 + tcol + 64 * c] = tw_hi[c];
+        lds_barrier();
+        // the next group's first twiddles and constants travel during the third block
+        double tw_lo = 0.0;
+        if (more) tw_lo = low_part(k + 1);
+        for (uint32_t rr = 0; rr < nr; rr++) {
+            const FpMod mod{uniform_f64(rconst[k & 1][rr][0]), uniform_f64(rconst[k & 1][rr][1])};
+            const uint32_t limb = __builtin_amdgcn_readfirstlane(rlimb[k & 1][rr]);
+            fuse_block<8, 8, 2, true, true>(tiles + rr * kMxStride, twl[rr], 6, mod, out + ((size_t)limb << 16), col0);
+        }
+        if (more) {
+            // entries 0..63 were last read by the second block, before the barrier above
+            twl[trow][tcol] = tw_lo;
+            stage_consts(k + 1, rec + kMxRecord);
+        }
+        lds_barrier();  // every read of the tiles is done before the next four rows overwrite them
     }
 }
 
@@ -1600,11 +1862,18 @@ hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, const Tuning 
     // (one operation: 3 and 6 equal, 4 and 8 slower; 8 operations: 207, 179, 168 us at 3, 8, 12 rows).  A CU with a
     // single workgroup has one wave per SIMD and nothing to cover its waits with (ModDown of one operation: 24.2 us in
     // 256 workgroups of 6 rows against 22.5 us in 512 of 3), so fewer than two per CU count as two.
-    uint32_t target = forced;
+    // the matrix-core kernel (N = 2^16) takes the output rows four at a time
+    // (merged ModDown + rescale: the matrix-core kernel first forms the rescale term for its whole tile, two rows' worth of
+    // work that pays once a workgroup has many rows, i.e. once the launch fills the chip without splitting the rows:
+    // 98 against 114 us for 8 operations, 27.8 against 25.3 us for one)
+    const bool mx = ld == 8 && b.mx_tab && !tune.no_matrix_bconv &&
+                    (!b.mdr || (b.mx_last && (uint64_t)b.n_units * items * tiles >= (tune.cus ? tune.cus : 256)));
+    const uint32_t step = mx ? 4 : 1;
+    uint32_t target = mx ? (forced + 3) / 4 * 4 : forced;
     if (!target) {
         const uint32_t cus = tune.cus ? tune.cus : 256;
         uint64_t best = ~0ull;
-        for (uint32_t r = 1; r <= kFuseMaxRows && r <= rows; r++) {
+        for (uint32_t r = step; r <= kFuseMaxRows && r < rows + step; r += step) {
             const uint64_t wgs = (uint64_t)b.n_units * items * tiles * ((rows + r - 1) / r);
             const uint64_t per_cu = (wgs + cus - 1) / cus;
             const uint64_t cost = (per_cu < 2 ? 2 : per_cu) * (2 * r + 3);
@@ -1619,6 +1888,13 @@ hipError_t launch_bconv_rows(const NttArgs &a, const BconvRows &b, const Tuning 
     const uint64_t wgs = (uint64_t)b.n_units * items * tiles * (p.compute_groups + p.copy_groups);
     if (wgs > 0x7fffffffu) return hipErrorInvalidValue;
     const dim3 grid((uint32_t)wgs);
+    if (mx) {
+        if (b.mdr)
+            hipLaunchKernelGGL(bconv_rows_mx_kernel<true>, grid, dim3(256), 0, s, a, p);
+        else
+            hipLaunchKernelGGL(bconv_rows_mx_kernel<false>, grid, dim3(256), 0, s, a, p);
+        return hipGetLastError();
+    }
     switch (ld) {
 #define HE_CASE(LD) \
     case LD: hipLaunchKernelGGL((bconv_rows_fp_kernel<LD, 8>), grid, dim3(kFuseWords / 8), 0, s, a, p); break;

@@ -1,5 +1,5 @@
-"""Base conversion fused with the rows pass of the forward transform (bconv_rows_fp_kernel: every prime below 2^50,
-N >= 2^12) against the oracle, through the C-ABI entry points that use it: he_modup (with the copy of a digit's own
+"""Base conversion fused with the rows pass of the forward transform (bconv_rows_fp_kernel, and bconv_rows_mx_kernel at
+N = 2^16: every prime below 2^50, N >= 2^12) against the oracle, through the C-ABI entry points that use it: he_modup (with the copy of a digit's own
 limbs), he_moddown (1 to 6 polynomials, overwriting and adding), he_keyswitch, he_keyswitch_rescale (the merged
 ModDown + rescale prologue) and its batch form; every degree from 2^12 to 2^16, full and partial last digits, and
 the same calls with the fusion switched off by the environment."""
@@ -17,6 +17,7 @@ CASES = [  # logn, bits, size_p, levels
     (15, [50, 50, 49, 50, 48], 1, (4, 2)),
     (16, [50] * 16, 8, (8, 3)),
     (16, [50, 49, 50, 50, 50, 50], 2, (4,)),
+    (16, [50, 49, 50, 48, 50, 50, 47, 50, 50, 50, 49, 50], 3, (7, 5)),   # 7 and 9, 5 and 7 output limbs: groups of four with a rest
 ]
 
 
@@ -34,10 +35,16 @@ def _evk(p, rng, capi):
     return host, dev, capi.evk_array([d.ptr for d in dev])
 
 
-@pytest.mark.parametrize("no_fused", ["0", "1"])
+@pytest.mark.parametrize("no_fused", ["0", "1", "vector_units"])
 @pytest.mark.parametrize("logn,bits,size_p,levels", CASES)
 def test_entry_points_with_fused_conversion(oracle, capi, monkeypatch, logn, bits, size_p, levels, no_fused):
-    monkeypatch.setenv("CAHEL_HIP_NO_FUSED_BCONV", no_fused)
+    if no_fused == "vector_units":
+        # N = 2^16 forms the conversion's products on the int8 matrix cores; this leg keeps them on the FP64 vector units
+        if logn != 16:
+            pytest.skip("the matrix-core kernel serves N = 2^16 only")
+        monkeypatch.setenv("CAHEL_HIP_NO_MATRIX_BCONV", "1")
+    else:
+        monkeypatch.setenv("CAHEL_HIP_NO_FUSED_BCONV", no_fused)
     cahel, parms, ctx, p = make_pair(oracle, logn, bits, size_p)
     rng = np.random.default_rng(100 + logn)
     lib, h = capi.lib(), ctx.he_handle()
