@@ -52,14 +52,14 @@ BLOCKS = 5
 # `--only batch`), per operation: L2-miss traffic in limbs of 8 N bytes (FETCH_SIZE scaled by 2, WRITE_SIZE by 1: the
 # factors a copy of known size gives) and SQ_INSTS_VALU summed over the kernels.  Constants of the profile, not
 # measured in this run.
-PROFILE = {"single": {"traffic_limbs": 1120.2, "valu_wave_instr": 33.41e6,
-                      "kernels": "tensor_intt_blocks_fp, ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp_inner, "
-                                 "ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp with the rescale "
-                                 "epilogue"},
-           "batch": {"traffic_limbs": 895.4, "valu_wave_instr": 30.9e6,
-                     "kernels": "per call of 8 operations: tensor_fp, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, "
+PROFILE = {"single": {"traffic_limbs": 1117.7, "valu_wave_instr": 30.88e6,
+                      "kernels": "tensor_intt_blocks_fp, ntt_rows (inverse), bconv_rows_mx (ModUp, conversion on the int8 "
+                                 "matrix cores), ntt_blocks_fp_inner, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, "
+                                 "ntt_blocks_fp with the rescale epilogue"},
+           "batch": {"traffic_limbs": 896.1, "valu_wave_instr": 27.3e6,
+                     "kernels": "per call of 8 operations: tensor_fp, ntt_blocks_fp + ntt_rows (inverse), bconv_rows_mx, "
                                 "ntt_blocks_fp_inner (items of a tile on one XCD, key tile shared through L2), "
-                                "ntt_blocks_fp + ntt_rows (inverse), bconv_rows_fp, ntt_blocks_fp with the rescale "
+                                "ntt_blocks_fp + ntt_rows (inverse), bconv_rows_mx, ntt_blocks_fp with the rescale "
                                 "epilogue"}}
 
 
