@@ -125,7 +125,7 @@ namespace {
     } while (0)
 
 // One record of BconvRows::mx_tab: up to four rows of a conversion matrix with at most 8 columns as 7-bit digits of
-// M[r][i] 2^(8 j) mod q_r, laid out as the A operands of v_mfma_i32_16x16x64_i8, and the offsets that undo the shift of
+// M[r][i] 2^(8 j) mod q_r, laid out as the A operands of v_mfma_i32_16x16x64_i8, and the constant that undoes the shift of
 // the input bytes by 128.  entry(rr, i) / modulus(rr): row rr of the record (rr < rows).  term = +1 / -1: byte 7 of limb i
 // carries byte i of a number that is added / subtracted (digits of +-2^(8 i) mod q_r there), see BconvRows::mx_last.
 template <typename Entry, typename Modulus>
@@ -157,6 +157,13 @@ void mx_record(std::vector<int32_t> &tab, uint32_t rows, uint32_t n_in, int term
                 }
                 offs[2 * rr + h] += (double)((128 * sum) << (7 * e));
             }
+    }
+    // one constant per row: (offset of the high group x 2^28 + offset of the low group) mod q
+    for (uint32_t rr = 0; rr < 4 && rr < rows; rr++) {
+        const uint64_t q = modulus(rr);
+        const unsigned __int128 v = ((unsigned __int128)(uint64_t)offs[2 * rr + 1] << 28) + (uint64_t)offs[2 * rr];
+        offs[2 * rr] = (double)(uint64_t)(v % q);
+        offs[2 * rr + 1] = 0.0;
     }
     memcpy(tab.data() + base + 4 * 128, offs, sizeof(offs));
 }

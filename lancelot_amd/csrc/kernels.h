@@ -237,8 +237,8 @@ struct BconvRows {
     // digits of 7 bits: sum_i x_i M[r][i] = sum over the bytes x_ij of x_i of x_ij M_ij (mod q_r), a 64-term product per
     // digit with the bytes as they lie in memory.  One record of kMxRecord 16-byte words per group of four output rows:
     // [half h = digits 4 h .. 4 h + 3][lane]: the lane's 16 bytes of the A operand (row 4 rr + e of the instruction is
-    // digit 4 h + e of output row rr; k = 8 limb + byte), then 8 doubles: for each row rr the offsets of its low and
-    // high digit groups, 128 x sum_e 2^(7 e) x (sum of the row of digit 4 h + e): the bytes enter as x - 128.
+    // digit 4 h + e of output row rr; k = 8 limb + byte), then 8 doubles: for each row rr the constant
+    // 128 x sum_e 2^(7 e) x (sum of the row of digit e) mod q_r that the sums lack (the bytes enter as x - 128), and a zero.
     const void *mx_tab;
     // mdr: the record of the dropped limb's row, alone and repeated in the four row slots of its record (every lane then
     // holds the row's sums for its coefficient).  Byte 7 of input limb i is free (the residues are below 2^50): the kernel

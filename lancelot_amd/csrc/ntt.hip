@@ -950,7 +950,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void bconv_rows_mx_kernel(NttArgs a, BconvRowsK p) {
     __shared__ double tiles[4 * kMxStride];
     __shared__ double twl[4][256];
-    __shared__ double rconst[2][4][4];         // per group parity and row: q, 1/q, and the two offsets of the digit sums
+    __shared__ double rconst[2][4][4];         // per group parity and row: q, 1/q, the constant that the digit sums lack
     __shared__ uint32_t rlimb[2][4];
     __shared__ uint32_t rtable[kFuseMaxRows + 4];
     constexpr int LOGC = 3;
@@ -1035,7 +1035,7 @@ void bconv_rows_mx_kernel(NttArgs a, BconvRowsK p) {
         const v4i *lrec = reinterpret_cast<const v4i *>(p.b.mx_last);
         const v4i la = lrec[lane], lh = lrec[64 + lane];
         const double *loff = reinterpret_cast<const double *>(lrec + 128);
-        const double off_lo = loff[0], off_hi = loff[1];
+        const double off = loff[0];
         const double c28 = fp_reduce(0x1p28, ml);
         const FpTw w28{c28, c28 * ml.qinv};
         const uint64_t *tl = reinterpret_cast<const uint64_t *>(tiles);
@@ -1050,8 +1050,8 @@ void bconv_rows_mx_kernel(NttArgs a, BconvRowsK p) {
                 const v4i hi = __builtin_amdgcn_mfma_i32_16x16x64_i8(lh, operand(8 * g + i), zero, 0, 0, 0);
                 const int l01 = lo.x + lo.y * 128, l23 = lo.z + lo.w * 128;
                 const int h01 = hi.x + hi.y * 128, h23 = hi.z + hi.w * 128;
-                const double ld = __builtin_fma((double)l23, 16384.0, (double)l01) + off_lo;
-                const double hd = __builtin_fma((double)h23, 16384.0, (double)h01) + off_hi;
+                const double ld = __builtin_fma((double)l23, 16384.0, (double)l01) + off;
+                const double hd = __builtin_fma((double)h23, 16384.0, (double)h01);
                 const double t = fp_from_u64(tl[e + ((uint32_t)(32 * i) << LOGC)]);
                 const uint64_t r = fp_to_u64(fp_canonical(t - (fp_mulmod(hd, w28, ml) + ld), ml));
                 const uint32_t b0 = (uint32_t)(r >> (16 * kg)) & 0xffu, b1 = (uint32_t)(r >> (16 * kg + 8)) & 0xffu;
@@ -1098,7 +1098,7 @@ void bconv_rows_mx_kernel(NttArgs a, BconvRowsK p) {
         {
             // first block, lane (rr, c) on row rr = kg
             const FpMod mod{rconst[k & 1][kg][0], rconst[k & 1][kg][1]};
-            const double off_lo = rconst[k & 1][kg][2], off_hi = rconst[k & 1][kg][3];
+            const double off = rconst[k & 1][kg][2];
             const double c28 = fp_reduce(0x1p28, mod);
             const FpTw w28{c28, c28 * mod.qinv};
             const double *tws = twl[kg];
@@ -1125,9 +1125,9 @@ void bconv_rows_mx_kernel(NttArgs a, BconvRowsK p) {
                     // signed digit sums (the bytes entered as x - 128): |S| < 2^21, the pairs below 2^29, lo and hi exact
                     const int l01 = lo.x + lo.y * 128, l23 = lo.z + lo.w * 128;
                     const int h01 = hi.x + hi.y * 128, h23 = hi.z + hi.w * 128;
-                    const double ld = __builtin_fma((double)l23, 16384.0, (double)l01) + off_lo;
-                    const double hd = __builtin_fma((double)h23, 16384.0, (double)h01) + off_hi;
-                    // |v| <= (1/2 + 2^-8) q + 2^43: within the 4 x 2^50 that the register blocks of this pass start from
+                    const double ld = __builtin_fma((double)l23, 16384.0, (double)l01) + off;
+                    const double hd = __builtin_fma((double)h23, 16384.0, (double)h01);
+                    // |v| <= (1/2 + 2^-8) q + 2^44 + q: within the 4 x 2^50 that the register blocks of this pass start from
                     v[i] = fp_mulmod(hd, w28, mod) + ld;
                 }
                 fp_ct_block<3, 2>(v, tws, 1u, mod);
