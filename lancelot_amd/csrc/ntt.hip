@@ -1237,7 +1237,12 @@ constexpr int kMaxGroup = 4;  // most jobs in one LimbGroup
 // and a single wave, which costs a third more time (three waves would spill, and measure slower).
 // GAL: the inverse pass gathers its input through a Galois permutation (a.in_galois); an instantiation of its own, so
 // that the index arithmetic costs the other launches no registers
-template <bool FWD, bool EPI, bool GAL>
+// TW_LDS (forward pass with an epilogue): the 30 twiddles of a thread live in LDS behind the tile instead of in 60
+// registers, which leaves room for the next tile's words in registers while the current one is transformed and its
+// epilogue operands travel: without it that fetch waits until the epilogue has stored, and every tile of the loop
+// exposes one round trip to memory.  LDS: the tile (17 T words), 15 T / 16 words of the first block's twiddles (one set
+// per 16 threads), 15 T of the second block's.
+template <bool FWD, bool EPI, bool GAL, bool TW_LDS = false>
 __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *lds) {
     const uint32_t nthreads = blockDim.x;
     const BlocksGeom g = blocks_geom(a);
@@ -1259,6 +1264,7 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
     double tw0[15], tw1[15];
     fp_load_block_tw<4>(tw0, fc.tw, g.idx0 + (gi >> 4));
     fp_load_block_tw<4>(tw1, fc.tw, g.idx1 + gi);
+    double *ltw0 = ld + 17 * nthreads, *ltw1 = ltw0 + 15 * (nthreads >> 4);
 
     // list mode: the unit's jobs are read before the first store, so that they stay scalar loads
     LimbJob pre[kMaxGroup];
@@ -1301,9 +1307,18 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
         }
     };
     fetch(job);
-    // the twiddles have arrived before the loop starts: inside it only the prefetch is in flight
+    if (TW_LDS) {
+        // (stride 15: the threads of a wave read their sets from distinct banks; 16 threads share a set of the first block)
 #pragma unroll
-    for (int i = 0; i < 15; i++) asm volatile("" ::"v"(tw0[i]), "v"(tw1[i]));
+        for (int i = 0; i < 15; i++) {
+            if ((gi & 15) == 0) ltw0[(gi >> 4) * 15 + i] = tw0[i];
+            ltw1[gi * 15 + i] = tw1[i];
+        }
+    } else {
+        // the twiddles have arrived before the loop starts: inside it only the prefetch is in flight
+#pragma unroll
+        for (int i = 0; i < 15; i++) asm volatile("" ::"v"(tw0[i]), "v"(tw1[i]));
+    }
     stage();
 
     for (uint32_t b = 0;; b++) {
@@ -1312,7 +1327,7 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
         // (with a fused epilogue the registers go to its operands instead and the next tile is fetched late)
         Job next = job;
         if (more) next = entry(b + 1);
-        if (more && !EPI) fetch(next);
+        if (more && (!EPI || TW_LDS)) fetch(next);
         const size_t epi_off = off + (size_t)job.limb * n;
         // SUB_MUL_ADD adds onto the polynomials named by epi_b_mask only (a rotation adds onto c0, not c1)
         const bool add_b = has_addend && (fma_mode || ((a.epi_b_mask >> (job.poly & 31)) & 1));
@@ -1331,13 +1346,27 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
         if (FWD) {
 #pragma unroll
             for (int j = 0; j < 16; j++) v[j] = ld[skew(base0 + (j << 4))];
-            fp_ct_block_tw<4, true>(v, tw0, m);
+            if (TW_LDS) {
+                double t[15];
+#pragma unroll
+                for (int i = 0; i < 15; i++) t[i] = ltw0[(gi >> 4) * 15 + i];
+                fp_ct_block_tw<4, true>(v, t, m);
+            } else {
+                fp_ct_block_tw<4, true>(v, tw0, m);
+            }
 #pragma unroll
             for (int j = 0; j < 16; j++) ld[skew(base0 + (j << 4))] = v[j];
             lds_barrier();
 #pragma unroll
             for (int j = 0; j < 16; j++) v[j] = ld[skew(base1 + j)];
-            fp_ct_block_tw<4, true>(v, tw1, m);
+            if (TW_LDS) {
+                double t[15];
+#pragma unroll
+                for (int i = 0; i < 15; i++) t[i] = ltw1[gi * 15 + i];
+                fp_ct_block_tw<4, true>(v, t, m);
+            } else {
+                fp_ct_block_tw<4, true>(v, tw1, m);
+            }
 #pragma unroll
             for (int j = 0; j < 16; j++) ld[skew(base1 + j)] = v[j];
             lds_barrier();
@@ -1386,7 +1415,7 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
             for (int i = 0; i < kPer; i++) dst[threadIdx.x + i * nthreads] = o[i];
         }
         if (!more) break;
-        if (EPI) fetch(next);
+        if (EPI && !TW_LDS) fetch(next);
         lds_barrier();  // every read of this tile is done before the next one overwrites it
         stage();
         job = next;
@@ -1398,6 +1427,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     __shared__ uint64_t lds[kLdsWords];
     ntt_blocks_fp_body<FWD, EPI, GAL>(a, lds);
 }
+
+// the forward pass with an epilogue: twiddles in LDS (blocks_epi_lds_bytes of dynamic LDS)
+extern __shared__ uint64_t dyn_lds[];
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void ntt_blocks_fp_epi_kernel(NttArgs a) {
+    ntt_blocks_fp_body<true, true, false, true>(a, dyn_lds);
+}
+inline size_t blocks_epi_lds_bytes(uint32_t threads) { return 8 * (size_t)(17 * threads + 15 * (threads >> 4) + 15 * threads); }
 
 // Forward blocks pass of ModUp fused with the key-switch inner product.  Workgroup = (limb t of Ql u P, tile of
 // 16 T words): its first T threads transform that tile of every digit in turn; all 2 T threads then multiply
@@ -1839,7 +1875,7 @@ hipError_t launch_blocks(NttArgs a, uint32_t n_polys, hipStream_t s) {
     else if (!FP)
         hipLaunchKernelGGL((ntt_blocks_int_kernel<FWD, false>), grid, block, 0, s, a);
     else if (epi)
-        hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, FWD, false>), grid, block, 0, s, a);
+        hipLaunchKernelGGL(ntt_blocks_fp_epi_kernel, grid, block, blocks_epi_lds_bytes(p.threads), s, a);
     else
         hipLaunchKernelGGL((ntt_blocks_fp_kernel<FWD, false, false>), grid, block, 0, s, a);
     return hipGetLastError();
