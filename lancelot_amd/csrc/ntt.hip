@@ -1146,17 +1146,29 @@ void bconv_rows_mx_kernel(NttArgs a, BconvRowsK p) {
         for (int c = 0; c < 3; c++) tw_hi[c] = a.tw_fp[((size_t)rtable[4 * k + trow] << 16) + 64 + tcol + 64 * c];
         // stages 3..5 inside the wave, tile by tile: lane (u, col) takes rows 32 u + 4 j + wave, which lanes of this wave wrote
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        for (uint32_t rr = 0; rr < nr; rr++) {
-            const FpMod mod{uniform_f64(rconst[k & 1][rr][0]), uniform_f64(rconst[k & 1][rr][1])};
-            double *tile_ld = tiles + rr * kMxStride;
+        {
+            // (all four tiles, also those of rows past the end: the words of the next tile are read before the block of
+            // the current one runs)
             const uint32_t u = lane >> 3;
             const uint32_t base = ((32 * u + wave) << LOGC) + (lane & 7);
-            double v[8];
+            double vn[8];
 #pragma unroll
-            for (int j = 0; j < 8; j++) v[j] = tile_ld[swz8(base + ((uint32_t)(4 * j) << LOGC))];
-            fp_ct_block<3, 2>(v, twl[rr], 8u + u, mod);
+            for (int j = 0; j < 8; j++) vn[j] = tiles[swz8(base + ((uint32_t)(4 * j) << LOGC))];
 #pragma unroll
-            for (int j = 0; j < 8; j++) tile_ld[swz8(base + ((uint32_t)(4 * j) << LOGC))] = v[j];
+            for (int rr = 0; rr < 4; rr++) {
+                const FpMod mod{uniform_f64(rconst[k & 1][rr][0]), uniform_f64(rconst[k & 1][rr][1])};
+                double *tile_ld = tiles + rr * kMxStride;
+                double v[8];
+#pragma unroll
+                for (int j = 0; j < 8; j++) v[j] = vn[j];
+                if (rr < 3) {
+#pragma unroll
+                    for (int j = 0; j < 8; j++) vn[j] = tile_ld[kMxStride + swz8(base + ((uint32_t)(4 * j) << LOGC))];
+                }
+                fp_ct_block<3, 2>(v, twl[rr], 8u + u, mod);
+#pragma unroll
+                for (int j = 0; j < 8; j++) tile_ld[swz8(base + ((uint32_t)(4 * j) << LOGC))] = v[j];
+            }
         }
         // (the third block of the previous group, the last reader of these entries, ended before that group's last barrier)
 #pragma unroll
