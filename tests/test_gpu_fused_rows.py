@@ -97,7 +97,7 @@ def test_entry_points_with_fused_conversion(oracle, capi, monkeypatch, logn, bit
                 assert (dout.numpy() == p.rescale(want)).all(), ("keyswitch_rescale", L, elt)
         # the batch form over three inputs (separate kernels for the inner product, same conversions)
         if L >= 2:
-            items = 3
+            items = 4 if logn == 16 else 3   # (four items: the merged ModDown + rescale then takes the matrix-core kernel at N = 2^16)
             c3 = rand_limbs(p, rng, range(L), n_polys=items)
             ct3 = np.stack([rand_limbs(p, rng, range(L), n_polys=2) for _ in range(items)])
             bws = DeviceArray(capi, shape=(lib.he_keyswitch_batch_workspace_words(h, L, items),))
