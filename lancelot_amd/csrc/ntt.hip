@@ -1383,7 +1383,9 @@ __device__ __forceinline__ void ntt_blocks_fp_body(const NttArgs &a, uint64_t *l
             for (int j = 0; j < 16; j++) ld[skew(base1 + j)] = v[j];
             lds_barrier();
 #pragma unroll
-            for (int i = 0; i < kPer; i++) v[i] = fp_canonical(ld[skew(threadIdx.x + i * nthreads)], m);
+            // (an epilogue subtracts the word as the second block left it, at most 5.3 q in magnitude: its difference from
+            // a minuend below 1.9 q stays below 2^53 and goes through one modular product)
+            for (int i = 0; i < kPer; i++) v[i] = EPI ? ld[skew(threadIdx.x + i * nthreads)] : fp_canonical(ld[skew(threadIdx.x + i * nthreads)], m);
             if (EPI) {
                 const double wd = fp_from_u64(a.w[2 * job.limb]);
                 const FpTw w{wd, wd * m.qinv};
