@@ -1417,8 +1417,10 @@ int he_ckks_encode_batch(const he_context *ctx, const double *re, const double *
     double *coeffs = reinterpret_cast<double *>(ws + head + (size_t)items * n);
     const FftTables ft{ctx->d_rot_group, ctx->d_ksi, ctx->log_n};
     // (the complex scratch of an item is `slots` values = at most N words: the items are packed `slots` apart)
-    HE_HIP(launch_ckks_encode(ft, re, im, count, slots, scale, v, coeffs, ws, items, value_stride, S(s)));
-    HE_HIP(launch_decompose_real(ctx->tables(), coeffs, out, limbs, 0, items, (size_t)out_poly_stride * n, S(s)));
+    // (the rounding kernel writes the residues itself: no pass over the coefficients as doubles)
+    const Tables tab = ctx->tables();
+    HE_HIP(launch_ckks_encode(ft, re, im, count, slots, scale, v, coeffs, ws, items, value_stride, S(s), &tab, out, limbs,
+                              (size_t)out_poly_stride * n));
     return he_ntt_forward(ctx, out, items, out_poly_stride, limbs, 0, limbs, 0, s);
 }
 
@@ -1447,11 +1449,11 @@ int he_encrypt_batch(const he_context *ctx, uint32_t L, uint32_t items, const ui
     const LimbMap map{LK, 0, L, Q};
     // item k draws u, e0, e1 from the stream ids stream_id + 3 k, + 1, + 2: what `items` encryptions in a row draw
     HE_HIP(launch_sample(ctx->tables(), SAMPLE_TERNARY, k, stream_id, u, map, nullptr, 0, items, 3, (size_t)LK * n, S(s)));
-    for (uint32_t i = 0; i < 2; i++)
-        HE_HIP(launch_sample(ctx->tables(), SAMPLE_ERROR, k, stream_id + 1 + i, wide + (size_t)i * LK * n, map, nullptr, 0,
-                             items, 3, 2 * (size_t)LK * n, S(s)));
-    if (int rc = he_ntt_forward(ctx, u, items, LK, LK, 0, L, Q, s)) return rc;
-    if (int rc = he_ntt_forward(ctx, wide, 2 * items, LK, LK, 0, L, Q, s)) return rc;
+    // (e0, e1 of all items in one launch: wide is [items][2] polynomials LK * N words apart)
+    HE_HIP(launch_sample(ctx->tables(), SAMPLE_ERROR, k, stream_id + 1, wide, map, nullptr, 0, 2 * items, 3, (size_t)LK * n,
+                         S(s), 2));
+    // u and wide lie one after the other: 3 * items polynomials of the same limbs
+    if (int rc = he_ntt_forward(ctx, u, 3 * items, LK, LK, 0, L, Q, s)) return rc;
     HE_HIP(launch_encrypt_fma(ctx->tables(), u, pk, wide, L, K, Q, items, S(s)));
     // divide by P; polynomial 0 of every ciphertext already holds the plaintext and is added onto
     return moddown_impl(ctx, L, wide, cts, 2 * items, 0x55555555u, tmp, s);

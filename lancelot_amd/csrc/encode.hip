@@ -6,8 +6,9 @@
 // contraction): a butterfly is u = a + b, t = (a - b) * w with the four-multiplication complex product, so
 // the result does not depend on how the butterflies are spread over threads.
 //
-// Layout: v = `slots` complex values as double2.  Stages whose span exceeds one tile of 2048 values run as
-// one kernel each over global memory; all the others run inside LDS in a single kernel.
+// Layout: v = `slots` complex values as double2.  The stages whose span exceeds one tile of 2048 values (at most 5)
+// run as one kernel over global memory, every thread holding the values that those stages combine; all the others
+// run inside LDS in a single kernel.
 #include "kernels.h"
 #include "modarith.cuh"
 
@@ -47,25 +48,69 @@ __device__ __forceinline__ void butterfly(double2 &a, double2 &b, double2 w) {
     }
 }
 
-// one stage over global memory; thread = one butterfly; blockIdx.y = item (vectors `slots` apart)
-template <bool INVERSE>
-__global__ __launch_bounds__(kThreads) void cfft_stage_kernel(double2 *v, uint32_t len, FftTables t, uint32_t slots) {
+// Where an encoding starts from: the caller's real and imaginary parts (zero padded from `count` on) instead of the
+// scratch vector.  re = nullptr: the scratch vector itself.
+struct FftSource {
+    const double *re, *im;
+    uint32_t count;
+    size_t value_stride;          // doubles between the items' values
+    unsigned long long *max_bits; // one per item, cleared here for the rounding kernel to accumulate into
+};
+
+__device__ __forceinline__ double2 source_value(const FftSource &src, uint32_t item, uint32_t i) {
+    if (i >= src.count) return double2{0.0, 0.0};
+    const size_t at = item * src.value_stride + i;
+    return double2{src.re[at], src.im ? src.im[at] : 0.0};
+}
+
+constexpr int kTopThreads = 64;
+
+// The R stages of span > tile in one kernel over global memory: thread `id` of an item holds the 2^R values
+// id + h * tile, which those stages combine among themselves only; every butterfly is the one that a launch per
+// stage with a thread per butterfly would compute (same operands, same twiddle).  blockIdx.y = item (vectors `slots`
+// apart).  INVERSE runs the spans slots, slots / 2, .., 2 tile; forward 2 tile, .., slots.
+template <bool INVERSE, int R>
+__global__ __launch_bounds__(kTopThreads) void cfft_top_kernel(double2 *v, uint32_t tile, FftTables t, uint32_t slots,
+                                                               FftSource src) {
+    constexpr int E = 1 << R;
+    const uint32_t id = blockIdx.x * kTopThreads + threadIdx.x;
     v += (size_t)blockIdx.y * slots;
-    const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
-    const uint32_t lenh = len >> 1;
-    const uint32_t j = b & (lenh - 1), pos = ((b / lenh) * len) + j;
-    double2 x = v[pos], y = v[pos + lenh];
-    butterfly<INVERSE>(x, y, stage_twiddle<INVERSE>(t, len, j));
-    v[pos] = x;
-    v[pos + lenh] = y;
+    double2 e[E];
+    if (INVERSE && src.re) {
+        if (id == 0) src.max_bits[blockIdx.y] = 0;
+#pragma unroll
+        for (int h = 0; h < E; h++) e[h] = source_value(src, blockIdx.y, id + h * tile);
+    } else {
+#pragma unroll
+        for (int h = 0; h < E; h++) e[h] = v[id + h * tile];
+    }
+#pragma unroll
+    for (int st = 0; st < R; st++) {
+        const int half = INVERSE ? E >> (st + 1) : 1 << st;   // distance of a butterfly's operands, in h
+        const uint32_t len = tile * 2 * half;
+#pragma unroll
+        for (int b = 0; b < E / 2; b++) {
+            const int lo = b & (half - 1), h0 = (b / half) * 2 * half + lo;
+            butterfly<INVERSE>(e[h0], e[h0 + half], stage_twiddle<INVERSE>(t, len, id + lo * tile));
+        }
+    }
+#pragma unroll
+    for (int h = 0; h < E; h++) v[id + h * tile] = e[h];
 }
 
 // every stage of span <= tile inside LDS; tile = min(slots, kFftTile) values per workgroup
 template <bool INVERSE>
-__global__ __launch_bounds__(kThreads) void cfft_lds_kernel(double2 *v, uint32_t tile, FftTables t, uint32_t slots) {
+__global__ __launch_bounds__(kThreads) void cfft_lds_kernel(double2 *v, uint32_t tile, FftTables t, uint32_t slots,
+                                                            FftSource src) {
     __shared__ double2 s[kFftTile];
     double2 *g = v + (size_t)blockIdx.y * slots + (size_t)blockIdx.x * tile;
-    for (uint32_t i = threadIdx.x; i < tile; i += kThreads) s[i] = g[i];
+    if (INVERSE && src.re) {
+        // (only when the whole vector is this one tile: otherwise the wider stages have run before)
+        if (threadIdx.x == 0) src.max_bits[blockIdx.y] = 0;
+        for (uint32_t i = threadIdx.x; i < tile; i += kThreads) s[i] = source_value(src, blockIdx.y, i);
+    } else {
+        for (uint32_t i = threadIdx.x; i < tile; i += kThreads) s[i] = g[i];
+    }
     __syncthreads();
     for (uint32_t k = 2; k <= tile; k <<= 1) {
         const uint32_t len = INVERSE ? (tile << 1) / k : k;   // tile, tile/2, ..., 2  or  2, 4, ..., tile
@@ -80,20 +125,6 @@ __global__ __launch_bounds__(kThreads) void cfft_lds_kernel(double2 *v, uint32_t
         __syncthreads();
     }
     for (uint32_t i = threadIdx.x; i < tile; i += kThreads) g[i] = s[i];
-}
-
-// values -> complex vector, zero padded; also clears the maximum that the rounding kernel accumulates
-__global__ __launch_bounds__(kThreads) void encode_load_kernel(const double *re, const double *im, uint32_t count,
-                                                               uint32_t slots, double2 *v,
-                                                               unsigned long long *max_bits, size_t value_stride) {
-    const uint32_t i = blockIdx.x * kThreads + threadIdx.x;
-    // blockIdx.y = item: its values value_stride doubles on, its vector `slots` on, its own maximum
-    re += blockIdx.y * value_stride;
-    if (im) im += blockIdx.y * value_stride;
-    v += (size_t)blockIdx.y * slots;
-    max_bits += blockIdx.y;
-    if (i == 0) *max_bits = 0;
-    if (i < slots) v[i] = i < count ? double2{re[i], im ? im[i] : 0.0} : double2{0.0, 0.0};
 }
 
 // The largest magnitude of an item's coefficients (the bit patterns of non-negative doubles order like the values):
@@ -116,14 +147,30 @@ __device__ __forceinline__ void block_max_to(unsigned long long *dst, unsigned l
     }
 }
 
+// Where the rounded coefficients go: as doubles to coeffs [items][N], or (out given) as residues of the first `limbs`
+// primes to out [items][limbs][N], items out_item_stride words apart.
+struct RoundSink {
+    double *coeffs;
+    uint64_t *out;
+    const uint64_t *moduli, *barrett;
+    uint32_t limbs;
+    size_t out_item_stride;
+};
+
+// residue of a rounded real coefficient (below 2^63 in magnitude: the caller checks the maximum)
+__device__ __forceinline__ uint64_t real_residue(double c, uint64_t q, uint64_t r1) {
+    const uint64_t r = barrett64((uint64_t)fabs(c), q, r1);
+    return c < 0 ? neg_mod(r, q) : r;
+}
+
 // coefficient c of the plaintext: real parts fill the first half, imaginary parts the second, `gap` apart;
 // value i comes from position bitrev(i) of the transformed vector
 __global__ __launch_bounds__(kThreads) void encode_round_kernel(const double2 *v, uint32_t log_slots, uint32_t gap,
-                                                                uint32_t half, double fix, double *coeffs,
+                                                                uint32_t half, double fix, RoundSink sink,
                                                                 unsigned long long *max_bits) {
     const uint32_t c = blockIdx.x * kThreads + threadIdx.x;
     v += (size_t)blockIdx.y << log_slots;
-    coeffs += (size_t)blockIdx.y * 2 * half;
+    double *coeffs = sink.coeffs + (size_t)blockIdx.y * 2 * half;
     max_bits += blockIdx.y;
     const bool imag = c >= half;
     const uint32_t k = imag ? c - half : c;
@@ -133,7 +180,13 @@ __global__ __launch_bounds__(kThreads) void encode_round_kernel(const double2 *v
         const double2 z = v[__brev(i) >> (32 - log_slots)];
         val = round((imag ? z.y : z.x) * fix);
     }
-    coeffs[c] = val;
+    if (sink.out) {
+        uint64_t *o = sink.out + blockIdx.y * sink.out_item_stride + c;
+        for (uint32_t l = 0; l < sink.limbs; l++)
+            o[(size_t)l * 2 * half] = real_residue(val, sink.moduli[l], sink.barrett[2 * l + 1]);
+    } else {
+        coeffs[c] = val;
+    }
     block_max_to(max_bits, (unsigned long long)__double_as_longlong(fabs(val)));
 }
 
@@ -144,11 +197,11 @@ __global__ __launch_bounds__(kThreads) void encode_round_kernel(const double2 *v
 // which sits at position (brev4(y) | brev(middle) | x) of the vector (consecutive in x), and writes the slot with low
 // bits x and top bits brev4(y) (consecutive in x), real part to coefficient i, imaginary part to coefficient N/2 + i.
 __global__ __launch_bounds__(kThreads) void encode_round_tiled_kernel(const double2 *v, uint32_t log_slots, uint32_t half,
-                                                                      double fix, double *coeffs, unsigned long long *max_bits) {
+                                                                      double fix, RoundSink sink, unsigned long long *max_bits) {
     __shared__ double2 tile[16][17];
     const uint32_t x = threadIdx.x & 15, y = threadIdx.x >> 4, mid = blockIdx.x, mid_bits = log_slots - 8;
     v += (size_t)blockIdx.y << log_slots;
-    coeffs += (size_t)blockIdx.y * 2 * half;
+    double *coeffs = sink.coeffs + (size_t)blockIdx.y * 2 * half;
     max_bits += blockIdx.y;
     const uint32_t rmid = mid_bits ? __brev(mid) >> (32 - mid_bits) : 0;
     const uint32_t brev4_y = __brev(y) >> 28;
@@ -157,8 +210,17 @@ __global__ __launch_bounds__(kThreads) void encode_round_tiled_kernel(const doub
     const double2 z = tile[x][y];
     const uint32_t i = (brev4_y << (log_slots - 4)) | (mid << 4) | x;
     const double re = round(z.x * fix), im = round(z.y * fix);
-    coeffs[i] = re;
-    coeffs[half + i] = im;
+    if (sink.out) {
+        uint64_t *o = sink.out + blockIdx.y * sink.out_item_stride + i;
+        for (uint32_t l = 0; l < sink.limbs; l++) {
+            const uint64_t q = sink.moduli[l], r1 = sink.barrett[2 * l + 1];
+            o[(size_t)l * 2 * half] = real_residue(re, q, r1);
+            o[(size_t)l * 2 * half + half] = real_residue(im, q, r1);
+        }
+    } else {
+        coeffs[i] = re;
+        coeffs[half + i] = im;
+    }
     const double big = fabs(re) > fabs(im) ? fabs(re) : fabs(im);
     block_max_to(max_bits, (unsigned long long)__double_as_longlong(big));
 }
@@ -234,17 +296,30 @@ __global__ __launch_bounds__(kThreads) void decode_compose_kernel(const uint64_t
 }
 
 template <bool INVERSE>
-hipError_t run_fft(double2 *v, uint32_t slots, uint32_t items, const FftTables &t, hipStream_t s) {
+hipError_t run_fft(double2 *v, uint32_t slots, uint32_t items, const FftTables &t, hipStream_t s, FftSource src) {
     const uint32_t tile = slots < kFftTile ? slots : kFftTile;
-    const dim3 stage_grid(slots / 2 / kThreads, items), lds_grid(slots / tile, items);
+    const dim3 top_grid(tile / kTopThreads, items), lds_grid(slots / tile, items);
+    const uint32_t wide = 31 - __builtin_clz(slots / tile);   // stages of span > tile
+    const FftSource none{nullptr, nullptr, 0, 0, nullptr};
+    auto top = [&](FftSource from) {
+        switch (wide) {
+            case 1: hipLaunchKernelGGL((cfft_top_kernel<INVERSE, 1>), top_grid, dim3(kTopThreads), 0, s, v, tile, t, slots, from); break;
+            case 2: hipLaunchKernelGGL((cfft_top_kernel<INVERSE, 2>), top_grid, dim3(kTopThreads), 0, s, v, tile, t, slots, from); break;
+            case 3: hipLaunchKernelGGL((cfft_top_kernel<INVERSE, 3>), top_grid, dim3(kTopThreads), 0, s, v, tile, t, slots, from); break;
+            case 4: hipLaunchKernelGGL((cfft_top_kernel<INVERSE, 4>), top_grid, dim3(kTopThreads), 0, s, v, tile, t, slots, from); break;
+            case 5: hipLaunchKernelGGL((cfft_top_kernel<INVERSE, 5>), top_grid, dim3(kTopThreads), 0, s, v, tile, t, slots, from); break;
+            default: return hipErrorInvalidValue;
+        }
+        return hipSuccess;
+    };
     if (INVERSE) {
-        for (uint32_t len = slots; len > tile; len >>= 1)
-            hipLaunchKernelGGL(cfft_stage_kernel<true>, stage_grid, dim3(kThreads), 0, s, v, len, t, slots);
-        hipLaunchKernelGGL(cfft_lds_kernel<true>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots);
+        if (wide)
+            if (hipError_t e = top(src)) return e;
+        hipLaunchKernelGGL(cfft_lds_kernel<true>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots, wide ? none : src);
     } else {
-        hipLaunchKernelGGL(cfft_lds_kernel<false>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots);
-        for (uint32_t len = tile << 1; len <= slots; len <<= 1)
-            hipLaunchKernelGGL(cfft_stage_kernel<false>, stage_grid, dim3(kThreads), 0, s, v, len, t, slots);
+        hipLaunchKernelGGL(cfft_lds_kernel<false>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots, none);
+        if (wide)
+            if (hipError_t e = top(none)) return e;
     }
     return hipGetLastError();
 }
@@ -259,20 +334,20 @@ __global__ __launch_bounds__(kThreads) void take_slots_kernel(const double2 *v, 
 
 hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double *im, uint32_t count, uint32_t slots,
                               double scale, double2 *v, double *coeffs, uint64_t *max_bits, uint32_t items,
-                              size_t value_stride, hipStream_t s) {
+                              size_t value_stride, hipStream_t s, const Tables *tab, uint64_t *out, uint32_t limbs,
+                              size_t out_item_stride) {
     const uint32_t n = 1u << t.log_n, log_slots = 31 - __builtin_clz(slots);
-    if (items == 0 || items > 65535) return hipErrorInvalidValue;
-    auto blocks = [&](uint32_t work) { return dim3((work + kThreads - 1) / kThreads, items); };
-    hipLaunchKernelGGL(encode_load_kernel, blocks(slots), dim3(kThreads), 0, s, re, im, count, slots, v,
-                       reinterpret_cast<unsigned long long *>(max_bits), value_stride);
-    hipError_t e = run_fft<true>(v, slots, items, t, s);
+    if (items == 0 || items > 65535 || (out && (!tab || limbs == 0))) return hipErrorInvalidValue;
+    unsigned long long *maxima = reinterpret_cast<unsigned long long *>(max_bits);
+    hipError_t e = run_fft<true>(v, slots, items, t, s, FftSource{re, im, count, value_stride, maxima});
     if (e != hipSuccess) return e;
+    const RoundSink sink{coeffs, out, out ? tab->moduli : nullptr, out ? tab->barrett : nullptr, limbs, out_item_stride};
     if (slots == n / 2 && log_slots >= 8)
         hipLaunchKernelGGL(encode_round_tiled_kernel, dim3(slots / kThreads, items), dim3(kThreads), 0, s, v, log_slots, n / 2,
-                           scale / (double)slots, coeffs, reinterpret_cast<unsigned long long *>(max_bits));
+                           scale / (double)slots, sink, maxima);
     else
-        hipLaunchKernelGGL(encode_round_kernel, blocks(n), dim3(kThreads), 0, s, v, log_slots, (n / 2) / slots, n / 2,
-                           scale / (double)slots, coeffs, reinterpret_cast<unsigned long long *>(max_bits));
+        hipLaunchKernelGGL(encode_round_kernel, dim3((n + kThreads - 1) / kThreads, items), dim3(kThreads), 0, s, v, log_slots,
+                           (n / 2) / slots, n / 2, scale / (double)slots, sink, maxima);
     return hipGetLastError();
 }
 
@@ -293,7 +368,7 @@ hipError_t launch_ckks_decode(const FftTables &t, const Tables &tab, const uint6
         default: HE_COMPOSE(0); break;
     }
 #undef HE_COMPOSE
-    return run_fft<false>(v, slots, items, t, s);
+    return run_fft<false>(v, slots, items, t, s, FftSource{nullptr, nullptr, 0, 0, nullptr});
 }
 
 hipError_t launch_take_slots(const double2 *v, uint32_t slots, uint32_t items, uint32_t count, double2 *out, hipStream_t s) {

@@ -174,28 +174,19 @@ void CAHELGPUPublicKey::encrypt_asymmetric(const CAHELGPUContext &context, const
             check_status(he_multiply_add(h, u.get(), pk_.data() + (std::size_t)i * QP * n, ci, ci, 1, limbs, 0, 0, st),
                          "he_multiply_add");
         }
+        check_status(he_add(h, cipher.data(), plain.data(), cipher.data(), 1, limbs, 0, st), "he_add");
     } else {
-        // encrypt over Ql u P, then divide by P (ModDown) onto the L limbs of the plaintext's level
-        const uint32_t L = (uint32_t)context.limbs_at(chain), LK = L + (uint32_t)K;
-        DeviceBuffer u((std::size_t)LK * n), wide(2 * (std::size_t)LK * n);
-        sample(context, 0, u.get(), LK, L, (uint32_t)Q);
-        check_status(he_ntt_forward(h, u.get(), 1, LK, LK, 0, L, (uint32_t)Q, st), "he_ntt_forward");
-        for (int i = 0; i < 2; i++) {
-            uint64_t *ci = wide.get() + (std::size_t)i * LK * n;
-            const uint64_t *pki = pk_.data() + (std::size_t)i * QP * n;
-            sample(context, 1, ci, LK, L, (uint32_t)Q);
-            check_status(he_ntt_forward(h, ci, 1, LK, LK, 0, L, (uint32_t)Q, st), "he_ntt_forward");
-            check_status(he_multiply_add(h, u.get(), pki, ci, ci, 1, L, 0, 0, st), "he_multiply_add");
-            check_status(he_multiply_add(h, u.get() + (std::size_t)L * n, pki + Q * n, ci + (std::size_t)L * n,
-                                         ci + (std::size_t)L * n, 1, (uint32_t)K, (uint32_t)Q, 0, st),
-                         "he_multiply_add");
-        }
+        // encrypt over Ql u P, then divide by P (ModDown) onto the L limbs of the plaintext's level: the batched
+        // pipeline with one item (u, e0, e1 from the next three stream ids; the plaintext lies in polynomial 0 and the
+        // division adds onto it)
+        const uint32_t L = (uint32_t)context.limbs_at(chain);
         cipher.resize(context, chain, 2);
-        DeviceBuffer ws(2 * (std::size_t)L * n);
-        check_status(he_moddown(h, L, wide.get(), cipher.data(), 2, 0, ws.get(), st), "he_moddown");
+        check_status(he_memcpy_d2d(cipher.data(), plain.data(), (std::size_t)L * n * sizeof(uint64_t), st), "copy");
+        DeviceBuffer ws(he_encrypt_batch_workspace_words(h, L, 1));
+        check_status(he_encrypt_batch(h, L, 1, pk_.data(), context.prng_key(), context.next_stream(3), cipher.data(),
+                                      ws.get(), st),
+                     "he_encrypt_batch");
     }
-    const uint32_t limbs = (uint32_t)context.limbs_at(chain);
-    check_status(he_add(h, cipher.data(), plain.data(), cipher.data(), 1, limbs, 0, st), "he_add");
     cipher.is_ntt_form() = true;
     cipher.is_asymmetric() = true;
     cipher.scale() = plain.scale();

@@ -321,10 +321,11 @@ enum : int { SAMPLE_TERNARY = 0, SAMPLE_ERROR = 1, SAMPLE_UNIFORM = 2, SAMPLE_GA
 struct ChaChaKey {
     uint32_t k[8];
 };
-// items polynomials in one launch: item k draws from stream_id + k * stream_stride and lands k * out_item_stride words on
+// items polynomials in one launch: polynomial k draws from stream_id + (k / stream_group) * stream_stride +
+// k % stream_group and lands k * out_item_stride words on
 hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
                          const uint64_t *cdt, uint32_t cdt_len, uint32_t items, uint32_t stream_stride,
-                         size_t out_item_stride, hipStream_t s);
+                         size_t out_item_stride, hipStream_t s, uint32_t stream_group = 1);
 // wide [items][2][L+K][N] += u [items][L+K][N] * pk [2][size_q+K][N] (both polynomials of the public key)
 hipError_t launch_encrypt_fma(const Tables &t, const uint64_t *u, const uint64_t *pk, uint64_t *wide, uint32_t L,
                               uint32_t K, uint32_t size_q, uint32_t items, hipStream_t s);
@@ -336,10 +337,13 @@ struct FftTables {
     uint32_t log_n;
 };
 // values (count <= slots, zero padded) -> rounded real coefficients [N]; *max_bits receives the bit pattern of the
-// largest |coefficient| (a non-negative double).  v: scratch of `slots` complex values.
+// largest |coefficient| (a non-negative double).  v: scratch of `slots` complex values.  With `out` the coefficients
+// leave as residues of the first `limbs` primes of `tab` instead (out [items][limbs][N], items out_item_stride words
+// apart) and coeffs is not written.
 hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double *im, uint32_t count, uint32_t slots,
                               double scale, double2 *v, double *coeffs, uint64_t *max_bits, uint32_t items,
-                              size_t value_stride, hipStream_t s);
+                              size_t value_stride, hipStream_t s, const Tables *tab = nullptr, uint64_t *out = nullptr,
+                              uint32_t limbs = 0, size_t out_item_stride = 0);
 // res: [limbs][N] coefficient-form residues of the first `limbs` primes -> v: `slots` complex values.
 // garner_inv[i * stride + j] = q_j^-1 mod q_i for j < i.
 // items: that many dense plaintexts res [items][limbs][N] -> v [items][slots].

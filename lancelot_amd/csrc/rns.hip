@@ -735,7 +735,7 @@ struct SampleArgs {
     LimbMap map;
     uint32_t log_n, cdt_len;
     int kind;
-    uint32_t stream_stride;
+    uint32_t stream_stride, stream_group;
     size_t out_item_stride;
 };
 
@@ -748,8 +748,9 @@ template <int KIND>
 __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
     const uint32_t n = 1u << p.log_n;
     const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
-    // blockIdx.y = item: its own stream id, its own polynomial
-    const uint64_t stream = p.stream + (uint64_t)blockIdx.y * p.stream_stride;
+    // blockIdx.y = polynomial: stream_group consecutive ones take consecutive stream ids, the next group starts
+    // stream_stride on
+    const uint64_t stream = p.stream + (uint64_t)(blockIdx.y / p.stream_group) * p.stream_stride + blockIdx.y % p.stream_group;
     uint64_t *out = p.out + blockIdx.y * p.out_item_stride;
     uint32_t w[16];
     if (KIND == SAMPLE_UNIFORM) {
@@ -1101,13 +1102,13 @@ hipError_t launch_hoist_inner(const Tables &t, const Tuning &tune, const uint64_
 
 hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
                          const uint64_t *cdt, uint32_t cdt_len, uint32_t items, uint32_t stream_stride,
-                         size_t out_item_stride, hipStream_t s) {
-    if (items == 0 || items > 65535) return hipErrorInvalidValue;
+                         size_t out_item_stride, hipStream_t s, uint32_t stream_group) {
+    if (items == 0 || items > 65535 || stream_group == 0) return hipErrorInvalidValue;
     const uint32_t n = 1u << t.log_n;
     uint32_t blocks = kind == SAMPLE_UNIFORM ? (n / 4) * map.limbs : (kind == SAMPLE_TERNARY ? n / 16 : n / 8);
     // (a thread's words leave as 16-byte stores)
     if ((reinterpret_cast<uintptr_t>(out) & 15) || (out_item_stride & 1)) return hipErrorInvalidValue;
-    SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind, stream_stride, out_item_stride};
+    SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind, stream_stride, stream_group, out_item_stride};
     const dim3 grid((blocks + kThreads - 1) / kThreads, items);
     switch (kind) {
         case SAMPLE_UNIFORM: hipLaunchKernelGGL(sample_kernel<SAMPLE_UNIFORM>, grid, dim3(kThreads), 0, s, p); break;
