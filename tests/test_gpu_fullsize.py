@@ -333,12 +333,15 @@ def _centred_distance(a, b, q):
     return np.minimum(d, q - d)
 
 
-@pytest.mark.parametrize("bits,size_p", [([50] * 32, 8), ([60, 40, 40, 60], 1)])
-@pytest.mark.parametrize("slots", [32768, 256])
+@pytest.mark.parametrize("bits,size_p,slots", [([50] * 32, 8, 32768), ([50] * 32, 8, 256),
+                                               ([60, 40, 40, 60], 1, 32768), ([60, 40, 40, 60], 1, 16384),
+                                               ([60, 40, 40, 60], 1, 8192), ([60, 40, 40, 60], 1, 4096),
+                                               ([60, 40, 40, 60], 1, 256)])
 def test_encoder_at_full_degree(oracle, bits, size_p, slots):
     """he_ckks_encode / he_ckks_decode and their batch forms (he_ckks_encode_batch, he_decrypt_decode_batch) at
-    N = 2^16 with all 32,768 slots (the special FFT then has stages wider than a workgroup's LDS tile) and with a
-    sparse slot count, on 24 limbs (the general Garner composition) and on Lancelot's 3 limbs (the one templated on
+    N = 2^16 with all 32,768 slots (the special FFT then has 4 stages wider than a workgroup's LDS tile, which one
+    kernel runs with 16 values per thread), with 16,384, 8,192 and 4,096 slots (3, 2 and 1 such stages: the other
+    instances of that kernel) and with a sparse slot count that fits the tile, on 24 limbs (the general Garner composition) and on Lancelot's 3 limbs (the one templated on
     the limb count): encoded coefficients within one unit of the oracle's encoder, decoded values within 2^-20 of its
     decoder and of the message (src/ckks.cu:104-209, 292-465)."""
     import ctypes as C
