@@ -1390,16 +1390,16 @@ int he_decompose_real(const he_context *ctx, const double *coeffs, uint64_t *out
 size_t he_ckks_workspace_words(const he_context *ctx, uint32_t limbs) {
     if (!ctx) return 0;
     const size_t n = ctx->n();
-    // encode: [8 words, the first holds the maximum] [N words: complex scratch] [N words: coefficients]
+    // encode: [8 words, the first holds the maximum] [N words: complex scratch]
     // decode: [limbs * N words: coefficient-form copy]
-    const size_t enc = 8 + 2 * n, dec = (size_t)limbs * n;
+    const size_t enc = 8 + n, dec = (size_t)limbs * n;
     return enc > dec ? enc : dec;
 }
 
 size_t he_ckks_encode_batch_workspace_words(const he_context *ctx, uint32_t items) {
     if (!ctx) return 0;
-    // [items words rounded up to 8: the maxima] [items][N words: complex scratch] [items][N words: coefficients]
-    return (((size_t)items + 7) & ~(size_t)7) + 2 * (size_t)items * ctx->n();
+    // [items words rounded up to 8: the maxima] [items][N words: complex scratch]
+    return (((size_t)items + 7) & ~(size_t)7) + (size_t)items * ctx->n();
 }
 
 int he_ckks_encode_batch(const he_context *ctx, const double *re, const double *im, uint32_t count, uint32_t slots,
@@ -1414,12 +1414,11 @@ int he_ckks_encode_batch(const he_context *ctx, const double *re, const double *
     const size_t n = ctx->n();
     const size_t head = ((size_t)items + 7) & ~(size_t)7;
     double2 *v = reinterpret_cast<double2 *>(ws + head);
-    double *coeffs = reinterpret_cast<double *>(ws + head + (size_t)items * n);
     const FftTables ft{ctx->d_rot_group, ctx->d_ksi, ctx->log_n};
     // (the complex scratch of an item is `slots` values = at most N words: the items are packed `slots` apart)
-    // (the rounding kernel writes the residues itself: no pass over the coefficients as doubles)
+    // (the rounding kernel writes the residues itself: the coefficients never exist as an array of doubles)
     const Tables tab = ctx->tables();
-    HE_HIP(launch_ckks_encode(ft, re, im, count, slots, scale, v, coeffs, ws, items, value_stride, S(s), &tab, out, limbs,
+    HE_HIP(launch_ckks_encode(ft, re, im, count, slots, scale, v, nullptr, ws, items, value_stride, S(s), &tab, out, limbs,
                               (size_t)out_poly_stride * n));
     return he_ntt_forward(ctx, out, items, out_poly_stride, limbs, 0, limbs, 0, s);
 }

@@ -337,7 +337,7 @@ hipError_t launch_ckks_encode(const FftTables &t, const double *re, const double
                               size_t value_stride, hipStream_t s, const Tables *tab, uint64_t *out, uint32_t limbs,
                               size_t out_item_stride) {
     const uint32_t n = 1u << t.log_n, log_slots = 31 - __builtin_clz(slots);
-    if (items == 0 || items > 65535 || (out && (!tab || limbs == 0))) return hipErrorInvalidValue;
+    if (items == 0 || items > 65535 || (out ? (!tab || limbs == 0) : !coeffs)) return hipErrorInvalidValue;
     unsigned long long *maxima = reinterpret_cast<unsigned long long *>(max_bits);
     hipError_t e = run_fft<true>(v, slots, items, t, s, FftSource{re, im, count, value_stride, maxima});
     if (e != hipSuccess) return e;
