@@ -227,6 +227,25 @@ int backend_for_level(const he_context *ctx, uint32_t L) {
     return capable && ctx->mixed_ok ? NTT_BACKEND_MIXED : NTT_BACKEND_INT;
 }
 
+// tables whose limbs a launch of this back end transforms in FP64
+uint64_t fp_mask_of(const he_context *ctx, int backend) {
+    return backend == NTT_BACKEND_INT ? 0 : (backend == NTT_BACKEND_FP ? ~(uint64_t)0 : ctx->fp_mask);
+}
+
+// A forward transform that reduces single-limb sources (K = 1) finishes those sources' inverse transform itself when
+// the launch is small (NTT_PRO_SOURCE_INTT_REDUCE): the inverse launch then stops after its blocks pass.
+// Environment CAHEL_HIP_NO_SOURCE_INTT=1 keeps the two rows passes apart.
+bool source_intt_ok(const he_context *ctx, uint32_t n_jobs) {
+    return !ctx->tune.no_source_intt && ntt_source_intt_ok(ctx->log_n, n_jobs, ctx->size_qp);
+}
+
+void set_source_intt(const he_context *ctx, NttArgs &fwd, int inverse_backend) {
+    fwd.pro_mode = NTT_PRO_SOURCE_INTT_REDUCE;
+    fwd.pro_src_fp_mask = fp_mask_of(ctx, inverse_backend);
+    fwd.pro_itw = ctx->d_ipsi;
+    fwd.pro_itw_fp = ctx->d_ipsi_fp;
+}
+
 // the FP64 back end applies when every table of the launch has a prime below 2^50
 bool fp_for(const he_context *ctx, const LimbMap &m) {
     if (!ctx->use_fp) return false;
@@ -456,6 +475,7 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->fuse_tensor = !(nt && nt[0] == '1');
         const char *nr = getenv("CAHEL_HIP_NO_REDUCE_IN_NTT");
         ctx->single_limb_digits = ctx->size_p == 1 && !(nr && nr[0] == '1');
+
         const char *nbf = getenv("CAHEL_HIP_NO_BATCH_FUSED_KS");
         ctx->batch_fused_inner = !(nbf && nbf[0] == '1');
         auto env_on = [](const char *name) { const char *e = getenv(name); return e && e[0] == '1'; };
@@ -468,6 +488,7 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->tune.hoist_no_xcd = env_on("CAHEL_HIP_NO_XCD_MAP");
         ctx->tune.hoist_no_contig = env_on("CAHEL_HIP_NO_XCD_CONTIG");
         ctx->tune.no_matrix_bconv = env_on("CAHEL_HIP_NO_MATRIX_BCONV");
+        ctx->tune.no_source_intt = env_on("CAHEL_HIP_NO_SOURCE_INTT");
         ctx->tune.fuse_rows_forced = env_count("CAHEL_HIP_FUSE_ROWS", 1, 24, 0);
         ctx->tune.bconv_rows = env_count("CAHEL_HIP_BCONV_ROWS", 1, 64, 6);
         int cus = 0;
@@ -865,15 +886,18 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     inv.map = plain_map(L, 0);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_part_hat_inv;
-    HE_HIP(launch_ntt_inverse(inv, items, backend_for(ctx, inv.map), S(s)));
     const bool fused = fuse_rows_ok(ctx, lv, L);
-    // skip_own (batched levels only): the consumer reads a digit's own limbs from c, their slots in out stay unwritten
-    if (skip_own && !lv->batched) return HE_E_INVALID_ARGUMENT;
-    const uint32_t copy_rows = skip_own ? 0 : lv->modup_max_copy;
     // digits of one limb each (K = 1): (Q_d / q_d)^-1 and the conversion matrix are all ones, so the conversion is the
     // reduction of the digit's coefficients modulo each other prime, which the forward transform does where it reads
     // its input; only the digits' own limbs are copied
     const bool reduce_in_ntt = ctx->single_limb_digits && !fused;
+    // ... and a small launch finishes the inverse transform there as well
+    const int inv_backend = backend_for(ctx, inv.map);
+    const bool source_intt = reduce_in_ntt && source_intt_ok(ctx, lv->n_modup_jobs * items);
+    HE_HIP(launch_ntt_inverse(inv, items, inv_backend, S(s), false, source_intt));
+    // skip_own (batched levels only): the consumer reads a digit's own limbs from c, their slots in out stay unwritten
+    if (skip_own && !lv->batched) return HE_E_INVALID_ARGUMENT;
+    const uint32_t copy_rows = skip_own ? 0 : lv->modup_max_copy;
     if (reduce_in_ntt) {
         for (uint32_t d = 0; d < lv->beta && !skip_own; d++)
             HE_HIP(hipMemcpy2DAsync(out + ((size_t)d * LK + d) * n, (size_t)lv->beta * LK * n * sizeof(uint64_t),
@@ -913,6 +937,7 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
         fwd.pro_src = ws;
         fwd.pro_item_stride = (size_t)L * n;
         fwd.pro_lk = LK;
+        if (source_intt) set_source_intt(ctx, fwd, inv_backend);
     }
     HE_HIP(launch_ntt_forward(fwd, 1, backend_for_level(ctx, L), S(s), fused));
     return HE_OK;
@@ -962,7 +987,6 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     inv.map = plain_map(K, ctx->size_q);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = ctx->d_phat_inv;
-    HE_HIP(launch_ntt_inverse(inv, n_polys, backend_for(ctx, inv.map), S(s)));
     const Level *lv = level_of(ctx, L);
     // the conversion tables describe up to 4 polynomials; more of them go as items of 2 (ciphertexts)
     const bool batched = lv && lv->batched && (n_polys <= 4 || n_polys % 2 == 0);
@@ -970,6 +994,10 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
     // one special prime: (P / p)^-1 and the conversion matrix are ones, the conversion is the reduction of the special
     // limb's coefficients modulo each q_j, done where the forward transform reads its input
     const bool reduce_in_ntt = ctx->single_limb_digits && !fused;
+    // ... and a small launch finishes the special limb's inverse transform there as well
+    const int inv_backend = backend_for(ctx, inv.map);
+    const bool source_intt = reduce_in_ntt && source_intt_ok(ctx, n_polys * L);
+    HE_HIP(launch_ntt_inverse(inv, n_polys, inv_backend, S(s), false, source_intt));
     if (reduce_in_ntt) {
     } else if (batched) {
         const uint32_t units = n_polys <= 4 ? n_polys : 2, items = n_polys / units;
@@ -1006,6 +1034,10 @@ int moddown_impl(const he_context *ctx, uint32_t L, uint64_t *cx, uint64_t *out,
         fwd.pro_mode = NTT_PRO_SOURCE_REDUCE;
         fwd.pro_src = cx + (size_t)L * n;
         fwd.pro_poly_stride = LK;
+        if (source_intt) {
+            set_source_intt(ctx, fwd, inv_backend);
+            fwd.pro_src_table = ctx->size_q;
+        }
     }
     HE_HIP(launch_ntt_forward(fwd, n_polys, backend_for(ctx, fwd.map), S(s), fused));
     return HE_OK;

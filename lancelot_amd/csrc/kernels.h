@@ -16,6 +16,8 @@ struct Tuning {
     bool hoist_no_xcd = false;       // CAHEL_HIP_NO_XCD_MAP=1
     bool hoist_no_contig = false;    // CAHEL_HIP_NO_XCD_CONTIG=1
     bool no_matrix_bconv = false;    // CAHEL_HIP_NO_MATRIX_BCONV=1: the fused base conversion stays on the FP64 vector units
+    bool no_source_intt = false;     // CAHEL_HIP_NO_SOURCE_INTT=1: K = 1, small launches: the inverse rows pass of a reduced
+                                     // source limb stays a launch of its own
 };
 
 // One limb-sized NTT job given explicitly: which limb of the buffer, which modulus table.
@@ -70,6 +72,15 @@ enum : int {
     // data_limb / pro_lk of pro_src + i * pro_item_stride: the base conversion of digits of one limb each (K = 1),
     // whose matrix is all ones, done where the forward transform of the converted limb reads its input
     NTT_PRO_SOURCE_REDUCE = 8,
+    // the same with the source limb still in the middle of its inverse transform: pro_src holds the words that the
+    // inverse blocks pass left (launch_ntt_inverse with rows_skipped), and the forward rows pass first runs the inverse
+    // rows pass on its tile of the source (the two passes work on the same rows x columns tile), without the round trip
+    // of the coefficients through memory and without a launch.  Every job repeats its source's inverse rows pass, so
+    // this is for launches of a few limbs, which are bound by the latency of one workgroup (ntt_source_intt_ok).
+    // Source of a job as for NTT_PRO_SOURCE_REDUCE; its prime is table data_limb / pro_lk in list mode, pro_src_table
+    // in map mode; bit t of pro_src_fp_mask says whether the blocks pass of table t ran on the FP64 back end.  The
+    // inverse transform's scaling must be N^-1 alone (digits of one limb each).
+    NTT_PRO_SOURCE_INTT_REDUCE = 9,
 };
 
 struct NttArgs {
@@ -101,6 +112,10 @@ struct NttArgs {
     uint32_t pro_poly_stride;
     size_t pro_item_stride;   // NTT_PRO_SOURCE_REDUCE in list mode: words between the sources of consecutive items
     uint32_t pro_lk;          // ... and limbs per digit of the list's buffer (L + K)
+    uint32_t pro_src_table;   // NTT_PRO_SOURCE_INTT_REDUCE in map mode: table of the source limb
+    uint64_t pro_src_fp_mask; // NTT_PRO_SOURCE_INTT_REDUCE: tables whose inverse blocks pass left FP64 lazy words
+    const uint64_t *pro_itw;  // ... and the inverse transform's twiddle tables (laid out like tw and tw_fp)
+    const double *pro_itw_fp;
     const uint64_t *epi_a;    // limb (poly, i) like `out`, with its own poly stride
     uint32_t epi_a_poly_stride;
     const uint64_t *epi_b;
@@ -131,7 +146,12 @@ hipError_t launch_ntt_forward(const NttArgs &a, uint32_t n_polys, int backend, h
 // a.out, epilogue NTT_EPI_MUL optional).
 // blocks_done: the blocks pass has run already (launch_tensor_intt_blocks left its lazy words in a.out), only the
 // rows pass is launched.
-hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool blocks_done = false);
+// rows_skipped: only the blocks pass is launched; a forward transform with NTT_PRO_SOURCE_INTT_REDUCE finishes it.
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool blocks_done = false,
+                              bool rows_skipped = false);
+// whether a forward launch of n_jobs limbs may take NTT_PRO_SOURCE_INTT_REDUCE (2^15 <= N <= 2^16, a launch small
+// enough to run on quarter tiles, every table below 64)
+bool ntt_source_intt_ok(uint32_t log_n, uint32_t n_jobs, uint32_t n_tables);
 
 // Tensor product of two size-2 ciphertexts fused with the blocks pass of the inverse transform of its third polynomial
 // (FP64 back end; every prime of the L limbs below 2^50).  `a`: inverse base arguments with map = the L data limbs

@@ -62,7 +62,8 @@ struct Job {
     uint32_t table;
     uint32_t poly;
     uint32_t limb;
-    const uint64_t *src;   // NTT_PRO_SOURCE_REDUCE (rows pass only): the limb that is reduced into this one
+    const uint64_t *src;   // NTT_PRO_SOURCE_[INTT_]REDUCE (rows pass only): the limb that is reduced into this one
+    uint32_t src_table;    // NTT_PRO_SOURCE_INTT_REDUCE: its prime
 };
 
 __device__ __forceinline__ Job decode_job(const NttArgs &a, uint32_t job) {
@@ -77,7 +78,9 @@ __device__ __forceinline__ Job decode_job(const NttArgs &a, uint32_t job) {
         j.table = lj.table;
         j.poly = 0;
         j.limb = 0;
-        j.src = a.pro_mode == NTT_PRO_SOURCE_REDUCE ? a.pro_src + item * a.pro_item_stride + (size_t)(lj.data_limb / a.pro_lk) * n : nullptr;
+        const bool sourced = a.pro_mode == NTT_PRO_SOURCE_REDUCE || a.pro_mode == NTT_PRO_SOURCE_INTT_REDUCE;
+        j.src_table = sourced ? lj.data_limb / a.pro_lk : 0;
+        j.src = sourced ? a.pro_src + item * a.pro_item_stride + (size_t)j.src_table * n : nullptr;
     } else {
         j.poly = job / a.map.limbs;
         j.limb = job % a.map.limbs;
@@ -85,6 +88,7 @@ __device__ __forceinline__ Job decode_job(const NttArgs &a, uint32_t job) {
         j.out = a.out + ((size_t)j.poly * a.out_poly_stride + j.limb) * n;
         j.table = map_table(a.map, j.limb);
         j.src = a.pro_src + ((size_t)j.poly * a.pro_poly_stride << a.log_n);
+        j.src_table = a.pro_src_table;
     }
     return j;
 }
@@ -188,7 +192,10 @@ __device__ __forceinline__ FpTw inverse_scale(const NttArgs &a, const Job &job, 
 //          ((g / C) << (LOGC + p1)) + g mod C + j C; twiddle index 2^p0 + g / C
 // Tile word e lives at row e / C, column col0 + e mod C of the limb's (N / 256) x 256 view.
 // ---------------------------------------------------------------------------------------------------
-template <int LD, bool FWD, int BE, int LOGC>
+// SRC_INTT (forward, NTT_PRO_SOURCE_INTT_REDUCE): the inverse rows pass of the source limb's tile runs first, on the
+// same registers: its last block leaves the coefficient of tile word t + T i in register i, which is where the forward
+// pass's first block takes its input from.
+template <int LD, bool FWD, int BE, int LOGC, bool SRC_INTT = false>
 __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, uint32_t col0, uint64_t *lds) {
     constexpr int p0 = Split<LD>::p0, p1 = Split<LD>::p1;
     constexpr int R0 = 1 << p0, R1 = 1 << p1, NG0 = 16 >> p0, NG1 = 16 >> p1;
@@ -220,13 +227,63 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
 #pragma unroll
         for (int k = 0; k < NG1; k++) block(v + k * R1, idx_near(k));
     };
+    // canonical coefficients of the source limb at the tile words t + T i
+    uint64_t s[SRC_INTT ? 16 : 1];
+    if constexpr (SRC_INTT) {
+        const uint32_t st = job.src_table;
+        // (the tables of the inverse transform lie behind the forward ones: a.tw / a.tw_fp are the forward launch's)
+        if ((a.pro_src_fp_mask >> st) & 1) {
+            const FpMod m = fp_ctx(a, st).m;
+            const double *itw = a.pro_itw_fp + ((size_t)st << a.log_n);
+            double v[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = __longlong_as_double((long long)job.src[p1 > 0 ? glob(e_near(j)) : glob(e_far(j))]);
+            if (p1 > 0) {
+                inner(v, [&](double *w, uint32_t idx) { fp_gs_block<(p1 > 0 ? p1 : 1), true>(w, itw, idx, m); });
+#pragma unroll
+                for (int j = 0; j < 16; j++) ld[skew(e_near(j))] = v[j];
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = ld[skew(e_far(j))];
+            }
+            outer(v, [&](double *w, uint32_t idx) { fp_gs_block<p0, true>(w, itw, idx, m); });
+            const double *cc = a.fp_consts + 4 * (size_t)st;
+            const FpTw ninv{cc[2], cc[3]};
+#pragma unroll
+            for (int j = 0; j < 16; j++) s[SRC_INTT ? j : 0] = fp_to_u64(fp_canonical(fp_mulmod(v[j], ninv, m), m));
+        } else {
+            const uint64_t q = a.moduli[st];
+            const uint64_t *itw = a.pro_itw + ((size_t)st << (a.log_n + 1));
+            uint64_t v[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = job.src[p1 > 0 ? glob(e_near(j)) : glob(e_far(j))];
+            if (p1 > 0) {
+                inner(v, [&](uint64_t *w, uint32_t idx) { gs_block<(p1 > 0 ? p1 : 1)>(w, itw, idx, q); });
+#pragma unroll
+                for (int j = 0; j < 16; j++) lds[skew(e_near(j))] = v[j];
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = lds[skew(e_far(j))];
+            }
+            outer(v, [&](uint64_t *w, uint32_t idx) { gs_block<p0>(w, itw, idx, q); });
+#pragma unroll
+            for (int j = 0; j < 16; j++) s[SRC_INTT ? j : 0] = reduce_2q(v[j], q);
+        }
+        // (the forward pass below writes and reads the same LDS slots in the same order as the inverse pass read and
+        // wrote them: a thread's own slots t + T i first, then a barrier)
+    }
     const bool fp = BE == NTT_BACKEND_FP || (BE == NTT_BACKEND_MIXED && ((a.fp_mask >> job.table) & 1));
     if (BE != NTT_BACKEND_INT && fp) {
         const FpCtx c = fp_ctx(a, job.table);
         double v[16];
         if (FWD) {
             bool reduce_first = true;
-            if (a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
+            if constexpr (SRC_INTT) {
+                const uint64_t q = a.moduli[job.table], r1 = a.barrett[2 * job.table + 1];
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = fp_from_u64(barrett64(s[SRC_INTT ? j : 0], q, r1));
+                reduce_first = false;
+            } else if (a.pro_mode == NTT_PRO_MODDOWN_RESCALE) {
                 const uint64_t *tsrc = a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
                 const uint64_t *dsrc = a.pro_src2 + ((size_t)job.poly * a.pro2_poly_stride << a.log_n);
                 const FpMod ml = fp_ctx(a, a.pro_last).m;
@@ -298,7 +355,11 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
     const uint64_t q = c.q;
     uint64_t v[16];
     if (FWD) {
-        if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE || a.pro_mode == NTT_PRO_SOURCE_REDUCE) {
+        if constexpr (SRC_INTT) {
+            const uint64_t r1 = a.barrett[2 * job.table + 1];
+#pragma unroll
+            for (int j = 0; j < 16; j++) v[j] = barrett64(s[SRC_INTT ? j : 0], q, r1);
+        } else if (a.pro_mode == NTT_PRO_BROADCAST_REDUCE || a.pro_mode == NTT_PRO_SOURCE_REDUCE) {
             const uint64_t r1 = a.barrett[2 * job.table + 1];
             const uint64_t *src = a.pro_mode == NTT_PRO_SOURCE_REDUCE ? job.src : a.pro_src + ((size_t)job.poly * a.pro_poly_stride << a.log_n);
 #pragma unroll
@@ -360,7 +421,7 @@ __device__ __forceinline__ void rows_direct(const NttArgs &a, const Job &job, ui
 // ---------------------------------------------------------------------------------------------------
 // rows pass: stages 0 .. LD-1 (forward) over an R = 2^LD rows x 256 matrix
 // ---------------------------------------------------------------------------------------------------
-template <int LD, bool FWD, int BE, int TL>
+template <int LD, bool FWD, int BE, int TL, bool SRC_INTT = false>
 __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     __shared__ uint64_t lds[(1 << TL) + (1 << (TL - 4))];
     constexpr uint32_t kRowThreads = (1u << TL) / 16;
@@ -376,9 +437,10 @@ __global__ __launch_bounds__((1 << TL) / 16) void ntt_rows_kernel(NttArgs a) {
     // (N = 2^17, 512 rows: the inner block would be five stages, 32 words a thread; that degree takes the tile
     // through LDS between its blocks, below)
     if constexpr (LD >= 4 && LD <= 8 && tile_elems == 16 * kRowThreads) {
-        rows_direct<LD, FWD, BE, LOGC>(a, job, col0, lds);
+        rows_direct<LD, FWD, BE, LOGC, SRC_INTT>(a, job, col0, lds);
         return;
     }
+    static_assert(!SRC_INTT || (LD >= 4 && LD <= 8 && tile_elems == 16 * kRowThreads), "only the register rows pass");
     double *ld = reinterpret_cast<double *>(lds);
 
     // the back end of this workgroup's limb: fixed by the launch, or (mixed) by the limb's prime
@@ -1797,6 +1859,19 @@ hipError_t launch_rows(const NttArgs &a, uint32_t n_jobs, hipStream_t s) {
     };
     // small launches (fewer 4096-word tiles than CUs) are bound by the latency of one workgroup: quarter tiles
     const bool small = ld >= 5 && n_jobs * (256u >> (kTileLog - ld < 8 ? kTileLog - ld : 8)) < 256;
+    if (a.pro_mode == NTT_PRO_SOURCE_INTT_REDUCE) {
+        // one instantiation per degree, on quarter tiles, which follows fp_mask limb by limb: the mask stands for the
+        // launch's back end here
+        if (!FWD || !ntt_source_intt_ok(a.log_n, n_jobs, 0) || !a.pro_itw || (a.pro_src_fp_mask && !a.pro_itw_fp))
+            return hipErrorInvalidValue;
+        NttArgs b = a;
+        b.fp_mask = FP == NTT_BACKEND_INT ? 0 : (FP == NTT_BACKEND_FP ? ~(uint64_t)0 : a.fp_mask);
+        if (ld == 7)
+            hipLaunchKernelGGL((ntt_rows_kernel<7, true, NTT_BACKEND_MIXED, 10, true>), grid(7, 10), dim3(64), 0, s, b);
+        else
+            hipLaunchKernelGGL((ntt_rows_kernel<8, true, NTT_BACKEND_MIXED, 10, true>), grid(8, 10), dim3(64), 0, s, b);
+        return hipGetLastError();
+    }
     switch (ld) {
 #define HE_CASE(LD)                                                                               \
     case LD:                                                                                      \
@@ -2003,16 +2078,23 @@ hipError_t launch_tensor_intt_blocks(NttArgs a, const TensorFuse &x, hipStream_t
     return hipGetLastError();
 }
 
-hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool blocks_done) {
+bool ntt_source_intt_ok(uint32_t log_n, uint32_t n_jobs, uint32_t n_tables) {
+    if (log_n < 15 || log_n > 16 || n_tables > 64) return false;
+    const uint32_t ld = log_n - 8;
+    return n_jobs * (256u >> (kTileLog - ld)) < 256;   // what launch_rows calls a small launch
+}
+
+hipError_t launch_ntt_inverse(const NttArgs &a, uint32_t n_polys, int backend, hipStream_t s, bool blocks_done,
+                              bool rows_skipped) {
     if (a.log_n < 9 || a.log_n > 17 || backend < NTT_BACKEND_INT || backend > NTT_BACKEND_MIXED) return hipErrorInvalidValue;
     const uint32_t n_jobs = a.jobs ? a.n_jobs * (a.items ? a.items : 1) : n_polys * a.map.limbs;
     if (n_jobs == 0) return hipSuccess;
-    if (!blocks_done && one_pass_ok(a, backend, false, n_jobs)) return launch_limb_fp<false>(a, n_jobs, s);
+    if (!blocks_done && !rows_skipped && one_pass_ok(a, backend, false, n_jobs)) return launch_limb_fp<false>(a, n_jobs, s);
     hipError_t e = blocks_done                    ? hipSuccess
                    : backend == NTT_BACKEND_MIXED ? launch_blocks<false, NTT_BACKEND_MIXED>(a, n_polys, s)
                    : backend                    ? launch_blocks<false, NTT_BACKEND_FP>(a, n_polys, s)
                                                 : launch_blocks<false, NTT_BACKEND_INT>(a, n_polys, s);
-    if (e != hipSuccess) return e;
+    if (e != hipSuccess || rows_skipped) return e;
     NttArgs rows = a;
     rows.in = a.out;  // the rows pass continues in place on the output buffer
     rows.in_poly_stride = a.out_poly_stride;

@@ -558,3 +558,56 @@ def test_largest_degree_scheme_flow(oracle):
     got = np.array(enc.decode(ctx, pt))
     err = np.abs(got - np.roll(x * y, -5))
     assert np.median(err) < 1e-4 and np.max(err) < 2e-2      # 2^30 of scale left; the floor-rescale bias in the first slots
+
+
+@pytest.mark.parametrize("logn,bits", [(16, [60, 40, 40, 60]), (15, [60, 40, 40, 60]), (16, [50, 45, 50, 49, 50])])
+@pytest.mark.parametrize("variant", ["default", "two_rows_passes", "integer", "integer_two_rows_passes"])
+def test_single_limb_digits_small_launches(oracle, monkeypatch, logn, bits, variant):
+    """One special prime (K = 1, Lancelot's chain): ModUp and ModDown reduce a single source limb into every other
+    prime, and a launch of a few limbs runs the source's inverse rows pass inside the forward rows pass
+    (CAHEL_HIP_NO_SOURCE_INTT=1 keeps the two passes apart).  he_modup, he_moddown (overwriting and adding), he_keyswitch
+    with and without a Galois element and he_rotate against the oracle, limb for limb, on the mixed, FP64 and integer
+    back ends, at every level of the chain (src/rns.cu:610-782 ModUp / ModDown, src/evaluate.cu:1622-1760 key switch)."""
+    import ctypes as C
+    from gpu_util import DeviceArray, make_pair, rand_limbs
+    from lancelot_amd import capi
+    monkeypatch.setenv("CAHEL_HIP_NO_SOURCE_INTT", "1" if variant.endswith("two_rows_passes") else "0")
+    monkeypatch.setenv("CAHEL_HIP_NO_FP64", "1" if variant.startswith("integer") else "0")
+    cahel, parms, ctx, p = make_pair(oracle, logn, bits, 1)
+    lib, h = capi.lib(), ctx.he_handle()
+    rng = np.random.default_rng(logn + len(bits))
+    K, n = 1, p.n
+    host_evk = [rand_limbs(p, rng, range(p.size_qp), n_polys=2) for _ in range(p.size_q)]
+    dev_evk = [DeviceArray(capi, host=k) for k in host_evk]
+    for L in range(p.size_q, 0, -1):
+        ptrs = capi.evk_array([dev_evk[d].ptr for d in range(L)])
+        tables = [p.table_index(L, t) for t in range(L + K)]
+        c = rand_limbs(p, rng, range(L))
+        c[:, :4] = np.array(p.moduli[:L], dtype=np.uint64)[:, None] - 1       # largest residues
+        dc = DeviceArray(capi, host=c)
+        dy = DeviceArray(capi, shape=(L, L + K, n))
+        ws = DeviceArray(capi, shape=(2 * L, n))
+        capi.check(lib.he_modup(h, L, dc.ptr, dy.ptr, ws.ptr, None))
+        assert (dy.numpy() == p.modup(c)).all(), L
+        assert (dc.numpy() == c).all()
+        cx = np.stack([rand_limbs(p, rng, tables) for _ in range(2)])
+        md = np.stack([p.moddown(cx[b]) for b in range(2)])
+        dcx, dout = DeviceArray(capi, host=cx), DeviceArray(capi, shape=(2, L, n))
+        capi.check(lib.he_moddown(h, L, dcx.ptr, dout.ptr, 2, 0, ws.ptr, None))
+        assert (dout.numpy() == md).all(), L
+        base = rand_limbs(p, rng, range(L), n_polys=2)
+        dcx, dacc = DeviceArray(capi, host=cx), DeviceArray(capi, host=base)
+        capi.check(lib.he_moddown(h, L, dcx.ptr, dacc.ptr, 2, 1, ws.ptr, None))
+        assert (dacc.numpy() == np.stack([p.add(base[b], md[b]) for b in range(2)])).all(), L
+        kws = DeviceArray(capi, shape=(lib.he_keyswitch_workspace_words(h, L),))
+        ct = rand_limbs(p, rng, range(L), n_polys=2)
+        for elt in (0, 5):
+            dct = DeviceArray(capi, host=ct)
+            capi.check(lib.he_keyswitch(h, L, dc.ptr, ptrs, dct.ptr, elt, kws.ptr, None))
+            ks = p.key_switch(p.galois_ntt(c, elt) if elt else c, host_evk)
+            assert (dct.numpy() == np.stack([p.add(ct[b], ks[b]) for b in range(2)])).all(), (L, elt)
+        dct, drot = DeviceArray(capi, host=ct), DeviceArray(capi, shape=(2, L, n))
+        elt = pow(5, 3, 2 * n)
+        capi.check(lib.he_rotate(h, L, dct.ptr, ptrs, drot.ptr, elt, kws.ptr, None))
+        ks = p.key_switch(p.galois_ntt(ct[1], elt), host_evk)
+        assert (drot.numpy() == np.stack([p.add(p.galois_ntt(ct[0], elt), ks[0]), ks[1]])).all(), L
