@@ -869,8 +869,9 @@ namespace {
 
 // ModUp of `items` polynomials: item k reads c + k * c_item_stride * N (stride in limbs), writes out [k][beta][L+K][N];
 // ws holds items * L limbs
+// in_galois != 0 (one item, skip_own): the input is sigma(c), X -> X^in_galois, gathered by the inverse blocks pass
 int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_item_stride, uint32_t items,
-               uint64_t *out, uint64_t *ws, he_stream s, bool skip_own = false) {
+               uint64_t *out, uint64_t *ws, he_stream s, bool skip_own = false, uint32_t in_galois = 0) {
     if (!ctx || !c || !out || !ws || ctx->size_p == 0 || items == 0 || c_item_stride < L) return HE_E_INVALID_ARGUMENT;
     const Level *lv = level_of(ctx, L);
     if (!lv) return HE_E_LEVEL_NOT_SET;
@@ -886,6 +887,8 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     inv.map = plain_map(L, 0);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_part_hat_inv;
+    if (in_galois && (items != 1 || !skip_own)) return HE_E_INVALID_ARGUMENT;   // (own limbs are copied from c as it is)
+    inv.in_galois = in_galois;
     const bool fused = fuse_rows_ok(ctx, lv, L);
     // digits of one limb each (K = 1): (Q_d / q_d)^-1 and the conversion matrix are all ones, so the conversion is the
     // reduction of the digit's coefficients modulo each other prime, which the forward transform does where it reads
@@ -1097,9 +1100,12 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
     const uint64_t *src = c;
     const bool fused_inner = ctx->fuse_inner && lv->batched && fp_for_level(ctx, L) &&
                              (items == 1 || (ctx->batch_fused_inner && !tin));
-    if (galois_elt && !fused_inner) {
+    // levels whose inner product reads a digit's own limbs from the input gather sigma(c) where they read c (the
+    // inverse blocks pass and the inner product); the others stage it
+    const bool gather = galois_elt && !fused_inner && lv->batched && items == 1;
+    if (galois_elt && !fused_inner && !gather) {
         // sigma(c) is staged in the second half of the ModDown workspace, which ModUp leaves alone and ModDown
-        // only touches after the inner product has read it (the fused path gathers sigma(c) where it reads c)
+        // only touches after the inner product has read it
         uint64_t *staged = tmp + (size_t)L * n;
         if (int rc = he_galois_ntt(ctx, c, staged, L, galois_elt, s)) return rc;
         src = staged;
@@ -1173,8 +1179,8 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         if (tin) return HE_E_INVALID_ARGUMENT;
         // (batched levels: neither kernel needs the copy of a digit's own limbs into y)
         const bool skip_own = fp_batch || lv->batched;
-        const uint32_t src_stride = galois_elt ? L : c_item_stride;
-        if (int rc = modup_impl(ctx, L, src, src_stride, items, y, tmp, s, skip_own)) return rc;
+        const uint32_t src_stride = (galois_elt && !gather) ? L : c_item_stride;
+        if (int rc = modup_impl(ctx, L, src, src_stride, items, y, tmp, s, skip_own, gather ? galois_elt : 0)) return rc;
         EvkPtrs ptrs;
         memset(&ptrs, 0, sizeof(ptrs));
         for (uint32_t d = 0; d < lv->beta; d++) {
@@ -1189,7 +1195,7 @@ int ks_accumulate(const he_context *ctx, const Level *lv, uint32_t L, const uint
         }
         HE_HIP(launch_inner_product(ctx->tables(), y, ptrs, cx, L, ctx->size_p, ctx->size_q, lv->beta, 0, false,
                                     fold_ct, fold_w, items, 2 * (size_t)L * n, S(s), add_c0, galois_elt, ctx->d_p_mod_q,
-                                    skip_own ? src : nullptr, (size_t)src_stride * n));
+                                    skip_own ? src : nullptr, (size_t)src_stride * n, gather ? galois_elt : 0));
     }
     return HE_OK;
 }

@@ -278,11 +278,14 @@ struct EvkPtrs {
 // items inputs (y and out dense, fold_ct fold_item_stride words apart) in one launch.
 // fold_ct / fold_w as in KsFuseArgs (nullptr: plain inner product).
 // add_c0 / add_elt / p_mod_q as in KsFuseArgs (add_elt = 0: add_c0 is added as it is; items must be 1).
+// own: the key switch's input in NTT form, from which a digit's own limbs are read instead of from y; own_elt != 0:
+// that input is sigma(own), X -> X^own_elt, gathered on load.
 hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtrs &evk, uint64_t *out, uint32_t L,
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
                                 const uint64_t *fold_ct, const uint64_t *fold_w, uint32_t items, size_t fold_item_stride,
                                 hipStream_t s, const uint64_t *add_c0 = nullptr, uint32_t add_elt = 0,
-                                const uint64_t *p_mod_q = nullptr, const uint64_t *own = nullptr, size_t own_item_stride = 0);
+                                const uint64_t *p_mod_q = nullptr, const uint64_t *own = nullptr, size_t own_item_stride = 0,
+                                uint32_t own_elt = 0);
 
 // The same product for a batch on the FP64 back end (every prime below 2^50, N >= 512): key words are loaded once
 // per group of up to 8 items, and a digit's own limbs come from own (the key switch's input in NTT form, items

@@ -393,6 +393,7 @@ struct InnerArgs {
     uint32_t add_elt;
     const uint64_t *own;            // optional: the key-switch input [L][N]; a digit's own limbs are read from it (their
     size_t own_item_stride;         // slots in y were left unwritten), items own_item_stride words apart
+    uint32_t own_elt;               // != 0: the key-switch input is sigma(own), gathered here (X -> X^own_elt)
 };
 
 // grid: (N / 256, L + K, items).  Streams beta digit limbs of y and 2 beta key limbs, writes (or accumulates) the
@@ -411,9 +412,10 @@ __global__ __launch_bounds__(kThreads) void inner_product_kernel(InnerArgs p) {
     uint64_t *out = p.out + blockIdx.z * p.out_item_stride;
     const uint64_t *own = p.own ? p.own + blockIdx.z * p.own_item_stride + ((size_t)t << p.log_n) : nullptr;
     const uint32_t own_d = (own && t < p.L) ? t / p.K : 0xffffffffu;
+    const uint32_t own_src = p.own_elt ? galois_index(j, p.own_elt, p.log_n) : src;
     U128 a0{0, 0}, a1{0, 0};
     for (uint32_t d = 0; d < p.beta; d++) {
-        const uint64_t v = d == own_d ? own[src] : y[(((size_t)d * LK + t) << p.log_n) + src];
+        const uint64_t v = d == own_d ? own[own_src] : y[(((size_t)d * LK + t) << p.log_n) + src];
         const uint64_t *k = p.evk.p[d];
         mac128(a0, v, k[key_off]);
         mac128(a1, v, k[key_off + key_poly]);
@@ -928,11 +930,11 @@ hipError_t launch_inner_product(const Tables &t, const uint64_t *y, const EvkPtr
                                 uint32_t K, uint32_t size_q, uint32_t beta, uint32_t galois_elt, bool accumulate,
                                 const uint64_t *fold_ct, const uint64_t *fold_w, uint32_t items, size_t fold_item_stride,
                                 hipStream_t s, const uint64_t *add_c0, uint32_t add_elt, const uint64_t *p_mod_q,
-                                const uint64_t *own, size_t own_item_stride) {
+                                const uint64_t *own, size_t own_item_stride, uint32_t own_elt) {
     const size_t n = (size_t)1 << t.log_n;
     InnerArgs p{y, out, t.moduli, t.barrett, evk, L, K, size_q, beta, t.log_n, galois_elt, accumulate ? 1 : 0,
                 fold_ct, fold_w, (size_t)beta * (L + K) * n, 2 * (size_t)(L + K) * n, fold_item_stride,
-                add_c0, p_mod_q, add_elt, own, own_item_stride};
+                add_c0, p_mod_q, add_elt, own, own_item_stride, own_elt};
     if (items == 0 || items > 65535 || (add_c0 && (items != 1 || !p_mod_q))) return hipErrorInvalidValue;
     hipLaunchKernelGGL(inner_product_kernel, dim3((1u << t.log_n) / kThreads, L + K, items), dim3(kThreads), 0, s, p);
     return hipGetLastError();
