@@ -1485,10 +1485,8 @@ int he_encrypt_batch(const he_context *ctx, uint32_t L, uint32_t items, const ui
     memcpy(k.k, key, sizeof(k.k));
     const LimbMap map{LK, 0, L, Q};
     // item k draws u, e0, e1 from the stream ids stream_id + 3 k, + 1, + 2: what `items` encryptions in a row draw
-    HE_HIP(launch_sample(ctx->tables(), SAMPLE_TERNARY, k, stream_id, u, map, nullptr, 0, items, 3, (size_t)LK * n, S(s)));
-    // (e0, e1 of all items in one launch: wide is [items][2] polynomials LK * N words apart)
-    HE_HIP(launch_sample(ctx->tables(), SAMPLE_ERROR, k, stream_id + 1, wide, map, nullptr, 0, 2 * items, 3, (size_t)LK * n,
-                         S(s), 2));
+    // (one launch: u and wide lie one after the other, 3 * items polynomials LK * N words apart)
+    HE_HIP(launch_sample_encrypt(ctx->tables(), k, stream_id, u, map, items, (size_t)LK * n, S(s)));
     // u and wide lie one after the other: 3 * items polynomials of the same limbs
     if (int rc = he_ntt_forward(ctx, u, 3 * items, LK, LK, 0, L, Q, s)) return rc;
     HE_HIP(launch_encrypt_fma(ctx->tables(), u, pk, wide, L, K, Q, items, S(s)));

@@ -127,6 +127,108 @@ __global__ __launch_bounds__(kThreads) void cfft_lds_kernel(double2 *v, uint32_t
     for (uint32_t i = threadIdx.x; i < tile; i += kThreads) g[i] = s[i];
 }
 
+// The same for a full tile of kFftTile = 2048 values, 8 values per thread: the 11 stages run as register blocks of
+// 3 + 3 + 3 + 2 stages with the tile in LDS between them (4 exchanges instead of 11), and the 24 twiddles a thread
+// needs are fetched ahead of everything (each is a table look-up behind a table look-up: inside the stages, 11 such
+// round trips to L2 in a row were most of the kernel's time).  Every butterfly has the operands and the twiddle it
+// has in cfft_lds_kernel, so the results are the same bit for bit.
+// Block of top span Lb = 8 S (S = 256, 32, 4): thread (hi, lo) = (tid / S, tid mod S) holds hi Lb + lo + k S, k < 8;
+// stage i of it (span Lb >> i) pairs k with k + (4 >> i) and takes twiddle lo + (k mod (4 >> i)) S.
+template <bool INVERSE>
+__global__ __launch_bounds__(kThreads) void cfft_lds8_kernel(double2 *v, FftTables t, uint32_t slots, FftSource src) {
+    constexpr uint32_t T = kFftTile;
+    static_assert(T == 2048 && kThreads == 256, "8 values per thread");
+    __shared__ double2 s[T + T / 32];
+    auto sk = [](uint32_t e) { return e + (e >> 5); };   // (a group of 4 lanes reads 32 values apart in the S = 4 block)
+    double2 *g = v + (size_t)blockIdx.y * slots + (size_t)blockIdx.x * T;
+    const uint32_t tid = threadIdx.x;
+    double2 tw[3][7], twd[3];
+#pragma unroll
+    for (int b = 0; b < 3; b++) {
+        const uint32_t S = 256u >> (3 * b), Lb = 8 * S, lo = tid & (S - 1);
+#pragma unroll
+        for (int k = 0; k < 4; k++) tw[b][k] = stage_twiddle<INVERSE>(t, Lb, lo + k * S);
+#pragma unroll
+        for (int k = 0; k < 2; k++) tw[b][4 + k] = stage_twiddle<INVERSE>(t, Lb / 2, lo + k * S);
+        tw[b][6] = stage_twiddle<INVERSE>(t, Lb / 4, lo);
+    }
+    twd[0] = stage_twiddle<INVERSE>(t, 4, 0);
+    twd[1] = stage_twiddle<INVERSE>(t, 4, 1);
+    twd[2] = stage_twiddle<INVERSE>(t, 2, 0);
+    if (INVERSE && src.re) {
+        // (only when the whole vector is this one tile: otherwise the wider stages have run before)
+        if (tid == 0) src.max_bits[blockIdx.y] = 0;
+#pragma unroll
+        for (int i = 0; i < 8; i++) s[sk(tid + i * kThreads)] = source_value(src, blockIdx.y, tid + i * kThreads);
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; i++) s[sk(tid + i * kThreads)] = g[tid + i * kThreads];
+    }
+    __syncthreads();
+    auto block3 = [&](int b) {
+        const uint32_t S = 256u >> (3 * b), Lb = 8 * S;
+        const uint32_t base = (tid / S) * Lb + (tid & (S - 1));
+        double2 e[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) e[k] = s[sk(base + k * S)];
+        if (INVERSE) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) butterfly<true>(e[k], e[k + 4], tw[b][k]);
+#pragma unroll
+            for (int k = 0; k < 4; k++) butterfly<true>(e[(k & 1) + 4 * (k >> 1)], e[(k & 1) + 4 * (k >> 1) + 2], tw[b][4 + (k & 1)]);
+#pragma unroll
+            for (int k = 0; k < 8; k += 2) butterfly<true>(e[k], e[k + 1], tw[b][6]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 8; k += 2) butterfly<false>(e[k], e[k + 1], tw[b][6]);
+#pragma unroll
+            for (int k = 0; k < 4; k++) butterfly<false>(e[(k & 1) + 4 * (k >> 1)], e[(k & 1) + 4 * (k >> 1) + 2], tw[b][4 + (k & 1)]);
+#pragma unroll
+            for (int k = 0; k < 4; k++) butterfly<false>(e[k], e[k + 4], tw[b][k]);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) s[sk(base + k * S)] = e[k];
+        __syncthreads();
+    };
+    // spans 4 and 2: two groups of 4 consecutive values per thread
+    auto block2 = [&]() {
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const uint32_t base = 4 * (tid + r * kThreads);
+            double2 e[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) e[k] = s[sk(base + k)];
+            if (INVERSE) {
+                butterfly<true>(e[0], e[2], twd[0]);
+                butterfly<true>(e[1], e[3], twd[1]);
+                butterfly<true>(e[0], e[1], twd[2]);
+                butterfly<true>(e[2], e[3], twd[2]);
+            } else {
+                butterfly<false>(e[0], e[1], twd[2]);
+                butterfly<false>(e[2], e[3], twd[2]);
+                butterfly<false>(e[0], e[2], twd[0]);
+                butterfly<false>(e[1], e[3], twd[1]);
+            }
+#pragma unroll
+            for (int k = 0; k < 4; k++) s[sk(base + k)] = e[k];
+        }
+        __syncthreads();
+    };
+    if (INVERSE) {
+        block3(0);
+        block3(1);
+        block3(2);
+        block2();
+    } else {
+        block2();
+        block3(2);
+        block3(1);
+        block3(0);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; i++) g[tid + i * kThreads] = s[sk(tid + i * kThreads)];
+}
+
 // The largest magnitude of an item's coefficients (the bit patterns of non-negative doubles order like the values):
 // reduced over the wave, then over the workgroup, one atomic per workgroup.  Atomics on one address are served one
 // after the other: one per thread took most of the rounding kernel's time, one per wave still half of it.  Every
@@ -315,9 +417,15 @@ hipError_t run_fft(double2 *v, uint32_t slots, uint32_t items, const FftTables &
     if (INVERSE) {
         if (wide)
             if (hipError_t e = top(src)) return e;
-        hipLaunchKernelGGL(cfft_lds_kernel<true>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots, wide ? none : src);
+        if (tile == kFftTile)
+            hipLaunchKernelGGL(cfft_lds8_kernel<true>, lds_grid, dim3(kThreads), 0, s, v, t, slots, wide ? none : src);
+        else
+            hipLaunchKernelGGL(cfft_lds_kernel<true>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots, wide ? none : src);
     } else {
-        hipLaunchKernelGGL(cfft_lds_kernel<false>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots, none);
+        if (tile == kFftTile)
+            hipLaunchKernelGGL(cfft_lds8_kernel<false>, lds_grid, dim3(kThreads), 0, s, v, t, slots, none);
+        else
+            hipLaunchKernelGGL(cfft_lds_kernel<false>, lds_grid, dim3(kThreads), 0, s, v, tile, t, slots, none);
         if (wide)
             if (hipError_t e = top(none)) return e;
     }

@@ -344,11 +344,14 @@ enum : int { SAMPLE_TERNARY = 0, SAMPLE_ERROR = 1, SAMPLE_UNIFORM = 2, SAMPLE_GA
 struct ChaChaKey {
     uint32_t k[8];
 };
-// items polynomials in one launch: polynomial k draws from stream_id + (k / stream_group) * stream_stride +
-// k % stream_group and lands k * out_item_stride words on
+// items polynomials in one launch: item k draws from stream_id + k * stream_stride and lands k * out_item_stride words on
 hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
                          const uint64_t *cdt, uint32_t cdt_len, uint32_t items, uint32_t stream_stride,
-                         size_t out_item_stride, hipStream_t s, uint32_t stream_group = 1);
+                         size_t out_item_stride, hipStream_t s);
+// u, e0, e1 of `items` public-key encryptions in one launch: out = [items] ternary polynomials, then [items][2]
+// error polynomials, poly_stride words apart; item k draws from the streams stream_id + 3 k, + 1, + 2
+hipError_t launch_sample_encrypt(const Tables &t, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
+                                 uint32_t items, size_t poly_stride, hipStream_t s);
 // wide [items][2][L+K][N] += u [items][L+K][N] * pk [2][size_q+K][N] (both polynomials of the public key)
 hipError_t launch_encrypt_fma(const Tables &t, const uint64_t *u, const uint64_t *pk, uint64_t *wide, uint32_t L,
                               uint32_t K, uint32_t size_q, uint32_t items, hipStream_t s);

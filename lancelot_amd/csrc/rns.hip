@@ -737,7 +737,7 @@ struct SampleArgs {
     LimbMap map;
     uint32_t log_n, cdt_len;
     int kind;
-    uint32_t stream_stride, stream_group;
+    uint32_t stream_stride;
     size_t out_item_stride;
 };
 
@@ -747,12 +747,14 @@ struct SampleArgs {
 // a run-time count the array lived in scratch memory); a thread's 16 or 8 consecutive output words leave as 16-byte
 // stores.
 template <int KIND>
+__device__ __forceinline__ void sample_signed(const SampleArgs &p, uint32_t b, uint64_t stream, uint64_t *out);
+
+template <int KIND>
 __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
     const uint32_t n = 1u << p.log_n;
     const uint32_t b = blockIdx.x * kThreads + threadIdx.x;
-    // blockIdx.y = polynomial: stream_group consecutive ones take consecutive stream ids, the next group starts
-    // stream_stride on
-    const uint64_t stream = p.stream + (uint64_t)(blockIdx.y / p.stream_group) * p.stream_stride + blockIdx.y % p.stream_group;
+    // blockIdx.y = item: its own stream id, its own polynomial
+    const uint64_t stream = p.stream + (uint64_t)blockIdx.y * p.stream_stride;
     uint64_t *out = p.out + blockIdx.y * p.out_item_stride;
     uint32_t w[16];
     if (KIND == SAMPLE_UNIFORM) {
@@ -774,6 +776,14 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
         dst[1] = ulonglong2{r[2], r[3]};
         return;
     }
+    sample_signed<KIND>(p, b, stream, out);
+}
+
+// ternary / error / gauss coefficients of ChaCha block b of `stream`, the same signed value to every limb of `out`
+template <int KIND>
+__device__ __forceinline__ void sample_signed(const SampleArgs &p, uint32_t b, uint64_t stream, uint64_t *out) {
+    const uint32_t n = 1u << p.log_n;
+    uint32_t w[16];
     constexpr int per_block = KIND == SAMPLE_TERNARY ? 16 : 8;
     if (b >= n / per_block) return;
     chacha20_block(p.key, b, stream, w);
@@ -800,6 +810,20 @@ __global__ __launch_bounds__(kThreads) void sample_kernel(SampleArgs p) {
         for (int e = 0; e < per_block; e += 2)
             dst[e / 2] = ulonglong2{v[e] < 0 ? q - (uint64_t)(-v[e]) : (uint64_t)v[e],
                                     v[e + 1] < 0 ? q - (uint64_t)(-v[e + 1]) : (uint64_t)v[e + 1]};
+    }
+}
+
+// The three polynomials of `items` public-key encryptions in one launch: out holds [items] ternary polynomials u and
+// behind them [items][2] error polynomials (e0, e1), all out_item_stride words apart; item k draws u, e0, e1 from the
+// streams p.stream + 3 k, + 1, + 2.  blockIdx.y = polynomial, blockIdx.z = 0.
+__global__ __launch_bounds__(kThreads) void sample_encrypt_kernel(SampleArgs p, uint32_t items) {
+    const uint32_t b = blockIdx.x * kThreads + threadIdx.x, y = blockIdx.y;
+    uint64_t *out = p.out + y * p.out_item_stride;
+    if (y < items) {
+        sample_signed<SAMPLE_TERNARY>(p, b, p.stream + 3 * (uint64_t)y, out);
+    } else {
+        const uint32_t e = y - items;
+        sample_signed<SAMPLE_ERROR>(p, b, p.stream + 3 * (uint64_t)(e >> 1) + 1 + (e & 1), out);
     }
 }
 
@@ -1104,13 +1128,13 @@ hipError_t launch_hoist_inner(const Tables &t, const Tuning &tune, const uint64_
 
 hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
                          const uint64_t *cdt, uint32_t cdt_len, uint32_t items, uint32_t stream_stride,
-                         size_t out_item_stride, hipStream_t s, uint32_t stream_group) {
-    if (items == 0 || items > 65535 || stream_group == 0) return hipErrorInvalidValue;
+                         size_t out_item_stride, hipStream_t s) {
+    if (items == 0 || items > 65535) return hipErrorInvalidValue;
     const uint32_t n = 1u << t.log_n;
     uint32_t blocks = kind == SAMPLE_UNIFORM ? (n / 4) * map.limbs : (kind == SAMPLE_TERNARY ? n / 16 : n / 8);
     // (a thread's words leave as 16-byte stores)
     if ((reinterpret_cast<uintptr_t>(out) & 15) || (out_item_stride & 1)) return hipErrorInvalidValue;
-    SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind, stream_stride, stream_group, out_item_stride};
+    SampleArgs p{out, t.moduli, t.barrett, cdt, key, stream_id, map, t.log_n, cdt_len, kind, stream_stride, out_item_stride};
     const dim3 grid((blocks + kThreads - 1) / kThreads, items);
     switch (kind) {
         case SAMPLE_UNIFORM: hipLaunchKernelGGL(sample_kernel<SAMPLE_UNIFORM>, grid, dim3(kThreads), 0, s, p); break;
@@ -1119,6 +1143,19 @@ hipError_t launch_sample(const Tables &t, int kind, ChaChaKey key, uint64_t stre
         case SAMPLE_GAUSS: hipLaunchKernelGGL(sample_kernel<SAMPLE_GAUSS>, grid, dim3(kThreads), 0, s, p); break;
         default: return hipErrorInvalidValue;
     }
+    return hipGetLastError();
+}
+
+hipError_t launch_sample_encrypt(const Tables &t, ChaChaKey key, uint64_t stream_id, uint64_t *out, LimbMap map,
+                                 uint32_t items, size_t poly_stride, hipStream_t s) {
+    if (items == 0 || 3 * (uint64_t)items > 65535) return hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(out) & 15) || (poly_stride & 1)) return hipErrorInvalidValue;
+    const uint32_t n = 1u << t.log_n;
+    SampleArgs p{out, t.moduli, t.barrett, nullptr, key, stream_id, map, t.log_n, 0, SAMPLE_ERROR, 0, poly_stride};
+    // (a ChaCha block yields 16 ternary or 8 error coefficients: the grid covers the error polynomials, the surplus
+    // threads of the ternary ones leave at once)
+    const dim3 grid((n / 8 + kThreads - 1) / kThreads, 3 * items);
+    hipLaunchKernelGGL(sample_encrypt_kernel, grid, dim3(kThreads), 0, s, p, items);
     return hipGetLastError();
 }
 
