@@ -49,6 +49,12 @@ int he_device_count(int *count);
 int he_malloc(void **dev_ptr, size_t bytes);
 int he_free(void *dev_ptr);
 int he_memcpy_h2d(void *dst_dev, const void *src_host, size_t bytes, he_stream stream);
+/* Page-locked host memory and an upload from it that does not wait: the copy is ordered on `stream` like a kernel, and
+ * the caller keeps the source unchanged until the stream has passed it (cudaMallocHost / cudaMemcpyAsync in the
+ * reference's terms; src/ckks.cu:143-152 uploads the values of every encoding with a blocking copy). */
+int he_host_malloc(void **host_ptr, size_t bytes);
+int he_host_free(void *host_ptr);
+int he_memcpy_h2d_async(void *dst_dev, const void *src_pinned, size_t bytes, he_stream stream);
 int he_memcpy_d2h(void *dst_host, const void *src_dev, size_t bytes, he_stream stream);
 int he_memcpy_d2d(void *dst_dev, const void *src_dev, size_t bytes, he_stream stream);
 /* `rows` runs of `width` bytes, the runs src_pitch bytes apart in the source and dst_pitch bytes apart in the

@@ -22,6 +22,9 @@ SIGNATURES = {
     "he_malloc": (C.c_int, [C.POINTER(vp), C.c_size_t]),
     "he_free": (C.c_int, [vp]),
     "he_memcpy_h2d": (C.c_int, [vp, vp, C.c_size_t, vp]),
+    "he_host_malloc": (C.c_int, [C.POINTER(vp), C.c_size_t]),
+    "he_host_free": (C.c_int, [vp]),
+    "he_memcpy_h2d_async": (C.c_int, [vp, vp, C.c_size_t, vp]),
     "he_memcpy_d2h": (C.c_int, [vp, vp, C.c_size_t, vp]),
     "he_memcpy_d2d": (C.c_int, [vp, vp, C.c_size_t, vp]),
     "he_memcpy2d_d2d": (C.c_int, [vp, C.c_size_t, vp, C.c_size_t, C.c_size_t, C.c_size_t, vp]),

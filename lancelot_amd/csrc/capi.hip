@@ -314,6 +314,25 @@ int he_memcpy_h2d(void *dst, const void *src, size_t bytes, he_stream s) {
     return HE_OK;
 }
 
+int he_host_malloc(void **host_ptr, size_t bytes) {
+    if (!host_ptr || bytes == 0) return HE_E_INVALID_ARGUMENT;
+    *host_ptr = nullptr;
+    HE_HIP(hipHostMalloc(host_ptr, bytes, hipHostMallocDefault));
+    return HE_OK;
+}
+
+int he_host_free(void *host_ptr) {
+    if (host_ptr) HE_HIP(hipHostFree(host_ptr));
+    return HE_OK;
+}
+
+int he_memcpy_h2d_async(void *dst, const void *src, size_t bytes, he_stream s) {
+    if (bytes == 0) return HE_OK;
+    if (!dst || !src) return HE_E_INVALID_ARGUMENT;
+    HE_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, S(s)));
+    return HE_OK;
+}
+
 int he_memcpy_d2h(void *dst, const void *src, size_t bytes, he_stream s) {
     if (bytes == 0) return HE_OK;
     HE_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, S(s)));

@@ -7,10 +7,39 @@
 // out and keeps the reference's argument checks.  Decoded values agree with the reference up to FP64 operation
 // order (bounded by the 2^-20 acceptance tolerance), not bit for bit.
 #include <cmath>
+#include <cstring>
 
 #include "cahel.h"
 
 using namespace cahel;
+
+namespace {
+
+// Page-locked staging for the values of an encoding, one buffer per host thread (the lanes of the host layer encode
+// from several threads), grown on demand and kept until the process ends.  The values are copied into it and uploaded
+// without waiting; every encoding ends with a blocking download (its largest coefficient), after which the buffer is
+// free for the thread's next call.
+struct PinnedStage {
+    void *ptr = nullptr;
+    std::size_t bytes = 0;
+    double *ensure(std::size_t want) {
+        if (want > bytes) {
+            if (ptr) check_status(he_host_free(ptr), "he_host_free");
+            ptr = nullptr;
+            bytes = 0;
+            check_status(he_host_malloc(&ptr, want), "he_host_malloc");
+            bytes = want;
+        }
+        return static_cast<double *>(ptr);
+    }
+};
+
+double *pinned_stage(std::size_t bytes) {
+    thread_local PinnedStage stage;
+    return stage.ensure(bytes);
+}
+
+}  // namespace
 
 CAHELGPUCKKSEncoder::CAHELGPUCKKSEncoder(const CAHELGPUContext &context) {
     if (context.scheme() != scheme_type::ckks) throw std::invalid_argument("unsupported scheme");
@@ -113,8 +142,14 @@ void CAHELGPUCKKSEncoder::encode_complex(const CAHELGPUContext &context, const d
     double *d_re = reinterpret_cast<double *>(staging.get());
     double *d_im = im ? d_re + ss : nullptr;
     if (count) {
-        check_status(he_memcpy_h2d(d_re, re, count * sizeof(double), context.stream()), "upload");
-        if (im) check_status(he_memcpy_h2d(d_im, im, count * sizeof(double), context.stream()), "upload");
+        // (through page-locked memory, without waiting: the download of the largest coefficient below is the wait)
+        double *host = pinned_stage((im ? 2 : 1) * count * sizeof(double));
+        std::memcpy(host, re, count * sizeof(double));
+        check_status(he_memcpy_h2d_async(d_re, host, count * sizeof(double), context.stream()), "upload");
+        if (im) {
+            std::memcpy(host + count, im, count * sizeof(double));
+            check_status(he_memcpy_h2d_async(d_im, host + count, count * sizeof(double), context.stream()), "upload");
+        }
     }
     check_status(he_ckks_encode(h, d_re, d_im, (uint32_t)count, (uint32_t)ss, scale, limbs, destination.data(),
                                 ws.get(), context.stream()),
