@@ -37,6 +37,8 @@ struct Level {
     uint32_t n_modup_jobs = 0;
     LimbGroup *d_modup_groups = nullptr; // runs of those jobs that share a modulus table
     uint32_t n_modup_groups = 0;
+    LimbGroup *d_modup_singles = nullptr; // every job a group of its own (n_modup_jobs of them): for launches so small
+                                          // that a workgroup which takes a run of limbs in turn is what they wait for
     // batched base conversion (all digits of ModUp / all polynomials of ModDown in one launch)
     BconvDesc *d_modup_descs = nullptr, *d_moddown_descs = nullptr;
     uint32_t *d_modup_limb = nullptr, *d_modup_table = nullptr;
@@ -720,6 +722,9 @@ int he_context_set_level(he_context *ctx, const he_level_desc *d) {
         lv.n_modup_groups = (uint32_t)groups.size();
         rc = upload(ctx, &lv.d_modup_jobs, jobs.data(), jobs.size());
         if (!rc) rc = upload(ctx, &lv.d_modup_groups, groups.data(), groups.size());
+        std::vector<LimbGroup> singles;
+        for (uint32_t j = 0; j < jobs.size(); j++) singles.push_back(LimbGroup{j, 1});
+        if (!rc) rc = upload(ctx, &lv.d_modup_singles, singles.data(), singles.size());
         if (rc) return rc;
     }
     lv.set = true;
@@ -950,8 +955,10 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     fwd.out = out;
     fwd.jobs = lv->d_modup_jobs;
     fwd.n_jobs = lv->n_modup_jobs;
-    fwd.groups = lv->d_modup_groups;
-    fwd.n_groups = lv->n_modup_groups;
+    // (a launch of at most 1024 workgroups of the smallest tile: one limb per workgroup)
+    const bool singles = (uint64_t)lv->n_modup_jobs * items * (n >> 10) <= 1024;
+    fwd.groups = singles ? lv->d_modup_singles : lv->d_modup_groups;
+    fwd.n_groups = singles ? lv->n_modup_jobs : lv->n_modup_groups;
     fwd.items = items;
     fwd.item_stride = (size_t)lv->beta * LK * n;
     if (reduce_in_ntt) {
