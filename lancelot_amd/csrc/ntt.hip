@@ -1756,7 +1756,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(1))) v
 // Integer back end (twiddles stay in the table: 30 Shoup pairs per thread do not fit in registers).  Three waves
 // per SIMD (168 registers, 24 bytes of spill in the forward kernel) hide the latency of the epilogue's operand loads
 // better than the two waves that 196 registers allow.
-template <bool FWD, bool GAL>
+// PRE: the operands of a fused epilogue are requested together with the tile, so that they travel while the
+// butterflies run (32 more registers: for the mixed kernel, which is compiled for two waves per SIMD and serves the
+// small launches, where nothing else covers that round trip).
+template <bool FWD, bool GAL, bool PRE = false>
 __device__ __forceinline__ void ntt_blocks_int_body(const NttArgs &a, uint64_t *lds) {
     const uint32_t nthreads = blockDim.x;
     const uint32_t tile_elems = nthreads << 4;
@@ -1781,17 +1784,24 @@ __device__ __forceinline__ void ntt_blocks_int_body(const NttArgs &a, uint64_t *
 #pragma unroll
             for (int i = 0; i < kPer; i++) lds[skew(threadIdx.x + i * nthreads)] = src[threadIdx.x + i * nthreads];
         }
-        __syncthreads();
         const size_t epi_off = off + (size_t)job.limb * n;
+        const uint64_t *minuend = epi ? a.epi_a + (size_t)job.poly * a.epi_a_poly_stride * n + epi_off : nullptr;
+        const bool add_b = has_addend && (fma_mode || ((a.epi_b_mask >> (job.poly & 31)) & 1));
+        const uint64_t *addend = add_b ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
+        uint64_t pre_a[PRE ? kPer : 1], pre_b[PRE ? kPer : 1];
+        if (PRE && epi) {
+#pragma unroll
+            for (int i = 0; i < kPer; i++) pre_a[PRE ? i : 0] = minuend[threadIdx.x + i * nthreads];
+#pragma unroll
+            for (int i = 0; i < kPer; i++) pre_b[PRE ? i : 0] = addend[threadIdx.x + i * nthreads];
+        }
+        __syncthreads();
         if (FWD) {
             tile_pass<4, true>(lds, tile_elems, 4, g.idx0, ic);
             __syncthreads();
             tile_pass<4, true>(lds, tile_elems, 0, g.idx1, ic);
             __syncthreads();
             if (epi) {
-                const uint64_t *minuend = a.epi_a + (size_t)job.poly * a.epi_a_poly_stride * n + epi_off;
-                const bool add_b = has_addend && (fma_mode || ((a.epi_b_mask >> (job.poly & 31)) & 1));
-                const uint64_t *addend = add_b ? a.epi_b + (size_t)job.poly * a.epi_b_poly_stride * n + epi_off : minuend;
                 uint64_t *dst = a.epi_dst + (size_t)job.poly * a.epi_dst_poly_stride * n + epi_off;
                 const Shoup w = load_shoup(a.w, job.limb);
                 const Shoup pw = fma_mode ? load_shoup(a.pro_w, job.limb) : w;
@@ -1799,12 +1809,14 @@ __device__ __forceinline__ void ntt_blocks_int_body(const NttArgs &a, uint64_t *
                 for (int i = 0; i < kPer; i++) {
                     const uint32_t e = threadIdx.x + i * nthreads;
                     const uint64_t c = reduce_4q(lds[skew(e)], q);
+                    const uint64_t ma = PRE ? pre_a[PRE ? i : 0] : minuend[e];
                     uint64_t r;
                     if (fma_mode) {
-                        r = mul_shoup(sub_mod(add_mod(mul_shoup(minuend[e], pw, q), addend[e], q), c, q), w, q);
+                        const uint64_t mb = PRE ? pre_b[PRE ? i : 0] : addend[e];
+                        r = mul_shoup(sub_mod(add_mod(mul_shoup(ma, pw, q), mb, q), c, q), w, q);
                     } else {
-                        r = mul_shoup(sub_mod(minuend[e], c, q), w, q);
-                        if (add_b) r = add_mod(r, addend[e], q);
+                        r = mul_shoup(sub_mod(ma, c, q), w, q);
+                        if (add_b) r = add_mod(r, PRE ? pre_b[PRE ? i : 0] : addend[e], q);
                     }
                     dst[e] = r;
                 }
@@ -1847,7 +1859,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     if ((a.fp_mask >> first.table) & 1)
         ntt_blocks_fp_body<FWD, EPI, GAL>(a, lds);
     else
-        ntt_blocks_int_body<FWD, GAL>(a, lds);
+        ntt_blocks_int_body<FWD, GAL, FWD && EPI>(a, lds);
 }
 
 template <bool FWD, int FP>
