@@ -560,19 +560,23 @@ def test_largest_degree_scheme_flow(oracle):
     assert np.median(err) < 1e-4 and np.max(err) < 2e-2      # 2^30 of scale left; the floor-rescale bias in the first slots
 
 
-@pytest.mark.parametrize("logn,bits", [(16, [60, 40, 40, 60]), (15, [60, 40, 40, 60]), (16, [50, 45, 50, 49, 50])])
-@pytest.mark.parametrize("variant", ["default", "two_rows_passes", "integer", "integer_two_rows_passes"])
+@pytest.mark.parametrize("logn,bits", [(16, [60, 40, 40, 60]), (15, [60, 40, 40, 60]), (16, [50, 45, 50, 49, 50]),
+                                       (15, [45, 40, 60])])
+@pytest.mark.parametrize("variant", ["default", "two_rows_passes", "integer", "integer_two_rows_passes", "no_mixed"])
 def test_single_limb_digits_small_launches(oracle, monkeypatch, logn, bits, variant):
     """One special prime (K = 1, Lancelot's chain): ModUp and ModDown reduce a single source limb into every other
     prime, and a launch of a few limbs runs the source's inverse rows pass inside the forward rows pass
     (CAHEL_HIP_NO_SOURCE_INTT=1 keeps the two passes apart).  he_modup, he_moddown (overwriting and adding), he_keyswitch
     with and without a Galois element and he_rotate against the oracle, limb for limb, on the mixed, FP64 and integer
-    back ends, at every level of the chain (src/rns.cu:610-782 ModUp / ModDown, src/evaluate.cu:1622-1760 key switch)."""
+    back ends (and with CAHEL_HIP_NO_MIXED=1, where the chain [45, 40, 60] transforms its sources in FP64 and their
+    targets on the integer back end), at every level of the chain (src/rns.cu:610-782 ModUp / ModDown,
+    src/evaluate.cu:1622-1760 key switch)."""
     import ctypes as C
     from gpu_util import DeviceArray, make_pair, rand_limbs
     from lancelot_amd import capi
     monkeypatch.setenv("CAHEL_HIP_NO_SOURCE_INTT", "1" if variant.endswith("two_rows_passes") else "0")
     monkeypatch.setenv("CAHEL_HIP_NO_FP64", "1" if variant.startswith("integer") else "0")
+    monkeypatch.setenv("CAHEL_HIP_NO_MIXED", "1" if variant == "no_mixed" else "0")
     cahel, parms, ctx, p = make_pair(oracle, logn, bits, 1)
     lib, h = capi.lib(), ctx.he_handle()
     rng = np.random.default_rng(logn + len(bits))
