@@ -16,12 +16,18 @@ using namespace cahel;
 namespace {
 
 // Page-locked staging for the values of an encoding, one buffer per host thread (the lanes of the host layer encode
-// from several threads), grown on demand and kept until the process ends.  The values are copied into it and uploaded
+// from several threads), grown on demand and kept until the thread ends.  The values are copied into it and uploaded
 // without waiting; every encoding ends with a blocking download (its largest coefficient), after which the buffer is
 // free for the thread's next call.
 struct PinnedStage {
     void *ptr = nullptr;
     std::size_t bytes = 0;
+    PinnedStage() = default;
+    PinnedStage(const PinnedStage &) = delete;
+    PinnedStage &operator=(const PinnedStage &) = delete;
+    ~PinnedStage() {
+        if (ptr) (void)he_host_free(ptr);   // (worker threads of a pool come and go: no buffer is left behind)
+    }
     double *ensure(std::size_t want) {
         if (want > bytes) {
             if (ptr) check_status(he_host_free(ptr), "he_host_free");
