@@ -496,7 +496,6 @@ int he_context_create(const he_context_desc *d, he_context **out) {
         ctx->fuse_tensor = !(nt && nt[0] == '1');
         const char *nr = getenv("CAHEL_HIP_NO_REDUCE_IN_NTT");
         ctx->single_limb_digits = ctx->size_p == 1 && !(nr && nr[0] == '1');
-
         const char *nbf = getenv("CAHEL_HIP_NO_BATCH_FUSED_KS");
         ctx->batch_fused_inner = !(nbf && nbf[0] == '1');
         auto env_on = [](const char *name) { const char *e = getenv(name); return e && e[0] == '1'; };
@@ -911,6 +910,8 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     inv.map = plain_map(L, 0);
     inv.epi_mode = NTT_EPI_MUL;
     inv.w = lv->d_part_hat_inv;
+    // skip_own (batched levels only): the consumer reads a digit's own limbs from c, their slots in out stay unwritten
+    if (skip_own && !lv->batched) return HE_E_INVALID_ARGUMENT;
     if (in_galois && (items != 1 || !skip_own)) return HE_E_INVALID_ARGUMENT;   // (own limbs are copied from c as it is)
     inv.in_galois = in_galois;
     const bool fused = fuse_rows_ok(ctx, lv, L);
@@ -922,8 +923,6 @@ int modup_impl(const he_context *ctx, uint32_t L, const uint64_t *c, uint32_t c_
     const int inv_backend = backend_for(ctx, inv.map);
     const bool source_intt = reduce_in_ntt && source_intt_ok(ctx, lv->n_modup_jobs * items);
     HE_HIP(launch_ntt_inverse(inv, items, inv_backend, S(s), false, source_intt));
-    // skip_own (batched levels only): the consumer reads a digit's own limbs from c, their slots in out stay unwritten
-    if (skip_own && !lv->batched) return HE_E_INVALID_ARGUMENT;
     const uint32_t copy_rows = skip_own ? 0 : lv->modup_max_copy;
     if (reduce_in_ntt) {
         for (uint32_t d = 0; d < lv->beta && !skip_own; d++)

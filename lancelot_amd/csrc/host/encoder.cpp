@@ -30,9 +30,10 @@ struct PinnedStage {
     }
     double *ensure(std::size_t want) {
         if (want > bytes) {
-            if (ptr) check_status(he_host_free(ptr), "he_host_free");
+            void *old = ptr;
             ptr = nullptr;
             bytes = 0;
+            if (old) check_status(he_host_free(old), "he_host_free");
             check_status(he_host_malloc(&ptr, want), "he_host_malloc");
             bytes = want;
         }
